@@ -1,0 +1,323 @@
+// Decode attention behind the reference's two entry points: score rows (q . K^T per head, through
+// map_matmul_t_dev) and softmax(prep(scores)) . V (map_attn_softmax_value_dev).
+//
+// Reference: shaders/src/f32/map_matmul_t.comp, map_attn_softmax_value.comp:39-89 (dispatch
+// adamah.c:6682-6781, 7894-8059), prep(s) = cap*tanh(s*scale/cap) when cap > 0 else s*scale.
+// The reference keeps all probabilities of a row in 2048 floats of shared memory and returns
+// without output for longer rows; here the row is split over workgroups with an online-softmax
+// merge (running max m, sum l, weighted values o), so any length works.  K/V rows are read from
+// the fp16 copy of the KV range when the operands lie inside it, else from the float32 map.
+#include "common.h"
+#include "../../include/adamah_hip.h"
+#include <algorithm>
+
+namespace adamah {
+
+__device__ __forceinline__ float ld(const float* p, uint64_t i) { return p[i]; }
+__device__ __forceinline__ float ld(const __half* p, uint64_t i) { return __half2float(p[i]); }
+
+__device__ __forceinline__ float wave_sum64(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max64(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// C[M,N] = A[M,K] . B[N,K]^T per op; one wave per output column, lanes over K.
+// B is read through `bsrc` (float map or fp16 KV copy, index = element - b_shift).
+template <typename TB>
+__global__ void __launch_bounds__(256)
+k_matmul_t(const float* A, float* C, const TB* bsrc, uint64_t b_shift, const uint32_t* __restrict__ la,
+           const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc, uint32_t M, uint32_t K, uint32_t N,
+           uint64_t a_elems, uint64_t b_elems) {
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const uint32_t col = blockIdx.x * 4u + wave, row = blockIdx.y, op = blockIdx.z;
+  if (col >= N) return;
+  const uint64_t a = (uint64_t)la[op] + (uint64_t)row * K, b = (uint64_t)lb[op] + (uint64_t)col * K;
+  const uint64_t c = (uint64_t)lc[op] + (uint64_t)row * N + col;
+  float s = 0.f;
+  if (a + K <= a_elems && b >= b_shift && b - b_shift + K <= b_elems)
+    for (uint32_t k = lane; k < K; k += 64u) s = fmaf(A[a + k], ld(bsrc, b - b_shift + k), s);
+  s = wave_sum64(s);
+  if (lane == 0 && c < a_elems) C[c] = s;
+}
+
+// C = A[M,K] . B[K,N] (non-transposed B), same indexing conventions.
+__global__ void __launch_bounds__(256)
+k_matmul_nt(const float* A, float* C, const float* B, const uint32_t* __restrict__ la, const uint32_t* __restrict__ lb,
+            const uint32_t* __restrict__ lc, uint32_t M, uint32_t K, uint32_t N, uint64_t a_elems, uint64_t b_elems) {
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const uint32_t col = blockIdx.x * 4u + wave, row = blockIdx.y, op = blockIdx.z;
+  if (col >= N) return;
+  const uint64_t a = (uint64_t)la[op] + (uint64_t)row * K, b = lb[op];
+  const uint64_t c = (uint64_t)lc[op] + (uint64_t)row * N + col;
+  float s = 0.f;
+  for (uint32_t k = lane; k < K; k += 64u) {
+    const uint64_t bi = b + (uint64_t)k * N + col;
+    if (a + k < a_elems && bi < b_elems) s = fmaf(A[a + k], B[bi], s);
+  }
+  s = wave_sum64(s);
+  if (lane == 0 && c < a_elems) C[c] = s;
+}
+
+__device__ __forceinline__ float prep(float v, float scale, float cap) {
+  v *= scale;
+  if (cap > 0.0f) v = tanhf(v / cap) * cap;
+  return v;
+}
+
+#define ATT_CHUNK 1024   // score rows handled by one workgroup
+
+// grid (n_splits, n_ops).  Workgroup (split s, op): rows [s*ATT_CHUNK, ...) of the op's score row.
+// Writes either the normalised output (n_splits == 1) or the partial (m, l, o[value_dim]).
+template <typename TV>
+__global__ void __launch_bounds__(256)
+k_attn_softmax_value(const float* data, float* out, const TV* vsrc, uint64_t v_shift, const uint32_t* __restrict__ lsc,
+                     const uint32_t* __restrict__ lv, const uint32_t* __restrict__ lo, uint32_t row_size,
+                     uint32_t value_dim, float scale, float cap, uint32_t n_splits, float* partial, uint64_t n_elems,
+                     uint64_t v_elems) {
+  __shared__ float p[ATT_CHUNK];
+  __shared__ float red[4];
+  __shared__ float osum[256];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t split = blockIdx.x, op = blockIdx.y;
+  const uint32_t t0 = split * ATT_CHUNK, t1 = min(row_size, t0 + ATT_CHUNK), nt = t1 - t0;
+  const uint64_t sb = lsc[op], vb = lv[op], ob = lo[op];
+  const bool ok = sb + row_size <= n_elems && vb >= v_shift &&
+                  vb - v_shift + (uint64_t)row_size * value_dim <= v_elems && ob + value_dim <= n_elems;
+  // pass 1: chunk maximum of prep(score)
+  float mx = -9.99999968e+37f;
+  if (ok)
+    for (uint32_t t = tid; t < nt; t += 256u) {
+      const float v = prep(data[sb + t0 + t], scale, cap);
+      p[t] = v;
+      mx = fmaxf(mx, v);
+    }
+  mx = wave_max64(mx);
+  if (lane == 0) red[wave] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  // pass 2: exponentials and their sum
+  float sum = 0.f;
+  if (ok)
+    for (uint32_t t = tid; t < nt; t += 256u) {
+      const float e = expf(p[t] - mx);
+      p[t] = e;
+      sum += e;
+    }
+  sum = wave_sum64(sum);
+  if (lane == 0) red[wave] = sum;
+  __syncthreads();
+  sum = (red[0] + red[1]) + (red[2] + red[3]);
+  // pass 3: o[d] = sum_t p[t] * V[t][d]; thread (slot, d): slot strides the rows
+  const uint32_t dpw = min(value_dim, 256u);       // columns handled per sweep
+  const uint32_t slots = 256u / dpw;               // rows in flight per sweep
+  for (uint32_t d0 = 0; d0 < value_dim; d0 += 256u) {
+    const uint32_t d = d0 + tid % dpw, slot = tid / dpw;
+    float acc = 0.f;
+    if (ok && d < value_dim && slot < slots) {
+      const uint64_t base = vb - v_shift + (uint64_t)t0 * value_dim + d;
+      for (uint32_t t = slot; t < nt; t += slots) acc = fmaf(p[t], ld(vsrc, base + (uint64_t)t * value_dim), acc);
+    }
+    osum[tid] = acc;
+    __syncthreads();
+    if (tid < dpw && d0 + tid < value_dim && ok) {
+      float o = 0.f;
+      for (uint32_t s = 0; s < slots; s++) {
+        o += osum[s * dpw + tid];
+      }
+      if (n_splits == 1) out[ob + d0 + tid] = o * (1.0f / sum);
+      else partial[((uint64_t)op * n_splits + split) * (value_dim + 2) + 2 + d0 + tid] = o;
+    }
+    __syncthreads();
+  }
+  if (n_splits > 1 && tid == 0) {
+    float* pp = partial + ((uint64_t)op * n_splits + split) * (value_dim + 2);
+    pp[0] = mx;
+    pp[1] = sum;
+  }
+}
+
+// Merge the split partials of one op: M = max m_s, L = sum l_s e^(m_s-M), o = sum o_s e^(m_s-M) / L.
+__global__ void __launch_bounds__(256)
+k_attn_combine(float* out, const float* partial, const uint32_t* __restrict__ lo, uint32_t value_dim,
+               uint32_t n_splits, uint64_t n_elems) {
+  const uint32_t op = blockIdx.x, tid = threadIdx.x;
+  const float* pp = partial + (uint64_t)op * n_splits * (value_dim + 2);
+  const uint64_t ob = lo[op];
+  if (ob + value_dim > n_elems) return;
+  float M = -9.99999968e+37f;
+  for (uint32_t s = 0; s < n_splits; s++) M = fmaxf(M, pp[(uint64_t)s * (value_dim + 2)]);
+  float L = 0.f;
+  for (uint32_t s = 0; s < n_splits; s++) {
+    const float* q = pp + (uint64_t)s * (value_dim + 2);
+    L += q[1] * expf(q[0] - M);
+  }
+  const float invL = 1.0f / L;
+  for (uint32_t d = tid; d < value_dim; d += 256u) {
+    float o = 0.f;
+    for (uint32_t s = 0; s < n_splits; s++) {
+      const float* q = pp + (uint64_t)s * (value_dim + 2);
+      o = fmaf(q[2 + d], expf(q[0] - M), o);
+    }
+    out[ob + d] = o * invL;
+  }
+}
+
+// Row softmax family (map_softmax.comp, map_softmax_abs.comp, map_attn_softmax_abs.comp):
+// one workgroup per row, source/destination bases from locs (multiplied by row_size when REL).
+template <bool REL>
+__global__ void __launch_bounds__(256)
+k_softmax_rows(float* data, const uint32_t* __restrict__ ls, const uint32_t* __restrict__ ldst, uint32_t row_size,
+               float scale, float cap, uint64_t n_elems) {
+  __shared__ float red[4];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, ri = blockIdx.x;
+  const uint64_t sb = REL ? (uint64_t)ls[ri] * row_size : ls[ri], db = REL ? (uint64_t)ldst[ri] * row_size : ldst[ri];
+  if (sb + row_size > n_elems || db + row_size > n_elems) return;
+  float mx = -9.99999968e+37f;
+  for (uint32_t i = tid; i < row_size; i += 256u) mx = fmaxf(mx, prep(data[sb + i], scale, cap));
+  mx = wave_max64(mx);
+  if (lane == 0) red[wave] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  float sum = 0.f;
+  for (uint32_t i = tid; i < row_size; i += 256u) sum += expf(prep(data[sb + i], scale, cap) - mx);
+  sum = wave_sum64(sum);
+  if (lane == 0) red[wave] = sum;
+  __syncthreads();
+  sum = (red[0] + red[1]) + (red[2] + red[3]);
+  const float inv = 1.0f / sum;
+  // src may equal dst: every thread rereads only the elements it then overwrites
+  for (uint32_t i = tid; i < row_size; i += 256u) data[db + i] = expf(prep(data[sb + i], scale, cap) - mx) * inv;
+}
+
+// All ops of a handle inside the fp16 KV range?  Needs the host copy of the locs.
+static bool all_in_kv(const Map* m, uint32_t h, uint32_t n_ops, uint64_t span) {
+  if (!m->kv16) return false;
+  const uint32_t* v = res_host(h, n_ops);
+  if (!v) return false;
+  for (uint32_t i = 0; i < n_ops; i++)
+    if (v[i] < m->kv_start || v[i] - m->kv_start + span > m->kv_count) return false;
+  return true;
+}
+
+}  // namespace adamah
+
+using namespace adamah;
+
+extern "C" {
+
+int map_matmul_t_dev(uint32_t map_id, uint32_t ha, uint32_t hb, uint32_t hc, uint32_t M, uint32_t K, uint32_t N,
+                     uint32_t n_ops) {
+  Map* m = get_f32_map(map_id);
+  if (!m) return ADAMAH_ERR_INVALID;
+  if (n_ops == 0 || M == 0 || N == 0) return ADAMAH_OK;
+  const uint32_t *la = res_u32(ha, n_ops), *lb = res_u32(hb, n_ops), *lc = res_u32(hc, n_ops);
+  if (!la || !lb || !lc) return ADAMAH_ERR_INVALID;
+  dim3 grid(cdiv(N, 4), M, n_ops);
+  float* d = (float*)m->buf;
+  if (all_in_kv(m, hb, n_ops, (uint64_t)N * K))
+    k_matmul_t<__half><<<grid, 256, 0, g.stream>>>(d, d, m->kv16, m->kv_start, la, lb, lc, M, K, N, m->n_elems,
+                                                   m->kv_count);
+  else
+    k_matmul_t<float><<<grid, 256, 0, g.stream>>>(d, d, d, 0, la, lb, lc, M, K, N, m->n_elems, m->n_elems);
+  count_launch();
+  return check_launch();
+}
+
+int map_matmul_t_x_dev(uint32_t map_act, uint32_t map_wt, uint32_t ha, uint32_t hb, uint32_t hc, uint32_t M, uint32_t K,
+                       uint32_t N, uint32_t n_ops) {
+  Map* ma = get_f32_map(map_act);
+  Map* mw = get_f32_map(map_wt);
+  if (!ma || !mw) return ADAMAH_ERR_INVALID;
+  if (n_ops == 0 || M == 0 || N == 0) return ADAMAH_OK;
+  const uint32_t *la = res_u32(ha, n_ops), *lb = res_u32(hb, n_ops), *lc = res_u32(hc, n_ops);
+  if (!la || !lb || !lc) return ADAMAH_ERR_INVALID;
+  dim3 grid(cdiv(N, 4), M, n_ops);
+  k_matmul_t<float><<<grid, 256, 0, g.stream>>>((const float*)ma->buf, (float*)ma->buf, (const float*)mw->buf, 0, la, lb,
+                                                lc, M, K, N, ma->n_elems, mw->n_elems);
+  count_launch();
+  return check_launch();
+}
+
+static int matmul_nt(uint32_t map_act, uint32_t map_wt, uint32_t ha, uint32_t hb, uint32_t hc, uint32_t M, uint32_t K,
+                     uint32_t N, uint32_t n_ops) {
+  Map* ma = get_f32_map(map_act);
+  Map* mw = get_f32_map(map_wt);
+  if (!ma || !mw) return ADAMAH_ERR_INVALID;
+  if (n_ops == 0 || M == 0 || N == 0) return ADAMAH_OK;
+  const uint32_t *la = res_u32(ha, n_ops), *lb = res_u32(hb, n_ops), *lc = res_u32(hc, n_ops);
+  if (!la || !lb || !lc) return ADAMAH_ERR_INVALID;
+  dim3 grid(cdiv(N, 4), M, n_ops);
+  k_matmul_nt<<<grid, 256, 0, g.stream>>>((const float*)ma->buf, (float*)ma->buf, (const float*)mw->buf, la, lb, lc, M,
+                                          K, N, ma->n_elems, mw->n_elems);
+  count_launch();
+  return check_launch();
+}
+int map_matmul_x_dev(uint32_t map_act, uint32_t map_wt, uint32_t ha, uint32_t hb, uint32_t hc, uint32_t M, uint32_t K,
+                     uint32_t N, uint32_t n_ops) {
+  return matmul_nt(map_act, map_wt, ha, hb, hc, M, K, N, n_ops);
+}
+int map_matmul_dev(uint32_t map_id, uint32_t ha, uint32_t hb, uint32_t hc, uint32_t M, uint32_t K, uint32_t N,
+                   uint32_t n_ops) {
+  return matmul_nt(map_id, map_id, ha, hb, hc, M, K, N, n_ops);
+}
+
+int map_attn_softmax_value_dev(uint32_t map_id, uint32_t hs, uint32_t hv, uint32_t ho, uint32_t n_ops,
+                               uint32_t row_size, uint32_t value_dim, float scale, float cap) {
+  Map* m = get_f32_map(map_id);
+  if (!m) return ADAMAH_ERR_INVALID;
+  if (n_ops == 0 || row_size == 0 || value_dim == 0) return ADAMAH_OK;
+  const uint32_t *ls = res_u32(hs, n_ops), *lv = res_u32(hv, n_ops), *lo = res_u32(ho, n_ops);
+  if (!ls || !lv || !lo) return ADAMAH_ERR_INVALID;
+  const uint32_t n_splits = cdiv(row_size, ATT_CHUNK);
+  if ((uint64_t)n_ops * n_splits * (value_dim + 2) > g.attn_scratch_floats) return ADAMAH_ERR_INVALID;
+  float* d = (float*)m->buf;
+  dim3 grid(n_splits, n_ops);
+  if (all_in_kv(m, hv, n_ops, (uint64_t)row_size * value_dim))
+    k_attn_softmax_value<__half><<<grid, 256, 0, g.stream>>>(d, d, m->kv16, m->kv_start, ls, lv, lo, row_size, value_dim,
+                                                             scale, cap, n_splits, g.attn_scratch, m->n_elems,
+                                                             m->kv_count);
+  else
+    k_attn_softmax_value<float><<<grid, 256, 0, g.stream>>>(d, d, d, 0, ls, lv, lo, row_size, value_dim, scale, cap,
+                                                            n_splits, g.attn_scratch, m->n_elems, m->n_elems);
+  count_launch();
+  int r = check_launch();
+  if (r || n_splits == 1) return r;
+  k_attn_combine<<<n_ops, 256, 0, g.stream>>>(d, g.attn_scratch, lo, value_dim, n_splits, m->n_elems);
+  count_launch();
+  return check_launch();
+}
+
+static int softmax_rows(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_rows, uint32_t row_size, float scale,
+                        float cap, bool rel) {
+  Map* m = get_f32_map(map_id);
+  if (!m) return ADAMAH_ERR_INVALID;
+  if (n_rows == 0 || row_size == 0) return ADAMAH_OK;
+  const uint32_t *ls = res_u32(hs, n_rows), *ld = res_u32(hd, n_rows);
+  if (!ls || !ld) return ADAMAH_ERR_INVALID;
+  if (rel)
+    k_softmax_rows<true><<<n_rows, 256, 0, g.stream>>>((float*)m->buf, ls, ld, row_size, scale, cap, m->n_elems);
+  else
+    k_softmax_rows<false><<<n_rows, 256, 0, g.stream>>>((float*)m->buf, ls, ld, row_size, scale, cap, m->n_elems);
+  count_launch();
+  return check_launch();
+}
+int map_softmax_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_rows, uint32_t row_size) {
+  return softmax_rows(map_id, hs, hd, n_rows, row_size, 1.0f, 0.0f, true);
+}
+int map_softmax_abs_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_rows, uint32_t row_size) {
+  return softmax_rows(map_id, hs, hd, n_rows, row_size, 1.0f, 0.0f, false);
+}
+int map_attn_softmax_abs_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_rows, uint32_t row_size, float scale,
+                             float cap) {
+  return softmax_rows(map_id, hs, hd, n_rows, row_size, scale, cap, false);
+}
+
+}  // extern "C"

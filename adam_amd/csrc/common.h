@@ -1,0 +1,135 @@
+// Shared state of libadamah_hip: maps, loc handles, the stream, staging and launch helpers.
+//
+// The library re-implements the native side of the ADAMAH op surface (reference:
+// adamah-MAIN/adamah/adamah.c) for one MI355X.  Everything is ordered on one HIP stream,
+// which replaces the reference's command-buffer batching and per-dispatch barriers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stddef.h>
+#include <vector>
+
+// Error codes of the reference C ABI (adamah.c:24-28).
+#define ADAMAH_OK 0
+#define ADAMAH_ERR_BACKEND -1
+#define ADAMAH_ERR_MEMORY -2
+#define ADAMAH_ERR_INVALID -3
+#define ADAMAH_ERR_NOT_FOUND -4
+
+#define MAX_MAPS 16
+#define MAX_RES 65536          // reference: 2048; ids stay 32-bit so a larger table is invisible to callers
+#define MAX_PLANS 8
+#define MAX_PLAN_OPS 4096
+
+#define DTYPE_F32 0
+#define DTYPE_BF16 1
+#define DTYPE_Q8 2
+#define DTYPE_Q4 3
+#define DTYPE_Q6 4
+#define DTYPE_COUNT 5
+
+#define WAVE 64
+
+namespace adamah {
+
+// How a quantised map's per-group parameters are held on the device.
+enum QLayout : int {
+  QL_AFFINE = 0,   // float2 (scale, zp) per group -- any qparams
+  QL_BLOCK16 = 1,  // additionally an fp16 scale plane: every group has zp == -off*scale with an
+                   // fp16-exact scale (off = 8 for Q4, 128 for Q8), i.e. GGUF Q4_0 / Q8_0 blocks
+};
+
+struct Map {
+  bool active = false;
+  uint32_t dtype = 0, word_size = 0, pack_size = 0, n_packs = 0, group_size = 0;
+  uint64_t n_elems = 0, total_bytes = 0, n_groups = 0;
+  uint8_t* buf = nullptr;   // f32 values, or packed codes (Q4: 2 per byte, Q8: 1 per byte)
+  float2* qp = nullptr;     // (scale, zp) per group
+  __half* d16 = nullptr;    // fp16 scale per group, valid for groups [0, block16_groups)
+  uint64_t block16_groups = 0;
+  // fp16 KV region of an f32 map: elements [kv_start, kv_start+kv_count) are mirrored in kv16
+  uint64_t kv_start = 0, kv_count = 0;
+  __half* kv16 = nullptr;
+};
+
+struct Res {
+  bool active = false;
+  uint32_t size_bytes = 0, cap_bytes = 0;
+  uint8_t* dptr = nullptr;
+  std::vector<uint8_t> host;  // last uploaded contents; empty when the device wrote the resource
+  bool host_valid = false;
+};
+
+struct Stats {
+  uint64_t dispatch = 0, submit = 0, barrier = 0, fusion_flush = 0;
+  uint32_t last_batch_dispatch = 0;
+};
+
+struct PlanOp {  // mirrors DecodePlanOp (adamah.c:175-194)
+  uint32_t kind, map_id, map_id2, op_code, h0, h1, h2, h3, h4, h5, u0, u1, u2, u3, u4, u5;
+  float f0, f1;
+};
+
+struct Ctx {
+  bool initialized = false;
+  int device = 0;
+  hipStream_t stream = nullptr;
+  hipDeviceProp_t prop;
+  int n_cu = 256;
+  Map maps[MAX_MAPS];
+  std::vector<Res> res;      // index = handle id (0 unused)
+  uint32_t res_next = 1;
+  // device arena for handles
+  std::vector<uint8_t*> arena_chunks;
+  uint8_t* arena_cur = nullptr;
+  size_t arena_left = 0;
+  // pinned staging, double buffered
+  uint8_t* stage[2] = {nullptr, nullptr};
+  size_t stage_cap = 0, stage_off = 0;
+  int stage_cur = 0;
+  bool stage_used[2] = {false, false};
+  // attention split-KV partials
+  float* attn_scratch = nullptr;
+  size_t attn_scratch_floats = 0;
+  int batch_depth = 0;
+  int fusion_enabled = 0;
+  int scheduler_mode = 0;
+  uint32_t active_dtype = 0;
+  Stats stats;
+  hipEvent_t timer_ev[2] = {nullptr, nullptr};
+  std::vector<PlanOp> plans[MAX_PLANS];
+  bool plan_active[MAX_PLANS] = {false};
+};
+
+extern Ctx g;
+
+// ---- runtime helpers (runtime.hip) -------------------------------------------------------
+Map* get_map(uint32_t id);                       // nullptr unless active
+Map* get_f32_map(uint32_t id);                   // nullptr unless active and DTYPE_F32
+Res* get_res(uint32_t h);                        // nullptr unless active
+// Device pointer to a handle's words, or nullptr if the handle is missing or shorter than n words.
+const uint32_t* res_u32(uint32_t h, uint64_t n_words);
+// Host copy of a handle's words (nullptr when the device produced it or it is too short).
+const uint32_t* res_host(uint32_t h, uint64_t n_words);
+uint32_t res_alloc(uint32_t n_bytes);            // 0 on failure
+// Library-owned handle `slot` (0..7) holding a copy of host data; reused across calls.
+uint32_t scratch_handle(int slot, const void* data, uint32_t n_bytes);
+void* stage_alloc(size_t n);                     // pinned region; enqueue its copy before allocating much more
+int h2d(void* dst, const void* src, size_t n);   // stream-ordered, source consumed before return
+int d2h(void* dst, const void* src, size_t n);   // stream-ordered copy + wait
+inline void count_launch(int n = 1) { g.stats.dispatch += n; g.stats.barrier += n; g.stats.last_batch_dispatch += n; }
+int check_launch();                              // hipGetLastError -> ADAMAH code
+
+inline uint32_t cdiv(uint64_t a, uint64_t b) { return (uint32_t)((a + b - 1) / b); }
+
+// True when [lo, lo+n) lies inside a map of n_elems elements.
+inline bool in_range(uint64_t lo, uint64_t n, uint64_t n_elems) { return lo <= n_elems && n <= n_elems - lo; }
+
+// ---- internal op entry points shared between translation units -----------------------------
+int op_matmul_t_xq(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t ha, uint32_t hb, uint32_t hc,
+                   uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops, bool transposed);
+int op_matvec_argmax(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t ha, uint32_t hb, uint32_t hidx,
+                     uint32_t hval, uint32_t hdst, uint32_t K, uint32_t N, uint32_t rows_per_group);
+
+}  // namespace adamah

@@ -1,0 +1,209 @@
+// RMSNorm (+ residual), half-split RoPE, fused per-head QK-norm + RoPE, and row copy (KV append).
+//
+// Reference kernels: shaders/src/f32/map_rmsnorm.comp, map_rmsnorm_x.comp:26-48,
+// map_rmsnorm_add.comp:14-44, map_rope.comp:11-37, map_qk_norm_rope_x.comp:32-84,
+// map_row_copy.comp:13-24; dispatchers adamah.c:7610-7878, 8476-8604, 8061-8085.
+// Row bases come from device-resident loc arrays, one entry per row, as in the reference.
+#include "common.h"
+#include "../../include/adamah_hip.h"
+
+namespace adamah {
+
+__device__ __forceinline__ float block_sum_256(float v, float* sh) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  if ((threadIdx.x & 63u) == 0) sh[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float t = (sh[0] + sh[1]) + (sh[2] + sh[3]);
+  __syncthreads();
+  return t;
+}
+
+// y = x * (1/sqrt(sum(x^2)/dim + eps)) * w (+ r); one 256-thread workgroup per row
+template <bool ADD>
+__global__ void __launch_bounds__(256)
+k_rmsnorm(const float* act, const float* wt, float* out, const uint32_t* __restrict__ ls,
+          const uint32_t* __restrict__ lw, const uint32_t* __restrict__ lr, const uint32_t* __restrict__ ld,
+          uint32_t dim, float eps, uint64_t act_elems, uint64_t wt_elems) {
+  __shared__ float sh[4];
+  const uint32_t ri = blockIdx.x, tid = threadIdx.x;
+  const uint64_t sb = ls[ri], wb = lw[ri], db = ld[ri], rb = ADD ? (uint64_t)lr[ri] : 0;
+  if (sb + dim > act_elems || db + dim > act_elems || wb + dim > wt_elems || (ADD && rb + dim > act_elems)) return;
+  float ss = 0.f;
+  for (uint32_t i = tid; i < dim; i += 256u) { float x = act[sb + i]; ss = fmaf(x, x, ss); }
+  ss = block_sum_256(ss, sh);
+  const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
+  for (uint32_t i = tid; i < dim; i += 256u) {
+    float y = act[sb + i] * inv * wt[wb + i];
+    if (ADD) y += act[rb + i];
+    out[db + i] = y;
+  }
+}
+
+// theta_i = pos * (1 / base^(2i/dim)).  The exponent and the reciprocal are float32 operations as
+// in the shader; the power itself is evaluated in double and rounded once, which makes the
+// frequency independent of the float32 pow implementation.
+__device__ __forceinline__ void rope_cs(uint32_t i, uint32_t dim, uint32_t pos, float base, float* c, float* s) {
+  const float e = (float)(2u * i) / (float)dim;
+  const float p = (float)pow((double)base, (double)e);
+  const float angle = (float)pos * (1.0f / p);
+  *c = cosf(angle);
+  *s = sinf(angle);
+}
+
+__global__ void __launch_bounds__(256)
+k_rope(float* data, const uint32_t* __restrict__ ls, const uint32_t* __restrict__ ld, uint32_t n_tokens,
+       uint32_t n_heads, uint32_t head_dim, uint32_t pos_offset, float base, uint64_t n_elems) {
+  const uint32_t half = head_dim >> 1;
+  const uint64_t tid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+  if (tid >= (uint64_t)n_tokens * n_heads * half) return;
+  const uint32_t token = (uint32_t)(tid / ((uint64_t)n_heads * half));
+  const uint32_t rem = (uint32_t)(tid % ((uint64_t)n_heads * half));
+  const uint32_t head = rem / half, d = rem % half;
+  const uint64_t bs = (uint64_t)ls[token] + (uint64_t)head * head_dim, bd = (uint64_t)ld[token] + (uint64_t)head * head_dim;
+  if (bs + head_dim > n_elems || bd + head_dim > n_elems) return;
+  float c, s;
+  rope_cs(d, head_dim, pos_offset + token, base, &c, &s);
+  const float x0 = data[bs + d], x1 = data[bs + d + half];
+  data[bd + d] = x0 * c - x1 * s;
+  data[bd + d + half] = x0 * s + x1 * c;
+}
+
+// One workgroup per Q or K row: RMSNorm with eps = 1e-6 (fixed in the shader), weight per row from
+// map_wt, then RoPE; rows written contiguously (Q rows, then K rows) from locs_qk_dst[0].
+__global__ void __launch_bounds__(256)
+k_qk_norm_rope(float* act, const float* wt, const uint32_t* __restrict__ lqs, const uint32_t* __restrict__ lqw,
+               const uint32_t* __restrict__ lks, const uint32_t* __restrict__ lkw, const uint32_t* __restrict__ ldst,
+               uint32_t q_rows, uint32_t q_dim, uint32_t k_rows, uint32_t k_dim, uint32_t pos, float base,
+               uint64_t act_elems, uint64_t wt_elems) {
+  __shared__ float sh[4];
+  const uint32_t row = blockIdx.x, tid = threadIdx.x;
+  const bool is_q = row < q_rows;
+  const uint32_t lr = is_q ? row : row - q_rows;
+  const uint32_t dim = is_q ? q_dim : k_dim, half = dim >> 1;
+  if (half == 0) return;
+  const uint64_t sb = is_q ? lqs[lr] : lks[lr], wb = is_q ? lqw[lr] : lkw[lr];
+  const uint64_t db = (uint64_t)ldst[0] + (is_q ? (uint64_t)lr * q_dim : (uint64_t)q_rows * q_dim + (uint64_t)lr * k_dim);
+  if (sb + dim > act_elems || db + dim > act_elems || wb + dim > wt_elems) return;
+  float ss = 0.f;
+  for (uint32_t i = tid; i < dim; i += 256u) { float x = act[sb + i]; ss = fmaf(x, x, ss); }
+  ss = block_sum_256(ss, sh);
+  const float inv = 1.0f / sqrtf(ss / (float)dim + 1e-6f);
+  for (uint32_t i = tid; i < half; i += 256u) {
+    const float y0 = act[sb + i] * inv * wt[wb + i];
+    const float y1 = act[sb + i + half] * inv * wt[wb + i + half];
+    float c, s;
+    rope_cs(i, dim, pos, base, &c, &s);
+    act[db + i] = y0 * c - y1 * s;
+    act[db + i + half] = y0 * s + y1 * c;
+  }
+}
+
+// spec = [src_row, dst_row] pairs; src = src_base[0] + src_row*row_size; dst = (dst_row+offset)*row_size.
+// Destinations inside the map's fp16 KV range are rounded to fp16 and mirrored.
+__global__ void __launch_bounds__(256)
+k_row_copy(float* data, const uint32_t* __restrict__ spec, const uint32_t* __restrict__ src_base, uint32_t n_copies,
+           uint32_t row_size, uint32_t dst_row_offset, uint64_t n_elems, __half* kv16, uint64_t kv_start,
+           uint64_t kv_count) {
+  const uint64_t tid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+  const uint32_t ci = (uint32_t)(tid / row_size), ei = (uint32_t)(tid % row_size);
+  if (ci >= n_copies) return;
+  const uint64_t so = (uint64_t)src_base[0] + (uint64_t)spec[2 * ci] * row_size + ei;
+  const uint64_t dof = ((uint64_t)spec[2 * ci + 1] + dst_row_offset) * row_size + ei;
+  if (so >= n_elems || dof >= n_elems) return;
+  float v = data[so];
+  if (kv16 && dof >= kv_start && dof - kv_start < kv_count) {
+    const __half h = __float2half(v);
+    kv16[dof - kv_start] = h;
+    v = __half2float(h);
+  }
+  data[dof] = v;
+}
+
+static int rmsnorm_impl(uint32_t map_act, uint32_t map_wt, uint32_t hs, uint32_t hw, uint32_t hr, uint32_t hd,
+                        uint32_t n_rows, uint32_t dim, float eps, bool add) {
+  Map* ma = get_f32_map(map_act);
+  Map* mw = get_f32_map(map_wt);
+  if (!ma || !mw) return ADAMAH_ERR_INVALID;
+  if (n_rows == 0) return ADAMAH_OK;
+  const uint32_t *ls = res_u32(hs, n_rows), *lw = res_u32(hw, n_rows), *ld = res_u32(hd, n_rows);
+  const uint32_t* lr = add ? res_u32(hr, n_rows) : ls;
+  if (!ls || !lw || !ld || !lr) return ADAMAH_ERR_INVALID;
+  float* a = (float*)ma->buf;
+  if (add)
+    k_rmsnorm<true><<<n_rows, 256, 0, g.stream>>>(a, (const float*)mw->buf, a, ls, lw, lr, ld, dim, eps, ma->n_elems,
+                                                  mw->n_elems);
+  else
+    k_rmsnorm<false><<<n_rows, 256, 0, g.stream>>>(a, (const float*)mw->buf, a, ls, lw, lr, ld, dim, eps, ma->n_elems,
+                                                   mw->n_elems);
+  count_launch();
+  return check_launch();
+}
+
+}  // namespace adamah
+
+using namespace adamah;
+
+extern "C" {
+
+int map_rmsnorm_dev(uint32_t map_id, uint32_t hs, uint32_t hw, uint32_t hd, uint32_t n_rows, uint32_t dim, float eps) {
+  return rmsnorm_impl(map_id, map_id, hs, hw, 0, hd, n_rows, dim, eps, false);
+}
+int map_rmsnorm_x_dev(uint32_t map_act, uint32_t map_wt, uint32_t hs, uint32_t hw, uint32_t hd, uint32_t n_rows,
+                      uint32_t dim, float eps) {
+  return rmsnorm_impl(map_act, map_wt, hs, hw, 0, hd, n_rows, dim, eps, false);
+}
+int map_rmsnorm_add_dev(uint32_t map_id, uint32_t hs, uint32_t hw, uint32_t hr, uint32_t hd, uint32_t n_rows,
+                        uint32_t dim, float eps) {
+  return rmsnorm_impl(map_id, map_id, hs, hw, hr, hd, n_rows, dim, eps, true);
+}
+
+int map_rope_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_tokens, uint32_t n_heads, uint32_t head_dim,
+                 uint32_t pos_offset, float freq_base) {
+  Map* m = get_f32_map(map_id);
+  if (!m) return ADAMAH_ERR_INVALID;
+  const uint64_t pairs = (uint64_t)n_tokens * n_heads * (head_dim / 2);
+  if (pairs == 0) return ADAMAH_OK;
+  const uint32_t *ls = res_u32(hs, n_tokens), *ld = res_u32(hd, n_tokens);
+  if (!ls || !ld) return ADAMAH_ERR_INVALID;
+  k_rope<<<cdiv(pairs, 256), 256, 0, g.stream>>>((float*)m->buf, ls, ld, n_tokens, n_heads, head_dim, pos_offset,
+                                                  freq_base, m->n_elems);
+  count_launch();
+  return check_launch();
+}
+
+int map_qk_norm_rope_x_dev(uint32_t map_act, uint32_t map_wt, uint32_t hqs, uint32_t hqw, uint32_t hks, uint32_t hkw,
+                           uint32_t hdst, uint32_t q_rows, uint32_t q_dim, uint32_t k_rows, uint32_t k_dim,
+                           uint32_t pos_offset, float freq_base) {
+  Map* ma = get_f32_map(map_act);
+  Map* mw = get_f32_map(map_wt);
+  if (!ma || !mw) return ADAMAH_ERR_INVALID;
+  if (q_rows + k_rows == 0) return ADAMAH_OK;
+  const uint32_t* one = res_u32(hdst, 1);
+  const uint32_t *lqs = q_rows ? res_u32(hqs, q_rows) : one, *lqw = q_rows ? res_u32(hqw, q_rows) : one;
+  const uint32_t *lks = k_rows ? res_u32(hks, k_rows) : one, *lkw = k_rows ? res_u32(hkw, k_rows) : one;
+  if (!one || !lqs || !lqw || !lks || !lkw) return ADAMAH_ERR_INVALID;
+  k_qk_norm_rope<<<q_rows + k_rows, 256, 0, g.stream>>>((float*)ma->buf, (const float*)mw->buf, lqs, lqw, lks, lkw, one,
+                                                        q_rows, q_dim, k_rows, k_dim, pos_offset, freq_base,
+                                                        ma->n_elems, mw->n_elems);
+  count_launch();
+  return check_launch();
+}
+
+int map_row_copy_offset_dev(uint32_t map_id, uint32_t hspec, uint32_t hbase, uint32_t dst_row_offset, uint32_t n_copies,
+                            uint32_t row_size) {
+  Map* m = get_f32_map(map_id);
+  if (!m) return ADAMAH_ERR_INVALID;
+  if (n_copies == 0 || row_size == 0) return ADAMAH_OK;
+  const uint32_t *spec = res_u32(hspec, 2ull * n_copies), *base = res_u32(hbase, 1);
+  if (!spec || !base) return ADAMAH_ERR_INVALID;
+  k_row_copy<<<cdiv((uint64_t)n_copies * row_size, 256), 256, 0, g.stream>>>(
+      (float*)m->buf, spec, base, n_copies, row_size, dst_row_offset, m->n_elems, m->kv16, m->kv_start, m->kv_count);
+  count_launch();
+  return check_launch();
+}
+int map_row_copy_dev(uint32_t map_id, uint32_t hspec, uint32_t hbase, uint32_t n_copies, uint32_t row_size) {
+  return map_row_copy_offset_dev(map_id, hspec, hbase, 0, n_copies, row_size);
+}
+
+}  // extern "C"

@@ -1,0 +1,480 @@
+"""Decode harness: issues the reference model engine's op sequence through the ADAMAH op surface.
+
+This is the caller side of the drop-in boundary.  It reproduces, for block-quantised
+(Q4_0 / Q8_0) models, what `ADAMEngine` does in the reference (adam/models/engine.py):
+
+* `_build_layout`      :518-609   tensors sorted with Q,K,V adjacent, packed back to back into the
+                                   Q4 map (and the Q8 map for Q8_0 tensors), norms into the workspace
+* `_alloc_workspace`   :1213-1576 slot order, score rows at element 0, per-head-contiguous KV cache
+                                   `[K|V][Hkv][kv_cap][d]` at the end of map 0, all loc handles
+* `_upload_all`        :929-1211  qparams + packed nibble upload (Q4), uint8+128 upload (Q8)
+* `_upload_locs`       :1601-1725 one base handle per weight, merged QKV / gate-up detection
+* `_forward`           :2971-3706 the per-token op order (default, non-Broadcom path)
+* `generate`           :3810-3944 token-by-token prefill, greedy decode loop, `decode_tps`
+
+It talks only to an object with the binding's methods, so the same harness runs on the HIP
+library and on any other implementation of the surface.  Two extensions beyond the
+reference, both optional: weights may be spread over several Q4 maps when they exceed the
+32-bit element range of one map, and the KV region may be declared fp16 (`kv_fp16`).
+"""
+import time
+from dataclasses import dataclass
+from typing import Optional
+
+import numpy as np
+
+from .quant import QTensor
+
+
+@dataclass
+class GenerationConfig:
+    max_tokens: int = 128
+    temperature: float = 0.0
+    top_k: int = 1
+    top_p: float = 1.0
+    repeat_penalty: float = 1.0
+    seed: Optional[int] = None
+    eos_token_ids: tuple = ()
+
+
+@dataclass
+class ModelConfig:
+    arch: str = "llama"
+    n_vocab: int = 32000
+    n_ctx: int = 4096
+    n_embd: int = 4096
+    n_head: int = 32
+    n_head_kv: int = 32
+    n_layer: int = 32
+    n_ff: int = 11008
+    head_dim: int = 128
+    head_dim_kv: int = 128
+    norm_eps: float = 1e-6
+    rope_base_global: float = 10000.0
+    rope_base_local: float = 10000.0
+    sliding_window: int = 0
+    ffn_act: str = 'silu'
+    emb_scale: float = 1.0
+    attn_softcap: float = 0.0
+    final_softcap: float = 0.0
+
+    def is_global(self, L):
+        # reference engine.py:52-54
+        if self.arch == "gemma3":
+            return (L + 1) % 6 == 0
+        return True
+
+
+class DecodeEngine:
+    WS_MAP = 0
+    Q8_MAP = 2
+    Q4_GROUP = 32
+    SAMPLE_TOPK_MAX = 64
+    SAMPLE_APPROX_SHORTLIST_MAX = 256
+
+    def __init__(self, gpu, cfg, tensors, A=None, kv_cap=1024, kv_fp16=False,
+                 fusion_scheduler_mode='legacy', gpu_fused_rows_per_group=256,
+                 q4_map_elem_limit=(1 << 32) - 64, verbose=False):
+        if A is None:
+            from . import adamah as A
+        self.gpu, self.cfg, self.tensors, self.A = gpu, cfg, tensors, A
+        self.verbose = verbose
+        self._kv_cap = int(kv_cap)
+        self._kv_fp16 = bool(kv_fp16)
+        self._rows_per_group = max(1, int(gpu_fused_rows_per_group))
+        self._q4_limit = int(q4_map_elem_limit)
+        self._build_layout()
+        self._alloc_workspace()
+        self._upload_all()
+        self._alloc_kv_cache()
+        self._upload_locs()
+        self._sched = str(fusion_scheduler_mode).strip().lower()
+        gpu.fusion_set_scheduler_mode(self._sched)
+        gpu.fusion_enable(True)
+        self._sample_token_ready = False
+        self.n_ops_last_forward = 0
+
+    # ------------------------------------------------------------------ layout
+    @staticmethod
+    def _qkv_sort_key(n):
+        for a, b in (('.attn_q.', '.attn_z0.'), ('.attn_k.', '.attn_z1.'), ('.attn_v.', '.attn_z2.')):
+            if a in n:
+                return n.replace(a, b)
+        return n
+
+    def _build_layout(self):
+        t = self.tensors
+        self._tied = 'output.weight' not in t
+        self._off, self._map_of, self._kind = {}, {}, {}
+        self._norm_names = []
+        q4_maps = [1] + [i for i in range(3, 16)]
+        mi, q4_pos, q8_pos = 0, 0, 0
+        self._q4_sizes = {}
+        for name in sorted(t.keys(), key=self._qkv_sort_key):
+            v = t[name]
+            if isinstance(v, QTensor):
+                if v.kind == 'q8_0':
+                    self._off[name], self._map_of[name], self._kind[name] = q8_pos, self.Q8_MAP, 'q8'
+                    q8_pos += v.size
+                else:
+                    if q4_pos and q4_pos + v.size > self._q4_limit:
+                        self._q4_sizes[q4_maps[mi]] = q4_pos
+                        mi += 1; q4_pos = 0
+                    self._off[name], self._map_of[name], self._kind[name] = q4_pos, q4_maps[mi], 'q4'
+                    q4_pos += v.size
+            elif isinstance(v, np.ndarray) and v.ndim == 1:
+                self._norm_names.append(name)
+        if q4_pos:
+            self._q4_sizes[q4_maps[mi]] = q4_pos
+        self._q8_total = q8_pos
+        self._lm_name = 'token_embd.weight' if self._tied else 'output.weight'
+
+    # ------------------------------------------------------------------ workspace
+    def _up(self, arr):
+        h, _ = self.gpu.upload_dev(np.ascontiguousarray(arr, dtype=np.uint32))
+        if h == 0:
+            raise RuntimeError("upload_dev failed")
+        return h
+
+    def _alloc_workspace(self):
+        c, g = self.cfg, self.gpu
+        kv_cap = self._kv_cap
+        q_dim, k_dim = c.n_head * c.head_dim, c.n_head_kv * c.head_dim_kv
+        gs = c.n_head // c.n_head_kv
+        self._ws = {}
+        self._fused_groups = (c.n_vocab + self._rows_per_group - 1) // self._rows_per_group
+
+        def span(name, sz, pos):
+            h = self._up(np.arange(pos, pos + sz))
+            self._ws[name] = (h, sz, pos)
+            g.register_loc_span(h, 0, pos, sz)
+
+        pos = 0
+        sc_sz = c.n_head * kv_cap
+        span('scores', sc_sz, 0)
+        self._scores_row_h = self._up(np.arange(0, sc_sz, kv_cap))
+        g.register_row_base_span(self._scores_row_h, 0, 0, c.n_head, kv_cap, kv_cap)
+        pos += sc_sz
+        self._pos_scale = pos; pos += 1
+        if c.emb_scale != 1.0:
+            h = self._up(np.full(c.n_embd, pos))
+            self._ws['emb_scale'] = (h, c.n_embd, pos)
+            g.register_loc_span(h, 0, pos, 1)
+            self._pos_emb_scale = pos; pos += 1
+        if c.attn_softcap > 0:
+            self._pos_attn_cap = pos; pos += 1
+        if c.final_softcap > 0:
+            self._pos_final_cap = pos; pos += 1
+
+        slots = [('hidden', c.n_embd), ('normed', c.n_embd), ('q', q_dim), ('k', k_dim), ('v', k_dim),
+                 ('attn_out', c.n_head * c.head_dim_kv), ('o_proj', c.n_embd), ('gate', c.n_ff),
+                 ('up', c.n_ff), ('act', c.n_ff), ('ffn_out', c.n_embd), ('logits', c.n_vocab),
+                 ('sample_token', 1), ('sample_rand', 1),
+                 ('sample_fused_idx', self._fused_groups), ('sample_fused_val', self._fused_groups),
+                 ('normed2', c.n_embd)]
+        for name, sz in slots:
+            span(name, sz, pos); pos += sz
+
+        for name in self._norm_names:
+            self._off[name] = pos; self._map_of[name] = 0
+            pos += self.tensors[name].size
+
+        pos_q, pos_k, pos_v = self._ws['q'][2], self._ws['k'][2], self._ws['v'][2]
+        self._q_rows_h = self._up(pos_q + np.arange(c.n_head) * c.head_dim)
+        g.register_row_base_span(self._q_rows_h, 0, pos_q, c.n_head, c.head_dim, c.head_dim)
+        self._k_rows_h = self._up(pos_k + np.arange(c.n_head_kv) * c.head_dim_kv)
+        g.register_row_base_span(self._k_rows_h, 0, pos_k, c.n_head_kv, c.head_dim_kv, c.head_dim_kv)
+        # separate source handles for RoPE (same positions as the q / k slots)
+        self._q_rope_src_h = self._up(np.arange(pos_q, pos_q + q_dim))
+        self._k_rope_src_h = self._up(np.arange(pos_k, pos_k + k_dim))
+        g.register_loc_span(self._q_rope_src_h, 0, pos_q, q_dim)
+        g.register_loc_span(self._k_rope_src_h, 0, pos_k, k_dim)
+        self._qk_out_h = None
+        if c.head_dim == c.head_dim_kv:
+            self._qk_out_h = self._up(np.arange(pos_q, pos_q + q_dim + k_dim))
+            g.register_loc_span(self._qk_out_h, 0, pos_q, q_dim + k_dim)
+        self._qkv_out_h = self._up(np.arange(pos_q, pos_q + q_dim + 2 * k_dim))
+        g.register_loc_span(self._qkv_out_h, 0, pos_q, q_dim + 2 * k_dim)
+        pos_gate = self._ws['gate'][2]
+        self._gateup_out_h = self._up(np.arange(pos_gate, pos_gate + 2 * c.n_ff))
+        g.register_loc_span(self._gateup_out_h, 0, pos_gate, 2 * c.n_ff)
+        self._k_src_base_h = self._up([pos_k])
+        g.register_loc_span(self._k_src_base_h, 0, pos_k, 1)
+
+        # KV cache: layer L -> K heads [Hkv, kv_cap, d] then V heads, start aligned to d
+        kv_step = kv_cap * c.head_dim_kv
+        kv_per_layer = 2 * c.n_head_kv * kv_step
+        if pos % c.head_dim_kv:
+            pos += c.head_dim_kv - pos % c.head_dim_kv
+        self._kv_start, self._kv_step, self._kv_per_layer = pos, kv_step, kv_per_layer
+        self._k_base = [pos + L * kv_per_layer for L in range(c.n_layer)]
+        self._v_base = [kb + c.n_head_kv * kv_step for kb in self._k_base]
+        pos += c.n_layer * kv_per_layer
+        self._k_locs_h, self._v_locs_h, self._kv_copy_h = [], [], []
+        heads = np.arange(c.n_head) // gs
+        for L in range(c.n_layer):
+            kb, vb = self._k_base[L], self._v_base[L]
+            hk = self._up(kb + heads * kv_step); hv = self._up(vb + heads * kv_step)
+            g.register_row_base_span(hk, 0, kb, c.n_head_kv, kv_step, kv_step)
+            g.register_row_base_span(hv, 0, vb, c.n_head_kv, kv_step, kv_step)
+            self._k_locs_h.append(hk); self._v_locs_h.append(hv)
+            spec = np.empty(4 * c.n_head_kv, np.uint32)
+            for gi in range(c.n_head_kv):
+                spec[4 * gi:4 * gi + 4] = (gi, kb // c.head_dim_kv + gi * kv_cap,
+                                           gi + c.n_head_kv, vb // c.head_dim_kv + gi * kv_cap)
+            self._kv_copy_h.append(self._up(spec))
+        pos_ao = self._ws['attn_out'][2]
+        self._ao_rows_h = self._up(pos_ao + np.arange(c.n_head) * c.head_dim_kv)
+        g.register_row_base_span(self._ao_rows_h, 0, pos_ao, c.n_head, c.head_dim_kv, c.head_dim_kv)
+
+        self._hid_locs = np.arange(self._ws['hidden'][2], self._ws['hidden'][2] + c.n_embd, dtype=np.uint32)
+        self._sample_locs = np.array([self._ws['sample_token'][2]], dtype=np.uint32)
+        self._ws_total = pos
+
+    # ------------------------------------------------------------------ upload
+    def _upload_all(self):
+        g, A, t = self.gpu, self.A, self.tensors
+        g.set_dtype(A.DTYPE_F32)
+        g.map_create(self.WS_MAP, 1, self._ws_total)
+        if self._kv_fp16:
+            g.kv_cache_fp16(self.WS_MAP, self._kv_start, self.cfg.n_layer * self._kv_per_layer)
+        chunk = 1 << 25
+        for mid, total in self._q4_sizes.items():
+            g.map_create_typed(mid, A.DTYPE_Q4, 1, total, self.Q4_GROUP)
+            names = [n for n in self._off if self._map_of.get(n) == mid and self._kind.get(n) == 'q4']
+            names.sort(key=lambda n: self._off[n])
+            ng = (total + self.Q4_GROUP - 1) // self.Q4_GROUP
+            sc = np.ones(ng, np.float32); zp = np.zeros(ng, np.float32)
+            for n in names:
+                s, z = t[n].qparams()
+                g0 = self._off[n] // self.Q4_GROUP
+                sc[g0:g0 + s.size] = s; zp[g0:g0 + z.size] = z
+            g.set_qparams(mid, sc, zp)
+            for n in names:
+                codes = t[n].codes
+                for b in range(0, codes.size, chunk):
+                    part = codes[b:b + chunk]
+                    g.scatter_q4_packed_contiguous(mid, self._off[n] + 2 * b, part, n_locs=2 * part.size)
+        if self._q8_total:
+            g.map_create_typed(self.Q8_MAP, A.DTYPE_Q8, 1, self._q8_total, self.Q4_GROUP)
+            ng = (self._q8_total + self.Q4_GROUP - 1) // self.Q4_GROUP
+            sc = np.ones(ng, np.float32); zp = np.zeros(ng, np.float32)
+            for n, kind in self._kind.items():
+                if kind != 'q8':
+                    continue
+                s, z = t[n].qparams()
+                g0 = self._off[n] // self.Q4_GROUP
+                sc[g0:g0 + s.size] = s; zp[g0:g0 + z.size] = z
+                codes = t[n].codes
+                for b in range(0, codes.size, chunk):
+                    g.scatter_contiguous(self.Q8_MAP, self._off[n] + b, codes[b:b + chunk])
+            g.set_qparams(self.Q8_MAP, sc, zp)
+        for n in self._norm_names:
+            off = self._off[n]
+            g.scatter(self.WS_MAP, np.arange(off, off + t[n].size, dtype=np.uint32),
+                      np.ascontiguousarray(t[n], np.float32))
+
+    def _alloc_kv_cache(self):
+        c, g = self.cfg, self.gpu
+        self.reset()
+        one = lambda p, v: g.scatter(self.WS_MAP, np.array([p], np.uint32), np.array([v], np.float32))
+        one(self._pos_scale, 1.0 / np.sqrt(c.head_dim))
+        if c.emb_scale != 1.0:
+            one(self._pos_emb_scale, c.emb_scale)
+        if c.attn_softcap > 0:
+            one(self._pos_attn_cap, c.attn_softcap)
+        if c.final_softcap > 0:
+            one(self._pos_final_cap, c.final_softcap)
+
+    def _upload_locs(self):
+        c = self.cfg
+        self._wh = {n: self._up([self._off[n]]) for n in self._kind}
+
+        def merged(names):
+            if len({self._map_of[n] for n in names}) != 1 or len({self._kind[n] for n in names}) != 1:
+                return None
+            for a, b in zip(names, names[1:]):
+                if self._off[b] != self._off[a] + self.tensors[a].size:
+                    return None
+            return self._wh[names[0]]
+
+        self._qkv_wt, self._gateup_wt = {}, {}
+        for L in range(c.n_layer):
+            p = f'blk.{L}'
+            h = merged([f'{p}.attn_q.weight', f'{p}.attn_k.weight', f'{p}.attn_v.weight'])
+            if h:
+                self._qkv_wt[L] = h
+            h = merged([f'{p}.ffn_gate.weight', f'{p}.ffn_up.weight'])
+            if h:
+                self._gateup_wt[L] = h
+        for n in self._norm_names:
+            off, sz = self._off[n], self.tensors[n].size
+            if 'attn_q_norm' in n:
+                rows, hd = c.n_head, c.head_dim
+                locs = [off] * rows if sz == hd else [off + i * hd for i in range(rows)]
+            elif 'attn_k_norm' in n:
+                rows, hd = c.n_head_kv, c.head_dim_kv
+                locs = [off] * rows if sz == hd else [off + i * hd for i in range(rows)]
+            else:
+                locs = [off]
+            self._wh[n] = self._up(locs)
+        # embedding fetch: tied Q4 matrix -> per-token gather locs; untied -> host rows
+        self._emb_gather_h = 0
+        if self._tied:
+            self._emb_base = (np.uint32(self._off[self._lm_name]) + np.arange(c.n_embd, dtype=np.uint32))
+            self._emb_locs = np.empty(c.n_embd, np.uint32)
+            self._emb_gather_h = self._up(self._emb_base)
+
+    # ------------------------------------------------------------------ op helpers
+    def _proj(self, in_h, name, out_h, K, N, wt_h=None):
+        g = self.gpu
+        fn = g.map_matmul_t_xq8_dev if self._kind[name] == 'q8' else g.map_matmul_t_xq4_dev
+        fn(self.WS_MAP, self._map_of[name], in_h, wt_h or self._wh[name], out_h, 1, K, N)
+
+    def _rms(self, src_h, name, dst_h, rows, dim):
+        self.gpu.map_rmsnorm_dev(self.WS_MAP, src_h, self._wh[name], dst_h, rows, dim, self.cfg.norm_eps)
+
+    # ------------------------------------------------------------------ forward
+    def _forward(self, tok, pos, sample=True):
+        """One decode step; op order of reference engine.py:2971-3402 (default discrete-GPU path)."""
+        c, g, A, ws = self.cfg, self.gpu, self.A, self.WS_MAP
+        q_dim, k_dim = c.n_head * c.head_dim, c.n_head_kv * c.head_dim_kv
+        seq_len = pos + 1
+        W = self._ws
+        hid_h, normed_h, q_h, k_h, v_h = (W[n][0] for n in ('hidden', 'normed', 'q', 'k', 'v'))
+        ao_h, op_h, n2_h, gate_h, up_h, act_h, ffn_h = (
+            W[n][0] for n in ('attn_out', 'o_proj', 'normed2', 'gate', 'up', 'act', 'ffn_out'))
+        alias_fast = self._sched != 'legacy'
+
+        if self._tied:
+            np.add(self._emb_base, np.uint32(tok * c.n_embd), out=self._emb_locs)
+            g.upload_dev(self._emb_locs, handle=self._emb_gather_h)
+        else:
+            row = self.tensors['token_embd.weight'].row(tok)
+            if c.emb_scale != 1.0:
+                row = row * np.float32(c.emb_scale)
+            g.scatter(ws, self._hid_locs, row)
+
+        g.batch_begin()
+        if self._tied:
+            src_h, _, _, _ = g.map_gather_dev(self._map_of[self._lm_name], self._emb_gather_h, c.n_embd)
+            g.map_scatter_dev(ws, hid_h, c.n_embd, src_h)
+            if c.emb_scale != 1.0:
+                g.map_broadcast_dev(ws, A.OP_MUL, hid_h, W['emb_scale'][0], hid_h, c.n_embd)
+
+        for L in range(c.n_layer):
+            p = f'blk.{L}'
+            freq = c.rope_base_global if c.is_global(L) else c.rope_base_local
+            self._rms(hid_h, f'{p}.attn_norm.weight', normed_h, 1, c.n_embd)
+            if alias_fast and L in self._qkv_wt:
+                self._proj(normed_h, f'{p}.attn_q.weight', self._qkv_out_h, c.n_embd,
+                           q_dim + 2 * k_dim, wt_h=self._qkv_wt[L])
+            else:
+                self._proj(normed_h, f'{p}.attn_q.weight', q_h, c.n_embd, q_dim)
+                self._proj(normed_h, f'{p}.attn_k.weight', k_h, c.n_embd, k_dim)
+                self._proj(normed_h, f'{p}.attn_v.weight', v_h, c.n_embd, k_dim)
+
+            qnn = f'{p}.attn_q_norm.weight'
+            if qnn in self._wh:
+                g.map_qk_norm_rope_x_dev(ws, ws, self._q_rows_h, self._wh[qnn], self._k_rows_h,
+                                         self._wh[f'{p}.attn_k_norm.weight'], self._qk_out_h,
+                                         c.n_head, c.head_dim, c.n_head_kv, c.head_dim_kv, pos, freq)
+            else:
+                g.map_rope_dev(ws, self._q_rope_src_h, q_h, 1, c.n_head, c.head_dim, pos, freq)
+                g.map_rope_dev(ws, self._k_rope_src_h, k_h, 1, c.n_head_kv, c.head_dim_kv, pos, freq)
+
+            g.map_row_copy_offset_dev(ws, self._kv_copy_h[L], self._k_src_base_h, pos,
+                                      2 * c.n_head_kv, c.head_dim_kv)
+            g.map_matmul_t_dev(ws, self._q_rows_h, self._k_locs_h[L], self._scores_row_h,
+                               1, c.head_dim, seq_len, c.n_head)
+            g.map_attn_softmax_value_dev(ws, self._scores_row_h, self._v_locs_h[L], self._ao_rows_h,
+                                         c.n_head, seq_len, c.head_dim_kv,
+                                         float(1.0 / np.sqrt(c.head_dim)), float(c.attn_softcap))
+            g.fusion_flush()
+            self._proj(ao_h, f'{p}.attn_output.weight', op_h, c.n_head * c.head_dim_kv, c.n_embd)
+            pan = f'{p}.post_attention_norm.weight'
+            if pan in self._wh:
+                g.map_rmsnorm_add_dev(ws, op_h, self._wh[pan], hid_h, hid_h, 1, c.n_embd, c.norm_eps)
+            else:
+                g.map_op2_dev(ws, A.OP_ADD, hid_h, op_h, hid_h, c.n_embd)
+
+            self._rms(hid_h, f'{p}.ffn_norm.weight', n2_h, 1, c.n_embd)
+            if alias_fast and L in self._gateup_wt:
+                self._proj(n2_h, f'{p}.ffn_gate.weight', self._gateup_out_h, c.n_embd, 2 * c.n_ff,
+                           wt_h=self._gateup_wt[L])
+            else:
+                self._proj(n2_h, f'{p}.ffn_gate.weight', gate_h, c.n_embd, c.n_ff)
+                self._proj(n2_h, f'{p}.ffn_up.weight', up_h, c.n_embd, c.n_ff)
+            g.map_op2_dev(ws, A.OP_GEGLU if c.ffn_act == 'gelu' else A.OP_SWIGLU, gate_h, up_h, act_h, c.n_ff)
+            self._proj(act_h, f'{p}.ffn_down.weight', ffn_h, c.n_ff, c.n_embd)
+            pfn = f'{p}.post_ffw_norm.weight'
+            if pfn in self._wh:
+                g.map_rmsnorm_add_dev(ws, ffn_h, self._wh[pfn], hid_h, hid_h, 1, c.n_embd, c.norm_eps)
+            else:
+                g.map_op2_dev(ws, A.OP_ADD, hid_h, ffn_h, hid_h, c.n_embd)
+
+        self._rms(hid_h, 'output_norm.weight', normed_h, 1, c.n_embd)
+        if sample:
+            fn = (g.map_matvec_argmax_t_xq8_dev if self._kind[self._lm_name] == 'q8'
+                  else g.map_matvec_argmax_t_xq4_dev)
+            fn(ws, self._map_of[self._lm_name], normed_h, self._wh[self._lm_name],
+               W['sample_fused_idx'][0], W['sample_fused_val'][0], W['sample_token'][0],
+               c.n_embd, c.n_vocab, self._rows_per_group)
+            self._sample_token_ready = True
+        g.batch_end()
+
+    def read_token(self):
+        # reference engine.py:1979-1981: token id crosses the boundary as float32
+        tok = self.gpu.gather(self.WS_MAP, self._sample_locs).view(np.float32)
+        return int(tok[0]) if tok.size else 0
+
+    def read_slot(self, name):
+        _, sz, pos = self._ws[name]
+        return self.gpu.gather(self.WS_MAP, np.arange(pos, pos + sz, dtype=np.uint32)).view(np.float32).copy()
+
+    def reset(self):
+        c = self.cfg
+        sc_sz = c.n_head * self._kv_cap
+        self.gpu.scatter(self.WS_MAP, np.arange(sc_sz, dtype=np.uint32), np.full(sc_sz, -1e30, np.float32))
+        self._sample_token_ready = False
+
+    # ------------------------------------------------------------------ generate
+    def generate(self, token_ids, config=None, forced=None):
+        """Greedy generation.  Prefill is the same `_forward` once per prompt token, LM head only
+        on the last one; `decode_tps = n_gen / wall(decode loop)` including the per-token
+        read-back (reference engine.py:3838-3931).  `forced`, when given, is a token list fed
+        back instead of the model's own choices (teacher forcing) while the choices are still
+        returned."""
+        config = config or GenerationConfig()
+        if len(token_ids) + config.max_tokens > self._kv_cap:
+            raise RuntimeError(
+                f"KV cache too small: need {len(token_ids) + config.max_tokens} tokens but "
+                f"kv_cap={self._kv_cap}. Reinitialize with kv_cap>={len(token_ids) + config.max_tokens}.")
+        self.reset()
+        tp = time.perf_counter()
+        last = len(token_ids) - 1
+        for i, t in enumerate(token_ids):
+            self._forward(int(t), i, sample=(i == last))
+        self.gpu.sync()
+        t_pre = time.perf_counter() - tp
+        out, ttimes = [], []
+        td = time.perf_counter()
+        for step in range(config.max_tokens):
+            t0 = time.perf_counter()
+            nt = self.read_token()
+            if nt in config.eos_token_ids:
+                break
+            out.append(nt)
+            feed = nt if forced is None else int(forced[step])
+            self._forward(feed, len(token_ids) + step, sample=True)
+            ttimes.append(time.perf_counter() - t0)
+        self.gpu.sync()
+        t_dec = time.perf_counter() - td
+        n_p, n_g = len(token_ids), len(out)
+        return out, {
+            'n_prompt': n_p, 'n_gen': n_g, 'prefill_s': t_pre, 'decode_s': t_dec,
+            'prefill_tps': n_p / t_pre if t_pre > 0 else 0.0,
+            'decode_tps': n_g / t_dec if t_dec > 0 else 0.0,
+            'avg_ms': float(np.mean(ttimes) * 1000) if ttimes else 0.0,
+            'sampling_mode': 'gpu_matvec_argmax',
+        }
