@@ -20,10 +20,12 @@ f32 = np.float32
 
 
 class CpuModel:
-    def __init__(self, cfg, tensors, kv_cap, kv_fp16=False):
+    def __init__(self, cfg, tensors, kv_cap, kv_fp16=False, acc64=True):
         """tensors: name -> float32 ndarray ([N,K] matrices, 1-D norms); the untied embedding may be
-        an object with .row(tok)."""
+        an object with .row(tok).  acc64=False keeps every matrix product in float32 BLAS, which is
+        how the reference's forward_cpu runs (used when this model is timed as the CPU baseline)."""
         self.c = cfg
+        self.acc64 = acc64
         self.t = tensors
         self.kv_fp16 = kv_fp16
         c = cfg
@@ -56,6 +58,8 @@ class CpuModel:
         return np.concatenate([x0 * ct - x1 * st, x0 * st + x1 * ct], axis=1).astype(np.float32)
 
     def mv(self, name, x):
+        if not self.acc64:
+            return self.t[name] @ x
         return (self.t[name].astype(np.float64) @ x.astype(np.float64)).astype(np.float32)
 
     def embed(self, tok):

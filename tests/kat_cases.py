@@ -238,7 +238,9 @@ def kat_decode_plan_runtime_args(g, A):
         g.decode_step(1, pos=8, seq_len=3)
     finally:
         g.clear_decode_plan(1)
-    for probe, lit in (([8, 9, 10], [10.0, 20.0, 30.0]), ([12, 13, 14], [2.0, 4.0, 6.0])):
+    # the copy's destination row (0 + pos 8) * 3 = 24 lies past the 24-element map in the reference's
+    # own scenario, so elements 8..10 stay 0 on both maps; the doubled values land at 12..14
+    for probe, lit in (([8, 9, 10], [0.0, 0.0, 0.0]), ([12, 13, 14], [2.0, 4.0, 6.0])):
         d, p = _read(g, 6, probe), _read(g, 7, probe)
         assert np.allclose(d, p, atol=1e-6) and np.allclose(p, lit, atol=1e-6)
 

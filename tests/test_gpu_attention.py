@@ -1,0 +1,100 @@
+"""GQA decode attention through the two reference entry points (scores, softmax.V): HIP vs oracle.
+
+BASELINE config 3: 32 q heads / 8 kv heads, head_dim 128, fp16 KV cache, contexts 1024 / 4096 /
+16384, q/K/V ~N(0,1), scale 1/sqrt(128), fp32 softmax; output compared per head (1e-3 rel L2)."""
+import numpy as np
+import pytest
+
+import oracle
+from adam_amd import adamah as A
+from gpu_util import note, up, f32map, put, read, rel_l2
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+def attention_case(g, q, K, V, ctx, cap_len, kv16, scale, softcap):
+    """K, V: [Hkv, ctx, d] float32.  Layout as the harness builds it: score rows at element 0 with
+    stride cap_len, then q, out, then the KV region [K heads | V heads], each head cap_len rows."""
+    Hq, d = q.shape
+    Hkv = K.shape[0]
+    gs = Hq // Hkv
+    sc_sz = Hq * cap_len
+    q_pos, out_pos = sc_sz, sc_sz + Hq * d
+    kv_start = (out_pos + Hq * d + d - 1) // d * d
+    step = cap_len * d
+    total = kv_start + 2 * Hkv * step
+    f32map(g, 0, total, None)
+    if kv16:
+        g.kv_cache_fp16(0, kv_start, 2 * Hkv * step)
+    put(g, 0, q_pos, q)
+    for h in range(Hkv):
+        put(g, 0, kv_start + h * step, K[h])
+        put(g, 0, kv_start + (Hkv + h) * step, V[h])
+    heads = np.arange(Hq) // gs
+    q_rows = up(g, q_pos + np.arange(Hq) * d)
+    k_locs = up(g, kv_start + heads * step)
+    v_locs = up(g, kv_start + (Hkv + heads) * step)
+    s_rows = up(g, np.arange(Hq) * cap_len)
+    o_rows = up(g, out_pos + np.arange(Hq) * d)
+    g.batch_begin()
+    g.map_matmul_t_dev(0, q_rows, k_locs, s_rows, 1, d, ctx, Hq)
+    g.map_attn_softmax_value_dev(0, s_rows, v_locs, o_rows, Hq, ctx, d, scale, softcap)
+    g.batch_end()
+    scores = np.stack([read(g, 0, h * cap_len, ctx) for h in range(0, Hq, max(1, Hq // 4))])
+    return read(g, 0, out_pos, Hq * d).reshape(Hq, d), scores
+
+
+@pytest.mark.parametrize("ctx", [1024, 4096, 16384])
+def test_config3_gqa_decode_attention_fp16_kv(hip, ctx):
+    Hq, Hkv, d = 32, 8, 128
+    rng = np.random.default_rng(ctx)
+    q = rng.standard_normal((Hq, d)).astype(np.float32)
+    K = rng.standard_normal((Hkv, ctx, d), dtype=np.float32)
+    V = rng.standard_normal((Hkv, ctx, d), dtype=np.float32)
+    outs = []
+    for name, g in (("hip", hip), ("oracle", oracle.init())):
+        note(f"attention ctx={ctx} on {name}")
+        outs.append(attention_case(g, q, K, V, ctx, ctx, True, float(1 / np.sqrt(d)), 0.0))
+    for h in range(Hq):
+        assert rel_l2(outs[0][0][h], outs[1][0][h]) < TOL, h
+    assert rel_l2(outs[0][1], outs[1][1]) < 1e-5          # raw q.k score rows
+    # the reference NumPy form (engine.py:2428-2441) on fp16-rounded K/V, independent of the op surface
+    K16 = K.astype(np.float16).astype(np.float64); V16 = V.astype(np.float16).astype(np.float64)
+    for h in (0, 13, 31):
+        s = K16[h // 4] @ q[h].astype(np.float64) / np.sqrt(d)
+        p = np.exp(s - s.max()); p /= p.sum()
+        assert rel_l2(outs[0][0][h], p @ V16[h // 4]) < TOL
+
+
+@pytest.mark.parametrize("ctx,kv16,softcap,Hq,Hkv,d", [
+    (1, True, 50.0, 4, 1, 256), (640, True, 50.0, 4, 1, 256), (1023, False, 0.0, 8, 2, 64),
+    (1025, True, 0.0, 8, 2, 64), (2049, False, 30.0, 4, 4, 128), (300, True, 0.0, 6, 2, 96)])
+def test_attention_variants(hip, ctx, kv16, softcap, Hq, Hkv, d):
+    rng = np.random.default_rng(ctx + d)
+    q = rng.standard_normal((Hq, d)).astype(np.float32)
+    K = rng.standard_normal((Hkv, ctx, d)).astype(np.float32)
+    V = rng.standard_normal((Hkv, ctx, d)).astype(np.float32)
+    outs = []
+    for name, g in (("hip", hip), ("oracle", oracle.init())):
+        note(f"attention variant ctx={ctx} kv16={kv16} cap={softcap} {Hq}/{Hkv}x{d} on {name}")
+        outs.append(attention_case(g, q, K, V, ctx, ctx + 7, kv16, float(1 / np.sqrt(d)), softcap)[0])
+    for h in range(Hq):
+        assert rel_l2(outs[0][h], outs[1][h]) < TOL, h
+    if ctx == 1:   # a single key: the output is the (fp16-rounded) V row exactly
+        want = V[:, 0].astype(np.float16).astype(np.float32) if kv16 else V[:, 0]
+        for h in range(Hq):
+            assert np.array_equal(outs[0][h], want[h // (Hq // Hkv)])
+
+
+def test_gqa_heads_with_equal_queries_agree(hip):
+    Hq, Hkv, d, ctx = 8, 2, 128, 1500
+    rng = np.random.default_rng(1)
+    q = np.repeat(rng.standard_normal((Hkv, d)).astype(np.float32), Hq // Hkv, axis=0)
+    K = rng.standard_normal((Hkv, ctx, d)).astype(np.float32)
+    V = rng.standard_normal((Hkv, ctx, d)).astype(np.float32)
+    note("gqa equal queries")
+    out, _ = attention_case(hip, q, K, V, ctx, ctx, True, float(1 / np.sqrt(d)), 0.0)
+    for g0 in range(Hkv):
+        for j in range(1, Hq // Hkv):
+            assert np.array_equal(out[g0 * 4], out[g0 * 4 + j])
