@@ -46,6 +46,57 @@ k_matmul_t(const float* A, float* C, const TB* bsrc, uint64_t b_shift, const uin
   if (lane == 0 && c < a_elems) C[c] = s;
 }
 
+// Decode scores, M == 1: out[op][t] = q_op . B_op[t].  LPR lanes share one B row (VEC contiguous
+// elements per 16-byte load, up to 4 loads per lane), 64/LPR rows per wave step; each lane keeps
+// its slice of the query in registers.  Needs K % VEC == 0, K <= 4*LPR*VEC and VEC-aligned bases.
+template <typename TB, int VEC>
+__global__ void __launch_bounds__(256)
+k_scores_vec(const float* A, float* C, const TB* bsrc, uint64_t b_shift, const uint32_t* __restrict__ la,
+             const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc, uint32_t K, uint32_t N, uint32_t lpr,
+             uint32_t rows_per_wg) {
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, op = blockIdx.y;
+  const uint32_t sub = lane % lpr, rslot = lane / lpr, rpw = 64u / lpr;   // lane's column slice / row slot
+  const uint64_t a = la[op], b = (uint64_t)lb[op] - b_shift, c = lc[op];
+  const uint32_t nvec = K / VEC;                                         // vectors per row
+  float q[4][VEC];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint32_t v = sub + i * lpr;
+#pragma unroll
+    for (int j = 0; j < VEC; j++) q[i][j] = v < nvec ? A[a + (uint64_t)v * VEC + j] : 0.f;
+  }
+  const uint32_t row0 = blockIdx.x * rows_per_wg, row1 = min(N, row0 + rows_per_wg);
+  for (uint32_t rb = row0 + wave * rpw; rb < row1; rb += 4u * rpw) {
+    const uint32_t r = rb + rslot;
+    float s = 0.f;
+    if (r < row1) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t v = sub + i * lpr;
+        if (v < nvec) {
+          const TB* bp = bsrc + b + (uint64_t)r * K + (uint64_t)v * VEC;
+          if (VEC == 8) {
+            const uint4 raw = *(const uint4*)bp;
+            const __half2* h = (const __half2*)&raw;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+              const float2 f = __half22float2(h[j]);
+              s = fmaf(q[i][2 * j], f.x, s);
+              s = fmaf(q[i][2 * j + 1], f.y, s);
+            }
+          } else {
+            const float4 f = *(const float4*)bp;
+            s = fmaf(q[i][0], f.x, s); s = fmaf(q[i][1], f.y, s);
+            s = fmaf(q[i][2], f.z, s); s = fmaf(q[i][3], f.w, s);
+          }
+        }
+      }
+    }
+    for (uint32_t o = lpr >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    if (r < row1 && sub == 0) C[c + r] = s;
+  }
+}
+
 // C = A[M,K] . B[K,N] (non-transposed B), same indexing conventions.
 __global__ void __launch_bounds__(256)
 k_matmul_nt(const float* A, float* C, const float* B, const uint32_t* __restrict__ la, const uint32_t* __restrict__ lb,
@@ -70,22 +121,22 @@ __device__ __forceinline__ float prep(float v, float scale, float cap) {
   return v;
 }
 
-#define ATT_CHUNK 1024   // score rows handled by one workgroup
+#define ATT_CHUNK 1024   // most score rows one workgroup handles (LDS array size)
 
 // grid (n_splits, n_ops).  Workgroup (split s, op): rows [s*ATT_CHUNK, ...) of the op's score row.
 // Writes either the normalised output (n_splits == 1) or the partial (m, l, o[value_dim]).
-template <typename TV>
+template <typename TV, int VEC>
 __global__ void __launch_bounds__(256)
 k_attn_softmax_value(const float* data, float* out, const TV* vsrc, uint64_t v_shift, const uint32_t* __restrict__ lsc,
                      const uint32_t* __restrict__ lv, const uint32_t* __restrict__ lo, uint32_t row_size,
-                     uint32_t value_dim, float scale, float cap, uint32_t n_splits, float* partial, uint64_t n_elems,
-                     uint64_t v_elems) {
+                     uint32_t value_dim, float scale, float cap, uint32_t n_splits, uint32_t chunk, float* partial,
+                     uint64_t n_elems, uint64_t v_elems) {
   __shared__ float p[ATT_CHUNK];
   __shared__ float red[4];
-  __shared__ float osum[256];
+  __shared__ float osum[VEC > 1 ? 2048 : 256];
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t split = blockIdx.x, op = blockIdx.y;
-  const uint32_t t0 = split * ATT_CHUNK, t1 = min(row_size, t0 + ATT_CHUNK), nt = t1 - t0;
+  const uint32_t t0 = split * chunk, t1 = min(row_size, t0 + chunk), nt = t1 - t0;
   const uint64_t sb = lsc[op], vb = lv[op], ob = lo[op];
   const bool ok = sb + row_size <= n_elems && vb >= v_shift &&
                   vb - v_shift + (uint64_t)row_size * value_dim <= v_elems && ob + value_dim <= n_elems;
@@ -114,6 +165,58 @@ k_attn_softmax_value(const float* data, float* out, const TV* vsrc, uint64_t v_s
   if (lane == 0) red[wave] = sum;
   __syncthreads();
   sum = (red[0] + red[1]) + (red[2] + red[3]);
+  if (VEC > 1) {
+    // pass 3, vector form: lpr = value_dim/VEC lanes cover one V row with 16-byte loads, 256/lpr rows
+    // are in flight per sweep, four sweeps unrolled; row-slot partials meet in LDS.
+    const uint32_t lpr = value_dim / VEC, slots = 256u / lpr, sub = tid % lpr, slot = tid / lpr;
+    float acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) acc[j] = 0.f;
+    if (ok && slot < slots) {
+      const TV* base = vsrc + (vb - v_shift) + (uint64_t)t0 * value_dim + (uint64_t)sub * VEC;
+#pragma unroll 4
+      for (uint32_t t = slot; t < nt; t += slots) {
+        const float w = p[t];
+        if (VEC == 8) {
+          const uint4 raw = *(const uint4*)(base + (uint64_t)t * value_dim);
+          const __half2* h = (const __half2*)&raw;
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            const float2 f = __half22float2(h[j]);
+            acc[2 * j] = fmaf(w, f.x, acc[2 * j]);
+            acc[2 * j + 1] = fmaf(w, f.y, acc[2 * j + 1]);
+          }
+        } else {
+          const float4 f = *(const float4*)(base + (uint64_t)t * value_dim);
+          acc[0] = fmaf(w, f.x, acc[0]); acc[1] = fmaf(w, f.y, acc[1]);
+          acc[2] = fmaf(w, f.z, acc[2]); acc[3] = fmaf(w, f.w, acc[3]);
+        }
+      }
+    }
+    // reduce the row slots: osum holds up to 2048 floats, so fold slots in rounds of (2048/value_dim)
+    const uint32_t fit = 2048u / value_dim;
+    float o = 0.f;
+    for (uint32_t s0 = 0; s0 < slots; s0 += fit) {
+      if (slot >= s0 && slot < s0 + fit && slot < slots) {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) osum[(slot - s0) * value_dim + sub * VEC + j] = acc[j];
+      }
+      __syncthreads();
+      if (tid < value_dim)
+        for (uint32_t s = 0; s < fit && s0 + s < slots; s++) o += osum[s * value_dim + tid];
+      __syncthreads();
+    }
+    if (tid < value_dim && ok) {
+      if (n_splits == 1) out[ob + tid] = o * (1.0f / sum);
+      else partial[((uint64_t)op * n_splits + split) * (value_dim + 2) + 2 + tid] = o;
+    }
+    if (n_splits > 1 && tid == 0) {
+      float* pp = partial + ((uint64_t)op * n_splits + split) * (value_dim + 2);
+      pp[0] = mx;
+      pp[1] = sum;
+    }
+    return;
+  }
   // pass 3: o[d] = sum_t p[t] * V[t][d]; thread (slot, d): slot strides the rows
   const uint32_t dpw = min(value_dim, 256u);       // columns handled per sweep
   const uint32_t slots = 256u / dpw;               // rows in flight per sweep
@@ -222,7 +325,26 @@ int map_matmul_t_dev(uint32_t map_id, uint32_t ha, uint32_t hb, uint32_t hc, uin
   if (!la || !lb || !lc) return ADAMAH_ERR_INVALID;
   dim3 grid(cdiv(N, 4), M, n_ops);
   float* d = (float*)m->buf;
-  if (all_in_kv(m, hb, n_ops, (uint64_t)N * K))
+  const bool kv = all_in_kv(m, hb, n_ops, (uint64_t)N * K);
+  // decode-score fast path: one query row per op, whole 16-byte vectors, operands verified on the host
+  const uint32_t vec = kv ? 8u : 4u;
+  const uint32_t *ah = res_host(ha, n_ops), *bh = res_host(hb, n_ops), *ch = res_host(hc, n_ops);
+  bool fast = M == 1 && ah && bh && ch && K % vec == 0 && K >= vec && K <= 4u * 64u * vec;
+  uint32_t lpr = 1;
+  if (fast) {
+    while (lpr < 64 && lpr * vec < K) lpr <<= 1;        // lanes per row: a power of two, at most 64
+    for (uint32_t op = 0; fast && op < n_ops; op++)
+      fast = in_range(ah[op], K, m->n_elems) && in_range(bh[op], (uint64_t)N * K, m->n_elems) &&
+             in_range(ch[op], N, m->n_elems) && (bh[op] - (kv ? m->kv_start : 0)) % vec == 0;
+  }
+  if (fast) {
+    const uint32_t rows_per_wg = std::max<uint32_t>(4u * (64u / lpr), std::min<uint32_t>(256u, cdiv(N, 2)));
+    dim3 g2(cdiv(N, rows_per_wg), n_ops);
+    if (kv)
+      k_scores_vec<__half, 8><<<g2, 256, 0, g.stream>>>(d, d, m->kv16, m->kv_start, la, lb, lc, K, N, lpr, rows_per_wg);
+    else
+      k_scores_vec<float, 4><<<g2, 256, 0, g.stream>>>(d, d, d, 0, la, lb, lc, K, N, lpr, rows_per_wg);
+  } else if (kv)
     k_matmul_t<__half><<<grid, 256, 0, g.stream>>>(d, d, m->kv16, m->kv_start, la, lb, lc, M, K, N, m->n_elems,
                                                    m->kv_count);
   else
@@ -276,17 +398,29 @@ int map_attn_softmax_value_dev(uint32_t map_id, uint32_t hs, uint32_t hv, uint32
   if (n_ops == 0 || row_size == 0 || value_dim == 0) return ADAMAH_OK;
   const uint32_t *ls = res_u32(hs, n_ops), *lv = res_u32(hv, n_ops), *lo = res_u32(ho, n_ops);
   if (!ls || !lv || !lo) return ADAMAH_ERR_INVALID;
-  const uint32_t n_splits = cdiv(row_size, ATT_CHUNK);
+  // rows per workgroup: enough workgroups to fill the chip (about 2 per CU over all ops), 32..1024 rows each
+  const uint32_t want_splits = std::max<uint32_t>(1u, cdiv(2u * (uint32_t)g.n_cu, n_ops));
+  uint32_t chunk = std::min<uint32_t>(ATT_CHUNK, std::max<uint32_t>(32u, cdiv(row_size, want_splits)));
+  chunk = (chunk + 31u) & ~31u;
+  const uint32_t n_splits = cdiv(row_size, chunk);
   if ((uint64_t)n_ops * n_splits * (value_dim + 2) > g.attn_scratch_floats) return ADAMAH_ERR_INVALID;
   float* d = (float*)m->buf;
   dim3 grid(n_splits, n_ops);
-  if (all_in_kv(m, hv, n_ops, (uint64_t)row_size * value_dim))
-    k_attn_softmax_value<__half><<<grid, 256, 0, g.stream>>>(d, d, m->kv16, m->kv_start, ls, lv, lo, row_size, value_dim,
-                                                             scale, cap, n_splits, g.attn_scratch, m->n_elems,
-                                                             m->kv_count);
-  else
-    k_attn_softmax_value<float><<<grid, 256, 0, g.stream>>>(d, d, d, 0, ls, lv, lo, row_size, value_dim, scale, cap,
-                                                            n_splits, g.attn_scratch, m->n_elems, m->n_elems);
+  const bool kv = all_in_kv(m, hv, n_ops, (uint64_t)row_size * value_dim);
+  // vector path: value rows made of whole 16-byte vectors, 256 % (value_dim/vec) == 0, operands host-verified
+  const uint32_t vec = kv ? 8u : 4u;
+  const uint32_t *sh = res_host(hs, n_ops), *vh = res_host(hv, n_ops), *oh = res_host(ho, n_ops);
+  bool fast = sh && vh && oh && value_dim % vec == 0 && value_dim / vec <= 256 && 256u % (value_dim / vec) == 0 &&
+              value_dim <= 2048 && value_dim <= 256;
+  for (uint32_t op = 0; fast && op < n_ops; op++)
+    fast = in_range(sh[op], row_size, m->n_elems) && in_range(vh[op], (uint64_t)row_size * value_dim, m->n_elems) &&
+           in_range(oh[op], value_dim, m->n_elems) && (vh[op] - (kv ? m->kv_start : 0)) % vec == 0;
+#define ASV(T, V, src, shift, elems)                                                                             \
+  k_attn_softmax_value<T, V><<<grid, 256, 0, g.stream>>>(d, d, src, shift, ls, lv, lo, row_size, value_dim, scale, \
+                                                         cap, n_splits, chunk, g.attn_scratch, m->n_elems, elems)
+  if (kv) { if (fast) ASV(__half, 8, m->kv16, m->kv_start, m->kv_count); else ASV(__half, 1, m->kv16, m->kv_start, m->kv_count); }
+  else { if (fast) ASV(float, 4, d, 0, m->n_elems); else ASV(float, 1, d, 0, m->n_elems); }
+#undef ASV
   count_launch();
   int r = check_launch();
   if (r || n_splits == 1) return r;

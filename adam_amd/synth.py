@@ -71,11 +71,16 @@ def _gen(name, shape, seed, sigma, quant, rows_per_chunk=8192):
     return out
 
 
-def make_model(cfg, seed=0, sigma=0.02, progress=None):
-    """dict name -> QTensor (matrices) / float32 array (norms) / SyntheticEmbedding (untied embd)."""
+def make_model(cfg, seed=0, sigma=0.02, workers=None):
+    """dict name -> QTensor (matrices) / float32 array (norms) / SyntheticEmbedding (untied embd).
+
+    Every tensor has its own generator seeded by (seed, crc32(name)), so the result does not
+    depend on `workers` (threads used to draw and quantise tensors in parallel)."""
+    import os
+    from concurrent.futures import ThreadPoolExecutor
     c = cfg
     q_dim, k_dim = c.n_head * c.head_dim, c.n_head_kv * c.head_dim_kv
-    t = {}
+    t, jobs = {}, []
     gemma = c.arch.startswith("gemma")
     for L in range(c.n_layer):
         p = f"blk.{L}"
@@ -83,7 +88,7 @@ def make_model(cfg, seed=0, sigma=0.02, progress=None):
                 "attn_output": (c.n_embd, c.n_head * c.head_dim_kv), "ffn_gate": (c.n_ff, c.n_embd),
                 "ffn_up": (c.n_ff, c.n_embd), "ffn_down": (c.n_embd, c.n_ff)}
         for nm, sh in mats.items():
-            t[f"{p}.{nm}.weight"] = _gen(f"{p}.{nm}.weight", sh, seed, sigma, quantize_q4_0)
+            jobs.append((f"{p}.{nm}.weight", sh, quantize_q4_0))
         t[f"{p}.attn_norm.weight"] = np.ones(c.n_embd, np.float32)
         t[f"{p}.ffn_norm.weight"] = np.ones(c.n_embd, np.float32)
         if gemma:
@@ -91,12 +96,15 @@ def make_model(cfg, seed=0, sigma=0.02, progress=None):
             t[f"{p}.attn_k_norm.weight"] = np.ones(c.head_dim_kv, np.float32)
             t[f"{p}.post_attention_norm.weight"] = np.ones(c.n_embd, np.float32)
             t[f"{p}.post_ffw_norm.weight"] = np.ones(c.n_embd, np.float32)
-        if progress:
-            progress(L)
     t["output_norm.weight"] = np.ones(c.n_embd, np.float32)
     if gemma:   # tied: the embedding matrix is also the LM head (Q4_0)
-        t["token_embd.weight"] = _gen("token_embd.weight", (c.n_vocab, c.n_embd), seed, sigma, quantize_q4_0)
+        jobs.append(("token_embd.weight", (c.n_vocab, c.n_embd), quantize_q4_0))
     else:       # untied: Q8_0 output head, host-side embedding rows
-        t["output.weight"] = _gen("output.weight", (c.n_vocab, c.n_embd), seed, sigma, quantize_q8_0)
+        jobs.append(("output.weight", (c.n_vocab, c.n_embd), quantize_q8_0))
         t["token_embd.weight"] = SyntheticEmbedding(c.n_vocab, c.n_embd, seed, sigma)
+    workers = workers or min(16, os.cpu_count() or 1)
+    jobs.sort(key=lambda j: -j[1][0] * j[1][1])
+    with ThreadPoolExecutor(max_workers=workers) as ex:
+        for (name, _, _), qt in zip(jobs, ex.map(lambda j: _gen(j[0], j[1], seed, sigma, j[2]), jobs)):
+            t[name] = qt
     return t

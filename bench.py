@@ -1,0 +1,218 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized decode hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemma3-1b|llama3-8b]
+
+A "step" is one bs=1 greedy decode step (embedding fetch, all layers, fused LM-head GEMV+argmax,
+token read-back) of a random-init Q4_0 model of the named architecture, issued through the
+ADAMAH op surface exactly as the decode harness does.  W untimed steps follow the prompt
+prefill, then exactly K steps are timed between two device synchronisations; weights, KV
+cache and activations are resident in HBM before the timed region starts.
+
+One JSON line is printed.  Besides the contract keys it carries
+  roofline      the Q4_0 GEMV kernel at the Llama-3-8B gate+up shape (28672x4096), timed with HIP
+                events on the library's stream while cycling through > 1 GB of distinct weights
+  gemv_shapes   the same measurement for the other Llama-3-8B GEMV shapes
+  cpu_baseline  the NumPy restatement of the reference forward pass (float32 BLAS, pre-dequantised
+                weights) timed on this host on a bounded sample of the same workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+LLAMA_GEMV_SHAPES = [(28672, 4096), (14336, 4096), (6144, 4096), (4096, 4096), (4096, 14336)]
+METRIC = "decode tok/s at bs=1 + Q4 GEMV achieved HBM GB/s (% of MI355X peak)"
+
+
+def log(msg):
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def gemv_bytes(N, K):
+    """Algorithmic bytes of one Q4_0 GEMV launch: 18 B per 32 weights + x + y."""
+    return N * K * 18 // 32 + 4 * K + 4 * N
+
+
+def measure_gemv(gpu, A, shapes, rounds=6):
+    """HBM GB/s of the Q4_0 GEMV at each shape.  A 1.88 G-element Q4 map (1.06 GB of codes + scales)
+    is carved into as many distinct [N, K] matrices as fit; each round launches every one of them
+    once through a registered decode plan (one host call per round), so consecutive launches
+    never touch the same weights and the 256 MB last-level cache cannot serve them."""
+    wmap, amap, plan_id = 3, 5, 7
+    total = 16 * 28672 * 4096
+    rng = np.random.default_rng(123)
+    gpu.map_create_typed(wmap, A.DTYPE_Q4, 1, total, 32)
+    s = rng.uniform(0.001, 0.01, total // 32).astype(np.float16).astype(np.float32)
+    gpu.set_qparams(wmap, s, np.float32(-8.0) * s)
+    chunk = 1 << 26
+    for b in range(0, total // 2, chunk):
+        n = min(chunk, total // 2 - b)
+        gpu.scatter_q4_packed_contiguous(wmap, 2 * b, rng.integers(0, 256, n, dtype=np.uint8), n_locs=2 * n)
+    assert gpu.map_layout(wmap) == 1
+    kmax = max(k for _, k in shapes); nmax = max(n for n, _ in shapes)
+    gpu.set_dtype(A.DTYPE_F32)
+    gpu.map_create(amap, 1, kmax + nmax)
+    gpu.scatter_contiguous(amap, 0, rng.standard_normal(kmax).astype(np.float32))
+    a_h = gpu.upload_dev(np.array([0], np.uint32))[0]
+    c_h = gpu.upload_dev(np.array([kmax], np.uint32))[0]
+    out = {}
+    for N, K in shapes:
+        n_mats = total // (N * K)
+        ops = []
+        for i in range(n_mats):
+            b_h = gpu.upload_dev(np.array([i * N * K], np.uint32))[0]
+            ops.append(A.DecodePlanOp(kind=A.DECODE_OP_MATMUL_T_XQ4, map_id=amap, map_id2=wmap,
+                                      h0=a_h, h1=b_h, h2=c_h, u0=1, u1=K, u2=N, u3=1))
+        gpu.register_decode_plan(plan_id, ops)
+        gpu.decode_step(plan_id, 0, 0)
+        gpu.sync()
+        gpu.timer_begin()
+        for _ in range(rounds):
+            gpu.decode_step(plan_id, 0, 0)
+        ms = gpu.timer_end()
+        gpu.clear_decode_plan(plan_id)
+        us = ms * 1e3 / (rounds * n_mats)
+        gbps = gemv_bytes(N, K) / (us * 1e-6) / 1e9
+        out[f"{N}x{K}"] = {"us_per_launch": round(us, 3), "GB/s": round(gbps, 1),
+                           "frac": round(gbps / HBM_PEAK_GBPS, 4), "launches": rounds * n_mats,
+                           "distinct_MB": round(n_mats * N * K * 18 / 32 / 1e6)}
+        log(f"gemv {N}x{K}: {us:.2f} us/launch, {gbps:.0f} GB/s ({100 * gbps / HBM_PEAK_GBPS:.1f}% of peak)")
+    gpu.map_destroy(wmap)
+    gpu.map_destroy(amap)
+    return out
+
+
+def cpu_baseline(cfg, tensors, prompt, n_prompt=8, n_steps=48):
+    """The oracle's NumPy forward pass (reference forward_cpu restated) on this host's cores."""
+    from oracle.forward_cpu import CpuModel
+    from adam_amd.quant import QTensor
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+    except Exception:
+        threads = 1
+    deq = {n: (v.dequant() if isinstance(v, QTensor) else v) for n, v in tensors.items()}
+    m = CpuModel(cfg, deq, kv_cap=n_prompt + n_steps + 1, kv_fp16=True, acc64=False)
+    logits = None
+    for i, t in enumerate(prompt[:n_prompt]):
+        logits = m.forward(int(t), i)
+    t0 = time.perf_counter()
+    for s in range(n_steps):
+        nt = int(np.argmax(logits))
+        logits = m.forward(nt, n_prompt + s)
+    dt = time.perf_counter() - t0
+    return {"value": round(n_steps / dt, 3), "unit": "tok/s", "cores": int(threads), "kind": "port",
+            "sample": f"{n_steps} greedy decode steps after a {n_prompt}-token prompt, same model, NumPy "
+                      f"float32 BLAS on pre-dequantised weights ({os.cpu_count()} logical CPUs visible)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--workload", default="gemma3-1b", choices=["gemma3-1b", "llama3-8b"])
+    ap.add_argument("--prompt", type=int, default=None, help="prompt length (default 512 / 3840)")
+    ap.add_argument("--scheduler", default="level_batched", choices=["legacy", "level_batched"])
+    ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
+
+    from adam_amd import adamah as A, synth
+    from adam_amd.engine import DecodeEngine
+
+    gemma = args.workload == "gemma3-1b"
+    cfg = synth.gemma3_1b_config() if gemma else synth.llama3_8b_config()
+    n_prompt = args.prompt if args.prompt is not None else (512 if gemma else 4096 - 256)
+    kv_cap = n_prompt + args.warmup + args.steps + 8
+    t0 = time.perf_counter()
+    tensors = synth.make_model(cfg, seed=0, sigma=0.02)
+    log(f"synthesised {args.workload} weights in {time.perf_counter() - t0:.1f}s")
+
+    gpu = A.init()
+    t0 = time.perf_counter()
+    eng = DecodeEngine(gpu, cfg, tensors, A=A, kv_cap=kv_cap, kv_fp16=True,
+                       fusion_scheduler_mode=args.scheduler)
+    gpu.sync()
+    log(f"uploaded in {time.perf_counter() - t0:.1f}s; maps {sorted(eng._q4_sizes)}")
+
+    rng = np.random.default_rng(0)
+    prompt = [int(t) for t in rng.integers(0, cfg.n_vocab, n_prompt)]
+    eng.reset()
+    t0 = time.perf_counter()
+    for i, t in enumerate(prompt):
+        eng._forward(t, i, sample=(i == n_prompt - 1))
+    gpu.sync()
+    prefill_s = time.perf_counter() - t0
+    log(f"prefill {n_prompt} tokens (token by token): {prefill_s:.2f}s")
+
+    tokens, pos = [], n_prompt
+    for _ in range(args.warmup):
+        nt = eng.read_token(); tokens.append(nt)
+        eng._forward(nt, pos); pos += 1
+    gpu.sync()
+    gpu.reset_native_stats()
+    gpu.timer_begin()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        nt = eng.read_token(); tokens.append(nt)
+        eng._forward(nt, pos); pos += 1
+    gpu.sync()
+    wall = time.perf_counter() - t0
+    dev_ms = gpu.timer_end()
+    stats = gpu.get_native_stats()
+    tok_s = args.steps / wall
+    launches = stats["dispatch_count"] / max(1, args.steps)
+
+    c = cfg
+    q4_w = sum(v.size for v in tensors.values() if getattr(v, "kind", "") == "q4_0")
+    q8_w = sum(v.size for v in tensors.values() if getattr(v, "kind", "") == "q8_0")
+    kv_b = 2 * c.n_layer * c.n_head_kv * c.head_dim_kv * 2 * (n_prompt + args.warmup + args.steps // 2)
+    step_bytes = q4_w * 18 // 32 + q8_w * 34 // 32 + kv_b
+    ceiling = HBM_PEAK_GBPS * 1e9 / step_bytes
+
+    res = {
+        "metric": METRIC, "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(1e3 * wall / args.steps, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}-shape Q4_0 random-init, bs=1 greedy decode, "
+                               f"{n_prompt}-token random prompt, fp16 KV, tokens {n_prompt}..{pos}",
+                   "scheduler": args.scheduler, "launches_per_token": round(launches, 1)},
+        "device_ms_per_step": round(dev_ms / args.steps, 4),
+        "algorithmic_bytes_per_token": int(step_bytes),
+        "tok_s_at_hbm_peak": round(ceiling, 1), "frac_of_hbm_roofline": round(tok_s / ceiling, 4),
+        "prefill_tok_s": round(n_prompt / prefill_s, 1), "first_tokens": tokens[args.warmup:args.warmup + 8],
+    }
+    del eng
+
+    if not args.no_roofline:
+        shapes = measure_gemv(gpu, A, LLAMA_GEMV_SHAPES)
+        top = shapes["28672x4096"]
+        res["roofline"] = {"bound": "hbm", "achieved": top["GB/s"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                           "frac": top["frac"], "traffic": None,
+                           "kernel": "k_gemv_block<Q4_0, store> 28672x4096, "
+                                     f"{gemv_bytes(28672, 4096)} algorithmic B/launch"}
+        res["gemv_shapes"] = shapes
+    gpu.shutdown()
+
+    if not args.no_cpu_baseline:
+        t0 = time.perf_counter()
+        n_cpu = 48 if gemma else 4
+        res["cpu_baseline"] = cpu_baseline(cfg, tensors, prompt, n_prompt=8 if gemma else 2, n_steps=n_cpu)
+        log(f"cpu baseline {res['cpu_baseline']['value']} tok/s ({time.perf_counter() - t0:.1f}s incl. dequant)")
+
+    print(json.dumps(res), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -220,11 +220,21 @@ class NumpyAdamah:
         elif m.dtype == DTYPE_Q8:
             m.data[idx] = np.ascontiguousarray(data).view(np.uint8).reshape(-1)[:idx.size]
         else:
-            m.data[idx] = np.ascontiguousarray(data).view(np.float32).reshape(-1)[:idx.size]
+            m.data[idx] = self._kv_round(map_id, idx, np.ascontiguousarray(data).view(np.float32).reshape(-1)[:idx.size])
         m.cache.clear()
         return 0
 
     map_scatter = scatter
+
+    def _kv_round(self, map_id, idx, vals):
+        """Values written into a declared fp16 KV range are rounded to fp16 (see kv_cache_fp16)."""
+        kv = getattr(self, "_kv_fp16", {}).get(map_id)
+        if kv is None:
+            return vals
+        inside = (idx >= kv[0]) & (idx < kv[0] + kv[1])
+        out = np.array(vals, dtype=np.float32, copy=True)
+        out[inside] = out[inside].astype(np.float16).astype(np.float32)
+        return out
 
     def scatter_contiguous(self, map_id, start_pack, data, n_locs=None):
         arr = np.ascontiguousarray(data)
@@ -323,7 +333,7 @@ class NumpyAdamah:
             return 0
         locs = lr.view(np.uint32)[:n_locs].astype(np.int64)
         idx = (locs[:, None] * m.pack_size + np.arange(m.pack_size)).reshape(-1)
-        m.data[idx] = sr.view(np.float32)[:idx.size]
+        m.data[idx] = self._kv_round(map_id, idx, sr.view(np.float32)[:idx.size])
         return 0
 
     # ------------------------------------------------------------------ elementwise
@@ -541,24 +551,23 @@ class NumpyAdamah:
         dst = ((spec[:, 1] + dst_row_offset) * row_size)[:, None] + np.arange(row_size)
         if max(src.max(), dst.max()) >= m.n:
             self._fail(fn, ERR_INVALID)
-        vals = m.data[src].copy()
-        kv = getattr(self, "_kv_fp16", {}).get(map_id)
-        if kv is not None:
-            inside = (dst >= kv[0]) & (dst < kv[0] + kv[1])
-            vals = np.where(inside, vals.astype(np.float16).astype(np.float32), vals)
-        m.data[dst] = vals
+        m.data[dst] = self._kv_round(map_id, dst, m.data[src].copy())
 
     def map_row_copy_dev(self, map_id, copy_spec_handle, src_base_handle, n_copies, row_size):
         self.map_row_copy_offset_dev(map_id, copy_spec_handle, src_base_handle, 0, n_copies, row_size)
 
     def kv_cache_fp16(self, map_id, start, count):
         """Extension shared with the HIP library: elements [start, start+count) of a float32
-        map are a KV cache kept in fp16.  Rows copied into that range are rounded to fp16
-        (round-to-nearest-even); reads see the rounded values."""
-        self._map("adamah_kv_cache_fp16", map_id, DTYPE_F32)
+        map are a KV cache kept in fp16.  Values copied or scattered into that range are rounded
+        to fp16 (round-to-nearest-even), as is whatever the range holds when it is declared; reads
+        see the rounded values."""
+        m = self._map("adamah_kv_cache_fp16", map_id, DTYPE_F32)
+        if count == 0 or start + count > m.n:
+            self._fail("adamah_kv_cache_fp16", ERR_INVALID)
         if not hasattr(self, "_kv_fp16"):
             self._kv_fp16 = {}
         self._kv_fp16[map_id] = (int(start), int(count))
+        m.data[start:start + count] = m.data[start:start + count].astype(np.float16).astype(np.float32)
 
     # ------------------------------------------------------------------ matmuls
     def _mm(self, fn, ma, wfun, la, lb, lc, M, K, N, n_ops, transposed=True):
