@@ -121,6 +121,7 @@ _SIGS = {
     "adamah_hip_timer_begin": (i32, []), "adamah_hip_timer_end": (f32c, []),
     "adamah_hip_debug_dequant": (i32, [_U, u64, u64, pf32]),
     "adamah_hip_map_layout": (i32, [_U]),
+    "adamah_hip_stream_probe": (f32c, [u64, u64, _U, _U, _U]),
 }
 
 # Symbols the reference treats as optional feature flags (__init__.py:579-600, 713-832, 878-1100).
@@ -586,6 +587,13 @@ class Adamah:
         if ret != 0:
             raise RuntimeError(f"adamah_hip_debug_dequant failed with code {ret}")
         return out
+
+    def stream_probe(self, bytes_per_launch, pool_bytes, mode=0, wg_per_cu=8, launches=64):
+        """Average microseconds per launch of a plain read (mode 0) or copy (mode 1) kernel."""
+        us = float(self._lib.adamah_hip_stream_probe(bytes_per_launch, pool_bytes, mode, wg_per_cu, launches))
+        if us < 0:
+            raise RuntimeError(f"adamah_hip_stream_probe failed with code {int(us)}")
+        return us
 
     def map_layout(self, map_id):
         """0 = generic affine qparams, 1 = fp16-scale block plane (Q4_0 / Q8_0 recognised)."""

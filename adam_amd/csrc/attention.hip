@@ -246,28 +246,38 @@ k_attn_softmax_value(const float* data, float* out, const TV* vsrc, uint64_t v_s
   }
 }
 
-// Merge the split partials of one op: M = max m_s, L = sum l_s e^(m_s-M), o = sum o_s e^(m_s-M) / L.
+// Merge the split partials of one op: M = max m_s, w_s = e^(m_s-M), L = sum l_s w_s,
+// out = sum_s o_s w_s / L.  n_splits <= 1024.
 __global__ void __launch_bounds__(256)
 k_attn_combine(float* out, const float* partial, const uint32_t* __restrict__ lo, uint32_t value_dim,
                uint32_t n_splits, uint64_t n_elems) {
-  const uint32_t op = blockIdx.x, tid = threadIdx.x;
-  const float* pp = partial + (uint64_t)op * n_splits * (value_dim + 2);
+  __shared__ float w[1024];
+  __shared__ float red[4];
+  const uint32_t op = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t stride = value_dim + 2;
+  const float* pp = partial + (uint64_t)op * n_splits * stride;
   const uint64_t ob = lo[op];
   if (ob + value_dim > n_elems) return;
   float M = -9.99999968e+37f;
-  for (uint32_t s = 0; s < n_splits; s++) M = fmaxf(M, pp[(uint64_t)s * (value_dim + 2)]);
+  for (uint32_t s = tid; s < n_splits; s += 256u) M = fmaxf(M, pp[(uint64_t)s * stride]);
+  M = wave_max64(M);
+  if (lane == 0) red[wave] = M;
+  __syncthreads();
+  M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
   float L = 0.f;
-  for (uint32_t s = 0; s < n_splits; s++) {
-    const float* q = pp + (uint64_t)s * (value_dim + 2);
-    L += q[1] * expf(q[0] - M);
+  for (uint32_t s = tid; s < n_splits; s += 256u) {
+    const float e = expf(pp[(uint64_t)s * stride] - M);
+    w[s] = e;
+    L = fmaf(pp[(uint64_t)s * stride + 1], e, L);
   }
-  const float invL = 1.0f / L;
+  L = wave_sum64(L);
+  if (lane == 0) red[wave] = L;
+  __syncthreads();
+  const float invL = 1.0f / ((red[0] + red[1]) + (red[2] + red[3]));
   for (uint32_t d = tid; d < value_dim; d += 256u) {
     float o = 0.f;
-    for (uint32_t s = 0; s < n_splits; s++) {
-      const float* q = pp + (uint64_t)s * (value_dim + 2);
-      o = fmaf(q[2 + d], expf(q[0] - M), o);
-    }
+    for (uint32_t s = 0; s < n_splits; s++) o = fmaf(pp[(uint64_t)s * stride + 2 + d], w[s], o);
     out[ob + d] = o * invL;
   }
 }
@@ -338,7 +348,9 @@ int map_matmul_t_dev(uint32_t map_id, uint32_t ha, uint32_t hb, uint32_t hc, uin
              in_range(ch[op], N, m->n_elems) && (bh[op] - (kv ? m->kv_start : 0)) % vec == 0;
   }
   if (fast) {
-    const uint32_t rows_per_wg = std::max<uint32_t>(4u * (64u / lpr), std::min<uint32_t>(256u, cdiv(N, 2)));
+    // rows per workgroup: about two workgroups per CU over all ops, at least one wave step each
+    const uint32_t want_wg = std::max<uint32_t>(1u, cdiv(2u * (uint32_t)g.n_cu, n_ops));
+    const uint32_t rows_per_wg = std::max<uint32_t>(4u * (64u / lpr), std::min<uint32_t>(1024u, cdiv(N, want_wg)));
     dim3 g2(cdiv(N, rows_per_wg), n_ops);
     if (kv)
       k_scores_vec<__half, 8><<<g2, 256, 0, g.stream>>>(d, d, m->kv16, m->kv_start, la, lb, lc, K, N, lpr, rows_per_wg);
@@ -403,7 +415,7 @@ int map_attn_softmax_value_dev(uint32_t map_id, uint32_t hs, uint32_t hv, uint32
   uint32_t chunk = std::min<uint32_t>(ATT_CHUNK, std::max<uint32_t>(32u, cdiv(row_size, want_splits)));
   chunk = (chunk + 31u) & ~31u;
   const uint32_t n_splits = cdiv(row_size, chunk);
-  if ((uint64_t)n_ops * n_splits * (value_dim + 2) > g.attn_scratch_floats) return ADAMAH_ERR_INVALID;
+  if ((uint64_t)n_ops * n_splits * (value_dim + 2) > g.attn_scratch_floats || n_splits > 1024) return ADAMAH_ERR_INVALID;
   float* d = (float*)m->buf;
   dim3 grid(n_splits, n_ops);
   const bool kv = all_in_kv(m, hv, n_ops, (uint64_t)row_size * value_dim);

@@ -19,6 +19,7 @@
 #include "common.h"
 #include "../../include/adamah_hip.h"
 #include <algorithm>
+#include <stdlib.h>
 
 namespace adamah {
 
@@ -49,6 +50,20 @@ template <int N> __device__ __forceinline__ float ubyte_f32(uint32_t w) {
   else if (N == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(w));
   else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(w));
   return r;
+}
+
+#define DPP_ADD(v, ctrl, rmask)                                                                    \
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, rmask, 0xF, false))
+
+// Sum over the 64 lanes; the total is valid in lane 63.
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+  DPP_ADD(v, 0xB1, 0xF);    // quad_perm [1,0,3,2]
+  DPP_ADD(v, 0x4E, 0xF);    // quad_perm [2,3,0,1]
+  DPP_ADD(v, 0x141, 0xF);   // row_half_mirror
+  DPP_ADD(v, 0x140, 0xF);   // row_mirror: every lane of a 16-lane row holds the row sum
+  DPP_ADD(v, 0x142, 0xA);   // row_bcast15 into rows 1 and 3
+  DPP_ADD(v, 0x143, 0xC);   // row_bcast31 into rows 2 and 3
+  return v;
 }
 
 // sum_j code[j] * x[j] for the 8 nibbles of one word; x = two float4 (elements 0..7)
@@ -162,19 +177,16 @@ k_gemv_block(const float* act, float* act_out, const uint8_t* __restrict__ W,
       }
 #pragma unroll
       for (int i = 0; i < ROWS; i++) {
-        const float y = wave_sum(acc[i]);
+        const float y = wave_sum_to_lane63(acc[i]);   // total valid in lane 63 only
         const uint32_t row = r + i;
-        if (row < row1) {
-          if (EPI == EPI_STORE) {
-            if (lane == 0) act_out[(uint64_t)lc[0] + row] = y;
-          } else if (better(y, row, best_v, best_i)) {
-            best_v = y; best_i = row;
-          }
+        if (row < row1 && lane == 63) {
+          if (EPI == EPI_STORE) act_out[(uint64_t)lc[0] + row] = y;
+          else if (better(y, row, best_v, best_i)) { best_v = y; best_i = row; }
         }
       }
     }
     if (EPI == EPI_ARGMAX) {
-      if (lane == 0) { red_v[wave] = best_v; red_i[wave] = best_i; }
+      if (lane == 63) { red_v[wave] = best_v; red_i[wave] = best_i; }
       __syncthreads();
       if (tid == 0) {
         float bv = red_v[0]; uint32_t bi = red_i[0];
@@ -184,6 +196,149 @@ k_gemv_block(const float* act, float* act_out, const uint8_t* __restrict__ W,
         act_out[lval[grp]] = bv;
       }
       __syncthreads();
+    }
+  }
+}
+
+// ---- register-resident activation variant --------------------------------------------------
+// Each lane keeps the 32 activations (and their sum) of its NB blocks in registers for the whole
+// workgroup lifetime, so the row loop touches no LDS: per row it issues NB 16-byte code loads and
+// NB scale loads, converts and FMAs.  KS waves share a row when K is long (each takes a slice of
+// 64*NB blocks) and meet through 64 bytes of LDS once per row step.
+typedef float float4_u __attribute__((ext_vector_type(4), aligned(4)));
+
+template <int FMT, int EPI, int NB, int KS>
+__global__ void __launch_bounds__(256)
+k_gemv_regx(const float* act, float* act_out, const uint8_t* __restrict__ W, const float2* __restrict__ qp,
+            const __half* __restrict__ d16, const uint32_t* __restrict__ la, const uint32_t* __restrict__ lb,
+            const uint32_t* __restrict__ lc, const uint32_t* __restrict__ lidx, const uint32_t* __restrict__ lval,
+            uint32_t K, uint32_t N, uint32_t rows_per_wg) {
+  constexpr bool Q4 = (FMT == FMT_Q4_B16 || FMT == FMT_Q4_AFF);
+  constexpr bool B16 = (FMT == FMT_Q4_B16 || FMT == FMT_Q8_B16);
+  constexpr float OFF = Q4 ? 8.0f : 128.0f;
+  constexpr int R = 4;             // rows in flight per wave
+  constexpr int G = 4 / KS;        // row groups per workgroup
+  __shared__ float part[G][KS][R];
+  __shared__ float red_v[4];
+  __shared__ uint32_t red_i[4];
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t kpart = wave % KS, grp = wave / KS;
+  const uint32_t nblk = K >> 5;
+  const uint64_t a = la[0], gbase = (uint64_t)lb[0] >> 5;
+
+  uint32_t blk[NB];
+  float x[NB][32], sx[NB];
+#pragma unroll
+  for (int i = 0; i < NB; i++) {
+    blk[i] = (kpart * NB + i) * 64u + lane;
+    const bool valid = blk[i] < nblk;
+    const float4_u* px = (const float4_u*)(act + a + (uint64_t)(valid ? blk[i] : 0u) * 32u);
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      float4_u v = px[j];
+      if (!valid) v = (float4_u)(0.f);
+      x[i][4 * j] = v.x; x[i][4 * j + 1] = v.y; x[i][4 * j + 2] = v.z; x[i][4 * j + 3] = v.w;
+      s += (v.x + v.y) + (v.z + v.w);
+    }
+    sx[i] = s;
+    if (!valid) blk[i] = nblk - 1;      // keep addresses in range; the zero activations cancel the block
+  }
+
+  const uint32_t row_begin = blockIdx.x * rows_per_wg;
+  const uint32_t row_end = min(N, row_begin + rows_per_wg);
+  const uint32_t iters = (rows_per_wg + G * R - 1) / (G * R);
+  float best_v = NEG_FLT_MAX;
+  uint32_t best_i = INVALID_IDX;
+
+  for (uint32_t it = 0; it < iters; it++) {
+    const uint32_t r0 = row_begin + it * (G * R) + grp * R;
+    float acc[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) acc[j] = 0.f;
+    if (r0 < row_end) {
+#pragma unroll
+      for (int i = 0; i < NB; i++) {
+        uint4 q0[R], q1[R];
+        float sc[R], zp[R];
+#pragma unroll
+        for (int j = 0; j < R; j++) {
+          const uint32_t row = min(r0 + j, row_end - 1);
+          const uint64_t gidx = gbase + (uint64_t)row * nblk + blk[i];
+          if (Q4) {
+            q0[j] = *(const uint4*)(W + (gidx << 4));
+          } else {
+            q0[j] = *(const uint4*)(W + (gidx << 5));
+            q1[j] = *(const uint4*)(W + (gidx << 5) + 16);
+          }
+          if (B16) { sc[j] = __half2float(d16[gidx]); zp[j] = 0.f; }
+          else { const float2 p = qp[gidx]; sc[j] = p.x; zp[j] = p.y; }
+        }
+#pragma unroll
+        for (int j = 0; j < R; j++) {
+          float d = 0.f;
+          const float* xv = x[i];
+          if (Q4) {
+            const uint32_t w[4] = {q0[j].x, q0[j].y, q0[j].z, q0[j].w};
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+              const uint32_t lo = w[u] & 0x0F0F0F0Fu, hi = (w[u] >> 4) & 0x0F0F0F0Fu;
+              d = fmaf(ubyte_f32<0>(lo), xv[8 * u + 0], d); d = fmaf(ubyte_f32<0>(hi), xv[8 * u + 1], d);
+              d = fmaf(ubyte_f32<1>(lo), xv[8 * u + 2], d); d = fmaf(ubyte_f32<1>(hi), xv[8 * u + 3], d);
+              d = fmaf(ubyte_f32<2>(lo), xv[8 * u + 4], d); d = fmaf(ubyte_f32<2>(hi), xv[8 * u + 5], d);
+              d = fmaf(ubyte_f32<3>(lo), xv[8 * u + 6], d); d = fmaf(ubyte_f32<3>(hi), xv[8 * u + 7], d);
+            }
+          } else {
+            const uint32_t w[8] = {q0[j].x, q0[j].y, q0[j].z, q0[j].w, q1[j].x, q1[j].y, q1[j].z, q1[j].w};
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+              d = fmaf(ubyte_f32<0>(w[u]), xv[4 * u + 0], d); d = fmaf(ubyte_f32<1>(w[u]), xv[4 * u + 1], d);
+              d = fmaf(ubyte_f32<2>(w[u]), xv[4 * u + 2], d); d = fmaf(ubyte_f32<3>(w[u]), xv[4 * u + 3], d);
+            }
+          }
+          if (B16) acc[j] = fmaf(sc[j], fmaf(-OFF, sx[i], d), acc[j]);
+          else acc[j] = fmaf(sc[j], d, fmaf(zp[j], sx[i], acc[j]));
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < R; j++) acc[j] = wave_sum_to_lane63(acc[j]);
+    if (KS > 1) {
+      if (lane == 63) {
+#pragma unroll
+        for (int j = 0; j < R; j++) part[grp][kpart][j] = acc[j];
+      }
+      __syncthreads();
+    }
+    // one lane per row group finishes the rows: lane 63 of the kpart-0 wave
+    if (kpart == 0 && lane == 63 && r0 < row_end) {
+#pragma unroll
+      for (int j = 0; j < R; j++) {
+        float y = acc[j];
+        if (KS > 1) {
+          y = part[grp][0][j];
+#pragma unroll
+          for (int p = 1; p < KS; p++) y += part[grp][p][j];
+        }
+        const uint32_t row = r0 + j;
+        if (row < row_end) {
+          if (EPI == EPI_STORE) act_out[(uint64_t)lc[0] + row] = y;
+          else if (better(y, row, best_v, best_i)) { best_v = y; best_i = row; }
+        }
+      }
+    }
+    if (KS > 1) __syncthreads();
+  }
+  if (EPI == EPI_ARGMAX) {
+    if (lane == 63) { red_v[wave] = best_v; red_i[wave] = best_i; }   // waves with kpart != 0 hold INVALID
+    __syncthreads();
+    if (tid == 0) {
+      float bv = red_v[0]; uint32_t bi = red_i[0];
+      for (int w = 1; w < 4; w++)
+        if (better(red_v[w], red_i[w], bv, bi)) { bv = red_v[w]; bi = red_i[w]; }
+      act_out[lidx[blockIdx.x]] = (float)(bi == INVALID_IDX ? 0u : bi);
+      act_out[lval[blockIdx.x]] = bv;
     }
   }
 }
@@ -316,7 +471,7 @@ struct XqArgs {
 static bool block_path_ok(const Map* ma, const Map* mw, uint32_t ha, uint32_t hb, uint32_t K, uint32_t N,
                           uint64_t* a_out, uint64_t* b_out) {
   if (mw->group_size != 32 || mw->pack_size != 1 || ma->pack_size != 1) return false;
-  if (K == 0 || (K & 31u) || (uint64_t)K * 4 + (K >> 5) * 4 > 64000) return false;
+  if (K == 0 || (K & 31u) || K > 16384) return false;
   const uint32_t* a = res_host(ha, 1);
   const uint32_t* b = res_host(hb, 1);
   if (!a || !b) return false;
@@ -332,13 +487,18 @@ static int fmt_of(const Map* mw, uint64_t b, uint64_t n_w) {
   return q4 ? (b16 ? FMT_Q4_B16 : FMT_Q4_AFF) : (b16 ? FMT_Q8_B16 : FMT_Q8_AFF);
 }
 
+static int tuning(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return v ? atoi(v) : dflt;
+}
+
 template <int EPI>
 static int launch_block(int fmt, const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb,
                         const uint32_t* lc, const uint32_t* lidx, const uint32_t* lval, uint32_t K, uint32_t N,
                         uint32_t rows_per_group) {
   const uint32_t n_groups = cdiv(N, rows_per_group);
   const size_t smem = (size_t)K * 4 + (size_t)(K >> 5) * 4;
-  const uint32_t per_cu = smem > 40000 ? 2 : 4;
+  const uint32_t per_cu = (uint32_t)tuning("ADAMAH_GEMV_PERCU", smem > 40000 ? 2 : 4);
   const uint32_t grid = std::min<uint32_t>(n_groups, (uint32_t)g.n_cu * per_cu);
   float* act = (float*)ma->buf;
 #define LAUNCH(F)                                                                                              \
@@ -353,6 +513,37 @@ static int launch_block(int fmt, const Map* ma, const Map* mw, const uint32_t* l
 #undef LAUNCH
   count_launch();
   return check_launch();
+}
+
+// Register-resident variant: K up to 16384.  For EPI_STORE rows_per_wg is chosen here; for
+// EPI_ARGMAX one workgroup handles one argmax group (rows_per_wg = rows_per_group).
+template <int EPI, int FMT>
+static int launch_regx_fmt(const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb, const uint32_t* lc,
+                           const uint32_t* lidx, const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rows_per_wg) {
+  float* act = (float*)ma->buf;
+  const uint32_t nblk = K >> 5;
+  const uint32_t grid = cdiv(N, rows_per_wg);
+#define RX(NB, KS)                                                                                             \
+  k_gemv_regx<FMT, EPI, NB, KS><<<grid, 256, 0, g.stream>>>(act, act, mw->buf, mw->qp, mw->d16, la, lb, lc, lidx, \
+                                                            lval, K, N, rows_per_wg)
+  if (nblk <= 64) RX(1, 1);
+  else if (nblk <= 128) RX(2, 1);
+  else if (nblk <= 256) RX(2, 2);
+  else RX(2, 4);
+#undef RX
+  count_launch();
+  return check_launch();
+}
+template <int EPI>
+static int launch_regx(int fmt, const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb,
+                       const uint32_t* lc, const uint32_t* lidx, const uint32_t* lval, uint32_t K, uint32_t N,
+                       uint32_t rows_per_wg) {
+  switch (fmt) {
+    case FMT_Q4_B16: return launch_regx_fmt<EPI, FMT_Q4_B16>(ma, mw, la, lb, lc, lidx, lval, K, N, rows_per_wg);
+    case FMT_Q4_AFF: return launch_regx_fmt<EPI, FMT_Q4_AFF>(ma, mw, la, lb, lc, lidx, lval, K, N, rows_per_wg);
+    case FMT_Q8_B16: return launch_regx_fmt<EPI, FMT_Q8_B16>(ma, mw, la, lb, lc, lidx, lval, K, N, rows_per_wg);
+    default: return launch_regx_fmt<EPI, FMT_Q8_AFF>(ma, mw, la, lb, lc, lidx, lval, K, N, rows_per_wg);
+  }
 }
 
 int op_matmul_t_xq(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t ha, uint32_t hb, uint32_t hc,
@@ -373,8 +564,20 @@ int op_matmul_t_xq(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t h
     if (ch && !in_range(ch[op], (uint64_t)M * N, ma->n_elems)) return ADAMAH_ERR_INVALID;
   }
   uint64_t a0 = 0, b0 = 0;
-  if (transposed && M == 1 && n_ops == 1 && ch && block_path_ok(ma, mw, ha, hb, K, N, &a0, &b0))
-    return launch_block<EPI_STORE>(fmt_of(mw, b0, (uint64_t)N * K), ma, mw, la, lb, lc, nullptr, nullptr, K, N, 16);
+  if (transposed && M == 1 && n_ops == 1 && ch && block_path_ok(ma, mw, ha, hb, K, N, &a0, &b0)) {
+    const int fmt = fmt_of(mw, b0, (uint64_t)N * K);
+    // long rows: activations in registers, waves share a row; otherwise activations staged in LDS
+    if (tuning("ADAMAH_GEMV_IMPL", K > 8192 ? 1 : 0) == 1) {
+      const uint32_t ks = K <= 4096 ? 1 : K <= 8192 ? 2 : 4;
+      const uint32_t step = (4 / ks) * 4;                       // rows one workgroup pass covers
+      const uint32_t passes = (uint32_t)tuning("ADAMAH_GEMV_PASSES", 2);
+      return launch_regx<EPI_STORE>(fmt, ma, mw, la, lb, lc, nullptr, nullptr, K, N, step * std::max(1u, passes));
+    }
+    if ((uint64_t)K * 4 + (K >> 5) * 4 > 64000) goto generic;
+    return launch_block<EPI_STORE>(fmt, ma, mw, la, lb, lc, nullptr, nullptr, K, N,
+                                   (uint32_t)tuning("ADAMAH_GEMV_RPG", 16));
+  }
+generic:
   dim3 grid(cdiv(N, 4), M, n_ops);
   float* act = (float*)ma->buf;
   const bool q4 = dtype == DTYPE_Q4;
@@ -407,8 +610,12 @@ int op_matvec_argmax(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t
   uint64_t a0 = 0, b0 = 0;
   int r;
   if (locs_ok && block_path_ok(ma, mw, ha, hb, K, N, &a0, &b0)) {
-    r = launch_block<EPI_ARGMAX>(fmt_of(mw, b0, (uint64_t)N * K), ma, mw, la, lb, nullptr, lidx, lval, K, N,
-                                 rows_per_group);
+    if (tuning("ADAMAH_GEMV_IMPL", K > 8192 ? 1 : 0) == 1)
+      r = launch_regx<EPI_ARGMAX>(fmt_of(mw, b0, (uint64_t)N * K), ma, mw, la, lb, nullptr, lidx, lval, K, N,
+                                  rows_per_group);
+    else
+      r = launch_block<EPI_ARGMAX>(fmt_of(mw, b0, (uint64_t)N * K), ma, mw, la, lb, nullptr, lidx, lval, K, N,
+                                   rows_per_group);
   } else {
     const uint32_t *ah = res_host(ha, 1), *bh = res_host(hb, 1);
     if (ah && !in_range(ah[0], K, ma->n_elems)) return ADAMAH_ERR_INVALID;

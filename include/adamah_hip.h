@@ -183,6 +183,10 @@ int adamah_hip_timer_begin(void);
 float adamah_hip_timer_end(void);
 /* Dequantise elements [start, start+count) of a Q4/Q8 map with the GEMV kernels' unpack code. */
 int adamah_hip_debug_dequant(uint32_t map_id, uint64_t start, uint64_t count, float* out);
+/* Streaming calibration: average microseconds per launch of a plain read (mode 0) or copy (mode 1)
+ * of bytes_per_launch bytes, walking a pool_bytes buffer; negative = error code. */
+float adamah_hip_stream_probe(uint64_t bytes_per_launch, uint64_t pool_bytes, uint32_t mode, uint32_t wg_per_cu,
+                              uint32_t launches);
 /* 0 = affine qparams only, 1 = fp16-scale block plane in use for the whole map, <0 = error. */
 int adamah_hip_map_layout(uint32_t map_id);
 
