@@ -29,6 +29,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 LLAMA_GEMV_SHAPES = [(28672, 4096), (14336, 4096), (6144, 4096), (4096, 4096), (4096, 14336)]
+# HBM bytes per 28672x4096 Q4_0 GEMV launch from rocprofv3 --pmc (profiles/gemv_q4_0_llama_shapes_pmc_
+# fetch_write.txt): FETCH_SIZE 32,365.3 counts x 1.999 KiB (factor from a plain read kernel of known
+# size) + WRITE_SIZE 112.1 counts x 1.000 KiB (factor from a plain copy kernel).
+GEMV_TRAFFIC_BYTES = int(32365.3 * 1.999 * 1024 + 112.1 * 1.000 * 1024)
 METRIC = "decode tok/s at bs=1 + Q4 GEMV achieved HBM GB/s (% of MI355X peak)"
 
 
@@ -122,6 +126,9 @@ def main():
     ap.add_argument("--workload", default="gemma3-1b", choices=["gemma3-1b", "llama3-8b"])
     ap.add_argument("--prompt", type=int, default=None, help="prompt length (default 512 / 3840)")
     ap.add_argument("--scheduler", default="level_batched", choices=["legacy", "level_batched"])
+    ap.add_argument("--only", default=None, choices=["gemv", "probe"],
+                    help="gemv: just the GEMV roofline leg; probe: plain read/copy kernels of known size "
+                         "(reference points for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -130,6 +137,22 @@ def main():
 
     from adam_amd import adamah as A, synth
     from adam_amd.engine import DecodeEngine
+
+    if args.only:
+        gpu = A.init()
+        if args.only == "gemv":
+            out = {"gemv_shapes": measure_gemv(gpu, A, LLAMA_GEMV_SHAPES[:1] + LLAMA_GEMV_SHAPES[3:], rounds=3)}
+        else:
+            nbytes = gemv_bytes(28672, 4096) // 4096 * 4096
+            pool = nbytes * 16
+            out = {"probe_bytes_per_launch": nbytes,
+                   "read_us": round(gpu.stream_probe(nbytes, pool, 0, 32, 48), 3),
+                   "copy_us": round(gpu.stream_probe(nbytes, pool, 1, 4, 48), 3)}
+            out["read_GB/s"] = round(nbytes / out["read_us"] / 1e3, 1)
+            out["copy_GB/s"] = round(2 * nbytes / out["copy_us"] / 1e3, 1)
+        gpu.shutdown()
+        print(json.dumps(out), flush=True)
+        return
 
     gemma = args.workload == "gemma3-1b"
     cfg = synth.gemma3_1b_config() if gemma else synth.llama3_8b_config()
@@ -199,7 +222,7 @@ def main():
         shapes = measure_gemv(gpu, A, LLAMA_GEMV_SHAPES)
         top = shapes["28672x4096"]
         res["roofline"] = {"bound": "hbm", "achieved": top["GB/s"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                           "frac": top["frac"], "traffic": None,
+                           "frac": top["frac"], "traffic": GEMV_TRAFFIC_BYTES,
                            "kernel": "k_gemv_block<Q4_0, store> 28672x4096, "
                                      f"{gemv_bytes(28672, 4096)} algorithmic B/launch"}
         res["gemv_shapes"] = shapes
