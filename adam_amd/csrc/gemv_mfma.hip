@@ -1,0 +1,322 @@
+// Q4 dequant-GEMV with the 4x4x4 int8 matrix instruction used as a dot-product unit.
+//
+// Semantics as in gemv_q.hip (reference: shaders/src/f32/map_matvec_t_xq4.comp:49-135; argmax tail
+// map_matvec_argmax_t_xq4.comp:66-158, map_argmax_pairs.comp:34-67).
+//
+// Why not plain VALU: with one convert and one FMA per weight (or one v_dot2 per two weights plus
+// unpacking) the kernel keeps the vector ALUs busy for most of its run time: it is bound by
+// instruction issue, not by HBM.  v_mfma_i32_4x4x4_16B_i8 multiplies sixteen independent 4x4x4
+// blocks per instruction; block g lives in lanes 4g..4g+3, operand A row i and operand B column j
+// both come from lane 4g+i / 4g+j (four k values, one byte each), and lane 4g+j receives column j
+// of the result.  Used here as
+//   B column j = four 4-bit codes of lane j's own weight row, one per byte:  w & 0x0F0F0F0F and
+//                (w >> 4) & 0x0F0F0F0F are all the unpacking there is (3 VALU ops per 8 weights);
+//   A row i    = digit i of the matching four activations, which are held as 22-bit fixed point
+//                x * 2^e = d0 * 2^14 + d1 * 2^7 + d2  (d0 signed, d1, d2 in 0..127; e per 32-block
+//                from the block's max |x|), rows 0..2 used, row 3 repeats row 0;
+// so every lane ends up with  sum q * d_i  for its own row and its own 32-weight block, exactly, in
+// int32.  The lane recombines the digits, subtracts the format's zero point through the precomputed
+// integer block sum of the activations, converts once to float and applies scale * 2^-e.
+// Everything up to that conversion is exact integer arithmetic; the activations keep 21 bits below
+// their block maximum.
+//
+// Lane = 4 * column + row: a wave works on bundles of four rows, the 16 columns are consecutive
+// 32-weight blocks.  Per step every lane loads four 16-byte blocks of its row (the wave covers
+// 4 rows x 2048 weights) and the next step's loads are issued before the current step is computed.
+#include "gemv_common.h"
+#include <algorithm>
+
+namespace adamah {
+
+typedef int i4_t __attribute__((ext_vector_type(4)));
+typedef float f4u_t __attribute__((ext_vector_type(4), aligned(4)));
+
+enum { MF_U = 4 };   // 16-byte blocks per lane and step
+
+// LDS layout: 128 bytes per activation block = 8 chunks of 16 bytes.  Chunk 2*d + h holds digit d of
+// words 2h, 2h+1 as {even(2h), odd(2h), even(2h+1), odd(2h+1)} (even/odd = elements 0,2,4,6 / 1,3,5,7 of
+// the 8-element word, one byte each, matching the byte order of the unpacked codes); chunk 6 holds
+// {zero-point term, 2^-e, sum(x) as float, 0}.  Chunk c of block b sits at position c ^ (b & 7), which
+// spreads the 16 blocks a wave reads at once over all banks.
+__device__ __forceinline__ uint32_t chunk_off(uint32_t c, uint32_t blk) { return ((c ^ (blk & 7u)) << 4); }
+
+struct PreM {
+  uint4 q[MF_U];
+  __half h[MF_U];
+  float2 p[MF_U];
+};
+
+template <int FMT, int EPI, bool RAGGED>
+__global__ void __launch_bounds__(1024)
+k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, const float2* __restrict__ qp,
+            const __half* __restrict__ d16, uint32_t a, uint32_t b_off, uint32_t c_out,
+            const uint32_t* __restrict__ lidx, const uint32_t* __restrict__ lval, uint32_t K, uint32_t N,
+            uint32_t rows_per_group, uint32_t n_groups) {
+  constexpr bool B16 = (FMT == FMT_Q4_B16);
+  extern __shared__ uint4 smem_u4[];
+  uint8_t* xs = (uint8_t*)smem_u4;                    // nblk * 128 bytes
+  __shared__ float red_f[16];
+  __shared__ uint32_t red_i[16];
+  const uint32_t nblk = K >> 5;
+  const uint32_t C = (nblk + 63u) >> 6;               // steps per row bundle
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, nthr = blockDim.x, nwav = nthr >> 6;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t l = lane & 3u, bcol = lane >> 2;      // row in bundle, block column 0..15
+  const uint64_t gbase = (uint64_t)b_off >> 5;
+
+  // ---- this wave's rows: store = contiguous balanced share of the 4-row bundles (waves that share
+  // a SIMD, w % 4, take neighbouring shares so that every SIMD gets the same load); argmax = the
+  // workgroup takes whole argmax groups, its waves interleave the bundles of a group ------------
+  uint32_t grp = blockIdx.x, first, stride, seg_end;
+  if (EPI == EPI_STORE) {
+    const uint32_t slot = (wave & 3u) * (nwav >> 2) + (wave >> 2);
+    const uint64_t n_q = (N + 3u) / 4u, gw = (uint64_t)blockIdx.x * nwav + slot, wt = (uint64_t)gridDim.x * nwav;
+    first = (uint32_t)(gw * n_q / wt) * 4u;
+    seg_end = min(N, (uint32_t)((gw + 1) * n_q / wt) * 4u);
+    stride = 4u;
+  } else {
+    first = grp * rows_per_group + wave * 4u;
+    seg_end = min(N, (grp + 1) * rows_per_group);
+    stride = 4u * nwav;
+  }
+
+  auto load = [&](PreM& R, uint32_t row0, uint32_t chunk, uint32_t end) {
+    const uint32_t row = min(row0 + l, end - 1u);
+    const uint64_t g0 = gbase + (uint64_t)row * nblk + chunk * 64u + bcol;
+#pragma unroll
+    for (uint32_t u = 0; u < MF_U; u++) {
+      uint64_t gi = g0 + u * 16u;
+      if (RAGGED) gi = gbase + (uint64_t)row * nblk + min(chunk * 64u + u * 16u + bcol, nblk - 1u);
+      R.q[u] = *(const uint4*)(W + (gi << 4));
+      if (B16) R.h[u] = d16[gi];
+      else R.p[u] = qp[gi];
+    }
+  };
+
+  PreM A, B;
+  if (first < seg_end) load(A, first, 0, seg_end);   // in flight while the activations are staged
+
+  // ---- activations -> fixed-point digits; one 8-element word per thread, four threads per block --
+  {
+    const uint32_t nw = nblk * 4u;
+    for (uint32_t i0 = 0; i0 < nw; i0 += nthr) {
+      const uint32_t i = i0 + tid;
+      const bool live = i < nw;             // uniform over a thread quad
+      const f4u_t* p = (const f4u_t*)(act + a + (uint64_t)min(i, nw - 1u) * 8u);
+      const f4u_t v0 = p[0], v1 = p[1];
+      const float x[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+      float m = 0.f, poison = 0.f;          // poison turns NaN as soon as one element is Inf or NaN
+#pragma unroll
+      for (int k = 0; k < 8; k++) { m = fmaxf(m, fabsf(x[k])); poison = fmaf(x[k], 0.f, poison); }
+      m = fmaxf(m, __shfl_xor(m, 1, 64)); m = fmaxf(m, __shfl_xor(m, 2, 64));
+      poison += __shfl_xor(poison, 1, 64); poison += __shfl_xor(poison, 2, 64);
+      const uint32_t e = (__float_as_uint(m) >> 23) & 0xFFu;
+      float s = 1.f, fs = 1.f;              // |x * s| < 2^21 when the block is finite and not tiny
+      if (e >= 21u && e <= 254u) { s = __uint_as_float((274u - e) << 23); fs = __uint_as_float((e - 20u) << 23); }
+      if (poison != poison) fs = poison;    // the block's result is NaN, as it would be in float arithmetic
+      int d0[8], d1[8], d2[8], sx = 0;
+#pragma unroll
+      for (int k = 0; k < 8; k++) {
+        int xi = (e >= 21u && e <= 254u) ? (int)rintf(x[k] * s) : 0;
+        xi = min(max(xi, -(1 << 21)), (1 << 21) - 1);
+        sx += xi;
+        d0[k] = xi >> 14; d1[k] = (xi >> 7) & 127; d2[k] = xi & 127;
+      }
+      sx += __shfl_xor(sx, 1, 64); sx += __shfl_xor(sx, 2, 64);
+      if (live) {
+        const uint32_t blk = i >> 2, j = i & 3u;
+        uint8_t* bp = xs + (size_t)blk * 128u;
+        auto pack = [](const int* d, int o) {
+          return (uint32_t)(d[o] & 255) | ((uint32_t)(d[o + 2] & 255) << 8) | ((uint32_t)(d[o + 4] & 255) << 16) |
+                 ((uint32_t)(d[o + 6] & 255) << 24);
+        };
+        const uint32_t h = j >> 1, wo = (j & 1u) * 8u;
+        *(uint2*)(bp + chunk_off(0u + h, blk) + wo) = make_uint2(pack(d0, 0), pack(d0, 1));
+        *(uint2*)(bp + chunk_off(2u + h, blk) + wo) = make_uint2(pack(d1, 0), pack(d1, 1));
+        *(uint2*)(bp + chunk_off(4u + h, blk) + wo) = make_uint2(pack(d2, 0), pack(d2, 1));
+        if (j == 0) {
+          uint4 prm;
+          prm.x = (uint32_t)(B16 ? 8 * sx : 0);              // zero-point term of the block format, integer
+          prm.y = __float_as_uint(fs);
+          prm.z = __float_as_uint((float)sx * fs);           // sum of the block's activations (affine format)
+          prm.w = 0;
+          *(uint4*)(bp + chunk_off(6u, blk)) = prm;
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  uint32_t nib = 0x0F0F0F0Fu;
+  asm volatile("" : "+s"(nib));             // opaque, so it stays in a register instead of a literal per use
+  const uint32_t dig = l < 3u ? l : 0u;     // lane 3 of a block repeats digit 0, its result row is unused
+  const uint32_t x_off0 = chunk_off(2u * dig, bcol), x_off1 = chunk_off(2u * dig + 1u, bcol), p_off = chunk_off(6u, bcol);
+  float acc = 0.f;
+  float best_v = NEG_FLT_MAX;
+  uint32_t best_i = INVALID_IDX;
+
+  auto compute = [&](const PreM& R, uint32_t row0, uint32_t chunk, uint32_t end) {
+    const uint8_t* base = xs + (size_t)(chunk * 64u + bcol) * 128u;
+    uint4 xa[MF_U], xb[MF_U], prm[MF_U];
+    bool valid[MF_U];
+    i4_t d[MF_U];
+#pragma unroll
+    for (uint32_t u = 0; u < MF_U; u++) {
+      valid[u] = true;
+      const uint8_t* bp = base + u * 2048u;
+      if (RAGGED) {
+        const uint32_t blk_raw = chunk * 64u + u * 16u + bcol;
+        valid[u] = blk_raw < nblk;
+        bp = xs + (size_t)min(blk_raw, nblk - 1u) * 128u;
+      }
+      xa[u] = *(const uint4*)(bp + x_off0); xb[u] = *(const uint4*)(bp + x_off1); prm[u] = *(const uint4*)(bp + p_off);
+      d[u] = (i4_t){0, 0, 0, 0};
+    }
+    // eight dependent matrix instructions per block; the four blocks of a step are interleaved so that
+    // consecutive instructions are independent
+#define MF_STEP(XV, WV, SH)                                                                                   \
+  _Pragma("unroll") for (uint32_t u = 0; u < MF_U; u++)                                                       \
+      d[u] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)XV, (int)(((WV) >> SH) & nib), d[u], 0, 0, 0)
+    MF_STEP(xa[u].x, R.q[u].x, 0); MF_STEP(xa[u].y, R.q[u].x, 4);
+    MF_STEP(xa[u].z, R.q[u].y, 0); MF_STEP(xa[u].w, R.q[u].y, 4);
+    MF_STEP(xb[u].x, R.q[u].z, 0); MF_STEP(xb[u].y, R.q[u].z, 4);
+    MF_STEP(xb[u].z, R.q[u].w, 0); MF_STEP(xb[u].w, R.q[u].w, 4);
+#undef MF_STEP
+#pragma unroll
+    for (uint32_t u = 0; u < MF_U; u++) {
+      // |d0| <= 15*128*32, so the recombination stays below 2^31
+      const int sq = d[u][0] * 16384 + d[u][1] * 128 + d[u][2];
+      // a block past the end of the row (ragged K) was clamped to a valid address: drop what it read
+      const float fsb = valid[u] ? __uint_as_float(prm[u].y) : 0.f, sxb = valid[u] ? __uint_as_float(prm[u].z) : 0.f;
+      if (B16) {
+        const float sc = valid[u] ? __half2float(R.h[u]) : 0.f;
+        acc = fmaf(sc, (float)(sq - (int)prm[u].x) * fsb, acc);
+      } else {
+        const float sc = valid[u] ? R.p[u].x : 0.f, zp = valid[u] ? R.p[u].y : 0.f;
+        acc = fmaf(sc, (float)sq * fsb, fmaf(zp, sxb, acc));
+      }
+    }
+    if (chunk == C - 1u) {   // row bundle complete: sum the 16 lanes that share a row
+      float y = acc;
+      y += __shfl_xor(y, 4, 64); y += __shfl_xor(y, 8, 64);
+      y += __shfl_xor(y, 16, 64); y += __shfl_xor(y, 32, 64);
+      acc = 0.f;
+      const uint32_t row = row0 + l;
+      if (row < end && bcol == 0u) {
+        if (EPI == EPI_STORE) act_out[(uint64_t)c_out + row] = y;
+        else if (better(y, row, best_v, best_i)) { best_v = y; best_i = row; }
+      }
+    }
+  };
+
+  while (true) {
+    if (first < seg_end) {
+      // steps t = 0..T-1 in (row bundle, chunk) order; register set A holds step 0 on entry.  The
+      // prefetch of the following step is issued unconditionally (past the end it re-reads the last
+      // rows, clamped in load()), so the number of loads in flight at every wait is known statically.
+      const uint32_t T = ((seg_end - first + stride - 1u) / stride) * C;
+      uint32_t row_a = first, ch_a = 0, row_b, ch_b, row_n = first, ch_n = 0;
+      if (++ch_n == C) { ch_n = 0; row_n += stride; }
+      for (uint32_t t = 0; t < T; t += 2) {
+        row_b = row_n; ch_b = ch_n;
+        load(B, row_b, ch_b, seg_end);
+        __builtin_amdgcn_sched_barrier(0);   // keep the prefetch ahead of the arithmetic
+        if (++ch_n == C) { ch_n = 0; row_n += stride; }
+        compute(A, row_a, ch_a, seg_end);
+        if (t + 1 >= T) break;
+        row_a = row_n; ch_a = ch_n;
+        load(A, row_a, ch_a, seg_end);
+        __builtin_amdgcn_sched_barrier(0);
+        if (++ch_n == C) { ch_n = 0; row_n += stride; }
+        compute(B, row_b, ch_b, seg_end);
+      }
+    }
+    if (EPI == EPI_STORE) break;
+    // argmax: next group's first loads go out before this group's partial is merged
+    const uint32_t done = grp;
+    grp += gridDim.x;
+    const bool more = grp < n_groups;
+    if (more) {
+      first = grp * rows_per_group + wave * 4u;
+      seg_end = min(N, (grp + 1) * rows_per_group);
+      if (first < seg_end) load(A, first, 0, seg_end);
+    }
+    // lanes 0..3 hold the best of their own rows
+#pragma unroll
+    for (int o = 1; o <= 2; o <<= 1) {
+      const float ov = __shfl_xor(best_v, o, 64);
+      const uint32_t oi = __shfl_xor(best_i, o, 64);
+      if (better(ov, oi, best_v, best_i)) { best_v = ov; best_i = oi; }
+    }
+    if (lane == 0u) { red_f[wave] = best_v; red_i[wave] = best_i; }
+    __syncthreads();
+    if (tid == 0) {
+      float bv = red_f[0]; uint32_t bi = red_i[0];
+      for (uint32_t w = 1; w < nwav; w++)
+        if (better(red_f[w], red_i[w], bv, bi)) { bv = red_f[w]; bi = red_i[w]; }
+      act_out[lidx[done]] = (float)(bi == INVALID_IDX ? 0u : bi);
+      act_out[lval[done]] = bv;
+    }
+    __syncthreads();
+    best_v = NEG_FLT_MAX; best_i = INVALID_IDX;
+    if (!more) break;
+  }
+}
+
+// ---- host side -----------------------------------------------------------------------------------
+static size_t mfma_smem(uint32_t K) { return (size_t)(K >> 5) * 128; }
+
+bool mfma_path_ok(const Map* mw, uint32_t K) {
+  return mw->dtype == DTYPE_Q4 && mw->group_size == 32 && K >= 32 && (K & 31u) == 0 && mfma_smem(K) <= 64000;
+}
+
+template <int EPI>
+static int launch_mfma(int fmt, uint32_t grid, uint32_t threads, const Map* ma, const Map* mw, uint32_t a, uint32_t b,
+                       uint32_t c, const uint32_t* lidx, const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rpg,
+                       uint32_t n_groups) {
+  float* act = (float*)ma->buf;
+  const size_t smem = mfma_smem(K);
+  const bool ragged = (K & 2047u) != 0;
+#define MK(F, R)                                                                                                   \
+  k_gemv_mfma<F, EPI, R><<<grid, threads, smem, g.stream>>>(act, act, mw->buf, mw->qp, mw->d16, a, b, c, lidx, lval, K, \
+                                                            N, rpg, n_groups)
+  if (fmt == FMT_Q4_B16) { if (ragged) MK(FMT_Q4_B16, true); else MK(FMT_Q4_B16, false); }
+  else { if (ragged) MK(FMT_Q4_AFF, true); else MK(FMT_Q4_AFF, false); }
+#undef MK
+  count_launch();
+  return check_launch();
+}
+
+// Launch shape for `units` wave-sized pieces of work: workgroups of 4, 8 or 16 waves (the activations
+// are converted once per workgroup), as many as give every SIMD four waves.
+static void mfma_shape(uint32_t K, uint32_t units, uint32_t* grid, uint32_t* threads) {
+  // largest workgroup (16, 8 or 4 waves) that still leaves a workgroup for every CU
+  uint32_t waves = 16;
+  while (waves > 4 && cdiv(units, waves) < (uint32_t)g.n_cu) waves >>= 1;
+  waves = (uint32_t)tuning("ADAMAH_MFMA_WAVES", (int)waves);
+  waves = waves >= 16 ? 16 : waves >= 8 ? 8 : 4;
+  const uint32_t per_simd = (uint32_t)std::max(1, tuning("ADAMAH_MFMA_PERSIMD", 4));
+  const size_t lds_fit = std::max<size_t>(1, (160 * 1024) / (mfma_smem(K) + 256));
+  const uint32_t wg_per_cu = (uint32_t)std::max<size_t>(1, std::min<size_t>(lds_fit, (size_t)per_simd * 4 / waves));
+  *threads = waves * 64;
+  *grid = std::max(1u, std::min<uint32_t>(cdiv(units, waves), (uint32_t)g.n_cu * wg_per_cu));
+}
+
+int launch_mfma_store(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32_t b, uint32_t c, uint32_t K,
+                      uint32_t N) {
+  uint32_t grid, threads;
+  mfma_shape(K, cdiv(N, 4), &grid, &threads);
+  return launch_mfma<EPI_STORE>(fmt, grid, threads, ma, mw, a, b, c, nullptr, nullptr, K, N, 0, 0);
+}
+
+int launch_mfma_argmax(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32_t b, const uint32_t* lidx,
+                       const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rows_per_group) {
+  const uint32_t n_groups = cdiv(N, rows_per_group);
+  uint32_t grid, threads;
+  mfma_shape(K, n_groups * 16u, &grid, &threads);   // one workgroup per group at a time
+  grid = std::min(grid, n_groups);
+  return launch_mfma<EPI_ARGMAX>(fmt, grid, threads, ma, mw, a, b, 0, lidx, lval, K, N, rows_per_group, n_groups);
+}
+
+}  // namespace adamah

@@ -16,55 +16,12 @@
 // access), read once per step and reused for ROWS weight rows.  Per block the kernel
 // accumulates  scale * sum(code*x) + zp * sum(x)  with sum(x) per block precomputed, so the
 // inner loop is one byte->float convert and one FMA per weight, fp32 throughout.
-#include "common.h"
+#include "gemv_common.h"
 #include "../../include/adamah_hip.h"
 #include <algorithm>
 #include <stdlib.h>
 
 namespace adamah {
-
-enum { FMT_Q4_B16 = 0, FMT_Q4_AFF = 1, FMT_Q8_B16 = 2, FMT_Q8_AFF = 3 };
-enum { EPI_STORE = 0, EPI_ARGMAX = 1 };
-
-#define NEG_FLT_MAX (-3.402823466e+38f)
-#define INVALID_IDX 0xffffffffu
-
-__device__ __forceinline__ bool better(float cv, uint32_t ci, float bv, uint32_t bi) {
-  // strict > or (== and lower index); an invalid best always loses (map_argmax.comp:15-19)
-  if (bi == INVALID_IDX) return true;
-  if (ci == INVALID_IDX) return false;
-  return (cv > bv) || ((cv == bv) && (ci < bi));
-}
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
-}
-
-// byte n of a 32-bit register -> float, one VALU op
-template <int N> __device__ __forceinline__ float ubyte_f32(uint32_t w) {
-  float r;
-  if (N == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(w));
-  else if (N == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(w));
-  else if (N == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(w));
-  else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(w));
-  return r;
-}
-
-#define DPP_ADD(v, ctrl, rmask)                                                                    \
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, rmask, 0xF, false))
-
-// Sum over the 64 lanes; the total is valid in lane 63.
-__device__ __forceinline__ float wave_sum_to_lane63(float v) {
-  DPP_ADD(v, 0xB1, 0xF);    // quad_perm [1,0,3,2]
-  DPP_ADD(v, 0x4E, 0xF);    // quad_perm [2,3,0,1]
-  DPP_ADD(v, 0x141, 0xF);   // row_half_mirror
-  DPP_ADD(v, 0x140, 0xF);   // row_mirror: every lane of a 16-lane row holds the row sum
-  DPP_ADD(v, 0x142, 0xA);   // row_bcast15 into rows 1 and 3
-  DPP_ADD(v, 0x143, 0xC);   // row_bcast31 into rows 2 and 3
-  return v;
-}
 
 // sum_j code[j] * x[j] for the 8 nibbles of one word; x = two float4 (elements 0..7)
 __device__ __forceinline__ float dot_q4_word(uint32_t w, const float4& xa, const float4& xb, float acc) {
@@ -487,7 +444,7 @@ static int fmt_of(const Map* mw, uint64_t b, uint64_t n_w) {
   return q4 ? (b16 ? FMT_Q4_B16 : FMT_Q4_AFF) : (b16 ? FMT_Q8_B16 : FMT_Q8_AFF);
 }
 
-static int tuning(const char* name, int dflt) {
+int tuning(const char* name, int dflt) {
   const char* v = getenv(name);
   return v ? atoi(v) : dflt;
 }
@@ -566,8 +523,11 @@ int op_matmul_t_xq(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t h
   uint64_t a0 = 0, b0 = 0;
   if (transposed && M == 1 && n_ops == 1 && ch && block_path_ok(ma, mw, ha, hb, K, N, &a0, &b0)) {
     const int fmt = fmt_of(mw, b0, (uint64_t)N * K);
-    // long rows: activations in registers, waves share a row; otherwise activations staged in LDS
-    if (tuning("ADAMAH_GEMV_IMPL", K > 8192 ? 1 : 0) == 1) {
+    // Q4: int8 matrix-instruction kernel.  Q8 (and Q4 on request): float32 kernels, activations in
+    // registers with waves sharing a row when K > 8192, else staged in LDS
+    const int impl = tuning("ADAMAH_GEMV_IMPL", mfma_path_ok(mw, K) ? 3 : K > 8192 ? 1 : 0);
+    if (impl == 3 && mfma_path_ok(mw, K)) return launch_mfma_store(fmt, ma, mw, (uint32_t)a0, (uint32_t)b0, ch[0], K, N);
+    if (impl == 1) {
       const uint32_t ks = K <= 4096 ? 1 : K <= 8192 ? 2 : 4;
       const uint32_t step = (4 / ks) * 4;                       // rows one workgroup pass covers
       const uint32_t passes = (uint32_t)tuning("ADAMAH_GEMV_PASSES", 2);
@@ -610,7 +570,11 @@ int op_matvec_argmax(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t
   uint64_t a0 = 0, b0 = 0;
   int r;
   if (locs_ok && block_path_ok(ma, mw, ha, hb, K, N, &a0, &b0)) {
-    if (tuning("ADAMAH_GEMV_IMPL", K > 8192 ? 1 : 0) == 1)
+    const int impl = tuning("ADAMAH_GEMV_IMPL", mfma_path_ok(mw, K) ? 3 : K > 8192 ? 1 : 0);
+    if (impl == 3 && mfma_path_ok(mw, K))
+      r = launch_mfma_argmax(fmt_of(mw, b0, (uint64_t)N * K), ma, mw, (uint32_t)a0, (uint32_t)b0, lidx, lval, K, N,
+                             rows_per_group);
+    else if (impl == 1)
       r = launch_regx<EPI_ARGMAX>(fmt_of(mw, b0, (uint64_t)N * K), ma, mw, la, lb, nullptr, lidx, lval, K, N,
                                   rows_per_group);
     else
