@@ -7,9 +7,12 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libadamah_hip.so")
-SOURCES = ["runtime.hip", "gemv_q.hip", "gemv_mfma.hip", "norm_rope.hip", "attention.hip", "elementwise.hip", "probe.hip"]
+SOURCES = ["runtime.hip", "gemv_q.hip", "gemv_mfma.hip", "fuse.hip", "norm_rope.hip", "attention.hip", "elementwise.hip", "probe.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", "-ffp-contract=off",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result", "-Wno-unused-value"]
+# gemv_mfma.hip draws a ticket with one atomic per workgroup and looks at it much later; the
+# compiler's wave-level aggregation of uniform-address atomics would wait for the result at once.
+EXTRA = {"gemv_mfma.hip": ["-mllvm", "-amdgpu-atomic-optimizer-strategy=None"]}
 
 
 def _hipcc():
@@ -36,7 +39,7 @@ def build(verbose=True, jobs=None):
     objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
 
     def one(i):
-        return _run([hipcc, *FLAGS, "-c", os.path.join(CSRC, SOURCES[i]), "-o", objs[i]])
+        return _run([hipcc, *FLAGS, *EXTRA.get(SOURCES[i], []), "-c", os.path.join(CSRC, SOURCES[i]), "-o", objs[i]])
 
     with ThreadPoolExecutor(max_workers=jobs or min(len(SOURCES), os.cpu_count() or 4)) as ex:
         for s, out in zip(SOURCES, ex.map(one, range(len(SOURCES)))):

@@ -11,7 +11,17 @@
 #include "../../include/adamah_hip.h"
 #include <algorithm>
 
+extern "C" int map_matmul_t_dev(uint32_t map_id, uint32_t ha, uint32_t hb, uint32_t hc, uint32_t M, uint32_t K, uint32_t N,
+                                uint32_t n_ops);
+
 namespace adamah {
+
+#ifdef ADAMAH_TRACE
+__device__ unsigned long long g_trace_attn[64];
+#define TRA(i) do { if (threadIdx.x == 0 && blockIdx.x == 0 && blockIdx.y == 0) g_trace_attn[i] = wall_clock64(); } while (0)
+#else
+#define TRA(i) do {} while (0)
+#endif
 
 __device__ __forceinline__ float ld(const float* p, uint64_t i) { return p[i]; }
 __device__ __forceinline__ float ld(const __half* p, uint64_t i) { return __half2float(p[i]); }
@@ -246,6 +256,199 @@ k_attn_softmax_value(const float* data, float* out, const TV* vsrc, uint64_t v_s
   }
 }
 
+// Scores and softmax . V of one chunk of the sequence in one launch (fp16 K and V rows, 8 elements
+// per 16-byte load): the two kernels above back to back inside a workgroup, with the prepared scores
+// handed over in LDS instead of through the score row in memory.  The raw scores are still stored
+// where the stand-alone score kernel would put them.  grid (n_splits, n_ops); lpr lanes share a K
+// row, vlpr = value_dim / 8 lanes a V row.
+template <int LPR>
+__global__ void __launch_bounds__(256)
+k_attn_fused(const float* data, float* out, const __half* kv, uint64_t kv_shift, const uint32_t* __restrict__ la,
+             const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc, const uint32_t* __restrict__ lv,
+             const uint32_t* __restrict__ lo, uint32_t K, uint32_t row_size, uint32_t value_dim, float scale,
+             float cap, uint32_t n_splits, uint32_t chunk, float* partial) {
+  constexpr int VEC = 8;
+  constexpr uint32_t lpr = LPR;
+  TRA(0);
+  __shared__ float p[ATT_CHUNK];
+  __shared__ float red[4];
+  __shared__ float osum[2048];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t split = blockIdx.x, op = blockIdx.y;
+  const uint32_t t0 = split * chunk, t1 = min(row_size, t0 + chunk), nt = t1 - t0;
+  const uint64_t a = la[op], kb = (uint64_t)lb[op] - kv_shift, c = lc[op], vb = (uint64_t)lv[op] - kv_shift, ob = lo[op];
+  // scores: the query slice of this lane in registers, 64/lpr K rows per wave step
+  {
+    const uint32_t sub = lane % lpr, rslot = lane / lpr, rpw = 64u / lpr, nvec = K / VEC;
+    float q[4][VEC];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t v = sub + i * lpr;
+#pragma unroll
+      for (int j = 0; j < VEC; j++) q[i][j] = v < nvec ? data[a + (uint64_t)v * VEC + j] : 0.f;
+    }
+    TRA(1);
+    if (lpr >= nvec) {
+      // every lane holds one 16-byte slice of a row (head dims up to 512): sixteen row groups per trip,
+      // all loads issued before the first is used; rows past the chunk are clamped and dropped
+      for (uint32_t rb = t0 + wave * rpw; rb < t1; rb += 64u * rpw) {
+        uint4 raw[16];
+        const uint32_t v = min(sub, nvec - 1u);
+#pragma unroll
+        for (int g16 = 0; g16 < 16; g16++) {
+          const uint32_t r = min(rb + g16 * 4u * rpw + rslot, t1 - 1u);
+          raw[g16] = *(const uint4*)(kv + kb + (uint64_t)r * K + (uint64_t)v * VEC);
+        }
+        // partial dot products of all sixteen groups, then the lane reductions stage by stage so that
+        // the sixteen shuffles of a stage are independent
+        float sg[16];
+#pragma unroll
+        for (int g16 = 0; g16 < 16; g16++) {
+          float s = 0.f;
+          if (sub < nvec) {
+            const __half2* h = (const __half2*)&raw[g16];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+              const float2 f = __half22float2(h[j]);
+              s = fmaf(q[0][2 * j], f.x, s);
+              s = fmaf(q[0][2 * j + 1], f.y, s);
+            }
+          }
+          sg[g16] = s;
+        }
+#pragma unroll
+        for (int o = LPR >> 1; o > 0; o >>= 1) {
+#pragma unroll
+          for (int g16 = 0; g16 < 16; g16++) sg[g16] += __shfl_xor(sg[g16], o, 64);
+        }
+#pragma unroll
+        for (int g16 = 0; g16 < 16; g16++) {
+          const uint32_t r = rb + g16 * 4u * rpw + rslot;
+          if (r < t1 && sub == 0) {
+            out[c + r] = sg[g16];
+            p[r - t0] = sg[g16];   // soft cap and scale are applied below, one row per thread
+          }
+        }
+      }
+    } else {
+      // long rows: up to four slices per lane, four row groups per trip
+      for (uint32_t rb = t0 + wave * rpw; rb < t1; rb += 16u * rpw) {
+        uint4 raw[4][4];
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+          const uint32_t r = min(rb + g4 * 4u * rpw + rslot, t1 - 1u);
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            if (i * lpr < nvec) {   // uniform: slices the row does not have are skipped
+              const uint32_t v = min(sub + i * lpr, nvec - 1u);
+              raw[g4][i] = *(const uint4*)(kv + kb + (uint64_t)r * K + (uint64_t)v * VEC);
+            }
+          }
+        }
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+          const uint32_t r = rb + g4 * 4u * rpw + rslot;
+          float s = 0.f;
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            if (sub + i * lpr < nvec) {
+              const __half2* h = (const __half2*)&raw[g4][i];
+#pragma unroll
+              for (int j = 0; j < 4; j++) {
+                const float2 f = __half22float2(h[j]);
+                s = fmaf(q[i][2 * j], f.x, s);
+                s = fmaf(q[i][2 * j + 1], f.y, s);
+              }
+            }
+          }
+          for (uint32_t o = lpr >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+          if (r < t1 && sub == 0) {
+            out[c + r] = s;
+            p[r - t0] = s;
+          }
+        }
+      }
+    }
+  }
+  TRA(2);
+  __syncthreads();
+  TRA(3);
+  float mx = -9.99999968e+37f;
+  for (uint32_t t = tid; t < nt; t += 256u) {
+    const float v = prep(p[t], scale, cap);
+    p[t] = v;
+    mx = fmaxf(mx, v);
+  }
+  mx = wave_max64(mx);
+  if (lane == 0) red[wave] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  float sum = 0.f;
+  for (uint32_t t = tid; t < nt; t += 256u) {
+    const float e = expf(p[t] - mx);
+    p[t] = e;
+    sum += e;
+  }
+  sum = wave_sum64(sum);
+  if (lane == 0) red[wave] = sum;
+  __syncthreads();
+  sum = (red[0] + red[1]) + (red[2] + red[3]);
+  TRA(4);
+  // values: vlpr lanes cover one V row, 256/vlpr rows in flight per sweep; row-slot partials meet in LDS
+  const uint32_t vlpr = value_dim / VEC, slots = 256u / vlpr, sub = tid % vlpr, slot = tid / vlpr;
+  float acc[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; j++) acc[j] = 0.f;
+  if (slot < slots) {
+    const __half* base = kv + vb + (uint64_t)t0 * value_dim + (uint64_t)sub * VEC;
+    // eight V rows per lane and trip, loads first (rows past the chunk: clamped, weight 0)
+    for (uint32_t tb = slot; tb < nt; tb += 8u * slots) {
+      uint4 raw[8];
+      float w[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const uint32_t t = tb + u * slots;
+        raw[u] = *(const uint4*)(base + (uint64_t)min(t, nt - 1u) * value_dim);
+        w[u] = t < nt ? p[min(t, nt - 1u)] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const __half2* h = (const __half2*)&raw[u];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const float2 f = __half22float2(h[j]);
+          acc[2 * j] = fmaf(w[u], f.x, acc[2 * j]);
+          acc[2 * j + 1] = fmaf(w[u], f.y, acc[2 * j + 1]);
+        }
+      }
+    }
+  }
+  TRA(5);
+  const uint32_t fit = 2048u / value_dim;
+  float o = 0.f;
+  for (uint32_t s0 = 0; s0 < slots; s0 += fit) {
+    if (slot >= s0 && slot < s0 + fit && slot < slots) {
+#pragma unroll
+      for (int j = 0; j < VEC; j++) osum[(slot - s0) * value_dim + sub * VEC + j] = acc[j];
+    }
+    __syncthreads();
+    if (tid < value_dim)
+      for (uint32_t s = 0; s < fit && s0 + s < slots; s++) o += osum[s * value_dim + tid];
+    __syncthreads();
+  }
+  if (tid < value_dim) {
+    if (n_splits == 1) out[ob + tid] = o * (1.0f / sum);
+    else partial[((uint64_t)op * n_splits + split) * (value_dim + 2) + 2 + tid] = o;
+  }
+  if (n_splits > 1 && tid == 0) {
+    float* pp = partial + ((uint64_t)op * n_splits + split) * (value_dim + 2);
+    pp[0] = mx;
+    pp[1] = sum;
+  }
+  TRA(6);
+}
+
 // Merge the split partials of one op: M = max m_s, w_s = e^(m_s-M), L = sum l_s w_s,
 // out = sum_s o_s w_s / L.  n_splits <= 1024.
 __global__ void __launch_bounds__(256)
@@ -320,7 +523,119 @@ static bool all_in_kv(const Map* m, uint32_t h, uint32_t n_ops, uint64_t span) {
   return true;
 }
 
+
+// Sequence split of softmax . V: rows per workgroup so that about two workgroups per CU exist over
+// all heads, 32..1024 rows each.
+#define ATT_FOLD_FLOATS 8192u   // most partial floats a consumer is asked to merge by itself
+static void attn_split(uint32_t n_ops, uint32_t row_size, uint32_t value_dim, bool few, uint32_t* chunk,
+                       uint32_t* n_splits) {
+  const uint32_t want_splits = std::max<uint32_t>(1u, cdiv(2u * (uint32_t)g.n_cu, n_ops));
+  uint32_t c = std::min<uint32_t>(ATT_CHUNK, std::max<uint32_t>(32u, cdiv(row_size, want_splits)));
+  c = (c + 31u) & ~31u;
+  // `few`: the consumer will merge the partials, every one of its workgroups reads all of them, so
+  // keep them few (longer chunks) as long as a chunk still fits a workgroup
+  while (few && c < ATT_CHUNK && (uint64_t)n_ops * cdiv(row_size, c) * (value_dim + 2) > ATT_FOLD_FLOATS) c += 32u;
+  *chunk = c;
+  *n_splits = cdiv(row_size, c);
+}
+
+// Operand checks of softmax . V against the host copies of the handles; *kv = K/V rows in the fp16
+// copy, *fast = whole 16-byte vectors and everything in range.
+static int attn_check(uint32_t map_id, uint32_t hs, uint32_t hv, uint32_t ho, uint32_t n_ops, uint32_t row_size,
+                      uint32_t value_dim, bool* kv, bool* fast) {
+  Map* m = get_f32_map(map_id);
+  if (!m) return ADAMAH_ERR_INVALID;
+  if (!res_u32(hs, n_ops) || !res_u32(hv, n_ops) || !res_u32(ho, n_ops)) return ADAMAH_ERR_INVALID;
+  uint32_t chunk, n_splits;
+  attn_split(n_ops, row_size, value_dim, false, &chunk, &n_splits);
+  if ((uint64_t)n_ops * n_splits * (value_dim + 2) > g.attn_scratch_floats || n_splits > 1024) return ADAMAH_ERR_INVALID;
+  *kv = all_in_kv(m, hv, n_ops, (uint64_t)row_size * value_dim);
+  const uint32_t vec = *kv ? 8u : 4u;
+  const uint32_t *sh = res_host(hs, n_ops), *vh = res_host(hv, n_ops), *oh = res_host(ho, n_ops);
+  bool f = sh && vh && oh && value_dim % vec == 0 && value_dim / vec <= 256 && 256u % (value_dim / vec) == 0 &&
+           value_dim <= 256;
+  for (uint32_t op = 0; f && op < n_ops; op++)
+    f = in_range(sh[op], row_size, m->n_elems) && in_range(vh[op], (uint64_t)row_size * value_dim, m->n_elems) &&
+        in_range(oh[op], value_dim, m->n_elems) && (vh[op] - (*kv ? m->kv_start : 0)) % vec == 0;
+  *fast = f;
+  return ADAMAH_OK;
+}
+
+int launch_scores(const PendOp& sc) {
+  g.no_defer++;
+  const int r = map_matmul_t_dev(sc.map_act, sc.h[0], sc.h[1], sc.h[2], 1, sc.k, sc.n, sc.rpg);
+  g.no_defer--;
+  return r;
+}
+
+// Can the queued score op be computed inside the softmax . V launch?  Same heads and length, the
+// score rows it writes are the ones softmax . V reads, K rows in the fp16 copy.
+bool attn_foldable(const PendOp& sc, const PendOp& at) {
+  if (sc.kind != PK_SCORES || at.kind != PK_ATTN || sc.map_act != at.map_act || sc.rpg != at.rpg || sc.n != at.n) return false;
+  const uint32_t *c = res_host(sc.h[2], sc.rpg), *s = res_host(at.h[0], at.rpg);
+  if (!c || !s) return false;
+  for (uint32_t i = 0; i < sc.rpg; i++) if (c[i] != s[i]) return false;
+  return true;
+}
+
+int launch_attn(const PendOp* sc, const PendOp& at, bool leave_partials, AttnPartials* ap) {
+  Map* m = get_f32_map(at.map_act);
+  if (!m) return ADAMAH_ERR_INVALID;
+  const uint32_t n_ops = at.rpg, row_size = at.n, value_dim = at.k;
+  bool kv = false, fast = false;
+  int r = attn_check(at.map_act, at.h[0], at.h[1], at.h[2], n_ops, row_size, value_dim, &kv, &fast);
+  if (r) return r;
+  const uint32_t *ls = res_u32(at.h[0], n_ops), *lv = res_u32(at.h[1], n_ops), *lo = res_u32(at.h[2], n_ops);
+  uint32_t chunk, n_splits;
+  attn_split(n_ops, row_size, value_dim, leave_partials, &chunk, &n_splits);
+  if ((uint64_t)n_ops * n_splits * (value_dim + 2) > ATT_FOLD_FLOATS) leave_partials = false;
+  float* d = (float*)m->buf;
+  dim3 grid(n_splits, n_ops);
+  if (sc && fast && kv) {
+    const uint32_t *la = res_u32(sc->h[0], n_ops), *lb = res_u32(sc->h[1], n_ops);
+    uint32_t lpr = 8;
+    while (lpr < 64 && lpr * 8u < sc->k) lpr <<= 1;
+#define AF(L)                                                                                                      \
+  k_attn_fused<L><<<grid, 256, 0, g.stream>>>(d, d, m->kv16, m->kv_start, la, lb, ls, lv, lo, sc->k, row_size, value_dim, \
+                                              at.eps, at.f2, n_splits, chunk, g.attn_scratch)
+    if (lpr == 8) AF(8); else if (lpr == 16) AF(16); else if (lpr == 32) AF(32); else AF(64);
+#undef AF
+  } else {
+    if (sc && (r = launch_scores(*sc))) return r;
+    const float scale = at.eps, cap = at.f2;
+#define ASV(T, V, src, shift, elems)                                                                             \
+  k_attn_softmax_value<T, V><<<grid, 256, 0, g.stream>>>(d, d, src, shift, ls, lv, lo, row_size, value_dim, scale, \
+                                                         cap, n_splits, chunk, g.attn_scratch, m->n_elems, elems)
+    if (kv) { if (fast) ASV(__half, 8, m->kv16, m->kv_start, m->kv_count); else ASV(__half, 1, m->kv16, m->kv_start, m->kv_count); }
+    else { if (fast) ASV(float, 4, d, 0, m->n_elems); else ASV(float, 1, d, 0, m->n_elems); }
+#undef ASV
+  }
+  count_launch();
+  r = check_launch();
+  if (r || n_splits == 1) { if (ap) ap->n_splits = 1; return r; }
+  AttnPartials loc = {g.attn_scratch, n_splits, value_dim, n_ops, 0};
+  if (leave_partials && ap) { *ap = loc; return ADAMAH_OK; }
+  if (ap) ap->n_splits = 1;
+  return launch_attn_combine(at, loc);
+}
+
+int launch_attn_combine(const PendOp& at, const AttnPartials& ap) {
+  Map* m = get_f32_map(at.map_act);
+  const uint32_t* lo = res_u32(at.h[2], at.rpg);
+  if (!m || !lo) return ADAMAH_ERR_INVALID;
+  k_attn_combine<<<at.rpg, 256, 0, g.stream>>>((float*)m->buf, ap.base, lo, ap.value_dim, ap.n_splits, m->n_elems);
+  count_launch();
+  return check_launch();
+}
+
 }  // namespace adamah
+
+#ifdef ADAMAH_TRACE
+extern "C" int adamah_hip_trace_read_attn(unsigned long long* out) {
+  hipStreamSynchronize(adamah::g.stream);
+  return hipMemcpyFromSymbol(out, HIP_SYMBOL(adamah::g_trace_attn), 64 * sizeof(unsigned long long)) == hipSuccess ? 0 : -1;
+}
+#endif
 
 using namespace adamah;
 
@@ -329,10 +644,10 @@ extern "C" {
 int map_matmul_t_dev(uint32_t map_id, uint32_t ha, uint32_t hb, uint32_t hc, uint32_t M, uint32_t K, uint32_t N,
                      uint32_t n_ops) {
   Map* m = get_f32_map(map_id);
-  if (!m) return ADAMAH_ERR_INVALID;
-  if (n_ops == 0 || M == 0 || N == 0) return ADAMAH_OK;
+  if (!m) { flush_pending(); return ADAMAH_ERR_INVALID; }
+  if (n_ops == 0 || M == 0 || N == 0) { flush_pending(); return ADAMAH_OK; }
   const uint32_t *la = res_u32(ha, n_ops), *lb = res_u32(hb, n_ops), *lc = res_u32(hc, n_ops);
-  if (!la || !lb || !lc) return ADAMAH_ERR_INVALID;
+  if (!la || !lb || !lc) { flush_pending(); return ADAMAH_ERR_INVALID; }
   dim3 grid(cdiv(N, 4), M, n_ops);
   float* d = (float*)m->buf;
   const bool kv = all_in_kv(m, hb, n_ops, (uint64_t)N * K);
@@ -347,6 +662,13 @@ int map_matmul_t_dev(uint32_t map_id, uint32_t ha, uint32_t hb, uint32_t hc, uin
       fast = in_range(ah[op], K, m->n_elems) && in_range(bh[op], (uint64_t)N * K, m->n_elems) &&
              in_range(ch[op], N, m->n_elems) && (bh[op] - (kv ? m->kv_start : 0)) % vec == 0;
   }
+  if (fast && kv && can_defer()) {   // decode scores over the fp16 cache: queue, softmax . V may absorb them
+    PendOp p;
+    p.kind = PK_SCORES; p.map_act = map_id; p.h[0] = ha; p.h[1] = hb; p.h[2] = hc; p.k = K; p.n = N; p.rpg = n_ops;
+    g.pend.push_back(p);
+    return ADAMAH_OK;
+  }
+  flush_pending();
   if (fast) {
     // rows per workgroup: about two workgroups per CU over all ops, at least one wave step each
     const uint32_t want_wg = std::max<uint32_t>(1u, cdiv(2u * (uint32_t)g.n_cu, n_ops));
@@ -366,7 +688,7 @@ int map_matmul_t_dev(uint32_t map_id, uint32_t ha, uint32_t hb, uint32_t hc, uin
 }
 
 int map_matmul_t_x_dev(uint32_t map_act, uint32_t map_wt, uint32_t ha, uint32_t hb, uint32_t hc, uint32_t M, uint32_t K,
-                       uint32_t N, uint32_t n_ops) {
+                       uint32_t N, uint32_t n_ops) { ADAMAH_API();
   Map* ma = get_f32_map(map_act);
   Map* mw = get_f32_map(map_wt);
   if (!ma || !mw) return ADAMAH_ERR_INVALID;
@@ -381,7 +703,7 @@ int map_matmul_t_x_dev(uint32_t map_act, uint32_t map_wt, uint32_t ha, uint32_t 
 }
 
 static int matmul_nt(uint32_t map_act, uint32_t map_wt, uint32_t ha, uint32_t hb, uint32_t hc, uint32_t M, uint32_t K,
-                     uint32_t N, uint32_t n_ops) {
+                     uint32_t N, uint32_t n_ops) { ADAMAH_API();
   Map* ma = get_f32_map(map_act);
   Map* mw = get_f32_map(map_wt);
   if (!ma || !mw) return ADAMAH_ERR_INVALID;
@@ -395,54 +717,33 @@ static int matmul_nt(uint32_t map_act, uint32_t map_wt, uint32_t ha, uint32_t hb
   return check_launch();
 }
 int map_matmul_x_dev(uint32_t map_act, uint32_t map_wt, uint32_t ha, uint32_t hb, uint32_t hc, uint32_t M, uint32_t K,
-                     uint32_t N, uint32_t n_ops) {
+                     uint32_t N, uint32_t n_ops) { ADAMAH_API();
   return matmul_nt(map_act, map_wt, ha, hb, hc, M, K, N, n_ops);
 }
 int map_matmul_dev(uint32_t map_id, uint32_t ha, uint32_t hb, uint32_t hc, uint32_t M, uint32_t K, uint32_t N,
-                   uint32_t n_ops) {
+                   uint32_t n_ops) { ADAMAH_API();
   return matmul_nt(map_id, map_id, ha, hb, hc, M, K, N, n_ops);
 }
 
 int map_attn_softmax_value_dev(uint32_t map_id, uint32_t hs, uint32_t hv, uint32_t ho, uint32_t n_ops,
                                uint32_t row_size, uint32_t value_dim, float scale, float cap) {
-  Map* m = get_f32_map(map_id);
-  if (!m) return ADAMAH_ERR_INVALID;
-  if (n_ops == 0 || row_size == 0 || value_dim == 0) return ADAMAH_OK;
-  const uint32_t *ls = res_u32(hs, n_ops), *lv = res_u32(hv, n_ops), *lo = res_u32(ho, n_ops);
-  if (!ls || !lv || !lo) return ADAMAH_ERR_INVALID;
-  // rows per workgroup: enough workgroups to fill the chip (about 2 per CU over all ops), 32..1024 rows each
-  const uint32_t want_splits = std::max<uint32_t>(1u, cdiv(2u * (uint32_t)g.n_cu, n_ops));
-  uint32_t chunk = std::min<uint32_t>(ATT_CHUNK, std::max<uint32_t>(32u, cdiv(row_size, want_splits)));
-  chunk = (chunk + 31u) & ~31u;
-  const uint32_t n_splits = cdiv(row_size, chunk);
-  if ((uint64_t)n_ops * n_splits * (value_dim + 2) > g.attn_scratch_floats || n_splits > 1024) return ADAMAH_ERR_INVALID;
-  float* d = (float*)m->buf;
-  dim3 grid(n_splits, n_ops);
-  const bool kv = all_in_kv(m, hv, n_ops, (uint64_t)row_size * value_dim);
-  // vector path: value rows made of whole 16-byte vectors, 256 % (value_dim/vec) == 0, operands host-verified
-  const uint32_t vec = kv ? 8u : 4u;
-  const uint32_t *sh = res_host(hs, n_ops), *vh = res_host(hv, n_ops), *oh = res_host(ho, n_ops);
-  bool fast = sh && vh && oh && value_dim % vec == 0 && value_dim / vec <= 256 && 256u % (value_dim / vec) == 0 &&
-              value_dim <= 2048 && value_dim <= 256;
-  for (uint32_t op = 0; fast && op < n_ops; op++)
-    fast = in_range(sh[op], row_size, m->n_elems) && in_range(vh[op], (uint64_t)row_size * value_dim, m->n_elems) &&
-           in_range(oh[op], value_dim, m->n_elems) && (vh[op] - (kv ? m->kv_start : 0)) % vec == 0;
-#define ASV(T, V, src, shift, elems)                                                                             \
-  k_attn_softmax_value<T, V><<<grid, 256, 0, g.stream>>>(d, d, src, shift, ls, lv, lo, row_size, value_dim, scale, \
-                                                         cap, n_splits, chunk, g.attn_scratch, m->n_elems, elems)
-  if (kv) { if (fast) ASV(__half, 8, m->kv16, m->kv_start, m->kv_count); else ASV(__half, 1, m->kv16, m->kv_start, m->kv_count); }
-  else { if (fast) ASV(float, 4, d, 0, m->n_elems); else ASV(float, 1, d, 0, m->n_elems); }
-#undef ASV
-  count_launch();
-  int r = check_launch();
-  if (r || n_splits == 1) return r;
-  k_attn_combine<<<n_ops, 256, 0, g.stream>>>(d, g.attn_scratch, lo, value_dim, n_splits, m->n_elems);
-  count_launch();
-  return check_launch();
+  if (n_ops == 0 || row_size == 0 || value_dim == 0) { flush_pending(); return get_f32_map(map_id) ? ADAMAH_OK : ADAMAH_ERR_INVALID; }
+  bool kv = false, fast = false;
+  int r = attn_check(map_id, hs, hv, ho, n_ops, row_size, value_dim, &kv, &fast);
+  if (r) { flush_pending(); return r; }
+  PendOp p;
+  p.kind = PK_ATTN; p.map_act = map_id; p.h[0] = hs; p.h[1] = hv; p.h[2] = ho; p.rpg = n_ops; p.n = row_size;
+  p.k = value_dim; p.eps = scale; p.f2 = cap;
+  if (fast && kv && can_defer()) {   // queue: the scores before it and the GEMV after it may be folded in
+    g.pend.push_back(p);
+    return ADAMAH_OK;
+  }
+  flush_pending();
+  return launch_attn(nullptr, p, false, nullptr);
 }
 
 static int softmax_rows(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_rows, uint32_t row_size, float scale,
-                        float cap, bool rel) {
+                        float cap, bool rel) { ADAMAH_API();
   Map* m = get_f32_map(map_id);
   if (!m) return ADAMAH_ERR_INVALID;
   if (n_rows == 0 || row_size == 0) return ADAMAH_OK;
@@ -455,14 +756,14 @@ static int softmax_rows(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_ro
   count_launch();
   return check_launch();
 }
-int map_softmax_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_rows, uint32_t row_size) {
+int map_softmax_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_rows, uint32_t row_size) { ADAMAH_API();
   return softmax_rows(map_id, hs, hd, n_rows, row_size, 1.0f, 0.0f, true);
 }
-int map_softmax_abs_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_rows, uint32_t row_size) {
+int map_softmax_abs_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_rows, uint32_t row_size) { ADAMAH_API();
   return softmax_rows(map_id, hs, hd, n_rows, row_size, 1.0f, 0.0f, false);
 }
 int map_attn_softmax_abs_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_rows, uint32_t row_size, float scale,
-                             float cap) {
+                             float cap) { ADAMAH_API();
   return softmax_rows(map_id, hs, hd, n_rows, row_size, scale, cap, false);
 }
 

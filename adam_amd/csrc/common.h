@@ -59,6 +59,24 @@ struct Res {
   uint8_t* dptr = nullptr;
   std::vector<uint8_t> host;  // last uploaded contents; empty when the device wrote the resource
   bool host_valid = false;
+  bool contig = false;        // host copy is the uint32 sequence host[0], host[0]+1, host[0]+2, ...
+};
+
+// A row-wise op recorded inside a batch instead of being launched at once, so that neighbours can be
+// folded into one kernel when the batch is flushed.  All offsets are element offsets resolved from
+// the host copies of the handles at record time (any later handle upload flushes the queue first).
+enum PendKind : uint32_t { PK_RMSNORM = 1, PK_GEMV = 2, PK_OP2 = 3, PK_ARGMAX = 4, PK_SCORES = 5, PK_ATTN = 6 };
+struct PendOp {
+  uint32_t kind = 0;
+  uint32_t map_act = 0, map_wt = 0;
+  uint32_t a = 0, b = 0, c = 0, d = 0;   // RMSNORM: src, weight, dst, residual.  GEMV: x, W, y.  OP2: a, b, dst.
+  uint32_t n = 0, k = 0;                 // RMSNORM: n = dim.  GEMV/ARGMAX: k = K, n = N.  OP2: n elements.
+  uint32_t op = 0;                       // RMSNORM: 1 = with residual.  GEMV/ARGMAX: weight format.  OP2: op code.
+  uint32_t h[3] = {0, 0, 0};             // ARGMAX: idx, val, dst handles.  SCORES: q, K, score rows.  ATTN: scores, V, out
+  uint32_t rpg = 0;                      // ARGMAX: rows per group.  SCORES / ATTN: number of heads (ops)
+  float eps = 0.f;                       // RMSNORM: eps.  ATTN: score scale
+  float f2 = 0.f;                        // ATTN: soft cap
+  // SCORES: k = head dim, n = sequence length.  ATTN: n = sequence length, k = value dim.
 };
 
 struct Stats {
@@ -100,6 +118,10 @@ struct Ctx {
   hipEvent_t timer_ev[2] = {nullptr, nullptr};
   std::vector<PlanOp> plans[MAX_PLANS];
   bool plan_active[MAX_PLANS] = {false};
+  // deferred row-wise ops of the open batch
+  std::vector<PendOp> pend;
+  int no_defer = 0;              // > 0 while an entry point runs on library-owned scratch handles
+  uint32_t* sync_ctr = nullptr;  // device counters for last-workgroup epilogues, zero between launches
 };
 
 extern Ctx g;
@@ -118,6 +140,26 @@ uint32_t scratch_handle(int slot, const void* data, uint32_t n_bytes);
 void* stage_alloc(size_t n);                     // pinned region; enqueue its copy before allocating much more
 int h2d(void* dst, const void* src, size_t n);   // stream-ordered, source consumed before return
 int d2h(void* dst, const void* src, size_t n);   // stream-ordered copy + wait
+// Deferral of row-wise ops (fuse.hip).  Every extern "C" entry point that is not itself deferred
+// starts with ADAMAH_API(), which launches whatever is pending, so stream order equals call order.
+bool can_defer();                // inside a batch, fusion not disabled, no scratch handles involved
+void flush_pending();
+#define ADAMAH_API() do { if (!adamah::g.pend.empty()) adamah::flush_pending(); } while (0)
+// Element offset held by a single-entry handle whose host copy is known; false otherwise.
+bool res_scalar(uint32_t h, uint32_t* out);
+// First element of a handle whose host copy is a run of n consecutive indices; false otherwise.
+bool res_run(uint32_t h, uint64_t n, uint32_t* start);
+int launch_rmsnorm_v(const PendOp& p);
+int launch_op2_v(const PendOp& p);
+// Attention (attention.hip): stand-alone launches of queued ops, and the fused form.  launch_attn
+// runs scores (when sc != nullptr) and softmax . V; with leave_partials it stops before the merge
+// of the sequence splits and reports their layout so that the consumer can merge them itself.
+struct AttnPartials { const float* base; uint32_t n_splits, value_dim, n_ops, out0; };
+int launch_scores(const PendOp& sc);
+int launch_attn(const PendOp* sc, const PendOp& at, bool leave_partials, AttnPartials* ap);
+int launch_attn_combine(const PendOp& at, const AttnPartials& ap);
+bool attn_foldable(const PendOp& sc, const PendOp& at);
+
 inline void count_launch(int n = 1) { g.stats.dispatch += n; g.stats.barrier += n; g.stats.last_batch_dispatch += n; }
 int check_launch();                              // hipGetLastError -> ADAMAH code
 

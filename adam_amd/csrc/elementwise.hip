@@ -235,7 +235,7 @@ using namespace adamah;
 
 extern "C" {
 
-int map_op1_dev(uint32_t map_id, uint32_t op, uint32_t hs, uint32_t hd, uint32_t n) {
+int map_op1_dev(uint32_t map_id, uint32_t op, uint32_t hs, uint32_t hd, uint32_t n) { ADAMAH_API();
   EwArgs a; uint32_t h[2] = {hs, hd};
   int r = ew_setup(map_id, h, 2, n, &a);
   if (r || n == 0) return r;
@@ -245,6 +245,18 @@ int map_op1_dev(uint32_t map_id, uint32_t op, uint32_t hs, uint32_t hd, uint32_t
   return check_launch();
 }
 int map_op2_dev(uint32_t map_id, uint32_t op, uint32_t ha, uint32_t hb, uint32_t hd, uint32_t n) {
+  if ((op == 0 || op == 34 || op == 35) && n > 0 && can_defer()) {
+    // ADD / GEGLU / SWIGLU over three contiguous ranges known on the host: queue it for fusion
+    Map* m = get_f32_map(map_id);
+    PendOp p;
+    if (m && m->pack_size == 1 && res_run(ha, n, &p.a) && res_run(hb, n, &p.b) && res_run(hd, n, &p.c) &&
+        in_range(p.a, n, m->n_elems) && in_range(p.b, n, m->n_elems) && in_range(p.c, n, m->n_elems)) {
+      p.kind = PK_OP2; p.map_act = map_id; p.n = n; p.op = op;
+      g.pend.push_back(p);
+      return ADAMAH_OK;
+    }
+  }
+  flush_pending();
   EwArgs a; uint32_t h[3] = {ha, hb, hd};
   int r = ew_setup(map_id, h, 3, n, &a);
   if (r || n == 0) return r;
@@ -253,7 +265,7 @@ int map_op2_dev(uint32_t map_id, uint32_t op, uint32_t ha, uint32_t hb, uint32_t
   count_launch();
   return check_launch();
 }
-int map_broadcast_dev(uint32_t map_id, uint32_t op, uint32_t hs, uint32_t hk, uint32_t hd, uint32_t n) {
+int map_broadcast_dev(uint32_t map_id, uint32_t op, uint32_t hs, uint32_t hk, uint32_t hd, uint32_t n) { ADAMAH_API();
   EwArgs a; uint32_t h[3] = {hs, hk, hd};
   int r = ew_setup(map_id, h, 3, n, &a);
   if (r || n == 0) return r;
@@ -262,7 +274,7 @@ int map_broadcast_dev(uint32_t map_id, uint32_t op, uint32_t hs, uint32_t hk, ui
   count_launch();
   return check_launch();
 }
-int map_fma_dev(uint32_t map_id, uint32_t ha, uint32_t hb, uint32_t hc, uint32_t hd, uint32_t n) {
+int map_fma_dev(uint32_t map_id, uint32_t ha, uint32_t hb, uint32_t hc, uint32_t hd, uint32_t n) { ADAMAH_API();
   EwArgs a; uint32_t h[4] = {ha, hb, hc, hd};
   int r = ew_setup(map_id, h, 4, n, &a);
   if (r || n == 0) return r;
@@ -271,7 +283,7 @@ int map_fma_dev(uint32_t map_id, uint32_t ha, uint32_t hb, uint32_t hc, uint32_t
   count_launch();
   return check_launch();
 }
-int map_reduce_dev(uint32_t map_id, uint32_t op, uint32_t hs, uint32_t hd, uint32_t n) {
+int map_reduce_dev(uint32_t map_id, uint32_t op, uint32_t hs, uint32_t hd, uint32_t n) { ADAMAH_API();
   EwArgs a; uint32_t h[2] = {hs, hd};
   int r = ew_setup(map_id, h, 2, n, &a);
   if (r || n == 0) return r;
@@ -281,7 +293,7 @@ int map_reduce_dev(uint32_t map_id, uint32_t op, uint32_t hs, uint32_t hd, uint3
   return check_launch();
 }
 int map_layernorm_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t hg, uint32_t hb, uint32_t n_rows,
-                      uint32_t dim, float eps) {
+                      uint32_t dim, float eps) { ADAMAH_API();
   EwArgs a; uint32_t h[4] = {hs, hd, hg, hb};
   int r = ew_setup(map_id, h, 4, n_rows, &a);
   if (r || n_rows == 0 || dim == 0) return r;
@@ -289,7 +301,7 @@ int map_layernorm_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t hg, ui
   count_launch();
   return check_launch();
 }
-int map_argmax_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n) {
+int map_argmax_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n) { ADAMAH_API();
   Map* m = get_f32_map(map_id);
   if (!m) return ADAMAH_ERR_INVALID;
   const uint32_t* ld = res_u32(hd, 1);
@@ -300,11 +312,11 @@ int map_argmax_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n) {
   return check_launch();
 }
 // Sampling beyond argmax is not part of this build.
-int map_topk_dev(uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t) { return ADAMAH_ERR_INVALID; }
-int map_topp_dev(uint32_t, uint32_t, uint32_t, uint32_t, float, float) { return ADAMAH_ERR_INVALID; }
+int map_topk_dev(uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t) { ADAMAH_API(); return ADAMAH_ERR_INVALID; }
+int map_topp_dev(uint32_t, uint32_t, uint32_t, uint32_t, float, float) { ADAMAH_API(); return ADAMAH_ERR_INVALID; }
 
 int map_row_gather_xq8_dev(uint32_t map_act, uint32_t map_wt, uint32_t src_base, uint32_t dst_base, uint32_t row_idx,
-                           uint32_t row_size, float scale) {
+                           uint32_t row_size, float scale) { ADAMAH_API();
   Map* ma = get_f32_map(map_act);
   Map* mw = get_map(map_wt);
   if (!ma || !mw || mw->dtype != DTYPE_Q8 || !mw->qp || mw->group_size == 0) return ADAMAH_ERR_INVALID;
@@ -319,45 +331,45 @@ int map_row_gather_xq8_dev(uint32_t map_act, uint32_t map_wt, uint32_t src_base,
 
 // ---- host-locs variants: copy the locs into library-owned handles, then run the handle op ----
 #define UP(slot, ptr, n) scratch_handle(slot, ptr, (uint32_t)((n) * 4u))
-int map_op1(uint32_t map_id, uint32_t op, const uint32_t* ls, const uint32_t* ld, uint32_t n) {
+int map_op1(uint32_t map_id, uint32_t op, const uint32_t* ls, const uint32_t* ld, uint32_t n) { ADAMAH_API();
   if (n == 0) return get_map(map_id) ? ADAMAH_OK : ADAMAH_ERR_INVALID;
   uint32_t a = UP(0, ls, n), b = UP(1, ld, n);
   if (!a || !b) return ADAMAH_ERR_INVALID;
   return map_op1_dev(map_id, op, a, b, n);
 }
-int map_op2(uint32_t map_id, uint32_t op, const uint32_t* la, const uint32_t* lb, const uint32_t* ld, uint32_t n) {
+int map_op2(uint32_t map_id, uint32_t op, const uint32_t* la, const uint32_t* lb, const uint32_t* ld, uint32_t n) { ADAMAH_API();
   if (n == 0) return get_map(map_id) ? ADAMAH_OK : ADAMAH_ERR_INVALID;
   uint32_t a = UP(0, la, n), b = UP(1, lb, n), d = UP(2, ld, n);
   if (!a || !b || !d) return ADAMAH_ERR_INVALID;
   return map_op2_dev(map_id, op, a, b, d, n);
 }
-int map_broadcast(uint32_t map_id, uint32_t op, const uint32_t* ls, const uint32_t* lk, const uint32_t* ld, uint32_t n) {
+int map_broadcast(uint32_t map_id, uint32_t op, const uint32_t* ls, const uint32_t* lk, const uint32_t* ld, uint32_t n) { ADAMAH_API();
   if (n == 0) return get_map(map_id) ? ADAMAH_OK : ADAMAH_ERR_INVALID;
   uint32_t a = UP(0, ls, n), b = UP(1, lk, n), d = UP(2, ld, n);
   if (!a || !b || !d) return ADAMAH_ERR_INVALID;
   return map_broadcast_dev(map_id, op, a, b, d, n);
 }
-int map_reduce(uint32_t map_id, uint32_t op, const uint32_t* ls, const uint32_t* ld, uint32_t n) {
+int map_reduce(uint32_t map_id, uint32_t op, const uint32_t* ls, const uint32_t* ld, uint32_t n) { ADAMAH_API();
   if (n == 0) return get_map(map_id) ? ADAMAH_OK : ADAMAH_ERR_INVALID;
   uint32_t a = UP(0, ls, n), b = UP(1, ld, n);
   if (!a || !b) return ADAMAH_ERR_INVALID;
   return map_reduce_dev(map_id, op, a, b, n);
 }
 int map_matmul(uint32_t map_id, const uint32_t* la, const uint32_t* lb, const uint32_t* lc, uint32_t M, uint32_t K,
-               uint32_t N, uint32_t n_ops) {
+               uint32_t N, uint32_t n_ops) { ADAMAH_API();
   if (n_ops == 0) return get_map(map_id) ? ADAMAH_OK : ADAMAH_ERR_INVALID;
   uint32_t a = UP(0, la, n_ops), b = UP(1, lb, n_ops), c = UP(2, lc, n_ops);
   if (!a || !b || !c) return ADAMAH_ERR_INVALID;
   return map_matmul_dev(map_id, a, b, c, M, K, N, n_ops);
 }
-int map_softmax(uint32_t map_id, const uint32_t* ls, const uint32_t* ld, uint32_t n_rows, uint32_t row_size) {
+int map_softmax(uint32_t map_id, const uint32_t* ls, const uint32_t* ld, uint32_t n_rows, uint32_t row_size) { ADAMAH_API();
   if (n_rows == 0) return get_map(map_id) ? ADAMAH_OK : ADAMAH_ERR_INVALID;
   uint32_t a = UP(0, ls, n_rows), b = UP(1, ld, n_rows);
   if (!a || !b) return ADAMAH_ERR_INVALID;
   return map_softmax_dev(map_id, a, b, n_rows, row_size);
 }
 int map_layernorm(uint32_t map_id, const uint32_t* ls, const uint32_t* ld, const uint32_t* lg, const uint32_t* lb,
-                  uint32_t n_rows, uint32_t dim, float eps) {
+                  uint32_t n_rows, uint32_t dim, float eps) { ADAMAH_API();
   if (n_rows == 0) return get_map(map_id) ? ADAMAH_OK : ADAMAH_ERR_INVALID;
   uint32_t a = UP(0, ls, n_rows), b = UP(1, ld, n_rows), c = UP(2, lg, n_rows), d = UP(3, lb, n_rows);
   if (!a || !b || !c || !d) return ADAMAH_ERR_INVALID;

@@ -1,0 +1,213 @@
+// Deferred row-wise ops and their fusion.
+//
+// The reference records the ops of a batch into one command buffer and lets its fusion scheduler
+// merge neighbours (adamah.c:1629-1721 batch_begin/batch_end, :4670-4691 and :5653-5714 fusion
+// enable/flush).  Here a HIP stream already gives the ordering, so only the ops that can be folded
+// into a neighbouring kernel are held back: single-row RMSNorm (+ residual), the M = 1 Q4 GEMV and
+// GEMV + argmax, and ADD / GEGLU / SWIGLU over contiguous ranges.  They are queued with their operand
+// offsets resolved on the host; when the batch ends, on adamah_fusion_flush, or as soon as any other
+// entry point is called, the queue is launched in order with these folds applied:
+//
+//   RMSNorm(x -> n); GEMV(n -> y)                         -> GEMV that normalises while staging n
+//   RMSNorm+residual(o, r -> r); RMSNorm(r -> n); GEMV(n)  -> GEMV that does both norms while staging
+//   GEMV(-> y); ADD(r, y -> d)                            -> GEMV that also stores r + y
+//   GEMV(-> [g; u]); GEGLU/SWIGLU(g, u -> t)              -> GEMV over paired rows that also stores t
+//
+// Every folded op still stores its own result where it would have stored it alone, so the contents
+// of the maps after a batch do not depend on whether anything was folded.
+#include "gemv_common.h"
+#include <stdlib.h>
+
+namespace adamah {
+
+bool can_defer() {
+  static const int off = getenv("ADAMAH_NO_FUSE") ? atoi(getenv("ADAMAH_NO_FUSE")) : 0;
+  return g.batch_depth > 0 && g.no_defer == 0 && !off;
+}
+
+bool res_scalar(uint32_t h, uint32_t* out) {
+  const uint32_t* p = res_host(h, 1);
+  if (!p) return false;
+  *out = p[0];
+  return true;
+}
+
+bool res_run(uint32_t h, uint64_t n, uint32_t* start) {
+  Res* r = get_res(h);
+  if (!r || !r->host_valid || !r->contig || n * 4 > r->size_bytes || n == 0) return false;
+  *start = ((const uint32_t*)r->host.data())[0];
+  return true;
+}
+
+// ---- stand-alone kernels with operands passed by value -------------------------------------------
+__global__ void __launch_bounds__(1024)
+k_rmsnorm_v(const float* act, const float* wt, float* out, uint32_t src, uint32_t w, uint32_t res, uint32_t dst,
+            uint32_t dim, float eps, int add) {
+  __shared__ float sh[16];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  float ss = 0.f;
+  for (uint32_t i = tid; i < dim; i += 1024u) { const float x = act[(uint64_t)src + i]; ss = fmaf(x, x, ss); }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+  if (lane == 0) sh[wave] = ss;
+  __syncthreads();
+  ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; i++) ss += sh[i];
+  const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
+  for (uint32_t i = tid; i < dim; i += 1024u) {
+    float y = act[(uint64_t)src + i] * inv * wt[(uint64_t)w + i];
+    if (add) y += act[(uint64_t)res + i];
+    out[(uint64_t)dst + i] = y;
+  }
+}
+
+__global__ void __launch_bounds__(256)
+k_op2_v(float* data, uint32_t op, uint32_t a, uint32_t b, uint32_t d, uint32_t n) {
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  if (i >= n) return;
+  const float x = data[(uint64_t)a + i], y = data[(uint64_t)b + i];
+  float r;
+  if (op == 0) r = x + y;
+  else if (op == 34) r = gelu_tanh(x) * y;
+  else r = (x / (1.0f + expf(-x))) * y;
+  data[(uint64_t)d + i] = r;
+}
+
+int launch_rmsnorm_v(const PendOp& p) {
+  Map* ma = get_f32_map(p.map_act);
+  Map* mw = get_f32_map(p.map_wt);
+  if (!ma || !mw) return ADAMAH_ERR_INVALID;
+  float* a = (float*)ma->buf;
+  k_rmsnorm_v<<<1, 1024, 0, g.stream>>>(a, (const float*)mw->buf, a, p.a, p.b, p.d, p.c, p.n, p.eps, (int)p.op);
+  count_launch();
+  return check_launch();
+}
+
+int launch_op2_v(const PendOp& p) {
+  Map* ma = get_f32_map(p.map_act);
+  if (!ma) return ADAMAH_ERR_INVALID;
+  k_op2_v<<<cdiv(p.n, 256), 256, 0, g.stream>>>((float*)ma->buf, p.op, p.a, p.b, p.c, p.n);
+  count_launch();
+  return check_launch();
+}
+
+static bool disjoint(uint64_t a, uint64_t na, uint64_t b, uint64_t nb) { return a + na <= b || b + nb <= a; }
+
+static int launch_gemv(const PendOp& gp, const GemvFuse* fz) {
+  Map* ma = get_f32_map(gp.map_act);
+  Map* mw = get_map(gp.map_wt);
+  if (!ma || !mw) return ADAMAH_ERR_INVALID;
+  if (gp.kind == PK_GEMV) return launch_mfma_store((int)gp.op, ma, mw, gp.a, gp.b, gp.c, gp.k, gp.n, fz);
+  const uint32_t n_groups = cdiv(gp.n, gp.rpg);
+  const uint32_t *lidx = res_u32(gp.h[0], n_groups), *lval = res_u32(gp.h[1], n_groups), *ldst = res_u32(gp.h[2], 1);
+  if (!lidx || !lval || !ldst) return ADAMAH_ERR_INVALID;
+  int r = launch_mfma_argmax((int)gp.op, ma, mw, gp.a, gp.b, lidx, lval, gp.k, gp.n, gp.rpg, fz);
+  if (r) return r;
+  return launch_argmax_pairs(ma, lidx, lval, ldst, n_groups);
+}
+
+// Prologue folds need the whole activation row in the registers of one workgroup.
+static bool row_fits(const PendOp& gp) {
+  const uint32_t threads = gp.kind == PK_GEMV ? mfma_store_threads(gp.k, gp.n) : 256u;
+  return gp.k <= 8u * PRO_WPT * threads;
+}
+
+void flush_pending() {
+  if (g.pend.empty()) return;
+  std::vector<PendOp> q;
+  q.swap(g.pend);   // launches below must not see a non-empty queue
+  const size_t n = q.size();
+  size_t i = 0;
+  while (i < n) {
+    const PendOp& p = q[i];
+    auto is_gemv = [&](size_t j) { return j < n && (q[j].kind == PK_GEMV || q[j].kind == PK_ARGMAX); };
+    size_t gi = n;    // the GEMV this group is built around, if any
+    GemvFuse fz = {};
+    if (p.kind == PK_SCORES || p.kind == PK_ATTN) {
+      // decode attention: scores computed inside the softmax . V launch; the merge of the sequence
+      // splits moves into the GEMV that consumes the heads' outputs when the partials are small
+      const PendOp* sc = nullptr;
+      size_t ai = i;
+      if (p.kind == PK_SCORES) {
+        if (i + 1 < n && attn_foldable(p, q[i + 1])) { sc = &p; ai = i + 1; }
+        else { launch_scores(p); i++; continue; }
+      }
+      const PendOp& at = q[ai];
+      bool fold = false;
+      if (ai + 1 < n && q[ai + 1].kind == PK_GEMV && q[ai + 1].map_act == at.map_act) {
+        const PendOp& gp = q[ai + 1];
+        const uint32_t* oh = res_host(at.h[2], at.rpg);
+        fold = oh && gp.a == oh[0] && gp.k == at.rpg * at.k && (at.k & 7u) == 0;
+        for (uint32_t h = 1; fold && h < at.rpg; h++) fold = oh[h] == oh[0] + h * at.k;
+      }
+      AttnPartials ap = {nullptr, 1, 0, 0, 0};
+      launch_attn(sc, at, fold, &ap);
+      if (fold && ap.n_splits > 1) {   // partials left for the GEMV to merge
+        fz.pro = PRO_COMBINE; fz.c_partial = ap.base; fz.c_splits = ap.n_splits; fz.c_vd = at.k;
+        fz.p_dst = q[ai + 1].a;
+        gi = ai + 1;
+      }
+      if (gi == n) { i = ai + 1; continue; }
+    } else if (is_gemv(i)) gi = i;
+    else if (p.kind == PK_RMSNORM && p.op == 1 && i + 2 < n && q[i + 1].kind == PK_RMSNORM && q[i + 1].op == 0 &&
+             is_gemv(i + 2)) {
+      // RMSNorm + residual (t), RMSNorm of t (x), GEMV of x
+      const PendOp &m = q[i + 1], &gp = q[i + 2];
+      Map *mw1 = get_f32_map(p.map_wt), *mw2 = get_f32_map(m.map_wt);
+      const bool chain = m.map_act == p.map_act && gp.map_act == p.map_act && m.a == p.c && m.n == p.n &&
+                         gp.a == m.c && gp.k == m.n;
+      // t may overwrite the residual (ticket-protected) but nothing else that is read; x must not
+      // overwrite any input
+      const bool safe = disjoint(p.c, p.n, p.a, p.n) && (p.c == p.d || disjoint(p.c, p.n, p.d, p.n)) &&
+                        disjoint(m.c, m.n, p.a, p.n) && disjoint(m.c, m.n, p.d, p.n) && disjoint(m.c, m.n, p.c, p.n);
+      if (chain && safe && mw1 && mw2 && (p.n & 31u) == 0 && row_fits(gp) && g.sync_ctr) {
+        fz.pro = PRO_NORM2; fz.p_src = p.a; fz.p_src2 = p.b; fz.p_eps = p.eps; fz.p_wt = (const float*)mw1->buf;
+        fz.p_res = p.d; fz.p_tdst = p.c; fz.p_w2 = m.b; fz.p_eps2 = m.eps; fz.p_wt2 = (const float*)mw2->buf;
+        fz.p_dst = m.c; fz.counter = g.sync_ctr;
+        gi = i + 2;
+      }
+    } else if (p.kind == PK_RMSNORM && p.op == 0 && is_gemv(i + 1)) {
+      const PendOp& gp = q[i + 1];
+      Map* mw = get_f32_map(p.map_wt);
+      // the prologue reads its source in every workgroup while workgroup 0 stores its result
+      if (gp.map_act == p.map_act && gp.a == p.c && gp.k == p.n && disjoint(p.a, p.n, p.c, p.n) && (p.n & 31u) == 0 &&
+          mw && row_fits(gp)) {
+        fz.pro = PRO_RMSNORM; fz.p_src = p.a; fz.p_src2 = p.b; fz.p_dst = p.c; fz.p_eps = p.eps;
+        fz.p_wt = (const float*)mw->buf;
+        gi = i + 1;
+      }
+    }
+    if (gi == n) {   // nothing to fold: launch the op alone
+      if (p.kind == PK_RMSNORM) launch_rmsnorm_v(p);
+      else launch_op2_v(p);
+      i++;
+      continue;
+    }
+    const PendOp& gp = q[gi];
+    size_t last = gi;
+    if (gp.kind == PK_GEMV && gi + 1 < n && q[gi + 1].kind == PK_OP2 && q[gi + 1].map_act == gp.map_act) {
+      const PendOp& e = q[gi + 1];
+      // Result rows are stored while other workgroups still read the kernel's inputs: the epilogue's
+      // destination must not touch any of them, nor the GEMV result.
+      bool clear = disjoint(e.c, e.n, gp.c, gp.n) && disjoint(e.c, e.n, gp.a, gp.k);
+      if (fz.pro) clear = clear && disjoint(e.c, e.n, fz.p_src, gp.k);
+      if (fz.pro == PRO_NORM2) clear = clear && disjoint(e.c, e.n, fz.p_res, gp.k) && disjoint(e.c, e.n, fz.p_tdst, gp.k);
+      if (e.op == 0 && e.n == gp.n && (e.a == gp.c) != (e.b == gp.c)) {
+        const uint32_t r = e.a == gp.c ? e.b : e.a;   // the residual may be updated in place
+        bool ok = clear && (r == e.c || disjoint(r, e.n, e.c, e.n));
+        if (fz.pro == PRO_NORM2) ok = ok && disjoint(r, e.n, fz.p_tdst, gp.k);
+        if (ok) { fz.e_mode = EPIX_ADD; fz.e_res = r; fz.e_dst = e.c; last = gi + 1; }
+      } else if ((e.op == 34 || e.op == 35) && gp.n == 2u * e.n && (e.n & 1u) == 0 && e.a == gp.c && e.b == gp.c + e.n &&
+                 clear) {
+        // gate rows then up rows in one matrix, activation over the two halves of its result
+        fz.e_mode = e.op == 34 ? EPIX_GEGLU : EPIX_SWIGLU; fz.e_dst = e.c;
+        last = gi + 1;
+      }
+    }
+    launch_gemv(gp, (fz.pro || fz.e_mode) ? &fz : nullptr);
+    i = last + 1;
+  }
+}
+
+}  // namespace adamah

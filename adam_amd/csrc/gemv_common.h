@@ -33,6 +33,11 @@ template <int N> __device__ __forceinline__ float ubyte_f32(uint32_t w) {
   return r;
 }
 
+// tanh-form GELU with the constants of the reference shader (map_op2.comp:34-44)
+__device__ __forceinline__ float gelu_tanh(float a) {
+  return 0.5f * a * (1.0f + tanhf(0.797884583f * (a + 0.0447149985f * a * a * a)));
+}
+
 #define DPP_ADD(v, ctrl, rmask)                                                                    \
   v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, rmask, 0xF, false))
 
@@ -52,11 +57,47 @@ __device__ __forceinline__ float wave_sum_to_lane63(float v) {
 // activation map (store), or per-group partial (index, value) pairs at lidx/lval (argmax).  The
 // offsets are passed by value (the caller read them from the host copies of the handles), which
 // spares the kernel a dependent load before its first weight load.  `fmt`: FMT_Q4_B16 / FMT_Q4_AFF.
+//
+// `fz` (optional) folds neighbouring row-wise ops into the launch: a prologue that produces the
+// activation vector, and for the store variant an epilogue applied to the result rows.  Every folded
+// op also stores its own result where it would have stored it alone.  Offsets are element offsets in
+// the activation map unless noted.
+enum { PRO_NONE = 0, PRO_RMSNORM = 1, PRO_NORM2 = 2, PRO_COMBINE = 3 };
+enum { PRO_WPT = 2 };   // 8-element words a thread keeps in registers: K <= 16 * workgroup size
+enum { EPIX_NONE = 0, EPIX_ADD = 1, EPIX_GEGLU = 2, EPIX_SWIGLU = 3 };
+struct GemvFuse {
+  // PRO_RMSNORM: x = rmsnorm(src; w, eps)                    -> p_dst
+  // PRO_NORM2:   t = rmsnorm(src; w, eps) + res               -> p_tdst
+  //              x = rmsnorm(t; w2, eps2)                     -> p_dst
+  uint32_t pro;
+  uint32_t p_src, p_src2;   // source vector; weight w (element offset in p_wt)
+  uint32_t p_dst;
+  float p_eps;
+  const float* p_wt;
+  uint32_t p_res, p_tdst, p_w2;   // residual, destination of t, weight w2 (element offset in p_wt2)
+  float p_eps2;
+  const float* p_wt2;
+  uint32_t* counter;        // PRO_NORM2: zero-initialised device counter, left at zero
+  // PRO_COMBINE: x = merge of the split-sequence attention partials, heads side by side  -> p_dst
+  //   partial[(head * c_splits + s) * (c_vd + 2)] = {max, sum, values[c_vd]}
+  const float* c_partial;
+  uint32_t c_splits, c_vd;
+  // EPIX_ADD:            e_dst[row] = e_res[row] + y[row]
+  // EPIX_GEGLU / SWIGLU: the matrix is [gate rows; up rows], e_dst[i] = act(y[i]) * y[N/2 + i]
+  uint32_t e_mode;
+  uint32_t e_res, e_dst;
+};
+// Threads per workgroup the launchers will use for a matrix with N rows (store variant).
+uint32_t mfma_store_threads(uint32_t K, uint32_t N);
 int launch_mfma_store(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32_t b, uint32_t c, uint32_t K,
-                      uint32_t N);
+                      uint32_t N, const GemvFuse* fz = nullptr);
 int launch_mfma_argmax(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32_t b, const uint32_t* lidx,
-                       const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rows_per_group);
+                       const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rows_per_group,
+                       const GemvFuse* fz = nullptr);
 bool mfma_path_ok(const Map* mw, uint32_t K);
+// Second pass of the fused GEMV + argmax: best of the per-group partials, token id stored as float.
+int launch_argmax_pairs(const Map* ma, const uint32_t* lidx, const uint32_t* lval, const uint32_t* ldst,
+                        uint32_t n_groups);
 int tuning(const char* name, int dflt);
 
 }  // namespace adamah

@@ -33,6 +33,14 @@ typedef float f4u_t __attribute__((ext_vector_type(4), aligned(4)));
 
 enum { MF_U = 4 };   // 16-byte blocks per lane and step
 
+#ifdef ADAMAH_TRACE
+__device__ unsigned long long g_trace[64];
+#define TR(i) do { if (threadIdx.x == 0 && (blockIdx.x == 0 || blockIdx.x == gridDim.x - 1)) \
+  g_trace[(blockIdx.x == 0 ? 0 : 16) + (i)] = wall_clock64(); } while (0)
+#else
+#define TR(i) do {} while (0)
+#endif
+
 // LDS layout: 128 bytes per activation block = 8 chunks of 16 bytes.  Chunk 2*d + h holds digit d of
 // words 2h, 2h+1 as {even(2h), odd(2h), even(2h+1), odd(2h+1)} (even/odd = elements 0,2,4,6 / 1,3,5,7 of
 // the 8-element word, one byte each, matching the byte order of the unpacked codes); chunk 6 holds
@@ -46,12 +54,17 @@ struct PreM {
   float2 p[MF_U];
 };
 
-template <int FMT, int EPI, bool RAGGED>
+// PRO selects where the activation vector comes from: the map as it is, or the result of preceding
+// row-wise ops that have been folded into this kernel (RMSNorm of another vector; or RMSNorm +
+// residual followed by a second RMSNorm).  Every workgroup recomputes those small ops while it
+// stages the activations; their results are also stored where the unfused ops would have put them.
+template <int FMT, int EPI, bool RAGGED, int PRO>
 __global__ void __launch_bounds__(1024)
 k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, const float2* __restrict__ qp,
             const __half* __restrict__ d16, uint32_t a, uint32_t b_off, uint32_t c_out,
             const uint32_t* __restrict__ lidx, const uint32_t* __restrict__ lval, uint32_t K, uint32_t N,
-            uint32_t rows_per_group, uint32_t n_groups) {
+            uint32_t rows_per_group, uint32_t n_groups, GemvFuse fz) {
+  TR(0);
   constexpr bool B16 = (FMT == FMT_Q4_B16);
   extern __shared__ uint4 smem_u4[];
   uint8_t* xs = (uint8_t*)smem_u4;                    // nblk * 128 bytes
@@ -81,12 +94,21 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
     stride = 4u * nwav;
   }
 
+  // Row of lane-row l in the bundle that starts at row0.  With the gated-activation epilogue the
+  // matrix is [gate rows; up rows] (N/2 each) and a bundle pairs two gate rows with their up rows.
+  const bool glu = EPI == EPI_STORE && (fz.e_mode == EPIX_GEGLU || fz.e_mode == EPIX_SWIGLU);
+  auto row_of = [&](uint32_t row0, uint32_t end) -> uint32_t {
+    if (glu) return (row0 >> 1) + (l & 1u) + (l >> 1) * (N >> 1);
+    return min(row0 + l, end - 1u);
+  };
   auto load = [&](PreM& R, uint32_t row0, uint32_t chunk, uint32_t end) {
-    const uint32_t row = min(row0 + l, end - 1u);
+    const uint32_t row = row_of(row0, end);
     const uint64_t g0 = gbase + (uint64_t)row * nblk + chunk * 64u + bcol;
 #pragma unroll
     for (uint32_t u = 0; u < MF_U; u++) {
       uint64_t gi = g0 + u * 16u;
+      // blocks past the end of the row are clamped, not skipped: the number of loads per step has to be
+      // fixed for the prefetch to stay ahead (see the step loop)
       if (RAGGED) gi = gbase + (uint64_t)row * nblk + min(chunk * 64u + u * 16u + bcol, nblk - 1u);
       R.q[u] = *(const uint4*)(W + (gi << 4));
       if (B16) R.h[u] = d16[gi];
@@ -94,60 +116,202 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
     }
   };
 
-  PreM A, B;
-  if (first < seg_end) load(A, first, 0, seg_end);   // in flight while the activations are staged
+  PreM A, B;   // A's first loads stay in flight while the activations are staged
+  if (PRO == PRO_NONE && first < seg_end) load(A, first, 0, seg_end);
 
-  // ---- activations -> fixed-point digits; one 8-element word per thread, four threads per block --
-  {
-    const uint32_t nw = nblk * 4u;
-    for (uint32_t i0 = 0; i0 < nw; i0 += nthr) {
-      const uint32_t i = i0 + tid;
-      const bool live = i < nw;             // uniform over a thread quad
-      const f4u_t* p = (const f4u_t*)(act + a + (uint64_t)min(i, nw - 1u) * 8u);
-      const f4u_t v0 = p[0], v1 = p[1];
-      const float x[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-      float m = 0.f, poison = 0.f;          // poison turns NaN as soon as one element is Inf or NaN
+  // ---- activations -> fixed-point digits; one 8-element word per thread and pass, four threads per
+  // block.  stage() turns one word into digits; the prologues below decide what the word is. ------
+  const uint32_t nw = nblk * 4u;
+  auto stage = [&](uint32_t i, bool live, const float* x) {
+    float m = 0.f, poison = 0.f;          // poison turns NaN as soon as one element is Inf or NaN
 #pragma unroll
-      for (int k = 0; k < 8; k++) { m = fmaxf(m, fabsf(x[k])); poison = fmaf(x[k], 0.f, poison); }
-      m = fmaxf(m, __shfl_xor(m, 1, 64)); m = fmaxf(m, __shfl_xor(m, 2, 64));
-      poison += __shfl_xor(poison, 1, 64); poison += __shfl_xor(poison, 2, 64);
-      const uint32_t e = (__float_as_uint(m) >> 23) & 0xFFu;
-      float s = 1.f, fs = 1.f;              // |x * s| < 2^21 when the block is finite and not tiny
-      if (e >= 21u && e <= 254u) { s = __uint_as_float((274u - e) << 23); fs = __uint_as_float((e - 20u) << 23); }
-      if (poison != poison) fs = poison;    // the block's result is NaN, as it would be in float arithmetic
-      int d0[8], d1[8], d2[8], sx = 0;
+    for (int k = 0; k < 8; k++) { m = fmaxf(m, fabsf(x[k])); poison = fmaf(x[k], 0.f, poison); }
+    m = fmaxf(m, __shfl_xor(m, 1, 64)); m = fmaxf(m, __shfl_xor(m, 2, 64));
+    poison += __shfl_xor(poison, 1, 64); poison += __shfl_xor(poison, 2, 64);
+    const uint32_t e = (__float_as_uint(m) >> 23) & 0xFFu;
+    float s = 1.f, fs = 1.f;              // |x * s| < 2^21 when the block is finite and not tiny
+    if (e >= 21u && e <= 254u) { s = __uint_as_float((274u - e) << 23); fs = __uint_as_float((e - 20u) << 23); }
+    if (poison != poison) fs = poison;    // the block's result is NaN, as it would be in float arithmetic
+    int d0[8], d1[8], d2[8], sx = 0;
 #pragma unroll
-      for (int k = 0; k < 8; k++) {
-        int xi = (e >= 21u && e <= 254u) ? (int)rintf(x[k] * s) : 0;
-        xi = min(max(xi, -(1 << 21)), (1 << 21) - 1);
-        sx += xi;
-        d0[k] = xi >> 14; d1[k] = (xi >> 7) & 127; d2[k] = xi & 127;
+    for (int k = 0; k < 8; k++) {
+      int xi = (e >= 21u && e <= 254u) ? (int)rintf(x[k] * s) : 0;
+      xi = min(max(xi, -(1 << 21)), (1 << 21) - 1);
+      sx += xi;
+      d0[k] = xi >> 14; d1[k] = (xi >> 7) & 127; d2[k] = xi & 127;
+    }
+    sx += __shfl_xor(sx, 1, 64); sx += __shfl_xor(sx, 2, 64);
+    if (live) {
+      const uint32_t blk = i >> 2, j = i & 3u;
+      uint8_t* bp = xs + (size_t)blk * 128u;
+      auto pack = [](const int* d, int o) {
+        return (uint32_t)(d[o] & 255) | ((uint32_t)(d[o + 2] & 255) << 8) | ((uint32_t)(d[o + 4] & 255) << 16) |
+               ((uint32_t)(d[o + 6] & 255) << 24);
+      };
+      const uint32_t h = j >> 1, wo = (j & 1u) * 8u;
+      *(uint2*)(bp + chunk_off(0u + h, blk) + wo) = make_uint2(pack(d0, 0), pack(d0, 1));
+      *(uint2*)(bp + chunk_off(2u + h, blk) + wo) = make_uint2(pack(d1, 0), pack(d1, 1));
+      *(uint2*)(bp + chunk_off(4u + h, blk) + wo) = make_uint2(pack(d2, 0), pack(d2, 1));
+      if (j == 0) {
+        uint4 prm;
+        prm.x = (uint32_t)(B16 ? 8 * sx : 0);              // zero-point term of the block format, integer
+        prm.y = __float_as_uint(fs);
+        prm.z = __float_as_uint((float)sx * fs);           // sum of the block's activations (affine format)
+        prm.w = 0;
+        *(uint4*)(bp + chunk_off(6u, blk)) = prm;
       }
-      sx += __shfl_xor(sx, 1, 64); sx += __shfl_xor(sx, 2, 64);
-      if (live) {
-        const uint32_t blk = i >> 2, j = i & 3u;
-        uint8_t* bp = xs + (size_t)blk * 128u;
-        auto pack = [](const int* d, int o) {
-          return (uint32_t)(d[o] & 255) | ((uint32_t)(d[o + 2] & 255) << 8) | ((uint32_t)(d[o + 4] & 255) << 16) |
-                 ((uint32_t)(d[o + 6] & 255) << 24);
-        };
-        const uint32_t h = j >> 1, wo = (j & 1u) * 8u;
-        *(uint2*)(bp + chunk_off(0u + h, blk) + wo) = make_uint2(pack(d0, 0), pack(d0, 1));
-        *(uint2*)(bp + chunk_off(2u + h, blk) + wo) = make_uint2(pack(d1, 0), pack(d1, 1));
-        *(uint2*)(bp + chunk_off(4u + h, blk) + wo) = make_uint2(pack(d2, 0), pack(d2, 1));
-        if (j == 0) {
-          uint4 prm;
-          prm.x = (uint32_t)(B16 ? 8 * sx : 0);              // zero-point term of the block format, integer
-          prm.y = __float_as_uint(fs);
-          prm.z = __float_as_uint((float)sx * fs);           // sum of the block's activations (affine format)
-          prm.w = 0;
-          *(uint4*)(bp + chunk_off(6u, blk)) = prm;
+    }
+  };
+  auto load8 = [&](const float* p, float* v) {
+    const f4u_t v0 = ((const f4u_t*)p)[0], v1 = ((const f4u_t*)p)[1];
+    v[0] = v0.x; v[1] = v0.y; v[2] = v0.z; v[3] = v0.w; v[4] = v1.x; v[5] = v1.y; v[6] = v1.z; v[7] = v1.w;
+  };
+  auto block_sum = [&](float v) {     // sum over the workgroup, same value in every thread
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    __syncthreads();                  // red_f may still be read from the previous use
+    if (lane == 0) red_f[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (uint32_t w = 0; w < nwav; w++) t += red_f[w];
+    return t;
+  };
+
+  float nrm1 = 1.f;
+  uint32_t ticket = 0;
+  if (PRO == PRO_NONE) {
+    // four passes of loads are issued before the first word is converted
+    for (uint32_t i0 = 0; i0 < nw; i0 += 4u * nthr) {
+      float x[4][8];
+#pragma unroll
+      for (uint32_t u = 0; u < 4; u++) load8(act + a + (uint64_t)min(i0 + u * nthr + tid, nw - 1u) * 8u, x[u]);
+#pragma unroll
+      for (uint32_t u = 0; u < 4; u++)
+        if (i0 + u * nthr + (tid & ~63u) < nw)   // wave-uniform: waves without words skip the conversion
+          stage(i0 + u * nthr + tid, i0 + u * nthr + tid < nw, x[u]);
+    }
+  } else if (PRO == PRO_COMBINE) {
+    // Folded merge of the attention partials (same arithmetic as the stand-alone merge kernel):
+    // M = max m_s, w_s = e^(m_s - M), L = sum l_s w_s, x = sum_s o_s w_s / L, per head.
+    if (first < seg_end) load(A, first, 0, seg_end);
+    const uint32_t stride = fz.c_vd + 2u;
+    for (uint32_t i0 = 0; i0 < nw; i0 += nthr) {
+      const uint32_t i = i0 + tid, ic = min(i, nw - 1u);
+      const uint32_t head = (ic * 8u) / fz.c_vd, j0 = (ic * 8u) % fz.c_vd;
+      const float* pp = fz.c_partial + (uint64_t)head * fz.c_splits * stride;
+      float M = -9.99999968e+37f;
+      for (uint32_t sp = 0; sp < fz.c_splits; sp++) M = fmaxf(M, pp[(uint64_t)sp * stride]);
+      float L = 0.f, x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      for (uint32_t sp = 0; sp < fz.c_splits; sp++) {
+        const float wgt = expf(pp[(uint64_t)sp * stride] - M);
+        L = fmaf(pp[(uint64_t)sp * stride + 1], wgt, L);
+        float o[8];
+        load8(pp + (uint64_t)sp * stride + 2 + j0, o);
+#pragma unroll
+        for (int k = 0; k < 8; k++) x[k] = fmaf(o[k], wgt, x[k]);
+      }
+      const float invL = 1.0f / L;
+#pragma unroll
+      for (int k = 0; k < 8; k++) x[k] *= invL;
+      if (i0 + (tid & ~63u) >= nw) continue;   // wave-uniform: nothing of this pass belongs to the wave
+      if (blockIdx.x == 0 && i < nw) {
+        f4u_t* o = (f4u_t*)(act_out + fz.p_dst + (uint64_t)i * 8u);
+        o[0] = (f4u_t){x[0], x[1], x[2], x[3]}; o[1] = (f4u_t){x[4], x[5], x[6], x[7]};
+      }
+      stage(i, i < nw, x);
+    }
+  } else {
+    // Folded row-wise ops.  Every thread keeps its (at most PRO_WPT) words in registers from one
+    // round of loads, so the norms cost block reductions but no further trips to memory.
+    //   PRO_RMSNORM:  x = src * rsqrt(mean(src^2) + eps) * w                       (stored at p_dst)
+    //   PRO_NORM2:    t = src * rsqrt(mean(src^2) + eps) * w + res                 (stored at p_tdst)
+    //                 x = t * rsqrt(mean(t^2) + eps2) * w2                          (stored at p_dst)
+    float v[PRO_WPT][8], wv[PRO_WPT][8], rv[PRO_WPT][8], w2v[PRO_WPT][8];
+    bool live[PRO_WPT];
+    float ss = 0.f;
+    bool mine[PRO_WPT];   // wave-uniform: the wave has words in this pass at all
+#pragma unroll
+    for (uint32_t u = 0; u < PRO_WPT; u++) {
+      const uint32_t i = u * nthr + tid;
+      live[u] = i < nw;
+      mine[u] = u * nthr + (tid & ~63u) < nw;
+#pragma unroll
+      for (int k = 0; k < 8; k++) { v[u][k] = 0.f; wv[u][k] = 0.f; rv[u][k] = 0.f; w2v[u][k] = 0.f; }
+      if (!mine[u]) continue;
+      const uint64_t e0 = (uint64_t)min(i, nw - 1u) * 8u;
+      load8(act + fz.p_src + e0, v[u]);
+      load8(fz.p_wt + fz.p_src2 + e0, wv[u]);
+      if (PRO == PRO_NORM2) { load8(act + fz.p_res + e0, rv[u]); load8(fz.p_wt2 + fz.p_w2 + e0, w2v[u]); }
+    }
+    __builtin_amdgcn_sched_barrier(0);   // activation loads first: they are waited for first
+    if (first < seg_end) load(A, first, 0, seg_end);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (uint32_t u = 0; u < PRO_WPT; u++)
+      if (mine[u]) {
+#pragma unroll
+        for (int k = 0; k < 8; k++) if (live[u]) ss = fmaf(v[u][k], v[u][k], ss);
+      }
+    // The ticket taken below tells other workgroups that this one has read `res`: its loads must have
+    // returned, not merely been issued.  Naming the registers as inputs of an (empty) asm makes the
+    // compiler wait for exactly those loads here.
+    if (PRO == PRO_NORM2) {
+#pragma unroll
+      for (uint32_t u = 0; u < PRO_WPT; u++)
+#pragma unroll
+        for (int k = 0; k < 8; k++) asm volatile("" ::"v"(rv[u][k]));
+    }
+    TR(1);
+    nrm1 = 1.0f / sqrtf(block_sum(ss) / (float)K + fz.p_eps);
+    TR(2);
+    const float nrm = nrm1;
+    if (PRO == PRO_NORM2) {
+      // Every thread of this workgroup has consumed `res` (the reduction above ends in a barrier).
+      // t usually goes back into `res` (residual updated in place), which other workgroups may not
+      // have read yet, so it is stored by whichever workgroup draws the last ticket.  The ticket is
+      // drawn here and looked at after staging, so nobody waits for the atomic's round trip.
+      if (wave == 0 && lane == 0) ticket = atomicAdd(fz.counter, 1u);
+      float ss2 = 0.f;
+#pragma unroll
+      for (uint32_t u = 0; u < PRO_WPT; u++)
+        if (mine[u]) {
+#pragma unroll
+          for (int k = 0; k < 8; k++) {
+            v[u][k] = v[u][k] * nrm * wv[u][k] + rv[u][k];
+            if (live[u]) ss2 = fmaf(v[u][k], v[u][k], ss2);
+          }
         }
+      const float nrm2 = 1.0f / sqrtf(block_sum(ss2) / (float)K + fz.p_eps2);
+      TR(3);
+#pragma unroll
+      for (uint32_t u = 0; u < PRO_WPT; u++)
+        if (mine[u]) {
+#pragma unroll
+          for (int k = 0; k < 8; k++) v[u][k] = v[u][k] * nrm2 * w2v[u][k];
+        }
+    } else {
+#pragma unroll
+      for (uint32_t u = 0; u < PRO_WPT; u++)
+        if (mine[u]) {
+#pragma unroll
+          for (int k = 0; k < 8; k++) v[u][k] = v[u][k] * nrm * wv[u][k];
+        }
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < PRO_WPT; u++) {
+      const uint32_t i = u * nthr + tid;
+      if (mine[u]) {
+        if (blockIdx.x == 0 && live[u]) {
+          f4u_t* o = (f4u_t*)(act_out + fz.p_dst + (uint64_t)i * 8u);
+          o[0] = (f4u_t){v[u][0], v[u][1], v[u][2], v[u][3]}; o[1] = (f4u_t){v[u][4], v[u][5], v[u][6], v[u][7]};
+        }
+        stage(i, live[u], v[u]);
       }
     }
   }
+  TR(4);
   __syncthreads();
-
+  TR(5);
   uint32_t nib = 0x0F0F0F0Fu;
   asm volatile("" : "+s"(nib));             // opaque, so it stays in a register instead of a literal per use
   const uint32_t dig = l < 3u ? l : 0u;     // lane 3 of a block repeats digit 0, its result row is unused
@@ -202,11 +366,46 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       y += __shfl_xor(y, 4, 64); y += __shfl_xor(y, 8, 64);
       y += __shfl_xor(y, 16, 64); y += __shfl_xor(y, 32, 64);
       acc = 0.f;
-      const uint32_t row = row0 + l;
-      if (row < end && bcol == 0u) {
-        if (EPI == EPI_STORE) act_out[(uint64_t)c_out + row] = y;
-        else if (better(y, row, best_v, best_i)) { best_v = y; best_i = row; }
+      if (glu) {
+        // lanes 0, 1 hold gate rows, lanes 2, 3 the matching up rows
+        const float yu = __shfl_down(y, 2, 64);
+        if (lane < 4u) {
+          const uint32_t row = row_of(row0, end);
+          act_out[(uint64_t)c_out + row] = y;
+          if (lane < 2u) {
+            const float t = fz.e_mode == EPIX_GEGLU ? gelu_tanh(y) * yu : (y / (1.0f + expf(-y))) * yu;
+            act_out[(uint64_t)fz.e_dst + row] = t;
+          }
+        }
+      } else {
+        const uint32_t row = row0 + l;
+        if (row < end && bcol == 0u) {
+          if (EPI == EPI_STORE) {
+            act_out[(uint64_t)c_out + row] = y;
+            if (fz.e_mode == EPIX_ADD) act_out[(uint64_t)fz.e_dst + row] = act[(uint64_t)fz.e_res + row] + y;
+          } else if (better(y, row, best_v, best_i)) { best_v = y; best_i = row; }
+        }
       }
+    }
+  };
+
+  // PRO_NORM2, last ticket: every other workgroup has read the residual, so t may now be stored over
+  // it.  Looked at only here, after the workgroup's own rows, so that nobody waits for the atomic; the
+  // whole workgroup then recomputes t for the row.
+  auto finish_norm2 = [&]() {
+    if (PRO != PRO_NORM2) return;
+    if (wave == 0 && lane == 0) red_i[0] = ticket;
+    __syncthreads();
+    if (red_i[0] != gridDim.x - 1u) return;
+    if (tid == 0) atomicExch(fz.counter, 0u);      // ready for the next launch on the stream
+    const f4u_t* ps = (const f4u_t*)(act + fz.p_src);
+    const f4u_t* pw = (const f4u_t*)(fz.p_wt + fz.p_src2);
+    const f4u_t* pr = (const f4u_t*)(act + fz.p_res);
+    f4u_t* pd = (f4u_t*)(act_out + fz.p_tdst);
+    for (uint32_t i = tid; i < (K >> 2); i += nthr) {
+      const f4u_t sv = ps[i], wv4 = pw[i], rv4 = pr[i];
+      pd[i] = (f4u_t){sv.x * nrm1 * wv4.x + rv4.x, sv.y * nrm1 * wv4.y + rv4.y, sv.z * nrm1 * wv4.z + rv4.z,
+                      sv.w * nrm1 * wv4.w + rv4.w};
     }
   };
 
@@ -218,7 +417,8 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       const uint32_t T = ((seg_end - first + stride - 1u) / stride) * C;
       uint32_t row_a = first, ch_a = 0, row_b, ch_b, row_n = first, ch_n = 0;
       if (++ch_n == C) { ch_n = 0; row_n += stride; }
-      for (uint32_t t = 0; t < T; t += 2) {
+      if (T == 1) compute(A, first, 0, seg_end);   // nothing to prefetch
+      else for (uint32_t t = 0; t < T; t += 2) {
         row_b = row_n; ch_b = ch_n;
         load(B, row_b, ch_b, seg_end);
         __builtin_amdgcn_sched_barrier(0);   // keep the prefetch ahead of the arithmetic
@@ -232,6 +432,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
         compute(B, row_b, ch_b, seg_end);
       }
     }
+    TR(6);
     if (EPI == EPI_STORE) break;
     // argmax: next group's first loads go out before this group's partial is merged
     const uint32_t done = grp;
@@ -262,6 +463,9 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
     best_v = NEG_FLT_MAX; best_i = INVALID_IDX;
     if (!more) break;
   }
+  TR(7);
+  finish_norm2();
+  TR(8);
 }
 
 // ---- host side -----------------------------------------------------------------------------------
@@ -271,19 +475,35 @@ bool mfma_path_ok(const Map* mw, uint32_t K) {
   return mw->dtype == DTYPE_Q4 && mw->group_size == 32 && K >= 32 && (K & 31u) == 0 && mfma_smem(K) <= 64000;
 }
 
-template <int EPI>
-static int launch_mfma(int fmt, uint32_t grid, uint32_t threads, const Map* ma, const Map* mw, uint32_t a, uint32_t b,
-                       uint32_t c, const uint32_t* lidx, const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rpg,
-                       uint32_t n_groups) {
+template <int EPI, int PRO>
+static void launch_mfma_p(int fmt, uint32_t grid, uint32_t threads, const Map* ma, const Map* mw, uint32_t a, uint32_t b,
+                          uint32_t c, const uint32_t* lidx, const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rpg,
+                          uint32_t n_groups, const GemvFuse& fz) {
   float* act = (float*)ma->buf;
   const size_t smem = mfma_smem(K);
   const bool ragged = (K & 2047u) != 0;
-#define MK(F, R)                                                                                                   \
-  k_gemv_mfma<F, EPI, R><<<grid, threads, smem, g.stream>>>(act, act, mw->buf, mw->qp, mw->d16, a, b, c, lidx, lval, K, \
-                                                            N, rpg, n_groups)
+#define MK(F, R)                                                                                                  \
+  k_gemv_mfma<F, EPI, R, PRO><<<grid, threads, smem, g.stream>>>(act, act, mw->buf, mw->qp, mw->d16, a, b, c, lidx, \
+                                                                 lval, K, N, rpg, n_groups, fz)
   if (fmt == FMT_Q4_B16) { if (ragged) MK(FMT_Q4_B16, true); else MK(FMT_Q4_B16, false); }
   else { if (ragged) MK(FMT_Q4_AFF, true); else MK(FMT_Q4_AFF, false); }
 #undef MK
+}
+
+template <int EPI>
+static int launch_mfma(int fmt, uint32_t grid, uint32_t threads, const Map* ma, const Map* mw, uint32_t a, uint32_t b,
+                       uint32_t c, const uint32_t* lidx, const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rpg,
+                       uint32_t n_groups, const GemvFuse* fzp) {
+  GemvFuse fz = {};
+  if (fzp) fz = *fzp;
+#define MP(P) launch_mfma_p<EPI, P>(fmt, grid, threads, ma, mw, a, b, c, lidx, lval, K, N, rpg, n_groups, fz)
+  switch (fz.pro) {
+    case PRO_RMSNORM: MP(PRO_RMSNORM); break;
+    case PRO_NORM2: MP(PRO_NORM2); break;
+    case PRO_COMBINE: MP(PRO_COMBINE); break;
+    default: MP(PRO_NONE); break;
+  }
+#undef MP
   count_launch();
   return check_launch();
 }
@@ -303,20 +523,33 @@ static void mfma_shape(uint32_t K, uint32_t units, uint32_t* grid, uint32_t* thr
   *grid = std::max(1u, std::min<uint32_t>(cdiv(units, waves), (uint32_t)g.n_cu * wg_per_cu));
 }
 
-int launch_mfma_store(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32_t b, uint32_t c, uint32_t K,
-                      uint32_t N) {
+uint32_t mfma_store_threads(uint32_t K, uint32_t N) {
   uint32_t grid, threads;
   mfma_shape(K, cdiv(N, 4), &grid, &threads);
-  return launch_mfma<EPI_STORE>(fmt, grid, threads, ma, mw, a, b, c, nullptr, nullptr, K, N, 0, 0);
+  return threads;
+}
+
+int launch_mfma_store(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32_t b, uint32_t c, uint32_t K,
+                      uint32_t N, const GemvFuse* fz) {
+  uint32_t grid, threads;
+  mfma_shape(K, cdiv(N, 4), &grid, &threads);
+  return launch_mfma<EPI_STORE>(fmt, grid, threads, ma, mw, a, b, c, nullptr, nullptr, K, N, 0, 0, fz);
 }
 
 int launch_mfma_argmax(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32_t b, const uint32_t* lidx,
-                       const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rows_per_group) {
+                       const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rows_per_group, const GemvFuse* fz) {
   const uint32_t n_groups = cdiv(N, rows_per_group);
   uint32_t grid, threads;
   mfma_shape(K, n_groups * 16u, &grid, &threads);   // one workgroup per group at a time
   grid = std::min(grid, n_groups);
-  return launch_mfma<EPI_ARGMAX>(fmt, grid, threads, ma, mw, a, b, 0, lidx, lval, K, N, rows_per_group, n_groups);
+  return launch_mfma<EPI_ARGMAX>(fmt, grid, threads, ma, mw, a, b, 0, lidx, lval, K, N, rows_per_group, n_groups, fz);
 }
 
 }  // namespace adamah
+
+#ifdef ADAMAH_TRACE
+extern "C" int adamah_hip_trace_read(unsigned long long* out) {
+  hipStreamSynchronize(adamah::g.stream);
+  return hipMemcpyFromSymbol(out, HIP_SYMBOL(adamah::g_trace), 64 * sizeof(unsigned long long)) == hipSuccess ? 0 : -1;
+}
+#endif

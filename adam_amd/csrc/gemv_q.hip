@@ -526,7 +526,18 @@ int op_matmul_t_xq(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t h
     // Q4: int8 matrix-instruction kernel.  Q8 (and Q4 on request): float32 kernels, activations in
     // registers with waves sharing a row when K > 8192, else staged in LDS
     const int impl = tuning("ADAMAH_GEMV_IMPL", mfma_path_ok(mw, K) ? 3 : K > 8192 ? 1 : 0);
-    if (impl == 3 && mfma_path_ok(mw, K)) return launch_mfma_store(fmt, ma, mw, (uint32_t)a0, (uint32_t)b0, ch[0], K, N);
+    if (impl == 3 && mfma_path_ok(mw, K)) {
+      if (can_defer()) {   // queue it: neighbouring row-wise ops may be folded into the launch
+        PendOp p;
+        p.kind = PK_GEMV; p.map_act = map_act; p.map_wt = map_wt; p.a = (uint32_t)a0; p.b = (uint32_t)b0; p.c = ch[0];
+        p.k = K; p.n = N; p.op = (uint32_t)fmt;
+        g.pend.push_back(p);
+        return ADAMAH_OK;
+      }
+      flush_pending();
+      return launch_mfma_store(fmt, ma, mw, (uint32_t)a0, (uint32_t)b0, ch[0], K, N);
+    }
+    flush_pending();
     if (impl == 1) {
       const uint32_t ks = K <= 4096 ? 1 : K <= 8192 ? 2 : 4;
       const uint32_t step = (4 / ks) * 4;                       // rows one workgroup pass covers
@@ -538,6 +549,7 @@ int op_matmul_t_xq(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t h
                                    (uint32_t)tuning("ADAMAH_GEMV_RPG", 16));
   }
 generic:
+  flush_pending();
   dim3 grid(cdiv(N, 4), M, n_ops);
   float* act = (float*)ma->buf;
   const bool q4 = dtype == DTYPE_Q4;
@@ -571,6 +583,14 @@ int op_matvec_argmax(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t
   int r;
   if (locs_ok && block_path_ok(ma, mw, ha, hb, K, N, &a0, &b0)) {
     const int impl = tuning("ADAMAH_GEMV_IMPL", mfma_path_ok(mw, K) ? 3 : K > 8192 ? 1 : 0);
+    if (impl == 3 && mfma_path_ok(mw, K) && can_defer()) {
+      PendOp p;
+      p.kind = PK_ARGMAX; p.map_act = map_act; p.map_wt = map_wt; p.a = (uint32_t)a0; p.b = (uint32_t)b0; p.k = K; p.n = N;
+      p.op = (uint32_t)fmt_of(mw, b0, (uint64_t)N * K); p.h[0] = hidx; p.h[1] = hval; p.h[2] = hdst; p.rpg = rows_per_group;
+      g.pend.push_back(p);
+      return ADAMAH_OK;
+    }
+    flush_pending();
     if (impl == 3 && mfma_path_ok(mw, K))
       r = launch_mfma_argmax(fmt_of(mw, b0, (uint64_t)N * K), ma, mw, (uint32_t)a0, (uint32_t)b0, lidx, lval, K, N,
                              rows_per_group);
@@ -581,6 +601,7 @@ int op_matvec_argmax(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t
       r = launch_block<EPI_ARGMAX>(fmt_of(mw, b0, (uint64_t)N * K), ma, mw, la, lb, nullptr, lidx, lval, K, N,
                                    rows_per_group);
   } else {
+    flush_pending();
     const uint32_t *ah = res_host(ha, 1), *bh = res_host(hb, 1);
     if (ah && !in_range(ah[0], K, ma->n_elems)) return ADAMAH_ERR_INVALID;
     if (bh && !in_range(bh[0], (uint64_t)N * K, mw->n_elems)) return ADAMAH_ERR_INVALID;
@@ -597,6 +618,11 @@ int op_matvec_argmax(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t
     r = check_launch();
   }
   if (r) return r;
+  return launch_argmax_pairs(ma, lidx, lval, ldst, n_groups);
+}
+
+int launch_argmax_pairs(const Map* ma, const uint32_t* lidx, const uint32_t* lval, const uint32_t* ldst,
+                        uint32_t n_groups) {
   k_argmax_pairs<<<1, 256, 0, g.stream>>>((float*)ma->buf, lidx, lval, ldst, n_groups, ma->n_elems);
   count_launch();
   return check_launch();
@@ -633,7 +659,7 @@ int map_matvec_argmax_t_xq8_dev(uint32_t ma, uint32_t mw, uint32_t a, uint32_t b
   return op_matvec_argmax(DTYPE_Q8, ma, mw, a, b, idx, val, dst, K, N, rpg);
 }
 
-int adamah_hip_debug_dequant(uint32_t map_id, uint64_t start, uint64_t count, float* out) {
+int adamah_hip_debug_dequant(uint32_t map_id, uint64_t start, uint64_t count, float* out) { ADAMAH_API();
   Map* m = get_map(map_id);
   if (!m || !m->qp || m->group_size != 32 || !out || count == 0 || !in_range(start, count, m->n_elems))
     return ADAMAH_ERR_INVALID;

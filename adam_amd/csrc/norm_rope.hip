@@ -126,6 +126,18 @@ static int rmsnorm_impl(uint32_t map_act, uint32_t map_wt, uint32_t hs, uint32_t
   Map* mw = get_f32_map(map_wt);
   if (!ma || !mw) return ADAMAH_ERR_INVALID;
   if (n_rows == 0) return ADAMAH_OK;
+  if (n_rows == 1 && dim > 0 && can_defer()) {
+    // single row with operands known on the host: queue it, a neighbouring GEMV may absorb it
+    PendOp p;
+    if (res_scalar(hs, &p.a) && res_scalar(hw, &p.b) && res_scalar(hd, &p.c) && (!add || res_scalar(hr, &p.d)) &&
+        in_range(p.a, dim, ma->n_elems) && in_range(p.c, dim, ma->n_elems) && in_range(p.b, dim, mw->n_elems) &&
+        (!add || in_range(p.d, dim, ma->n_elems))) {
+      p.kind = PK_RMSNORM; p.map_act = map_act; p.map_wt = map_wt; p.n = dim; p.op = add ? 1u : 0u; p.eps = eps;
+      g.pend.push_back(p);
+      return ADAMAH_OK;
+    }
+  }
+  flush_pending();
   const uint32_t *ls = res_u32(hs, n_rows), *lw = res_u32(hw, n_rows), *ld = res_u32(hd, n_rows);
   const uint32_t* lr = add ? res_u32(hr, n_rows) : ls;
   if (!ls || !lw || !ld || !lr) return ADAMAH_ERR_INVALID;
@@ -159,7 +171,7 @@ int map_rmsnorm_add_dev(uint32_t map_id, uint32_t hs, uint32_t hw, uint32_t hr, 
 }
 
 int map_rope_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_tokens, uint32_t n_heads, uint32_t head_dim,
-                 uint32_t pos_offset, float freq_base) {
+                 uint32_t pos_offset, float freq_base) { ADAMAH_API();
   Map* m = get_f32_map(map_id);
   if (!m) return ADAMAH_ERR_INVALID;
   const uint64_t pairs = (uint64_t)n_tokens * n_heads * (head_dim / 2);
@@ -174,7 +186,7 @@ int map_rope_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_tokens, u
 
 int map_qk_norm_rope_x_dev(uint32_t map_act, uint32_t map_wt, uint32_t hqs, uint32_t hqw, uint32_t hks, uint32_t hkw,
                            uint32_t hdst, uint32_t q_rows, uint32_t q_dim, uint32_t k_rows, uint32_t k_dim,
-                           uint32_t pos_offset, float freq_base) {
+                           uint32_t pos_offset, float freq_base) { ADAMAH_API();
   Map* ma = get_f32_map(map_act);
   Map* mw = get_f32_map(map_wt);
   if (!ma || !mw) return ADAMAH_ERR_INVALID;
@@ -191,7 +203,7 @@ int map_qk_norm_rope_x_dev(uint32_t map_act, uint32_t map_wt, uint32_t hqs, uint
 }
 
 int map_row_copy_offset_dev(uint32_t map_id, uint32_t hspec, uint32_t hbase, uint32_t dst_row_offset, uint32_t n_copies,
-                            uint32_t row_size) {
+                            uint32_t row_size) { ADAMAH_API();
   Map* m = get_f32_map(map_id);
   if (!m) return ADAMAH_ERR_INVALID;
   if (n_copies == 0 || row_size == 0) return ADAMAH_OK;

@@ -38,7 +38,7 @@ extern "C" {
 // average microseconds per launch over `launches` launches (HIP events on the library stream),
 // or a negative error code.
 float adamah_hip_stream_probe(uint64_t bytes_per_launch, uint64_t pool_bytes, uint32_t mode, uint32_t wg_per_cu,
-                              uint32_t launches) {
+                              uint32_t launches) { ADAMAH_API();
   if (!g.initialized || bytes_per_launch < 4096 || pool_bytes < bytes_per_launch || launches == 0 || wg_per_cu == 0)
     return (float)ADAMAH_ERR_INVALID;
   uint8_t *src = nullptr, *dst = nullptr;

@@ -82,7 +82,22 @@ uint32_t res_alloc(uint32_t n_bytes) {
   r.dptr = p;
   r.host.clear();
   r.host_valid = false;
+  r.contig = false;
   return id;
+}
+
+// Remember what was uploaded into a handle, and whether it is a run of consecutive indices.
+static void note_host(Res* r, const void* data, uint32_t n_bytes) {
+  r->host.assign((const uint8_t*)data, (const uint8_t*)data + n_bytes);
+  r->host_valid = true;
+  r->contig = false;
+  if (n_bytes >= 4 && (n_bytes & 3u) == 0) {
+    const uint32_t* v = (const uint32_t*)r->host.data();
+    const uint32_t n = n_bytes >> 2;
+    bool run = true;
+    for (uint32_t i = 1; run && i < n; i++) run = v[i] == v[0] + i;
+    r->contig = run;
+  }
 }
 
 static uint32_t g_scratch_h[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -95,8 +110,7 @@ uint32_t scratch_handle(int slot, const void* data, uint32_t n_bytes) {
     if (!r) return 0;
   }
   r->size_bytes = n_bytes;
-  r->host.assign((const uint8_t*)data, (const uint8_t*)data + n_bytes);
-  r->host_valid = true;
+  note_host(r, data, n_bytes);
   if (h2d(r->dptr, data, n_bytes) != ADAMAH_OK) return 0;
   return g_scratch_h[slot];
 }
@@ -322,6 +336,9 @@ int adamah_init_ex(uint64_t hot_bytes, uint64_t cold_bytes) {
   g.res_next = 1;
   g.attn_scratch_floats = (size_t)4 << 20;   // 16 MiB of split-KV partials
   HIPCHK(hipMalloc((void**)&g.attn_scratch, g.attn_scratch_floats * sizeof(float)));
+  HIPCHK(hipMalloc((void**)&g.sync_ctr, 256));
+  HIPCHK(hipMemsetAsync(g.sync_ctr, 0, 256, g.stream));
+  g.pend.clear();
   g.batch_depth = 0; g.fusion_enabled = 0; g.scheduler_mode = 0; g.active_dtype = 0;
   g.stats = Stats();
   g.initialized = true;
@@ -330,7 +347,7 @@ int adamah_init_ex(uint64_t hot_bytes, uint64_t cold_bytes) {
 
 int adamah_init(void) { return adamah_init_ex(0, 0); }
 
-void adamah_shutdown(void) {
+void adamah_shutdown(void) { ADAMAH_API();
   if (!g.initialized) return;
   hipStreamSynchronize(g.stream);
   for (int i = 0; i < MAX_MAPS; i++)
@@ -348,13 +365,16 @@ void adamah_shutdown(void) {
   }
   if (g.attn_scratch) hipFree(g.attn_scratch);
   g.attn_scratch = nullptr;
+  if (g.sync_ctr) hipFree(g.sync_ctr);
+  g.sync_ctr = nullptr;
+  g.pend.clear();
   for (int i = 0; i < MAX_PLANS; i++) { g.plans[i].clear(); g.plan_active[i] = false; }
   hipStreamDestroy(g.stream);
   g.stream = nullptr;
   g.initialized = false;
 }
 
-void adamah_sync(void) { if (g.initialized) hipStreamSynchronize(g.stream); }
+void adamah_sync(void) { ADAMAH_API(); if (g.initialized) hipStreamSynchronize(g.stream); }
 void adamah_synchronize(uint64_t ticket) { (void)ticket; adamah_sync(); }
 void adamah_synchronize_all(void) { adamah_sync(); }
 
@@ -382,25 +402,27 @@ void batch_begin(void) {
   if (!g.initialized) return;
   if (g.batch_depth++ == 0) g.stats.last_batch_dispatch = 0;
 }
-void batch_end(void) {
+void batch_end(void) { ADAMAH_API();
   if (!g.initialized || g.batch_depth == 0) return;
   if (--g.batch_depth == 0) g.stats.submit++;
 }
 void adamah_fusion_enable(int enable) { g.fusion_enabled = enable ? 1 : 0; }
 int adamah_fusion_is_enabled(void) { return g.fusion_enabled; }
+// A scheduling hint in the reference (submit what has been fused so far); results only become
+// observable at a sync or a read-back, so the pending queue is left alone.
 int adamah_fusion_flush(void) { g.stats.fusion_flush++; return ADAMAH_OK; }
 void adamah_fusion_set_scheduler_mode(int mode) { if (mode >= 0 && mode <= 2) g.scheduler_mode = mode; }
 int adamah_fusion_get_scheduler_mode(void) { return g.scheduler_mode; }
-int adamah_register_loc_span(uint32_t h, uint32_t map_id, uint32_t, uint32_t) {
+int adamah_register_loc_span(uint32_t h, uint32_t map_id, uint32_t, uint32_t) { ADAMAH_API();
   return (get_res(h) && map_id < MAX_MAPS) ? ADAMAH_OK : ADAMAH_ERR_INVALID;
 }
-int adamah_register_row_base_span(uint32_t h, uint32_t map_id, uint32_t, uint32_t, uint32_t, uint32_t) {
+int adamah_register_row_base_span(uint32_t h, uint32_t map_id, uint32_t, uint32_t, uint32_t, uint32_t) { ADAMAH_API();
   return (get_res(h) && map_id < MAX_MAPS) ? ADAMAH_OK : ADAMAH_ERR_INVALID;
 }
-void adamah_clear_loc_alias_meta(uint32_t) {}
-void adamah_stats_reset(void) { g.stats = Stats(); }
+void adamah_clear_loc_alias_meta(uint32_t) { ADAMAH_API();}
+void adamah_stats_reset(void) { ADAMAH_API(); g.stats = Stats(); }
 void adamah_stats_get(uint64_t* dispatch, uint64_t* submit, uint64_t* barrier, uint64_t* flush, uint64_t* dsu,
-                      uint64_t* hit, uint64_t* miss, uint64_t* alias, uint64_t* mode) {
+                      uint64_t* hit, uint64_t* miss, uint64_t* alias, uint64_t* mode) { ADAMAH_API();
   if (dispatch) *dispatch = g.stats.dispatch;   // kernel launches
   if (submit) *submit = g.stats.submit;
   if (barrier) *barrier = g.stats.barrier;      // in-order stream: one implicit dependency per launch
@@ -411,7 +433,7 @@ void adamah_stats_get(uint64_t* dispatch, uint64_t* submit, uint64_t* barrier, u
   if (alias) *alias = 0;
   if (mode) *mode = (uint64_t)g.scheduler_mode;
 }
-uint32_t adamah_get_last_barrier_count(void) { return g.stats.last_batch_dispatch; }
+uint32_t adamah_get_last_barrier_count(void) { ADAMAH_API(); return g.stats.last_batch_dispatch; }
 
 // ---- maps ------------------------------------------------------------------------------------------
 int adamah_set_dtype(uint32_t dtype) {
@@ -422,7 +444,7 @@ int adamah_set_dtype(uint32_t dtype) {
 }
 uint32_t adamah_get_dtype(void) { return g.active_dtype; }
 
-int map_init_dtype(uint32_t id, uint32_t dtype, uint32_t pack_size, uint32_t n_packs, uint32_t group_size) {
+int map_init_dtype(uint32_t id, uint32_t dtype, uint32_t pack_size, uint32_t n_packs, uint32_t group_size) { ADAMAH_API();
   if (!g.initialized || id >= MAX_MAPS || dtype >= DTYPE_COUNT) return ADAMAH_ERR_INVALID;
   if (dtype == DTYPE_BF16 || dtype == DTYPE_Q6) return ADAMAH_ERR_INVALID;
   Map* m = &g.maps[id];
@@ -454,21 +476,21 @@ int map_init_dtype(uint32_t id, uint32_t dtype, uint32_t pack_size, uint32_t n_p
   return check_launch();
 }
 
-int map_init(uint32_t id, uint32_t word_size, uint32_t pack_size, uint32_t n_packs) {
+int map_init(uint32_t id, uint32_t word_size, uint32_t pack_size, uint32_t n_packs) { ADAMAH_API();
   uint32_t dtype = word_size == 2 ? DTYPE_BF16 : word_size == 1 ? DTYPE_Q8 : DTYPE_F32;
   return map_init_dtype(id, dtype, pack_size, n_packs, 128);
 }
 
-int map_destroy(uint32_t id) {
+int map_destroy(uint32_t id) { ADAMAH_API();
   Map* m = get_map(id);
   if (!m) return ADAMAH_ERR_INVALID;
   destroy_map(m);
   return ADAMAH_OK;
 }
-uint64_t map_size(uint32_t id) { Map* m = get_map(id); return m ? m->n_packs : 0; }
-uint32_t map_get_dtype(uint32_t id) { Map* m = get_map(id); return m ? m->dtype : 0; }
+uint64_t map_size(uint32_t id) { ADAMAH_API(); Map* m = get_map(id); return m ? m->n_packs : 0; }
+uint32_t map_get_dtype(uint32_t id) { ADAMAH_API(); Map* m = get_map(id); return m ? m->dtype : 0; }
 
-int map_set_qparams(uint32_t map_id, const float* scales, const float* zps, uint32_t n_groups) {
+int map_set_qparams(uint32_t map_id, const float* scales, const float* zps, uint32_t n_groups) { ADAMAH_API();
   Map* m = get_map(map_id);
   if (!m || !m->qp || !scales || !zps) return ADAMAH_ERR_INVALID;
   if ((uint64_t)n_groups > m->n_groups) return ADAMAH_ERR_INVALID;
@@ -500,13 +522,13 @@ int map_set_qparams(uint32_t map_id, const float* scales, const float* zps, uint
   return ADAMAH_OK;
 }
 
-int adamah_hip_map_layout(uint32_t map_id) {
+int adamah_hip_map_layout(uint32_t map_id) { ADAMAH_API();
   Map* m = get_map(map_id);
   if (!m) return ADAMAH_ERR_INVALID;
   return (m->qp && m->n_groups > 0 && m->block16_groups == m->n_groups) ? QL_BLOCK16 : QL_AFFINE;
 }
 
-int adamah_kv_cache_fp16(uint32_t map_id, uint32_t start, uint32_t count) {
+int adamah_kv_cache_fp16(uint32_t map_id, uint32_t start, uint32_t count) { ADAMAH_API();
   Map* m = get_f32_map(map_id);
   if (!m || count == 0 || !in_range(start, count, m->n_elems)) return ADAMAH_ERR_INVALID;
   hipStreamSynchronize(g.stream);
@@ -520,7 +542,7 @@ int adamah_kv_cache_fp16(uint32_t map_id, uint32_t start, uint32_t count) {
 
 // ---- host -> map ---------------------------------------------------------------------------------
 static int scatter_impl(Map* m, const uint32_t* locs, uint64_t start_pack, bool contiguous, const void* data,
-                        uint32_t n_locs) {
+                        uint32_t n_locs) { ADAMAH_API();
   uint64_t n_vals = (uint64_t)n_locs * m->pack_size;
   if (m->dtype == DTYPE_Q4) {
     if (!m->qp) return ADAMAH_ERR_INVALID;
@@ -578,7 +600,7 @@ static bool locs_contiguous(const uint32_t* locs, uint32_t n, uint32_t n_packs, 
   return true;
 }
 
-uint64_t map_scatter(uint32_t map_id, const uint32_t* locs, const void* data, uint32_t n_locs) {
+uint64_t map_scatter(uint32_t map_id, const uint32_t* locs, const void* data, uint32_t n_locs) { ADAMAH_API();
   Map* m = get_map(map_id);
   if (!m) return (uint64_t)(int64_t)ADAMAH_ERR_INVALID;
   if (n_locs == 0) return ADAMAH_OK;
@@ -588,7 +610,7 @@ uint64_t map_scatter(uint32_t map_id, const uint32_t* locs, const void* data, ui
   return (uint64_t)(int64_t)scatter_impl(m, locs, start, cont, data, n_locs);
 }
 
-uint64_t map_scatter_contiguous(uint32_t map_id, uint32_t start_pack, const void* data, uint32_t n_locs) {
+uint64_t map_scatter_contiguous(uint32_t map_id, uint32_t start_pack, const void* data, uint32_t n_locs) { ADAMAH_API();
   Map* m = get_map(map_id);
   if (!m) return (uint64_t)(int64_t)ADAMAH_ERR_INVALID;
   if (n_locs == 0) return ADAMAH_OK;
@@ -597,7 +619,7 @@ uint64_t map_scatter_contiguous(uint32_t map_id, uint32_t start_pack, const void
   return (uint64_t)(int64_t)scatter_impl(m, nullptr, start_pack, true, data, n_locs);
 }
 
-uint64_t map_scatter_q4_packed_contiguous(uint32_t map_id, uint32_t start_pack, const void* packed, uint32_t n_locs) {
+uint64_t map_scatter_q4_packed_contiguous(uint32_t map_id, uint32_t start_pack, const void* packed, uint32_t n_locs) { ADAMAH_API();
   Map* m = get_map(map_id);
   if (!m) return (uint64_t)(int64_t)ADAMAH_ERR_INVALID;
   if (!packed || n_locs == 0) return ADAMAH_OK;
@@ -607,7 +629,7 @@ uint64_t map_scatter_q4_packed_contiguous(uint32_t map_id, uint32_t start_pack, 
   return (uint64_t)(int64_t)h2d(m->buf + start_pack / 2, packed, n_locs / 2);
 }
 
-uint64_t map_gather(uint32_t map_id, const uint32_t* locs, void* data, uint32_t n_locs) {
+uint64_t map_gather(uint32_t map_id, const uint32_t* locs, void* data, uint32_t n_locs) { ADAMAH_API();
   Map* m = get_map(map_id);
   if (!m) return (uint64_t)(int64_t)ADAMAH_ERR_INVALID;
   if (n_locs == 0) return ADAMAH_OK;
@@ -635,6 +657,8 @@ uint64_t map_gather(uint32_t map_id, const uint32_t* locs, void* data, uint32_t 
 
 // ---- handles ---------------------------------------------------------------------------------------
 uint64_t map_upload_dev(uint32_t handle, const void* data, uint32_t n_bytes) {
+  // a new handle cannot be an operand of anything queued; rewriting an existing one can
+  if (handle != 0) ADAMAH_API();
   if (!g.initialized || !data || n_bytes == 0) return 0;
   uint32_t id = handle;
   if (id == 0) {
@@ -643,20 +667,19 @@ uint64_t map_upload_dev(uint32_t handle, const void* data, uint32_t n_bytes) {
   }
   Res* r = get_res(id);
   if (!r || r->size_bytes != n_bytes) return 0;   // re-upload must keep the byte size (adamah.c:3601-3608)
-  r->host.assign((const uint8_t*)data, (const uint8_t*)data + n_bytes);
-  r->host_valid = true;
+  note_host(r, data, n_bytes);
   if (h2d(r->dptr, data, n_bytes) != ADAMAH_OK) return 0;
   return (uint64_t)id;
 }
 
-int map_download_dev(uint32_t handle, void* data, uint32_t n_bytes) {
+int map_download_dev(uint32_t handle, void* data, uint32_t n_bytes) { ADAMAH_API();
   if (!g.initialized || !data || n_bytes == 0) return ADAMAH_ERR_INVALID;
   Res* r = get_res(handle);
   if (!r || n_bytes > r->size_bytes) return ADAMAH_ERR_INVALID;
   return d2h(data, r->dptr, n_bytes);
 }
 
-uint64_t map_gather_dev(uint32_t map_id, uint32_t locs_handle, uint32_t n_locs) {
+uint64_t map_gather_dev(uint32_t map_id, uint32_t locs_handle, uint32_t n_locs) { ADAMAH_API();
   Map* m = get_map(map_id);
   if (!m || n_locs == 0) return 0;
   const uint32_t* locs = res_u32(locs_handle, n_locs);
@@ -678,7 +701,7 @@ uint64_t map_gather_dev(uint32_t map_id, uint32_t locs_handle, uint32_t n_locs) 
   return (uint64_t)id;
 }
 
-uint64_t map_scatter_dev(uint32_t map_id, uint32_t locs_handle, uint32_t n_locs, uint32_t src_handle) {
+uint64_t map_scatter_dev(uint32_t map_id, uint32_t locs_handle, uint32_t n_locs, uint32_t src_handle) { ADAMAH_API();
   Map* m = get_f32_map(map_id);
   if (!m || n_locs == 0) return 0;
   const uint32_t* locs = res_u32(locs_handle, n_locs);
@@ -693,11 +716,11 @@ uint64_t map_scatter_dev(uint32_t map_id, uint32_t locs_handle, uint32_t n_locs,
 }
 
 // ---- stopwatch -------------------------------------------------------------------------------------
-int adamah_hip_timer_begin(void) {
+int adamah_hip_timer_begin(void) { ADAMAH_API();
   if (!g.initialized) return ADAMAH_ERR_INVALID;
   return hipEventRecord(g.timer_ev[0], g.stream) == hipSuccess ? ADAMAH_OK : ADAMAH_ERR_BACKEND;
 }
-float adamah_hip_timer_end(void) {
+float adamah_hip_timer_end(void) { ADAMAH_API();
   if (!g.initialized) return -1.0f;
   float ms = -1.0f;
   if (hipEventRecord(g.timer_ev[1], g.stream) != hipSuccess) return -1.0f;
@@ -709,14 +732,14 @@ float adamah_hip_timer_end(void) {
 // ---- decode plan (adamah.c:10244-10398): a recorded op list replayed with runtime pos / seq_len ---
 #define RT_POS 0xFFFFFFFEu
 #define RT_SEQ 0xFFFFFFFDu
-int adamah_register_decode_plan(uint32_t plan_id, const AdamahDecodePlanOp* ops, uint32_t n_ops) {
+int adamah_register_decode_plan(uint32_t plan_id, const AdamahDecodePlanOp* ops, uint32_t n_ops) { ADAMAH_API();
   if (plan_id >= MAX_PLANS || n_ops > MAX_PLAN_OPS || (n_ops > 0 && !ops)) return ADAMAH_ERR_INVALID;
   g.plans[plan_id].resize(n_ops);
   if (n_ops) memcpy(g.plans[plan_id].data(), ops, sizeof(PlanOp) * n_ops);
   g.plan_active[plan_id] = true;
   return ADAMAH_OK;
 }
-void adamah_clear_decode_plan(uint32_t plan_id) {
+void adamah_clear_decode_plan(uint32_t plan_id) { ADAMAH_API();
   if (plan_id >= MAX_PLANS) return;
   g.plans[plan_id].clear();
   g.plan_active[plan_id] = false;

@@ -74,7 +74,7 @@ class DecodeEngine:
 
     def __init__(self, gpu, cfg, tensors, A=None, kv_cap=1024, kv_fp16=False,
                  fusion_scheduler_mode='legacy', gpu_fused_rows_per_group=256,
-                 q4_map_elem_limit=(1 << 32) - 64, verbose=False):
+                 q4_map_elem_limit=(1 << 32) - 64, verbose=False, decode_plan=True, plan_id=0):
         if A is None:
             from . import adamah as A
         self.gpu, self.cfg, self.tensors, self.A = gpu, cfg, tensors, A
@@ -93,6 +93,14 @@ class DecodeEngine:
         gpu.fusion_enable(True)
         self._sample_token_ready = False
         self.n_ops_last_forward = 0
+        # The per-token op list is the same every step except for pos / seq_len, so it is registered
+        # once as a native decode plan (reference API adamah.c:10341-10398) and replayed with one call.
+        self._plan_id = None
+        if decode_plan and getattr(gpu, '_has_decode_plan', False):
+            ops = self._plan_ops()
+            if len(ops) <= 4096:
+                gpu.register_decode_plan(plan_id, ops)
+                self._plan_id = plan_id
 
     # ------------------------------------------------------------------ layout
     @staticmethod
@@ -334,6 +342,87 @@ class DecodeEngine:
     def _rms(self, src_h, name, dst_h, rows, dim):
         self.gpu.map_rmsnorm_dev(self.WS_MAP, src_h, self._wh[name], dst_h, rows, dim, self.cfg.norm_eps)
 
+    # ------------------------------------------------------------------ decode plan
+    def _plan_ops(self):
+        """The layer loop of `_forward` (plus the output norm) as DecodePlanOp records; `pos` and
+        `seq_len` are the runtime sentinels.  Field use per kind: adamah.c:10265-10338."""
+        c, A, ws = self.cfg, self.A, self.WS_MAP
+        P, S = A.DECODE_RUNTIME_POS, A.DECODE_RUNTIME_SEQ_LEN
+        q_dim, k_dim = c.n_head * c.head_dim, c.n_head_kv * c.head_dim_kv
+        W = self._ws
+        hid_h, normed_h, q_h, k_h, v_h = (W[n][0] for n in ('hidden', 'normed', 'q', 'k', 'v'))
+        ao_h, op_h, n2_h, gate_h, up_h, act_h, ffn_h = (
+            W[n][0] for n in ('attn_out', 'o_proj', 'normed2', 'gate', 'up', 'act', 'ffn_out'))
+        alias_fast = self._sched != 'legacy'
+        Op = A.DecodePlanOp
+        ops = []
+
+        def rms(src, name, dst, dim):
+            ops.append(Op(kind=A.DECODE_OP_RMSNORM, map_id=ws, h0=src, h1=self._wh[name], h2=dst, u0=1, u1=dim,
+                          f0=c.norm_eps))
+
+        def rms_add(src, name, res, dst, dim):
+            ops.append(Op(kind=A.DECODE_OP_RMSNORM_ADD, map_id=ws, h0=src, h1=self._wh[name], h2=res, h3=dst, u0=1,
+                          u1=dim, f0=c.norm_eps))
+
+        def proj(in_h, name, out_h, K, N, wt_h=None):
+            kind = A.DECODE_OP_MATMUL_T_XQ8 if self._kind[name] == 'q8' else A.DECODE_OP_MATMUL_T_XQ4
+            ops.append(Op(kind=kind, map_id=ws, map_id2=self._map_of[name], h0=in_h, h1=wt_h or self._wh[name],
+                          h2=out_h, u0=1, u1=K, u2=N, u3=1))
+
+        def op2(code, a, b, d, n):
+            ops.append(Op(kind=A.DECODE_OP_OP2, map_id=ws, op_code=code, h0=a, h1=b, h2=d, u0=n))
+
+        for L in range(c.n_layer):
+            p = f'blk.{L}'
+            freq = c.rope_base_global if c.is_global(L) else c.rope_base_local
+            rms(hid_h, f'{p}.attn_norm.weight', normed_h, c.n_embd)
+            if alias_fast and L in self._qkv_wt:
+                proj(normed_h, f'{p}.attn_q.weight', self._qkv_out_h, c.n_embd, q_dim + 2 * k_dim, self._qkv_wt[L])
+            else:
+                proj(normed_h, f'{p}.attn_q.weight', q_h, c.n_embd, q_dim)
+                proj(normed_h, f'{p}.attn_k.weight', k_h, c.n_embd, k_dim)
+                proj(normed_h, f'{p}.attn_v.weight', v_h, c.n_embd, k_dim)
+            qnn = f'{p}.attn_q_norm.weight'
+            if qnn in self._wh:
+                ops.append(Op(kind=A.DECODE_OP_QK_NORM_ROPE_X, map_id=ws, map_id2=ws, h0=self._q_rows_h, h1=self._wh[qnn],
+                              h2=self._k_rows_h, h3=self._wh[f'{p}.attn_k_norm.weight'], h4=self._qk_out_h,
+                              u0=c.n_head, u1=c.head_dim, u2=c.n_head_kv, u3=c.head_dim_kv, u4=P, f0=freq))
+            else:
+                ops.append(Op(kind=A.DECODE_OP_ROPE, map_id=ws, h0=self._q_rope_src_h, h1=q_h, u0=1, u1=c.n_head,
+                              u2=c.head_dim, u3=P, f0=freq))
+                ops.append(Op(kind=A.DECODE_OP_ROPE, map_id=ws, h0=self._k_rope_src_h, h1=k_h, u0=1, u1=c.n_head_kv,
+                              u2=c.head_dim_kv, u3=P, f0=freq))
+            ops.append(Op(kind=A.DECODE_OP_ROW_COPY_OFFSET, map_id=ws, h0=self._kv_copy_h[L], h1=self._k_src_base_h,
+                          u0=P, u1=2 * c.n_head_kv, u2=c.head_dim_kv))
+            ops.append(Op(kind=A.DECODE_OP_MATMUL_T, map_id=ws, h0=self._q_rows_h, h1=self._k_locs_h[L],
+                          h2=self._scores_row_h, u0=1, u1=c.head_dim, u2=S, u3=c.n_head))
+            ops.append(Op(kind=A.DECODE_OP_ATTN_SOFTMAX_VALUE, map_id=ws, h0=self._scores_row_h, h1=self._v_locs_h[L],
+                          h2=self._ao_rows_h, u0=c.n_head, u1=S, u2=c.head_dim_kv,
+                          f0=float(1.0 / np.sqrt(c.head_dim)), f1=float(c.attn_softcap)))
+            ops.append(Op(kind=A.DECODE_OP_FUSION_FLUSH))
+            proj(ao_h, f'{p}.attn_output.weight', op_h, c.n_head * c.head_dim_kv, c.n_embd)
+            pan = f'{p}.post_attention_norm.weight'
+            if pan in self._wh:
+                rms_add(op_h, pan, hid_h, hid_h, c.n_embd)
+            else:
+                op2(A.OP_ADD, hid_h, op_h, hid_h, c.n_embd)
+            rms(hid_h, f'{p}.ffn_norm.weight', n2_h, c.n_embd)
+            if alias_fast and L in self._gateup_wt:
+                proj(n2_h, f'{p}.ffn_gate.weight', self._gateup_out_h, c.n_embd, 2 * c.n_ff, self._gateup_wt[L])
+            else:
+                proj(n2_h, f'{p}.ffn_gate.weight', gate_h, c.n_embd, c.n_ff)
+                proj(n2_h, f'{p}.ffn_up.weight', up_h, c.n_embd, c.n_ff)
+            op2(A.OP_GEGLU if c.ffn_act == 'gelu' else A.OP_SWIGLU, gate_h, up_h, act_h, c.n_ff)
+            proj(act_h, f'{p}.ffn_down.weight', ffn_h, c.n_ff, c.n_embd)
+            pfn = f'{p}.post_ffw_norm.weight'
+            if pfn in self._wh:
+                rms_add(ffn_h, pfn, hid_h, hid_h, c.n_embd)
+            else:
+                op2(A.OP_ADD, hid_h, ffn_h, hid_h, c.n_embd)
+        rms(hid_h, 'output_norm.weight', normed_h, c.n_embd)
+        return ops
+
     # ------------------------------------------------------------------ forward
     def _forward(self, tok, pos, sample=True):
         """One decode step; op order of reference engine.py:2971-3402 (default discrete-GPU path)."""
@@ -362,7 +451,7 @@ class DecodeEngine:
             if c.emb_scale != 1.0:
                 g.map_broadcast_dev(ws, A.OP_MUL, hid_h, W['emb_scale'][0], hid_h, c.n_embd)
 
-        for L in range(c.n_layer):
+        for L in range(c.n_layer if self._plan_id is None else 0):
             p = f'blk.{L}'
             freq = c.rope_base_global if c.is_global(L) else c.rope_base_local
             self._rms(hid_h, f'{p}.attn_norm.weight', normed_h, 1, c.n_embd)
@@ -413,7 +502,10 @@ class DecodeEngine:
             else:
                 g.map_op2_dev(ws, A.OP_ADD, hid_h, ffn_h, hid_h, c.n_embd)
 
-        self._rms(hid_h, 'output_norm.weight', normed_h, 1, c.n_embd)
+        if self._plan_id is None:
+            self._rms(hid_h, 'output_norm.weight', normed_h, 1, c.n_embd)
+        else:
+            g.decode_step(self._plan_id, pos, seq_len)
         if sample:
             fn = (g.map_matvec_argmax_t_xq8_dev if self._kind[self._lm_name] == 'q8'
                   else g.map_matvec_argmax_t_xq4_dev)

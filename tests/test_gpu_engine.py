@@ -76,3 +76,21 @@ def test_many_tokens_do_not_exhaust_handles(hip):
     note("2500 decode steps")
     out, _ = eng.generate([1, 2], GenerationConfig(max_tokens=2500))
     assert len(out) == 2500
+
+
+@pytest.mark.parametrize("arch", ["gemma3", "llama"])
+def test_decode_plan_replay_equals_op_by_op(hip, arch):
+    """The engine registers its per-token op list as a native decode plan; replaying it must give
+    the tokens and the hidden state of issuing the ops one by one."""
+    cfg = synth.tiny_config(arch, n_layer=3, n_embd=256, n_head=4, n_head_kv=2, head_dim=64, n_ff=512, n_vocab=1000)
+    tensors = synth.make_model(cfg, seed=9, sigma=0.1)
+    res = []
+    for plan in (True, False):
+        note(f"engine {arch} decode_plan={plan}")
+        eng = DecodeEngine(hip, cfg, tensors, A=A, kv_cap=64, kv_fp16=True, fusion_scheduler_mode="level_batched",
+                           gpu_fused_rows_per_group=128, decode_plan=plan)
+        assert (eng._plan_id is not None) == plan
+        tok, _ = eng.generate([5, 17, 900, 2], GenerationConfig(max_tokens=16))
+        res.append((tok, eng.read_slot('hidden')))
+    assert res[0][0] == res[1][0]
+    assert np.array_equal(res[0][1], res[1][1])

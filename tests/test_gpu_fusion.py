@@ -1,0 +1,227 @@
+"""Ops that the HIP library folds into a neighbouring GEMV launch when they are issued inside a
+batch, against the oracle running the same ops one by one (needs an MI355X).
+
+Covered folds: RMSNorm -> GEMV, RMSNorm+residual -> RMSNorm -> GEMV, GEMV -> ADD, GEMV over
+[gate; up] rows -> GEGLU/SWIGLU, the combinations of a prologue with an epilogue, RMSNorm ->
+GEMV+argmax; sequences of the same ops that are not folded (activation before the GEMV, norm after
+it) and sequences that must NOT be folded (aliasing operands).  Every slot an unfused run would
+write is compared, because the fused kernels have to leave the maps exactly as the separate ops
+would.  Tolerance: 1e-3 relative L2
+(the bar for GEMV outputs); the vectors produced by the folded row-wise ops themselves are held
+to 1e-5."""
+import numpy as np
+import pytest
+
+import oracle
+from adam_amd import adamah as A
+from adam_amd import quant
+from gpu_util import note, up, read, rel_l2, load_qtensor
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+class Slots:
+    """Workspace layout shared by the scenarios: named float ranges in map 0, weights in map 1."""
+
+    def __init__(self, K, N):
+        self.K, self.N = K, N
+        self.off, pos = {}, 0
+        for name, n in (("src", K), ("src2", K), ("x", K), ("y", N), ("res", N), ("dst", N), ("nw", K), ("nw2", N),
+                        ("resk", K), ("nwk", K), ("idx", 64), ("val", 64), ("tok", 8)):
+            self.off[name] = pos
+            pos += n + 32          # keep the ranges apart and 32-element aligned
+        self.total = pos
+
+    def fill(self, g, rng_seed):
+        rng = np.random.default_rng(rng_seed)
+        g.set_dtype(A.DTYPE_F32)
+        g.map_create(0, 1, self.total)
+        vals = {"src": rng.standard_normal(self.K), "src2": rng.standard_normal(self.K),
+                "x": rng.standard_normal(self.K), "res": rng.standard_normal(self.N),
+                "nw": rng.uniform(0.5, 1.5, self.K), "nw2": rng.uniform(0.5, 1.5, self.N),
+                "resk": rng.standard_normal(self.K), "nwk": rng.uniform(0.5, 1.5, self.K)}
+        for k, v in vals.items():
+            g.scatter_contiguous(0, self.off[k], v.astype(np.float32))
+
+    def h(self, g, name):
+        return up(g, [self.off[name]])
+
+    def run(self, g, name, n):
+        return up(g, np.arange(self.off[name], self.off[name] + n, dtype=np.uint32))
+
+
+def make_weights(N, K, seed):
+    rng = np.random.default_rng(seed)
+    return quant.quantize_q4_0((rng.standard_normal((N, K)) * 0.02).astype(np.float32))
+
+
+def scenario(g, s, qt, pro, epi, batch=True):
+    """pro in (None, 'rms', 'norm2', 'geglu', 'swiglu');
+    epi in (None, 'add', 'add_swapped', 'norm_add', 'geglu_after', 'swiglu_after')."""
+    K, N = s.K, s.N
+    if batch:
+        g.batch_begin()
+    if pro == 'rms':
+        g.map_rmsnorm_dev(0, s.h(g, "src"), s.h(g, "nw"), s.h(g, "x"), 1, K, 1e-6)
+    elif pro == 'norm2':
+        g.map_rmsnorm_add_dev(0, s.h(g, "src"), s.h(g, "nw"), s.h(g, "resk"), s.h(g, "resk"), 1, K, 1e-6)
+        g.map_rmsnorm_dev(0, s.h(g, "resk"), s.h(g, "nwk"), s.h(g, "x"), 1, K, 1e-5)
+    elif pro in ('geglu', 'swiglu'):
+        g.map_op2_dev(0, A.OP_GEGLU if pro == 'geglu' else A.OP_SWIGLU, s.run(g, "src", K), s.run(g, "src2", K),
+                      s.run(g, "x", K), K)
+    g.map_matmul_t_xq4_dev(0, 1, s.h(g, "x"), up(g, [0]), s.h(g, "y"), 1, K, N)
+    if epi == 'add':
+        g.map_op2_dev(0, A.OP_ADD, s.run(g, "res", N), s.run(g, "y", N), s.run(g, "res", N), N)   # in place
+    elif epi == 'add_swapped':
+        g.map_op2_dev(0, A.OP_ADD, s.run(g, "y", N), s.run(g, "res", N), s.run(g, "dst", N), N)
+    elif epi == 'norm_add':
+        g.map_rmsnorm_add_dev(0, s.h(g, "y"), s.h(g, "nw2"), s.h(g, "res"), s.h(g, "res"), 1, N, 1e-6)
+    elif epi in ('geglu_after', 'swiglu_after'):
+        half = N // 2
+        g.map_op2_dev(0, A.OP_GEGLU if epi == 'geglu_after' else A.OP_SWIGLU, s.run(g, "y", half),
+                      up(g, np.arange(s.off["y"] + half, s.off["y"] + N, dtype=np.uint32)), s.run(g, "dst", half), half)
+    if batch:
+        g.batch_end()
+    return {n: read(g, 0, s.off[n], s.K if n in ("x", "resk") else s.N) for n in ("x", "resk", "y", "res", "dst")}
+
+
+@pytest.mark.parametrize("K,N", [(1152, 1536), (4096, 4096), (6912, 1152), (2048, 100)])
+@pytest.mark.parametrize("pro", [None, 'rms', 'norm2', 'geglu', 'swiglu'])
+@pytest.mark.parametrize("epi", [None, 'add', 'add_swapped', 'norm_add', 'geglu_after', 'swiglu_after'])
+def test_folded_sequences_match_separate_ops(hip, K, N, pro, epi):
+    s = Slots(K, N)
+    qt = make_weights(N, K, K + N)
+    out = {}
+    for name, g in (("hip", hip), ("oracle", oracle.init())):
+        note(f"fusion {name} K={K} N={N} pro={pro} epi={epi}")
+        s.fill(g, 5)
+        load_qtensor(g, 1, qt)
+        out[name] = scenario(g, s, qt, pro, epi)
+    for slot, tol in (("x", 1e-5), ("resk", 1e-5), ("y", TOL), ("res", TOL), ("dst", TOL)):
+        assert rel_l2(out["hip"][slot], out["oracle"][slot]) < tol or not np.any(out["oracle"][slot]), slot
+
+
+def test_folded_equals_unbatched_on_device(hip):
+    """The same sequence outside a batch launches the separate kernels; both routes must agree to
+    float rounding on every slot."""
+    K, N = 4096, 2048
+    s = Slots(K, N)
+    qt = make_weights(N, K, 3)
+    res = []
+    for batch in (True, False):
+        note(f"fusion batched={batch}")
+        s.fill(hip, 9)
+        load_qtensor(hip, 1, qt)
+        res.append(scenario(hip, s, qt, 'norm2', 'geglu_after', batch=batch))
+    for slot in ("x", "resk", "y", "dst"):
+        assert rel_l2(res[0][slot], res[1][slot]) < 1e-5, slot
+
+
+def test_aliasing_sequences_are_not_folded(hip):
+    """RMSNorm in place (dst == src) feeding a GEMV, and an ADD whose destination is the GEMV input:
+    folding either would race, so they have to run as separate kernels and still be right."""
+    K = N = 1024
+    s = Slots(K, N)
+    qt = make_weights(N, K, 8)
+    out = {}
+    for name, g in (("hip", hip), ("oracle", oracle.init())):
+        note(f"fusion aliasing {name}")
+        s.fill(g, 13)
+        load_qtensor(g, 1, qt)
+        g.batch_begin()
+        g.map_rmsnorm_dev(0, s.h(g, "x"), s.h(g, "nw"), s.h(g, "x"), 1, K, 1e-6)              # in place
+        g.map_matmul_t_xq4_dev(0, 1, s.h(g, "x"), up(g, [0]), s.h(g, "y"), 1, K, N)
+        g.map_op2_dev(0, A.OP_ADD, s.run(g, "x", N), s.run(g, "y", N), s.run(g, "x", N), N)   # writes the GEMV input
+        g.batch_end()
+        out[name] = {n: read(g, 0, s.off[n], K) for n in ("x", "y")}
+    assert rel_l2(out["hip"]["y"], out["oracle"]["y"]) < TOL
+    assert rel_l2(out["hip"]["x"], out["oracle"]["x"]) < TOL
+
+
+@pytest.mark.parametrize("K,N,rpg", [(1152, 4096, 256), (2048, 1000, 64)])
+def test_rmsnorm_folded_into_matvec_argmax(hip, K, N, rpg):
+    s = Slots(K, N)
+    qt = make_weights(N, K, 77)
+    n_groups = (N + rpg - 1) // rpg
+    assert n_groups <= 64
+    tok = {}
+    for name, g in (("hip", hip), ("oracle", oracle.init())):
+        note(f"fusion argmax {name} K={K} N={N}")
+        s.fill(g, 21)
+        load_qtensor(g, 1, qt)
+        g.batch_begin()
+        g.map_rmsnorm_dev(0, s.h(g, "src"), s.h(g, "nw"), s.h(g, "x"), 1, K, 1e-6)
+        g.map_matvec_argmax_t_xq4_dev(0, 1, s.h(g, "x"), up(g, [0]), s.run(g, "idx", n_groups), s.run(g, "val", n_groups),
+                                      s.h(g, "tok"), K, N, rpg)
+        g.batch_end()
+        tok[name] = (read(g, 0, s.off["tok"], 1)[0], read(g, 0, s.off["x"], K), read(g, 0, s.off["idx"], n_groups),
+                     read(g, 0, s.off["val"], n_groups))
+    assert tok["hip"][0] == tok["oracle"][0]
+    assert rel_l2(tok["hip"][1], tok["oracle"][1]) < 1e-5
+    assert np.array_equal(tok["hip"][2], tok["oracle"][2])
+    assert rel_l2(tok["hip"][3], tok["oracle"][3]) < TOL
+
+
+def test_host_write_between_deferred_ops_keeps_order(hip):
+    """A scatter issued between two ops of a batch must land between them (the queue is flushed
+    before any other entry point runs)."""
+    K, N = 1024, 512
+    s = Slots(K, N)
+    qt = make_weights(N, K, 4)
+    out = {}
+    for name, g in (("hip", hip), ("oracle", oracle.init())):
+        note(f"fusion ordering {name}")
+        s.fill(g, 2)
+        load_qtensor(g, 1, qt)
+        g.batch_begin()
+        g.map_rmsnorm_dev(0, s.h(g, "src"), s.h(g, "nw"), s.h(g, "x"), 1, K, 1e-6)
+        g.scatter_contiguous(0, s.off["x"] + 7, np.array([3.5], np.float32))    # overwrites one normalised value
+        g.map_matmul_t_xq4_dev(0, 1, s.h(g, "x"), up(g, [0]), s.h(g, "y"), 1, K, N)
+        g.batch_end()
+        out[name] = (read(g, 0, s.off["x"], K), read(g, 0, s.off["y"], N))
+    assert out["hip"][0][7] == np.float32(3.5)
+    assert rel_l2(out["hip"][0], out["oracle"][0]) < 1e-5
+    assert rel_l2(out["hip"][1], out["oracle"][1]) < TOL
+
+
+@pytest.mark.parametrize("ctx,Hq,Hkv,d,N", [(640, 4, 1, 256, 1152), (3000, 8, 2, 128, 512), (40, 4, 2, 64, 96)])
+def test_attention_chain_folded_into_output_projection(hip, ctx, Hq, Hkv, d, N):
+    """scores -> softmax.V -> Q4 GEMV over the heads' outputs in one batch: the scores move into the
+    softmax.V launch and the merge of the sequence splits into the GEMV's staging.  Raw scores, the
+    attention output and the projection are all compared."""
+    from gpu_util import f32map, put
+    rng = np.random.default_rng(ctx + N)
+    q = rng.standard_normal((Hq, d)).astype(np.float32)
+    Kc = rng.standard_normal((Hkv, ctx, d)).astype(np.float32)
+    Vc = rng.standard_normal((Hkv, ctx, d)).astype(np.float32)
+    qt = make_weights(N, Hq * d, 31)
+    gs = Hq // Hkv
+    sc_sz = Hq * ctx
+    q_pos, out_pos, y_pos = sc_sz, sc_sz + Hq * d, sc_sz + 2 * Hq * d
+    kv_start = (y_pos + N + d - 1) // d * d
+    step = ctx * d
+    res = {}
+    for name, g in (("hip", hip), ("oracle", oracle.init())):
+        note(f"attention+projection {name} ctx={ctx} {Hq}/{Hkv}x{d} N={N}")
+        f32map(g, 0, kv_start + 2 * Hkv * step, None)
+        g.kv_cache_fp16(0, kv_start, 2 * Hkv * step)
+        put(g, 0, q_pos, q)
+        for h in range(Hkv):
+            put(g, 0, kv_start + h * step, Kc[h])
+            put(g, 0, kv_start + (Hkv + h) * step, Vc[h])
+        load_qtensor(g, 1, qt)
+        heads = np.arange(Hq) // gs
+        s_rows = up(g, np.arange(Hq) * ctx)
+        o_rows = up(g, out_pos + np.arange(Hq) * d)
+        g.batch_begin()
+        g.map_matmul_t_dev(0, up(g, q_pos + np.arange(Hq) * d), up(g, kv_start + heads * step), s_rows, 1, d, ctx, Hq)
+        g.map_attn_softmax_value_dev(0, s_rows, up(g, kv_start + (Hkv + heads) * step), o_rows, Hq, ctx, d,
+                                     float(1 / np.sqrt(d)), 50.0)
+        g.fusion_flush()
+        g.map_matmul_t_xq4_dev(0, 1, up(g, [out_pos]), up(g, [0]), up(g, [y_pos]), 1, Hq * d, N)
+        g.batch_end()
+        res[name] = (read(g, 0, 0, sc_sz), read(g, 0, out_pos, Hq * d), read(g, 0, y_pos, N))
+    assert rel_l2(res["hip"][0], res["oracle"][0]) < 1e-5
+    assert rel_l2(res["hip"][1], res["oracle"][1]) < TOL
+    assert rel_l2(res["hip"][2], res["oracle"][2]) < TOL
