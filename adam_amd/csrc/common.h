@@ -149,6 +149,7 @@ void flush_pending();
 bool res_scalar(uint32_t h, uint32_t* out);
 // First element of a handle whose host copy is a run of n consecutive indices; false otherwise.
 bool res_run(uint32_t h, uint64_t n, uint32_t* start);
+void gemm_q4_mfma_release();   // frees the GEMM's scratch (shutdown)
 int launch_rmsnorm_v(const PendOp& p);
 int launch_op2_v(const PendOp& p);
 // Attention (attention.hip): stand-alone launches of queued ops, and the fused form.  launch_attn

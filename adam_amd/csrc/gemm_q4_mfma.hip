@@ -1,0 +1,228 @@
+// Batched (M > 1) quantised matmul  C[M, N] = A[M, K] . W[N, K]^T  for Q4_0 weights on the fp16
+// matrix cores: prefill chunks and batched decode.
+//
+// Reference: shaders/src/f32/map_matmul_t_xq4.comp:33-73 (one thread per output, scalar K loop;
+// dispatch adamah.c:8693-8803).  With more than one activation row the weights are reused, so this
+// is the one place on the path where the work is a dense contraction and belongs on MFMA.
+//
+// v_mfma_f32_16x16x16_f16:  D[i][j] += sum_k A[i][k] B[k][j];  lane l supplies A[l % 16][4g..4g+3] and
+// B[4g..4g+3][l % 16] with g = l / 16, and receives D[4g..4g+3][l % 16].  Here i runs over 16 weight
+// rows, j over 16 activation rows, and the sixteen k of one instruction are four weights out of each
+// of four consecutive 32-weight blocks: lane (row, g) loads block g of its row as one 16-byte word
+// group, dequantises it in registers to fp16 (exactly (q - 8), then times the block's fp16 scale:
+// one rounding per weight) and feeds eight instructions from it.  The activations of the tile are
+// converted once per step to fp16 in LDS, scaled per row by a power of two so that no row can
+// overflow fp16 (the scale is divided out of the fp32 result), in the element order the unpacking
+// produces.  Accumulation is fp32 in the matrix core.
+//
+// Workgroup = 4 waves = 64 weight rows x (16 * MT) activation rows; one step = 128 weights of K.
+// KSPLIT (few activation rows): the four waves share 16 weight rows and take every fourth step of K
+// each, so that small matrices still spread over the whole chip; their partial tiles are summed
+// through LDS in a fixed order.
+#include "gemv_common.h"
+#include <algorithm>
+
+namespace adamah {
+
+typedef _Float16 h2q_t __attribute__((ext_vector_type(2)));
+typedef _Float16 h4q_t __attribute__((ext_vector_type(4)));
+typedef float f4q_t __attribute__((ext_vector_type(4)));
+typedef float f4qu_t __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u2q_t __attribute__((ext_vector_type(2)));
+
+// Per activation row: s = 2^e with max|x| * s in [2^13, 2^14) (1 when the row is zero, tiny or not
+// finite), and 1 / s.  One workgroup per row.
+__global__ void __launch_bounds__(256)
+k_row_pow2_scale(const float* act, const uint32_t* __restrict__ la, uint32_t M, uint32_t K, float* scale) {
+  __shared__ float red[4];
+  const uint32_t row = blockIdx.x, op = blockIdx.y, tid = threadIdx.x;
+  const float* x = act + (uint64_t)la[op] + (uint64_t)row * K;
+  float m = 0.f;
+  for (uint32_t i = tid; i < K; i += 256u) m = fmaxf(m, fabsf(x[i]));
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  if ((tid & 63u) == 0) red[tid >> 6] = m;
+  __syncthreads();
+  if (tid == 0) {
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    const uint32_t e = (__float_as_uint(m) >> 23) & 0xFFu;
+    float s = 1.f, inv = 1.f;
+    if (e >= 14u && e <= 254u) { s = __uint_as_float((267u - e) << 23); inv = __uint_as_float((e - 13u) << 23); }
+    scale[2 * ((uint64_t)op * M + row)] = s;
+    scale[2 * ((uint64_t)op * M + row) + 1] = inv;
+  }
+}
+
+template <int MT, bool KSPLIT>
+__global__ void __launch_bounds__(256)
+k_gemm_q4_f16(const float* act, float* out, const uint8_t* __restrict__ W, const __half* __restrict__ d16,
+              const uint32_t* __restrict__ la, const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc,
+              const float* __restrict__ scale, uint32_t M, uint32_t K, uint32_t N) {
+  constexpr uint32_t BM = 16u * MT;
+  // activation tile: [row][block 0..3][64 bytes]; a row is padded to 272 bytes so that the sixteen rows
+  // a wave reads side by side fall into different banks
+  constexpr uint32_t ROWB = 272u;
+  constexpr uint32_t TILES = KSPLIT ? 4u : 1u;       // KSPLIT: one activation tile per wave
+  __shared__ __attribute__((aligned(16))) uint8_t xs_all[TILES * BM * ROWB];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t r16 = lane & 15u, g = lane >> 4;
+  uint8_t* xs = xs_all + (KSPLIT ? wave * BM * ROWB : 0u);
+  const uint32_t n0 = KSPLIT ? blockIdx.x * 16u : blockIdx.x * 64u + wave * 16u, m0 = blockIdx.y * BM, op = blockIdx.z;
+  const uint64_t a_off = la[op], c_off = lc[op], gbase = (uint64_t)lb[op] >> 5;
+  const uint32_t nblk = K >> 5;
+  const uint32_t nrow = min(n0 + r16, N - 1u);          // rows past N are clamped here and not stored
+
+  f4q_t acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; t++) acc[t] = (f4q_t){0.f, 0.f, 0.f, 0.f};
+
+  uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u, nib_lo = 0x000F000Fu, nib_hi = 0x00F000F0u;
+  asm volatile("" : "+v"(magic_lo));   // opaque: lets instruction selection use the three-operand and-or
+  asm volatile("" : "+v"(magic_hi));
+  asm volatile("" : "+s"(nib_lo));
+  asm volatile("" : "+s"(nib_hi));
+  const h2q_t off_lo = {(_Float16)-1032.f, (_Float16)-1032.f}, off_hi = {(_Float16)-72.f, (_Float16)-72.f};
+
+  // One step ahead: the weights and activation words of the next step are loaded into registers while
+  // the matrix cores work on the current one.
+  constexpr uint32_t NTH = KSPLIT ? 64u : 256u, WPT = BM * 16u / NTH;   // staging threads per tile, words per thread
+  const uint32_t st = KSPLIT ? lane : tid;
+  float xr[WPT][8], rs[WPT];
+  uint4 qn;
+  _Float16 dn;
+#pragma unroll
+  for (uint32_t u = 0; u < WPT; u++) {
+    const uint32_t row = m0 + ((st + u * NTH) >> 4);
+    rs[u] = row < M ? scale[2 * ((uint64_t)op * M + row)] : 0.f;     // rows past M become zeros
+  }
+  auto fetch = [&](uint32_t kb_raw) {   // always executed; steps past K re-read the last one and are not used
+    const uint32_t kb = min(kb_raw, nblk - 4u);
+    const uint64_t gi = gbase + (uint64_t)nrow * nblk + kb + g;
+    qn = *(const uint4*)(W + (gi << 4));
+    dn = __builtin_bit_cast(_Float16, d16[gi]);
+#pragma unroll
+    for (uint32_t u = 0; u < WPT; u++) {
+      const uint32_t w = st + u * NTH, row = min(m0 + (w >> 4), M - 1u), wi = w & 15u;
+      const f4qu_t* p = (const f4qu_t*)(act + a_off + (uint64_t)row * K + (uint64_t)kb * 32u + wi * 8u);
+      const f4qu_t v0 = p[0], v1 = p[1];
+      xr[u][0] = v0.x; xr[u][1] = v0.y; xr[u][2] = v0.z; xr[u][3] = v0.w;
+      xr[u][4] = v1.x; xr[u][5] = v1.y; xr[u][6] = v1.z; xr[u][7] = v1.w;
+    }
+  };
+  fetch(KSPLIT ? wave * 4u : 0u);
+
+  for (uint32_t kb0 = 0; kb0 < nblk; kb0 += KSPLIT ? 16u : 4u) {
+    // KSPLIT: wave w takes step kb0/4 + w; a wave whose step lies past K idles through the barriers
+    const uint32_t kb_raw = kb0 + (KSPLIT ? wave * 4u : 0u);
+    const bool busy = kb_raw < nblk;
+    const uint4 q = qn;
+    const _Float16 d = dn;
+    // activations of the step -> fp16 in LDS, element order inside a word following the nibble pairs of
+    // the unpacking: (0,4)(1,5) | (2,6)(3,7)
+#pragma unroll
+    for (uint32_t u = 0; u < WPT; u++) {
+      const uint32_t w = st + u * NTH, m = w >> 4, wi = w & 15u;
+      const float sc = rs[u];
+      const h2q_t p0 = {(_Float16)(xr[u][0] * sc), (_Float16)(xr[u][4] * sc)}, p1 = {(_Float16)(xr[u][1] * sc), (_Float16)(xr[u][5] * sc)};
+      const h2q_t p2 = {(_Float16)(xr[u][2] * sc), (_Float16)(xr[u][6] * sc)}, p3 = {(_Float16)(xr[u][3] * sc), (_Float16)(xr[u][7] * sc)};
+      *(uint4*)(xs + m * ROWB + wi * 16u) =
+          make_uint4(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1),
+                     __builtin_bit_cast(uint32_t, p2), __builtin_bit_cast(uint32_t, p3));
+    }
+    // dequantise: (1024 + n) - 1032 = n - 8 and (64 + n) - 72 = n - 8 exactly, then one rounding in d * (n - 8)
+    uint32_t wq[8][2];
+    const h2q_t d2 = {d, d};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const uint32_t w = j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w, w8 = w >> 8;
+      const h2q_t t0 = __builtin_bit_cast(h2q_t, (w & nib_lo) | magic_lo), t1 = __builtin_bit_cast(h2q_t, (w & nib_hi) | magic_hi);
+      const h2q_t t2 = __builtin_bit_cast(h2q_t, (w8 & nib_lo) | magic_lo), t3 = __builtin_bit_cast(h2q_t, (w8 & nib_hi) | magic_hi);
+      wq[2 * j][0] = __builtin_bit_cast(uint32_t, (h2q_t)((t0 + off_lo) * d2));
+      wq[2 * j][1] = __builtin_bit_cast(uint32_t, (h2q_t)((t1 + off_hi) * d2));
+      wq[2 * j + 1][0] = __builtin_bit_cast(uint32_t, (h2q_t)((t2 + off_lo) * d2));
+      wq[2 * j + 1][1] = __builtin_bit_cast(uint32_t, (h2q_t)((t3 + off_hi) * d2));
+    }
+    __syncthreads();
+    fetch(kb_raw + (KSPLIT ? 16u : 4u));
+    if (busy) {
+#pragma unroll
+    for (int t = 0; t < MT; t++) {
+      const uint8_t* xp = xs + (t * 16u + r16) * ROWB + g * 64u;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const uint4 xv = *(const uint4*)(xp + j * 16);
+        const u2q_t a0 = {wq[2 * j][0], wq[2 * j][1]}, a1 = {wq[2 * j + 1][0], wq[2 * j + 1][1]};
+        const u2q_t b0 = {xv.x, xv.y}, b1 = {xv.z, xv.w};
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4q_t, a0), __builtin_bit_cast(h4q_t, b0), acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4q_t, a1), __builtin_bit_cast(h4q_t, b1), acc[t], 0, 0, 0);
+      }
+    }
+    }
+    __syncthreads();
+  }
+  if (KSPLIT) {   // sum the four waves' tiles in wave order; wave 0 stores
+    float* part = (float*)xs_all;             // 3 * 64 * 4 * MT floats, the activation tiles are done with
+    if (wave > 0) {
+#pragma unroll
+      for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) part[(((wave - 1u) * MT + t) * 4u + r) * 64u + lane] = acc[t][r];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (uint32_t w = 0; w < 3; w++)
+#pragma unroll
+      for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[t][r] += part[((w * MT + t) * 4u + r) * 64u + lane];
+  }
+  // lane (j = r16, g) holds D[4g + r][j]: weight rows n0 + 4g + r, activation row m0 + 16 t + r16
+#pragma unroll
+  for (int t = 0; t < MT; t++) {
+    const uint32_t row = m0 + t * 16u + r16;
+    if (row >= M) continue;
+    const float inv = scale[2 * ((uint64_t)op * M + row) + 1];
+    float* c = out + c_off + (uint64_t)row * N;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const uint32_t n = n0 + 4u * g + r;
+      if (n < N) c[n] = acc[t][r] * inv;
+    }
+  }
+}
+
+static float* g_scale_buf = nullptr;
+static size_t g_scale_cap = 0;
+
+// Preconditions (checked by the caller against the host copies of the handles): Q4 map whose blocks
+// in range are in the block16 layout, K a multiple of 128, weight bases block aligned, all operands
+// in range.
+int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb, const uint32_t* lc,
+                        uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops) {
+  const size_t need = (size_t)2 * M * n_ops;
+  if (need > g_scale_cap) {
+    if (g_scale_buf) { hipStreamSynchronize(g.stream); hipFree(g_scale_buf); }
+    g_scale_cap = std::max<size_t>(need, 8192);
+    if (hipMalloc((void**)&g_scale_buf, g_scale_cap * sizeof(float)) != hipSuccess) { g_scale_buf = nullptr; g_scale_cap = 0; return ADAMAH_ERR_MEMORY; }
+  }
+  float* act = (float*)ma->buf;
+  k_row_pow2_scale<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf);
+  count_launch();
+  const uint32_t mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8;
+  const bool ksplit = mt <= 2;    // few activation rows: bandwidth bound, spread K over the waves
+  dim3 grid(cdiv(N, ksplit ? 16 : 64), cdiv(M, 16 * mt), n_ops);
+#define GQ(T, S) k_gemm_q4_f16<T, S><<<grid, 256, 0, g.stream>>>(act, act, mw->buf, mw->d16, la, lb, lc, g_scale_buf, M, K, N)
+  if (mt == 1) GQ(1, true); else if (mt == 2) GQ(2, true); else if (mt == 4) GQ(4, false); else GQ(8, false);
+#undef GQ
+  count_launch();
+  return check_launch();
+}
+
+void gemm_q4_mfma_release() {
+  if (g_scale_buf) hipFree(g_scale_buf);
+  g_scale_buf = nullptr;
+  g_scale_cap = 0;
+}
+
+}  // namespace adamah

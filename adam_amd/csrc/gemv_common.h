@@ -95,6 +95,9 @@ int launch_mfma_argmax(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32
                        const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rows_per_group,
                        const GemvFuse* fz = nullptr);
 bool mfma_path_ok(const Map* mw, uint32_t K);
+// M > 1: fp16 matrix-core GEMM over Q4 block16 weights (gemm_q4_mfma.hip); operands already validated.
+int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb, const uint32_t* lc,
+                        uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops);
 // Second pass of the fused GEMV + argmax: best of the per-group partials, token id stored as float.
 int launch_argmax_pairs(const Map* ma, const uint32_t* lidx, const uint32_t* lval, const uint32_t* ldst,
                         uint32_t n_groups);

@@ -516,7 +516,7 @@ static void mfma_shape(uint32_t K, uint32_t units, uint32_t* grid, uint32_t* thr
   while (waves > 4 && cdiv(units, waves) < (uint32_t)g.n_cu) waves >>= 1;
   waves = (uint32_t)tuning("ADAMAH_MFMA_WAVES", (int)waves);
   waves = waves >= 16 ? 16 : waves >= 8 ? 8 : 4;
-  const uint32_t per_simd = (uint32_t)std::max(1, tuning("ADAMAH_MFMA_PERSIMD", 4));
+  const uint32_t per_simd = (uint32_t)std::max(1, tuning("ADAMAH_MFMA_PERSIMD", 2));
   const size_t lds_fit = std::max<size_t>(1, (160 * 1024) / (mfma_smem(K) + 256));
   const uint32_t wg_per_cu = (uint32_t)std::max<size_t>(1, std::min<size_t>(lds_fit, (size_t)per_simd * 4 / waves));
   *threads = waves * 64;

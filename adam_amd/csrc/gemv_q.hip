@@ -548,6 +548,17 @@ int op_matmul_t_xq(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t h
     return launch_block<EPI_STORE>(fmt, ma, mw, la, lb, lc, nullptr, nullptr, K, N,
                                    (uint32_t)tuning("ADAMAH_GEMV_RPG", 16));
   }
+  // several activation rows over Q4_0 blocks: fp16 matrix-core GEMM
+  if (transposed && M > 1 && dtype == DTYPE_Q4 && mw->group_size == 32 && K >= 128 && (K & 127u) == 0 && ah && bh && ch &&
+      mw->pack_size == 1 && ma->pack_size == 1 && tuning("ADAMAH_GEMM_IMPL", 1) == 1) {
+    bool ok = true;
+    for (uint32_t op = 0; ok && op < n_ops; op++)
+      ok = (bh[op] & 31u) == 0 && fmt_of(mw, bh[op], (uint64_t)N * K) == FMT_Q4_B16;
+    if (ok) {
+      flush_pending();
+      return launch_gemm_q4_mfma(ma, mw, la, lb, lc, M, K, N, n_ops);
+    }
+  }
 generic:
   flush_pending();
   dim3 grid(cdiv(N, 4), M, n_ops);
