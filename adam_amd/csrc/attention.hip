@@ -534,7 +534,12 @@ static void attn_split(uint32_t n_ops, uint32_t row_size, uint32_t value_dim, bo
   c = (c + 31u) & ~31u;
   // `few`: the consumer will merge the partials, every one of its workgroups reads all of them, so
   // keep them few (longer chunks) as long as a chunk still fits a workgroup
-  while (few && c < ATT_CHUNK && (uint64_t)n_ops * cdiv(row_size, c) * (value_dim + 2) > ATT_FOLD_FLOATS) c += 32u;
+  if (few) {
+    uint32_t cf = c;
+    while (cf < ATT_CHUNK && (uint64_t)n_ops * cdiv(row_size, cf) * (value_dim + 2) > ATT_FOLD_FLOATS) cf += 32u;
+    // partials still too many at the longest chunk: the consumer will not merge them, keep the wide split
+    if ((uint64_t)n_ops * cdiv(row_size, cf) * (value_dim + 2) <= ATT_FOLD_FLOATS) c = cf;
+  }
   *chunk = c;
   *n_splits = cdiv(row_size, c);
 }

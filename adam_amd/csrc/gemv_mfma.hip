@@ -63,13 +63,14 @@ __global__ void __launch_bounds__(1024)
 k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, const float2* __restrict__ qp,
             const __half* __restrict__ d16, uint32_t a, uint32_t b_off, uint32_t c_out,
             const uint32_t* __restrict__ lidx, const uint32_t* __restrict__ lval, uint32_t K, uint32_t N,
-            uint32_t rows_per_group, uint32_t n_groups, GemvFuse fz) {
+            uint32_t rows_per_group, uint32_t n_groups, uint32_t ks, GemvFuse fz) {
   TR(0);
   constexpr bool B16 = (FMT == FMT_Q4_B16);
   extern __shared__ uint4 smem_u4[];
   uint8_t* xs = (uint8_t*)smem_u4;                    // nblk * 128 bytes
   __shared__ float red_f[16];
   __shared__ uint32_t red_i[16];
+  __shared__ float part[16 * 64];                     // ks > 1: per-wave partial sums of a shared bundle
   const uint32_t nblk = K >> 5;
   const uint32_t C = (nblk + 63u) >> 6;               // steps per row bundle
 
@@ -81,8 +82,17 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
   // ---- this wave's rows: store = contiguous balanced share of the 4-row bundles (waves that share
   // a SIMD, w % 4, take neighbouring shares so that every SIMD gets the same load); argmax = the
   // workgroup takes whole argmax groups, its waves interleave the bundles of a group ------------
+  // ks > 1 (store only, short matrices with long rows): ks neighbouring waves share one bundle and take
+  // every ks-th step of K each; a workgroup holds nwav / ks bundles, one round.
   uint32_t grp = blockIdx.x, first, stride, seg_end;
-  if (EPI == EPI_STORE) {
+  const uint32_t kpart = ks > 1u ? wave % ks : 0u;
+  if (EPI == EPI_STORE && ks > 1u) {
+    const uint32_t bundle = blockIdx.x * (nwav / ks) + wave / ks;
+    first = bundle * 4u;
+    seg_end = kpart < C ? min(N, first + 4u) : 0u;      // nothing to do: no bundle, or no step of K left for this wave
+    if (first >= N) seg_end = 0u;
+    stride = 4u;
+  } else if (EPI == EPI_STORE) {
     const uint32_t slot = (wave & 3u) * (nwav >> 2) + (wave >> 2);
     const uint64_t n_q = (N + 3u) / 4u, gw = (uint64_t)blockIdx.x * nwav + slot, wt = (uint64_t)gridDim.x * nwav;
     first = (uint32_t)(gw * n_q / wt) * 4u;
@@ -117,7 +127,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
   };
 
   PreM A, B;   // A's first loads stay in flight while the activations are staged
-  if (PRO == PRO_NONE && first < seg_end) load(A, first, 0, seg_end);
+  if (PRO == PRO_NONE && first < seg_end) load(A, first, kpart, seg_end);
 
   // ---- activations -> fixed-point digits; one 8-element word per thread and pass, four threads per
   // block.  stage() turns one word into digits; the prologues below decide what the word is. ------
@@ -193,7 +203,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
   } else if (PRO == PRO_COMBINE) {
     // Folded merge of the attention partials (same arithmetic as the stand-alone merge kernel):
     // M = max m_s, w_s = e^(m_s - M), L = sum l_s w_s, x = sum_s o_s w_s / L, per head.
-    if (first < seg_end) load(A, first, 0, seg_end);
+    if (first < seg_end) load(A, first, kpart, seg_end);
     const uint32_t stride = fz.c_vd + 2u;
     for (uint32_t i0 = 0; i0 < nw; i0 += nthr) {
       const uint32_t i = i0 + tid, ic = min(i, nw - 1u);
@@ -244,7 +254,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       if (PRO == PRO_NORM2) { load8(act + fz.p_res + e0, rv[u]); load8(fz.p_wt2 + fz.p_w2 + e0, w2v[u]); }
     }
     __builtin_amdgcn_sched_barrier(0);   // activation loads first: they are waited for first
-    if (first < seg_end) load(A, first, 0, seg_end);
+    if (first < seg_end) load(A, first, kpart, seg_end);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (uint32_t u = 0; u < PRO_WPT; u++)
@@ -361,7 +371,9 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
         acc = fmaf(sc, (float)sq * fsb, fmaf(zp, sxb, acc));
       }
     }
-    if (chunk == C - 1u) {   // row bundle complete: sum the 16 lanes that share a row
+    if (ks > 1u) {
+      if (chunk + ks >= C) part[wave * 64u + lane] = acc;   // this wave's share of the bundle is done
+    } else if (chunk == C - 1u) {   // row bundle complete: sum the 16 lanes that share a row
       float y = acc;
       y += __shfl_xor(y, 4, 64); y += __shfl_xor(y, 8, 64);
       y += __shfl_xor(y, 16, 64); y += __shfl_xor(y, 32, 64);
@@ -414,25 +426,43 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       // steps t = 0..T-1 in (row bundle, chunk) order; register set A holds step 0 on entry.  The
       // prefetch of the following step is issued unconditionally (past the end it re-reads the last
       // rows, clamped in load()), so the number of loads in flight at every wait is known statically.
-      const uint32_t T = ((seg_end - first + stride - 1u) / stride) * C;
-      uint32_t row_a = first, ch_a = 0, row_b, ch_b, row_n = first, ch_n = 0;
-      if (++ch_n == C) { ch_n = 0; row_n += stride; }
-      if (T == 1) compute(A, first, 0, seg_end);   // nothing to prefetch
+      const uint32_t Cw = (C - kpart + ks - 1u) / ks;     // steps of K this wave takes per bundle
+      const uint32_t T = ((seg_end - first + stride - 1u) / stride) * Cw;
+      uint32_t row_a = first, ch_a = kpart, row_b, ch_b, row_n = first, ch_n = kpart;
+      if ((ch_n += ks) >= C) { ch_n = kpart; row_n += stride; }
+      if (T == 1) compute(A, first, kpart, seg_end);   // nothing to prefetch
       else for (uint32_t t = 0; t < T; t += 2) {
         row_b = row_n; ch_b = ch_n;
         load(B, row_b, ch_b, seg_end);
         __builtin_amdgcn_sched_barrier(0);   // keep the prefetch ahead of the arithmetic
-        if (++ch_n == C) { ch_n = 0; row_n += stride; }
+        if ((ch_n += ks) >= C) { ch_n = kpart; row_n += stride; }
         compute(A, row_a, ch_a, seg_end);
         if (t + 1 >= T) break;
         row_a = row_n; ch_a = ch_n;
         load(A, row_a, ch_a, seg_end);
         __builtin_amdgcn_sched_barrier(0);
-        if (++ch_n == C) { ch_n = 0; row_n += stride; }
+        if ((ch_n += ks) >= C) { ch_n = kpart; row_n += stride; }
         compute(B, row_b, ch_b, seg_end);
       }
     }
     TR(6);
+    if (EPI == EPI_STORE && ks > 1u) {
+      // the ks waves of a bundle meet: the first of them adds the shares in wave order and stores
+      if (!(first < seg_end)) part[wave * 64u + lane] = 0.f;
+      __syncthreads();
+      if (kpart == 0u && first < N) {
+        float y = part[wave * 64u + lane];
+        for (uint32_t pk = 1; pk < ks; pk++) y += part[(wave + pk) * 64u + lane];
+        y += __shfl_xor(y, 4, 64); y += __shfl_xor(y, 8, 64);
+        y += __shfl_xor(y, 16, 64); y += __shfl_xor(y, 32, 64);
+        const uint32_t row = first + l;
+        if (row < N && bcol == 0u) {
+          act_out[(uint64_t)c_out + row] = y;
+          if (fz.e_mode == EPIX_ADD) act_out[(uint64_t)fz.e_dst + row] = act[(uint64_t)fz.e_res + row] + y;
+        }
+      }
+      break;
+    }
     if (EPI == EPI_STORE) break;
     // argmax: next group's first loads go out before this group's partial is merged
     const uint32_t done = grp;
@@ -478,13 +508,13 @@ bool mfma_path_ok(const Map* mw, uint32_t K) {
 template <int EPI, int PRO>
 static void launch_mfma_p(int fmt, uint32_t grid, uint32_t threads, const Map* ma, const Map* mw, uint32_t a, uint32_t b,
                           uint32_t c, const uint32_t* lidx, const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rpg,
-                          uint32_t n_groups, const GemvFuse& fz) {
+                          uint32_t n_groups, uint32_t ks, const GemvFuse& fz) {
   float* act = (float*)ma->buf;
   const size_t smem = mfma_smem(K);
   const bool ragged = (K & 2047u) != 0;
 #define MK(F, R)                                                                                                  \
   k_gemv_mfma<F, EPI, R, PRO><<<grid, threads, smem, g.stream>>>(act, act, mw->buf, mw->qp, mw->d16, a, b, c, lidx, \
-                                                                 lval, K, N, rpg, n_groups, fz)
+                                                                 lval, K, N, rpg, n_groups, ks, fz)
   if (fmt == FMT_Q4_B16) { if (ragged) MK(FMT_Q4_B16, true); else MK(FMT_Q4_B16, false); }
   else { if (ragged) MK(FMT_Q4_AFF, true); else MK(FMT_Q4_AFF, false); }
 #undef MK
@@ -493,10 +523,10 @@ static void launch_mfma_p(int fmt, uint32_t grid, uint32_t threads, const Map* m
 template <int EPI>
 static int launch_mfma(int fmt, uint32_t grid, uint32_t threads, const Map* ma, const Map* mw, uint32_t a, uint32_t b,
                        uint32_t c, const uint32_t* lidx, const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rpg,
-                       uint32_t n_groups, const GemvFuse* fzp) {
+                       uint32_t n_groups, uint32_t ks, const GemvFuse* fzp) {
   GemvFuse fz = {};
   if (fzp) fz = *fzp;
-#define MP(P) launch_mfma_p<EPI, P>(fmt, grid, threads, ma, mw, a, b, c, lidx, lval, K, N, rpg, n_groups, fz)
+#define MP(P) launch_mfma_p<EPI, P>(fmt, grid, threads, ma, mw, a, b, c, lidx, lval, K, N, rpg, n_groups, ks, fz)
   switch (fz.pro) {
     case PRO_RMSNORM: MP(PRO_RMSNORM); break;
     case PRO_NORM2: MP(PRO_NORM2); break;
@@ -523,17 +553,40 @@ static void mfma_shape(uint32_t K, uint32_t units, uint32_t* grid, uint32_t* thr
   *grid = std::max(1u, std::min<uint32_t>(cdiv(units, waves), (uint32_t)g.n_cu * wg_per_cu));
 }
 
+// Store launches of short matrices with long rows leave most SIMDs without work when a bundle of four
+// rows belongs to one wave: there, 2 or 4 waves share a bundle and split K (one step of 2048 at a time).
+static uint32_t mfma_ksplit(uint32_t K, uint32_t N, bool paired_rows) {
+  const uint32_t C = cdiv(K, 2048u), n_q = cdiv(N, 4u);
+  const uint32_t want = (uint32_t)std::max(1, tuning("ADAMAH_MFMA_KSPLIT_WAVES", 4096));
+  uint32_t ks = 1;
+  // every wave keeps at least one full step and a partial one, so its loads still overlap its arithmetic
+  while (ks < 4u && ks * 2u * 3u <= C * 2u && n_q * ks * 2u <= want) ks *= 2u;
+  const int forced = tuning("ADAMAH_MFMA_KS", 0);
+  if (forced == 1 || forced == 2 || forced == 4) ks = std::min<uint32_t>((uint32_t)forced, std::max(1u, C));
+  if (ks == 3u) ks = 2u;
+  return paired_rows ? 1u : ks;
+}
+
+static void mfma_store_shape(uint32_t K, uint32_t N, uint32_t ks, uint32_t* grid, uint32_t* threads) {
+  const uint32_t n_q = cdiv(N, 4u);
+  mfma_shape(K, n_q * ks, grid, threads);
+  if (ks > 1u) *grid = cdiv(n_q, *threads / 64u / ks);   // one bundle per ks waves, one round
+}
+
 uint32_t mfma_store_threads(uint32_t K, uint32_t N) {
-  uint32_t grid, threads;
-  mfma_shape(K, cdiv(N, 4), &grid, &threads);
-  return threads;
+  uint32_t grid, t1, tk;
+  mfma_store_shape(K, N, 1u, &grid, &t1);
+  mfma_store_shape(K, N, mfma_ksplit(K, N, false), &grid, &tk);
+  return std::min(t1, tk);
 }
 
 int launch_mfma_store(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32_t b, uint32_t c, uint32_t K,
                       uint32_t N, const GemvFuse* fz) {
   uint32_t grid, threads;
-  mfma_shape(K, cdiv(N, 4), &grid, &threads);
-  return launch_mfma<EPI_STORE>(fmt, grid, threads, ma, mw, a, b, c, nullptr, nullptr, K, N, 0, 0, fz);
+  const bool paired = fz && (fz->e_mode == EPIX_GEGLU || fz->e_mode == EPIX_SWIGLU);
+  const uint32_t ks = mfma_ksplit(K, N, paired);
+  mfma_store_shape(K, N, ks, &grid, &threads);
+  return launch_mfma<EPI_STORE>(fmt, grid, threads, ma, mw, a, b, c, nullptr, nullptr, K, N, 0, 0, ks, fz);
 }
 
 int launch_mfma_argmax(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32_t b, const uint32_t* lidx,
@@ -542,7 +595,7 @@ int launch_mfma_argmax(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32
   uint32_t grid, threads;
   mfma_shape(K, n_groups * 16u, &grid, &threads);   // one workgroup per group at a time
   grid = std::min(grid, n_groups);
-  return launch_mfma<EPI_ARGMAX>(fmt, grid, threads, ma, mw, a, b, 0, lidx, lval, K, N, rows_per_group, n_groups, fz);
+  return launch_mfma<EPI_ARGMAX>(fmt, grid, threads, ma, mw, a, b, 0, lidx, lval, K, N, rows_per_group, n_groups, 1u, fz);
 }
 
 }  // namespace adamah

@@ -126,9 +126,10 @@ def main():
     ap.add_argument("--workload", default="gemma3-1b", choices=["gemma3-1b", "llama3-8b"])
     ap.add_argument("--prompt", type=int, default=None, help="prompt length (default 512 / 3840)")
     ap.add_argument("--scheduler", default="level_batched", choices=["legacy", "level_batched"])
-    ap.add_argument("--only", default=None, choices=["gemv", "probe"],
-                    help="gemv: just the GEMV roofline leg; probe: plain read/copy kernels of known size "
-                         "(reference points for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--only", default=None, choices=["roofline", "gemv", "probe"],
+                    help="roofline: just the 28672x4096 GEMV (one kernel row in a rocprofv3 --stats table); "
+                         "gemv: that shape, 4096x4096 and 4096x14336; probe: plain read/copy kernels of known "
+                         "size (reference points for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -140,7 +141,9 @@ def main():
 
     if args.only:
         gpu = A.init()
-        if args.only == "gemv":
+        if args.only == "roofline":
+            out = {"gemv_shapes": measure_gemv(gpu, A, LLAMA_GEMV_SHAPES[:1], rounds=8)}
+        elif args.only == "gemv":
             out = {"gemv_shapes": measure_gemv(gpu, A, LLAMA_GEMV_SHAPES[:1] + LLAMA_GEMV_SHAPES[3:], rounds=3)}
         else:
             nbytes = gemv_bytes(28672, 4096) // 4096 * 4096
@@ -223,7 +226,7 @@ def main():
         top = shapes["28672x4096"]
         res["roofline"] = {"bound": "hbm", "achieved": top["GB/s"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                            "frac": top["frac"], "traffic": GEMV_TRAFFIC_BYTES,
-                           "kernel": "k_gemv_block<Q4_0, store> 28672x4096, "
+                           "kernel": "k_gemv_mfma<Q4_0 block16, store> 28672x4096, "
                                      f"{gemv_bytes(28672, 4096)} algorithmic B/launch"}
         res["gemv_shapes"] = shapes
     gpu.shutdown()
