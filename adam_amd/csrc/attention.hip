@@ -8,6 +8,7 @@
 // merge (running max m, sum l, weighted values o), so any length works.  K/V rows are read from
 // the fp16 copy of the KV range when the operands lie inside it, else from the float32 map.
 #include "common.h"
+#include "attn_common.h"
 #include "../../include/adamah_hip.h"
 #include <algorithm>
 
@@ -125,11 +126,6 @@ k_matmul_nt(const float* A, float* C, const float* B, const uint32_t* __restrict
   if (lane == 0 && c < a_elems) C[c] = s;
 }
 
-__device__ __forceinline__ float prep(float v, float scale, float cap) {
-  v *= scale;
-  if (cap > 0.0f) v = tanhf(v / cap) * cap;
-  return v;
-}
 
 #define ATT_CHUNK 1024   // most score rows one workgroup handles (LDS array size)
 
@@ -450,12 +446,14 @@ k_attn_fused(const float* data, float* out, const __half* kv, uint64_t kv_shift,
 }
 
 // Merge the split partials of one op: M = max m_s, w_s = e^(m_s-M), L = sum l_s w_s,
-// out = sum_s o_s w_s / L.  n_splits <= 1024.
+// out = sum_s o_s w_s / L.  n_splits <= 1024.  grid (n_ops, ceil(value_dim / 32)): a workgroup owns 32
+// output elements, eight groups of 32 threads take every eighth split each and meet in LDS.
 __global__ void __launch_bounds__(256)
 k_attn_combine(float* out, const float* partial, const uint32_t* __restrict__ lo, uint32_t value_dim,
                uint32_t n_splits, uint64_t n_elems) {
   __shared__ float w[1024];
   __shared__ float red[4];
+  __shared__ float osum[8][32];
   const uint32_t op = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t stride = value_dim + 2;
   const float* pp = partial + (uint64_t)op * n_splits * stride;
@@ -478,9 +476,22 @@ k_attn_combine(float* out, const float* partial, const uint32_t* __restrict__ lo
   if (lane == 0) red[wave] = L;
   __syncthreads();
   const float invL = 1.0f / ((red[0] + red[1]) + (red[2] + red[3]));
-  for (uint32_t d = tid; d < value_dim; d += 256u) {
+  const uint32_t d = blockIdx.y * 32u + (tid & 31u), sg = tid >> 5;
+  float o0 = 0.f, o1 = 0.f;
+  if (d < value_dim) {
+    uint32_t s = sg;
+    for (; s + 8u < n_splits; s += 16u) {
+      o0 = fmaf(pp[(uint64_t)s * stride + 2 + d], w[s], o0);
+      o1 = fmaf(pp[(uint64_t)(s + 8u) * stride + 2 + d], w[s + 8u], o1);
+    }
+    if (s < n_splits) o0 = fmaf(pp[(uint64_t)s * stride + 2 + d], w[s], o0);
+  }
+  osum[sg][tid & 31u] = o0 + o1;
+  __syncthreads();
+  if (tid < 32u && d < value_dim) {
     float o = 0.f;
-    for (uint32_t s = 0; s < n_splits; s++) o = fmaf(pp[(uint64_t)s * stride + 2 + d], w[s], o);
+#pragma unroll
+    for (int i = 0; i < 8; i++) o += osum[i][tid];
     out[ob + d] = o * invL;
   }
 }
@@ -596,6 +607,23 @@ int launch_attn(const PendOp* sc, const PendOp& at, bool leave_partials, AttnPar
   if ((uint64_t)n_ops * n_splits * (value_dim + 2) > ATT_FOLD_FLOATS) leave_partials = false;
   float* d = (float*)m->buf;
   dim3 grid(n_splits, n_ops);
+  if (sc && fast && kv && sc->k == value_dim) {
+    // all query heads of a KV head in one workgroup, K and V rows read once
+    AttnDecodeArgs da = {d, m->kv16, m->kv_start,
+                         res_u32(sc->h[0], n_ops), res_u32(sc->h[1], n_ops), ls, lv, lo,
+                         res_host(sc->h[0], n_ops), res_host(sc->h[1], n_ops), res_host(at.h[0], n_ops),
+                         res_host(at.h[1], n_ops), res_host(at.h[2], n_ops),
+                         n_ops, value_dim, row_size, at.eps, at.f2, leave_partials, ATT_FOLD_FLOATS};
+    int drc = 0;
+    bool left = false;
+    AttnPartials dp = {};
+    if (launch_attn_decode(da, &dp, &left, &drc)) {
+      if (ap) ap->n_splits = 1;
+      if (drc || dp.n_splits == 1) return drc;
+      if (left && ap) { *ap = dp; return ADAMAH_OK; }
+      return launch_attn_combine(at, dp);
+    }
+  }
   if (sc && fast && kv) {
     const uint32_t *la = res_u32(sc->h[0], n_ops), *lb = res_u32(sc->h[1], n_ops);
     uint32_t lpr = 8;
@@ -628,7 +656,7 @@ int launch_attn_combine(const PendOp& at, const AttnPartials& ap) {
   Map* m = get_f32_map(at.map_act);
   const uint32_t* lo = res_u32(at.h[2], at.rpg);
   if (!m || !lo) return ADAMAH_ERR_INVALID;
-  k_attn_combine<<<at.rpg, 256, 0, g.stream>>>((float*)m->buf, ap.base, lo, ap.value_dim, ap.n_splits, m->n_elems);
+  k_attn_combine<<<dim3(at.rpg, cdiv(ap.value_dim, 32)), 256, 0, g.stream>>>((float*)m->buf, ap.base, lo, ap.value_dim, ap.n_splits, m->n_elems);
   count_launch();
   return check_launch();
 }

@@ -1,0 +1,373 @@
+// Grouped decode attention: scores and softmax . V of one token for all query heads that share a
+// KV head, in one pass over the fp16 K and V rows.
+//
+// Reference: the pair map_matmul_t_dev (scores, shaders/src/f32/map_matmul_t.comp) and
+// map_attn_softmax_value_dev (map_attn_softmax_value.comp:39-89; dispatch adamah.c:6682-6781,
+// 7894-8059) as the decode loop issues them (adam/models/engine.py:2428-2441 for the arithmetic).
+// The reference runs one workgroup per query head, so every KV row is fetched once per head of its
+// group and twice more through the score row; here a workgroup owns (KV head, slice of the sequence)
+// and reads each K and V row once for the whole group.
+//
+// Workgroup = NW (4 or 8) waves; a wave takes 16-row tiles of the slice.  Per tile a lane issues its K and V
+// loads together (16 bytes each, rows contiguous across lanes), then
+//   scores  v_mfma_f32_16x16x16_f16 with A = queries (matrix row = head, zero beyond the group) and
+//           B = K tile (column = row of the tile).  The queries are scaled per head by a power of two
+//           into fp16 range and split into a high and a low fp16 part, so the products are exact and
+//           the sum is fp32: the raw scores stored to the score rows match a float32 dot product.
+//   softmax online per wave (running maximum m, sum l), weights handed to the V phase through LDS
+//   values  every lane owns D/64 dims of the output and sees all 16 rows of the tile: fp32 FMAs, one
+//           accumulator set per head of the group, no reduction across lanes.
+// With more than one tile per wave (PF) the next tile's loads are issued before the current tile's
+// arithmetic (two register sets).  The queries reach the lanes through LDS, so their rows need no
+// alignment.  The waves merge through LDS; slices merge through partials (m, l, o[D]) per head and slice, by
+// the consumer when they are few, else by the merge kernel.  (A merge by the last workgroup to
+// finish, found with an atomic ticket, needs a device-scope release and acquire in every workgroup;
+// each of those writes back and invalidates the L2 of its XCD and the kernel got 4x slower.)
+#include "attn_common.h"
+#include <algorithm>
+
+namespace adamah {
+
+typedef _Float16 h4a_t __attribute__((ext_vector_type(4)));
+typedef float f4a_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u2a_t __attribute__((ext_vector_type(2)));
+
+#ifdef ADAMAH_TRACE
+__device__ unsigned long long g_trace_attd[64];
+#define TRD(i) do { if (threadIdx.x == 0 && blockIdx.x == 0 && blockIdx.y == 0) g_trace_attd[i] = wall_clock64(); } while (0)
+#else
+#define TRD(i) do {} while (0)
+#endif
+
+#define ATTD_NEG (-1.0e30f)
+#define ATTD_MAX_SPLITS 256u
+#define ATTD_MAX_GROUPS 128u
+
+// Operand bases by value (the handles' host copies): saves a dependent load before the first K row.
+#define ATTD_MAX_OPS 64u
+struct AttdBases { uint32_t q[ATTD_MAX_OPS], sc[ATTD_MAX_OPS], o[ATTD_MAX_OPS], kb[ATTD_MAX_OPS], vb[ATTD_MAX_OPS]; };
+
+#define ATTD_DPP(v, ctrl) __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, 0xF, 0xF, false))
+// all-reduce over each 16-lane row: quad_perm [1,0,3,2], [2,3,0,1], row_half_mirror, row_mirror
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, ATTD_DPP(v, 0xB1)); v = fmaxf(v, ATTD_DPP(v, 0x4E));
+  v = fmaxf(v, ATTD_DPP(v, 0x141)); v = fmaxf(v, ATTD_DPP(v, 0x140));
+  return v;
+}
+__device__ __forceinline__ float row16_sum(float v) {
+  v += ATTD_DPP(v, 0xB1); v += ATTD_DPP(v, 0x4E); v += ATTD_DPP(v, 0x141); v += ATTD_DPP(v, 0x140);
+  return v;
+}
+
+template <int D, int G, int NW, bool PF>
+__global__ void __launch_bounds__(NW * 64)
+k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift, const AttdBases bs,
+              uint32_t row_size, float scale, float cap, uint32_t n_splits, uint32_t chunk, float* partial) {
+  constexpr int NI = D / 32;           // 16-byte K loads per lane and tile
+  constexpr int DPL = D / 64;          // V dims per lane (every lane sees all 16 rows of the tile)
+  constexpr int DW = DPL > 2 ? DPL / 2 : 1;
+  constexpr uint32_t NT = NW * 64;     // threads
+  __shared__ float pbuf[NW][16][G];    // softmax weights of the wave's tile, [row][head]
+  __shared__ float abuf[NW][G];        // per head: rescale factor of the tile
+  __shared__ float obuf[NW][G][D];     // wave results; first the queries of the group, [head][dim]
+  __shared__ float mlbuf[NW][G][2];
+  __shared__ h4a_t qop[2 * NI][2][64]; // query operands of the matrix product: [k-step][hi, lo][lane]
+  __shared__ uint32_t hmax[G];         // per head: bits of max |q|
+  __shared__ float qinv[G];            // per head: 1 / (power-of-two scale of the queries)
+
+  TRD(0);
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));   // scalar: row numbers below are too
+  const uint32_t c = lane & 15u, kc = lane >> 4;
+  const uint32_t split = blockIdx.x, group = blockIdx.y, op0 = group * G;
+  const uint32_t t0 = split * chunk, t1 = min(row_size, t0 + chunk);
+  // wave-uniform bases plus 32-bit byte offsets: the V row of a load is the same for all lanes
+  const char* kbase = (const char*)(kv + ((uint64_t)bs.kb[group] - kv_shift));
+  const char* vbase = (const char*)(kv + ((uint64_t)bs.vb[group] - kv_shift));
+  const uint32_t klane = 16u * kc, vlane = 2u * (uint32_t)DPL * lane;
+
+  auto fetch = [&](uint4 (&kr)[NI], uint32_t (&vr)[16][DW], uint32_t rb) {
+    const uint32_t koff = min(rb + c, t1 - 1u) * (2u * D) + klane;
+#pragma unroll
+    for (int i = 0; i < NI; i++) kr[i] = *(const uint4*)(kbase + koff + 64u * i);
+#pragma unroll
+    for (int u = 0; u < 16; u++) {
+      const char* src = vbase + (uint64_t)(min(rb + u, t1 - 1u) * (2u * D)) + vlane;
+      if (DPL == 1) vr[u][0] = *(const uint16_t*)src;
+      else if (DPL == 2) vr[u][0] = *(const uint32_t*)src;
+      else { const uint2 t = *(const uint2*)src; vr[u][0] = t.x; vr[u][DW - 1] = t.y; }
+    }
+  };
+
+  // Queries: coalesced scalar loads into LDS (obuf[0] is free until the end) with the per-head
+  // maximum on the way; then the first tile's K and V loads go out; then the matrix-A operands (lane
+  // (head c, kc) of operand 2i+j: dims 32i + 8kc + 4j .. +3 of head c, zero beyond the group), scaled
+  // by 2^e into [2^13, 2^14) and split hi + lo, are written to LDS once for all waves.
+  uint4 kA[NI], kB[NI];
+  uint32_t vA[16][DW], vB[16][DW];
+  uint32_t rbase = t0 + wave * 16u;
+  const bool any = rbase < t1;
+  {
+    float* qs = &obuf[0][0][0];
+    if (tid < (uint32_t)G) hmax[tid] = 0u;
+    __syncthreads();
+    for (uint32_t i = tid; i < (uint32_t)(G * D); i += NT) {   // a wave's 64 elements belong to one head
+      const uint32_t hq = (uint32_t)__builtin_amdgcn_readfirstlane((int)(i / D));   // scalar: read from the arguments
+      const float x = data[(uint64_t)bs.q[op0 + hq] + i % D];
+      qs[i] = x;
+      float m = fabsf(x);
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+      if (lane == 0u) atomicMax(&hmax[i / D], __float_as_uint(m));
+    }
+    if (any) fetch(kA, vA, rbase);
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    const uint32_t e = c < G ? (hmax[c] >> 23) & 0xFFu : 0u;
+    float s = 1.f, inv = 1.f;
+    if (e >= 14u && e <= 254u) { s = __uint_as_float((267u - e) << 23); inv = __uint_as_float((e - 13u) << 23); }
+    if (wave == 0u && c < G && kc == 0u) qinv[c] = inv;
+    for (uint32_t idx = wave; idx < 2u * NI; idx += NW) {
+      const float4 q4 = c < G ? *(const float4*)(qs + c * D + 32u * (idx >> 1) + 8u * kc + 4u * (idx & 1u))
+                              : make_float4(0.f, 0.f, 0.f, 0.f);
+      const float x[4] = {q4.x * s, q4.y * s, q4.z * s, q4.w * s};
+      h4a_t hi4, lo4;
+#pragma unroll
+      for (int t = 0; t < 4; t++) {
+        const _Float16 hi = (_Float16)x[t];
+        hi4[t] = hi;
+        lo4[t] = (_Float16)(x[t] - (float)hi);
+      }
+      qop[idx][0][lane] = hi4;
+      qop[idx][1][lane] = lo4;
+    }
+    __syncthreads();
+  }
+  TRD(1);
+  // after the matrix product lane (c, kc) holds heads 4kc..4kc+3 of tile row c
+  float inv_s[4], m_run[4], l_run[4];
+  bool hval[4];
+  uint32_t crow[4];
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    hval[r] = 4u * kc + r < (uint32_t)G;
+    inv_s[r] = hval[r] ? qinv[4u * kc + r] : 0.f;
+    // scalar reads of the arguments, then a per-lane choice
+    crow[r] = 0u;
+    if (r < G) crow[r] = bs.sc[op0 + r];
+    if (G > 4 && kc == 1u) crow[r] = bs.sc[op0 + (4 + r) % G];
+    m_run[r] = ATTD_NEG;
+    l_run[r] = 0.f;
+  }
+
+  float acc[G][DPL];
+#pragma unroll
+  for (int h = 0; h < G; h++)
+#pragma unroll
+    for (int j = 0; j < DPL; j++) acc[h][j] = 0.f;
+
+  auto tile = [&](const uint4 (&kr)[NI], const uint32_t (&vr)[16][DW], uint32_t rb) {
+    // scores of the tile: 2 * NI k-steps, high and low query part each, four independent sums
+    f4a_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = s0, s2 = s0, s3 = s0;
+#pragma unroll
+    for (int i = 0; i < NI; i++) {
+      const u2a_t b0 = {kr[i].x, kr[i].y}, b1 = {kr[i].z, kr[i].w};
+      s0 = __builtin_amdgcn_mfma_f32_16x16x16f16(qop[2 * i][0][lane], __builtin_bit_cast(h4a_t, b0), s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x16f16(qop[2 * i][1][lane], __builtin_bit_cast(h4a_t, b0), s1, 0, 0, 0);
+      s2 = __builtin_amdgcn_mfma_f32_16x16x16f16(qop[2 * i + 1][0][lane], __builtin_bit_cast(h4a_t, b1), s2, 0, 0, 0);
+      s3 = __builtin_amdgcn_mfma_f32_16x16x16f16(qop[2 * i + 1][1][lane], __builtin_bit_cast(h4a_t, b1), s3, 0, 0, 0);
+    }
+    TRD(3);
+    const uint32_t row = rb + c;
+    const bool rok = row < t1;
+    float v[4], mt[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const float raw = ((s0[r] + s2[r]) + (s1[r] + s3[r])) * inv_s[r];
+      if (rok && hval[r]) out[(uint64_t)crow[r] + row] = raw;
+      v[r] = rok && hval[r] ? prep(raw, scale, cap) : ATTD_NEG;
+      mt[r] = row16_max(v[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const float m_new = fmaxf(m_run[r], mt[r]);
+      const float alpha = __expf(m_run[r] - m_new);
+      const float p = rok && hval[r] ? __expf(v[r] - m_new) : 0.f;
+      l_run[r] = l_run[r] * alpha + p;
+      m_run[r] = m_new;
+      if (hval[r]) {
+        pbuf[wave][c][4u * kc + r] = p;
+        if (c == 0u) abuf[wave][4u * kc + r] = alpha;
+      }
+    }
+    TRD(4);
+    __builtin_amdgcn_wave_barrier();
+    // values: rescale the running sums, then the sixteen rows of the tile
+#pragma unroll
+    for (int h = 0; h < G; h++) {
+      const float al = abuf[wave][h];
+#pragma unroll
+      for (int j = 0; j < DPL; j++) acc[h][j] *= al;
+    }
+#pragma unroll
+    for (int u = 0; u < 16; u++) {
+      float f[DPL];
+      if (DPL == 1) f[0] = __half2float(__ushort_as_half((unsigned short)vr[u][0]));
+      else {
+#pragma unroll
+        for (int w = 0; w < DW; w++) {
+          const float2 t = __half22float2(*(const __half2*)&vr[u][w]);
+          f[2 * w] = t.x; f[(2 * w + 1) % DPL] = t.y;
+        }
+      }
+#pragma unroll
+      for (int h = 0; h < G; h++) {
+        const float pw = pbuf[wave][u][h];
+#pragma unroll
+        for (int j = 0; j < DPL; j++) acc[h][j] = fmaf(pw, f[j], acc[h][j]);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+
+  TRD(2);
+  if (any) {
+    if (PF) {
+      while (true) {
+        fetch(kB, vB, rbase + NW * 16u);     // next tile (clamped into the slice when there is none)
+        __builtin_amdgcn_sched_barrier(0);
+        tile(kA, vA, rbase);
+        rbase += NW * 16u;
+        if (rbase >= t1) break;
+        fetch(kA, vA, rbase + NW * 16u);
+        __builtin_amdgcn_sched_barrier(0);
+        tile(kB, vB, rbase);
+        rbase += NW * 16u;
+        if (rbase >= t1) break;
+      }
+    } else {
+      while (true) {
+        tile(kA, vA, rbase);
+        rbase += NW * 16u;
+        if (rbase >= t1) break;
+        fetch(kA, vA, rbase);
+      }
+    }
+  }
+  TRD(5);
+
+  // wave results to LDS: l summed over the 16 tile rows; each lane owns its dims of the output
+#pragma unroll
+  for (int r = 0; r < 4; r++) l_run[r] = row16_sum(l_run[r]);
+#pragma unroll
+  for (int h = 0; h < G; h++)
+#pragma unroll
+    for (int j = 0; j < DPL; j++) obuf[wave][h][(uint32_t)DPL * lane + j] = acc[h][j];
+  if (c == 0u) {
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+      if (hval[r]) { mlbuf[wave][4u * kc + r][0] = m_run[r]; mlbuf[wave][4u * kc + r][1] = l_run[r]; }
+  }
+  TRD(6);
+  __syncthreads();
+  for (uint32_t idx = tid; idx < (uint32_t)(G * D); idx += NT) {
+    const uint32_t h = idx / D, d = idx % D;
+    float M = mlbuf[0][h][0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) M = fmaxf(M, mlbuf[w][h][0]);
+    float o = 0.f, L = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; w++) {
+      const float e = __expf(mlbuf[w][h][0] - M);
+      o = fmaf(obuf[w][h][d], e, o);
+      L = fmaf(mlbuf[w][h][1], e, L);
+    }
+    if (n_splits == 1u) {
+      out[(uint64_t)bs.o[op0 + h] + d] = o * (1.0f / L);
+    } else {
+      float* pp = partial + ((uint64_t)(op0 + h) * n_splits + split) * (D + 2);
+      pp[2 + d] = o;
+      if (d == 0u) { pp[0] = M; pp[1] = L; }
+    }
+  }
+  TRD(7);
+}
+
+template <int D, int NW, bool PF>
+static void launch_dg(uint32_t G, dim3 grid, const AttnDecodeArgs& a, const AttdBases& bs, uint32_t n_splits,
+                      uint32_t chunk) {
+#define ADL(GG)                                                                                       \
+  k_attn_decode<D, GG, NW, PF><<<grid, NW * 64, 0, g.stream>>>(a.data, a.data, a.kv, a.kv_shift, bs, a.row_size, \
+                                                               a.scale, a.cap, n_splits, chunk, g.attn_scratch)
+  if (G == 1) ADL(1); else if (G == 2) ADL(2); else if (G == 4) ADL(4); else ADL(8);
+#undef ADL
+}
+
+template <int D>
+static void launch_d(uint32_t G, uint32_t nw, bool pf, dim3 grid, const AttnDecodeArgs& a, const AttdBases& bs,
+                     uint32_t n_splits, uint32_t chunk) {
+  if (nw == 8) launch_dg<D, 8, false>(G, grid, a, bs, n_splits, chunk);
+  else if (pf) launch_dg<D, 4, true>(G, grid, a, bs, n_splits, chunk);
+  else launch_dg<D, 4, false>(G, grid, a, bs, n_splits, chunk);
+}
+
+bool launch_attn_decode(const AttnDecodeArgs& a, AttnPartials* ap, bool* left, int* rc) {
+  if (tuning("ADAMAH_ATTN_IMPL", 1) == 0) return false;
+  const uint32_t D = a.head_dim, n_ops = a.n_ops;
+  if (D != 64 && D != 128 && D != 256) return false;
+  if (!a.ha || !a.hb || !a.hc || !a.hv || !a.ho || !a.kv || n_ops == 0 || n_ops > ATTD_MAX_OPS || a.row_size == 0) return false;
+  uint32_t G = 1;
+  while (G < n_ops && G < 8 && a.hb[G] == a.hb[0] && a.hv[G] == a.hv[0]) G++;
+  if (G != 1 && G != 2 && G != 4 && G != 8) G = G > 4 ? 4 : G == 3 ? 2 : 1;
+  while (G > 1 && n_ops % G) G >>= 1;
+  for (uint32_t op = 0; op < n_ops; op++) {
+    const uint32_t o0 = op - op % G;
+    if (a.hb[op] != a.hb[o0] || a.hv[op] != a.hv[o0]) return false;
+    if ((a.hb[op] - a.kv_shift) % 8u || (a.hv[op] - a.kv_shift) % 8u) return false;
+  }
+  const uint32_t n_groups = n_ops / G;
+  if (n_groups > ATTD_MAX_GROUPS) return false;
+
+  // Slices of the sequence.  Short sequences (at most one 16-row tile per wave when the chip holds
+  // `target` waves): workgroups of 8 waves, one tile each, no prefetch; longer ones: 4 waves and as
+  // many tiles per wave as it takes.
+  const uint32_t target = (uint32_t)std::max(1, tuning("ADAMAH_ATTN_WAVES", 4 * g.n_cu));
+  const uint64_t tiles = (uint64_t)n_groups * cdiv(a.row_size, 16u);
+  uint32_t nw = (tiles <= target && G * D <= 1024u) ? 8u : 4u;
+  nw = (uint32_t)tuning("ADAMAH_ATTN_NW", (int)nw) == 8u && G * D <= 1024u ? 8u : 4u;
+  const uint32_t step = nw * 16u;
+  uint32_t chunk = step * std::max<uint32_t>(1u, cdiv(tiles, target));
+  while (cdiv(a.row_size, chunk) > ATTD_MAX_SPLITS) chunk += step;
+  bool leave = a.leave_partials;
+  if (leave) {
+    uint32_t cf = chunk;
+    while (cf < 4096u && (uint64_t)n_ops * cdiv(a.row_size, cf) * (D + 2) > a.fold_floats) cf += step;
+    if ((uint64_t)n_ops * cdiv(a.row_size, cf) * (D + 2) <= a.fold_floats) chunk = cf; else leave = false;
+  }
+  if (nw == 8u && chunk > step) { nw = 4u; }   // several tiles per wave: the prefetching 4-wave form
+  const bool pf = chunk > nw * 16u;
+  const uint32_t n_splits = cdiv(a.row_size, chunk);
+  if ((uint64_t)n_ops * n_splits * (D + 2) > g.attn_scratch_floats) return false;
+  AttdBases bs;
+  for (uint32_t op = 0; op < n_ops; op++) { bs.q[op] = a.ha[op]; bs.sc[op] = a.hc[op]; bs.o[op] = a.ho[op]; }
+  for (uint32_t gi = 0; gi < n_groups; gi++) { bs.kb[gi] = a.hb[gi * G]; bs.vb[gi] = a.hv[gi * G]; }
+  // the slices are merged by the consumer (leave) or by the caller's merge kernel
+  dim3 grid(n_splits, n_groups);
+  if (D == 64) launch_d<64>(G, nw, pf, grid, a, bs, n_splits, chunk);
+  else if (D == 128) launch_d<128>(G, nw, pf, grid, a, bs, n_splits, chunk);
+  else launch_d<256>(G, nw, pf, grid, a, bs, n_splits, chunk);
+  count_launch();
+  *rc = check_launch();
+  *ap = AttnPartials{g.attn_scratch, *rc == 0 ? n_splits : 1u, D, n_ops, 0};
+  *left = leave;
+  return true;
+}
+
+}  // namespace adamah
+
+#ifdef ADAMAH_TRACE
+extern "C" int adamah_hip_trace_read_attd(unsigned long long* out) {
+  hipStreamSynchronize(adamah::g.stream);
+  return hipMemcpyFromSymbol(out, HIP_SYMBOL(adamah::g_trace_attd), 64 * sizeof(unsigned long long)) == hipSuccess ? 0 : -1;
+}
+#endif

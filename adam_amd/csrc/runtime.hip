@@ -336,8 +336,8 @@ int adamah_init_ex(uint64_t hot_bytes, uint64_t cold_bytes) {
   g.res_next = 1;
   g.attn_scratch_floats = (size_t)4 << 20;   // 16 MiB of split-KV partials
   HIPCHK(hipMalloc((void**)&g.attn_scratch, g.attn_scratch_floats * sizeof(float)));
-  HIPCHK(hipMalloc((void**)&g.sync_ctr, 256));
-  HIPCHK(hipMemsetAsync(g.sync_ctr, 0, 256, g.stream));
+  HIPCHK(hipMalloc((void**)&g.sync_ctr, 1024));   // [0..63] GEMV prologues, [64..191] attention groups
+  HIPCHK(hipMemsetAsync(g.sync_ctr, 0, 1024, g.stream));
   g.pend.clear();
   g.batch_depth = 0; g.fusion_enabled = 0; g.scheduler_mode = 0; g.active_dtype = 0;
   g.stats = Stats();
