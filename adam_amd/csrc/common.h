@@ -65,18 +65,22 @@ struct Res {
 // A row-wise op recorded inside a batch instead of being launched at once, so that neighbours can be
 // folded into one kernel when the batch is flushed.  All offsets are element offsets resolved from
 // the host copies of the handles at record time (any later handle upload flushes the queue first).
-enum PendKind : uint32_t { PK_RMSNORM = 1, PK_GEMV = 2, PK_OP2 = 3, PK_ARGMAX = 4, PK_SCORES = 5, PK_ATTN = 6 };
+enum PendKind : uint32_t { PK_RMSNORM = 1, PK_GEMV = 2, PK_OP2 = 3, PK_ARGMAX = 4, PK_SCORES = 5, PK_ATTN = 6,
+                           PK_ROPE = 7, PK_QKNR = 8, PK_ROWCOPY = 9 };
 struct PendOp {
   uint32_t kind = 0;
   uint32_t map_act = 0, map_wt = 0;
   uint32_t a = 0, b = 0, c = 0, d = 0;   // RMSNORM: src, weight, dst, residual.  GEMV: x, W, y.  OP2: a, b, dst.
   uint32_t n = 0, k = 0;                 // RMSNORM: n = dim.  GEMV/ARGMAX: k = K, n = N.  OP2: n elements.
   uint32_t op = 0;                       // RMSNORM: 1 = with residual.  GEMV/ARGMAX: weight format.  OP2: op code.
-  uint32_t h[3] = {0, 0, 0};             // ARGMAX: idx, val, dst handles.  SCORES: q, K, score rows.  ATTN: scores, V, out
+  uint32_t h[5] = {0, 0, 0, 0, 0};       // ARGMAX: idx, val, dst handles.  SCORES: q, K, score rows.  ATTN: scores, V, out
   uint32_t rpg = 0;                      // ARGMAX: rows per group.  SCORES / ATTN: number of heads (ops)
   float eps = 0.f;                       // RMSNORM: eps.  ATTN: score scale
   float f2 = 0.f;                        // ATTN: soft cap
   // SCORES: k = head dim, n = sequence length.  ATTN: n = sequence length, k = value dim.
+  // ROPE (one token): a = src, c = dst, rpg = heads, k = head dim, n = position, eps = frequency base.
+  // QKNR: h = q rows, q weights, k rows, k weights, dst; rpg/k = q rows/dim, op/d = k rows/dim, n, eps as ROPE.
+  // ROWCOPY: h = spec, source base; rpg = copies, k = row size, n = destination row offset.
 };
 
 struct Stats {
@@ -151,6 +155,8 @@ bool res_scalar(uint32_t h, uint32_t* out);
 bool res_run(uint32_t h, uint64_t n, uint32_t* start);
 void gemm_q4_mfma_release();   // frees the GEMM's scratch (shutdown)
 int launch_rmsnorm_v(const PendOp& p);
+bool row_op_deferrable(const PendOp& p);                                  // rowprep.hip
+size_t launch_row_run(const std::vector<PendOp>& q, size_t i, int* rc);   // rowprep.hip
 int launch_op2_v(const PendOp& p);
 // Attention (attention.hip): stand-alone launches of queued ops, and the fused form.  launch_attn
 // runs scores (when sc != nullptr) and softmax . V; with leave_partials it stops before the merge

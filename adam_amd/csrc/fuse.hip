@@ -12,6 +12,7 @@
 //   RMSNorm+residual(o, r -> r); RMSNorm(r -> n); GEMV(n)  -> GEMV that does both norms while staging
 //   GEMV(-> y); ADD(r, y -> d)                            -> GEMV that also stores r + y
 //   GEMV(-> [g; u]); GEGLU/SWIGLU(g, u -> t)              -> GEMV over paired rows that also stores t
+//   RoPE(q); RoPE(k) | QK-norm+RoPE; row copy (KV append)  -> one launch of row tasks (rowprep.hip)
 //
 // Every folded op still stores its own result where it would have stored it alone, so the contents
 // of the maps after a batch do not depend on whether anything was folded.
@@ -124,6 +125,12 @@ void flush_pending() {
     auto is_gemv = [&](size_t j) { return j < n && (q[j].kind == PK_GEMV || q[j].kind == PK_ARGMAX); };
     size_t gi = n;    // the GEMV this group is built around, if any
     GemvFuse fz = {};
+    if (p.kind == PK_ROPE || p.kind == PK_QKNR || p.kind == PK_ROWCOPY) {
+      // rotation of the new Q / K rows and the KV append: one launch for the run
+      int rc = 0;
+      i += launch_row_run(q, i, &rc);
+      continue;
+    }
     if (p.kind == PK_SCORES || p.kind == PK_ATTN) {
       // decode attention: scores computed inside the softmax . V launch; the merge of the sequence
       // splits moves into the GEMV that consumes the heads' outputs when the partials are small

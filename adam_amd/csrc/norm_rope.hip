@@ -171,11 +171,18 @@ int map_rmsnorm_add_dev(uint32_t map_id, uint32_t hs, uint32_t hw, uint32_t hr, 
 }
 
 int map_rope_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_tokens, uint32_t n_heads, uint32_t head_dim,
-                 uint32_t pos_offset, float freq_base) { ADAMAH_API();
+                 uint32_t pos_offset, float freq_base) {
   Map* m = get_f32_map(map_id);
   if (!m) return ADAMAH_ERR_INVALID;
   const uint64_t pairs = (uint64_t)n_tokens * n_heads * (head_dim / 2);
   if (pairs == 0) return ADAMAH_OK;
+  if (n_tokens == 1 && can_defer()) {
+    // one token with operands known on the host: queue it, it may share a launch with the KV append
+    PendOp p;
+    p.kind = PK_ROPE; p.map_act = map_id; p.rpg = n_heads; p.k = head_dim; p.n = pos_offset; p.eps = freq_base;
+    if (res_scalar(hs, &p.a) && res_scalar(hd, &p.c) && row_op_deferrable(p)) { g.pend.push_back(p); return ADAMAH_OK; }
+  }
+  flush_pending();
   const uint32_t *ls = res_u32(hs, n_tokens), *ld = res_u32(hd, n_tokens);
   if (!ls || !ld) return ADAMAH_ERR_INVALID;
   k_rope<<<cdiv(pairs, 256), 256, 0, g.stream>>>((float*)m->buf, ls, ld, n_tokens, n_heads, head_dim, pos_offset,
@@ -186,11 +193,19 @@ int map_rope_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_tokens, u
 
 int map_qk_norm_rope_x_dev(uint32_t map_act, uint32_t map_wt, uint32_t hqs, uint32_t hqw, uint32_t hks, uint32_t hkw,
                            uint32_t hdst, uint32_t q_rows, uint32_t q_dim, uint32_t k_rows, uint32_t k_dim,
-                           uint32_t pos_offset, float freq_base) { ADAMAH_API();
+                           uint32_t pos_offset, float freq_base) {
   Map* ma = get_f32_map(map_act);
   Map* mw = get_f32_map(map_wt);
   if (!ma || !mw) return ADAMAH_ERR_INVALID;
   if (q_rows + k_rows == 0) return ADAMAH_OK;
+  if (map_act == map_wt && can_defer()) {
+    PendOp p;
+    p.kind = PK_QKNR; p.map_act = map_act; p.map_wt = map_wt; p.rpg = q_rows; p.k = q_dim; p.op = k_rows; p.d = k_dim;
+    p.n = pos_offset; p.eps = freq_base;
+    p.h[0] = hqs; p.h[1] = hqw; p.h[2] = hks; p.h[3] = hkw; p.h[4] = hdst;
+    if (row_op_deferrable(p)) { g.pend.push_back(p); return ADAMAH_OK; }
+  }
+  flush_pending();
   const uint32_t* one = res_u32(hdst, 1);
   const uint32_t *lqs = q_rows ? res_u32(hqs, q_rows) : one, *lqw = q_rows ? res_u32(hqw, q_rows) : one;
   const uint32_t *lks = k_rows ? res_u32(hks, k_rows) : one, *lkw = k_rows ? res_u32(hkw, k_rows) : one;
@@ -203,10 +218,17 @@ int map_qk_norm_rope_x_dev(uint32_t map_act, uint32_t map_wt, uint32_t hqs, uint
 }
 
 int map_row_copy_offset_dev(uint32_t map_id, uint32_t hspec, uint32_t hbase, uint32_t dst_row_offset, uint32_t n_copies,
-                            uint32_t row_size) { ADAMAH_API();
+                            uint32_t row_size) {
   Map* m = get_f32_map(map_id);
   if (!m) return ADAMAH_ERR_INVALID;
   if (n_copies == 0 || row_size == 0) return ADAMAH_OK;
+  if (can_defer()) {
+    PendOp p;
+    p.kind = PK_ROWCOPY; p.map_act = map_id; p.h[0] = hspec; p.h[1] = hbase; p.rpg = n_copies; p.k = row_size;
+    p.n = dst_row_offset;
+    if (row_op_deferrable(p)) { g.pend.push_back(p); return ADAMAH_OK; }
+  }
+  flush_pending();
   const uint32_t *spec = res_u32(hspec, 2ull * n_copies), *base = res_u32(hbase, 1);
   if (!spec || !base) return ADAMAH_ERR_INVALID;
   k_row_copy<<<cdiv((uint64_t)n_copies * row_size, 256), 256, 0, g.stream>>>(

@@ -15,7 +15,7 @@ import pytest
 import oracle
 from adam_amd import adamah as A
 from adam_amd import quant
-from gpu_util import note, up, read, rel_l2, load_qtensor
+from gpu_util import note, up, read, rel_l2, load_qtensor, f32map, put
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
@@ -225,3 +225,65 @@ def test_attention_chain_folded_into_output_projection(hip, ctx, Hq, Hkv, d, N):
     assert rel_l2(res["hip"][0], res["oracle"][0]) < 1e-5
     assert rel_l2(res["hip"][1], res["oracle"][1]) < TOL
     assert rel_l2(res["hip"][2], res["oracle"][2]) < TOL
+
+
+# ---- rotation of the new Q / K rows + KV append as one launch ---------------------------------------
+def _kv_prep_case(g, style, batch, Hq, Hkv, d, pos, seed, hazard=None):
+    """Layout: q | k | v | weights | (gap) | KV cache [K heads | V heads] of `cap` rows each (fp16 mirrored)."""
+    cap = 8
+    rng = np.random.default_rng(seed)
+    qn, kn = Hq * d, Hkv * d
+    q = rng.standard_normal(qn).astype(np.float32); k = rng.standard_normal(kn).astype(np.float32)
+    v = rng.standard_normal(kn).astype(np.float32)
+    wq = rng.uniform(0.5, 1.5, d).astype(np.float32); wk = rng.uniform(0.5, 1.5, d).astype(np.float32)
+    q0, k0, v0, w0 = 3, 3 + qn, 3 + qn + kn, 3 + qn + 2 * kn          # odd start: rows need no alignment
+    kv_start = (w0 + 2 * d + d - 1) // d * d
+    total = kv_start + 2 * Hkv * cap * d
+    f32map(g, 0, total, None)
+    put(g, 0, q0, np.concatenate([q, k, v, wq, wk]))
+    g.kv_cache_fp16(0, kv_start, 2 * Hkv * cap * d)
+    spec = []
+    for gi in range(Hkv):
+        spec += [gi, kv_start // d + gi * cap, gi + Hkv, kv_start // d + (Hkv + gi) * cap]
+    hq, hk = up(g, [q0]), up(g, [k0])
+    q_rows, k_rows = up(g, q0 + np.arange(Hq) * d), up(g, k0 + np.arange(Hkv) * d)
+    hspec, hbase, hdst = up(g, spec), up(g, [k0]), up(g, [q0])
+    hwq, hwk = up(g, [w0] * Hq), up(g, [w0 + d] * Hkv)
+    if batch:
+        g.batch_begin()
+    if style == "rope":
+        g.map_rope_dev(0, hq, hq, 1, Hq, d, pos, 5e5)
+        g.map_rope_dev(0, hk, hk, 1, Hkv, d, pos, 5e5)
+    else:
+        g.map_qk_norm_rope_x_dev(0, 0, q_rows, hwq, k_rows, hwk, hdst, Hq, d, Hkv, d, pos, 1e6)
+    if hazard == "copy_twice":       # second append of the same rows to another position: rides or runs alone
+        g.map_row_copy_offset_dev(0, hspec, hbase, pos % cap, 2 * Hkv, d)
+        g.map_row_copy_offset_dev(0, hspec, hbase, (pos + 1) % cap, 2 * Hkv, d)
+    elif hazard == "rope_after_copy":  # the copy must see the rows before the second rotation
+        g.map_row_copy_offset_dev(0, hspec, hbase, pos % cap, 2 * Hkv, d)
+        g.map_rope_dev(0, hk, hk, 1, Hkv, d, pos + 1, 5e5)
+    elif hazard == "shifted_source":   # source rows straddle two produced rows: no ride
+        g.map_row_copy_offset_dev(0, hspec, up(g, [k0 - d // 2]), pos % cap, 2 * Hkv, d)
+    else:
+        g.map_row_copy_offset_dev(0, hspec, hbase, pos % cap, 2 * Hkv, d)
+    launches = None
+    if batch:
+        g.batch_end()
+        launches = g.get_last_barrier_count()
+    return read(g, 0, 0, total), launches
+
+
+@pytest.mark.parametrize("style,Hq,Hkv,d,pos", [("rope", 32, 8, 128, 4095), ("rope", 4, 2, 64, 1), ("qknr", 4, 1, 256, 611),
+                                               ("qknr", 8, 4, 128, 77)])
+@pytest.mark.parametrize("hazard", [None, "copy_twice", "rope_after_copy", "shifted_source"])
+def test_kv_prep_run_equals_separate_ops(hip, style, Hq, Hkv, d, pos, hazard):
+    note(f"kv prep {style} {Hq}/{Hkv}x{d} pos={pos} hazard={hazard}")
+    folded, launches = _kv_prep_case(hip, style, True, Hq, Hkv, d, pos, 11, hazard)
+    apart, _ = _kv_prep_case(hip, style, False, Hq, Hkv, d, pos, 11, hazard)
+    assert np.array_equal(folded.view(np.uint32), apart.view(np.uint32))
+    want, _ = _kv_prep_case(oracle.init(), style, False, Hq, Hkv, d, pos, 11, hazard)
+    assert rel_l2(folded, want) < 1e-5
+    if hazard is None:
+        assert launches == 1          # rotation(s) and append shared one launch
+    elif hazard in ("rope_after_copy", "shifted_source"):
+        assert launches >= 2          # the dependent op was kept out of the first launch
