@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized decode hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemma3-1b|llama3-8b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemma3-1b|llama3-8b] [--only LEG]
 
 A "step" is one bs=1 greedy decode step (embedding fetch, all layers, fused LM-head GEMV+argmax,
 token read-back) of a random-init Q4_0 model of the named architecture, issued through the
@@ -13,6 +13,7 @@ One JSON line is printed.  Besides the contract keys it carries
   roofline      the Q4_0 GEMV kernel at the Llama-3-8B gate+up shape (28672x4096), timed with HIP
                 events on the library's stream while cycling through > 1 GB of distinct weights
   gemv_shapes   the same measurement for the other Llama-3-8B GEMV shapes
+  attention_32q8kv_d128  GQA decode attention over an fp16 KV cache at context 1024 / 4096 / 16384
   cpu_baseline  the NumPy restatement of the reference forward pass (float32 BLAS, pre-dequantised
                 weights) timed on this host on a bounded sample of the same workload
 """
@@ -30,9 +31,9 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 LLAMA_GEMV_SHAPES = [(28672, 4096), (14336, 4096), (6144, 4096), (4096, 4096), (4096, 14336)]
 # HBM bytes per 28672x4096 Q4_0 GEMV launch from rocprofv3 --pmc (profiles/gemv_q4_0_llama_shapes_pmc_
-# fetch_write.txt): FETCH_SIZE 32,365.3 counts x 1.999 KiB (factor from a plain read kernel of known
-# size) + WRITE_SIZE 112.1 counts x 1.000 KiB (factor from a plain copy kernel).
-GEMV_TRAFFIC_BYTES = int(32365.3 * 1.999 * 1024 + 112.1 * 1.000 * 1024)
+# fetch_write.txt): FETCH_SIZE 32,528.8 counts x 1.999 KiB (factor from a plain read kernel of known
+# size) + WRITE_SIZE 130.5 counts x 1.000 KiB (factor from a plain copy kernel).
+GEMV_TRAFFIC_BYTES = int(32528.8 * 1.999 * 1024 + 130.5 * 1.000 * 1024)
 METRIC = "decode tok/s at bs=1 + Q4 GEMV achieved HBM GB/s (% of MI355X peak)"
 
 
@@ -94,6 +95,93 @@ def measure_gemv(gpu, A, shapes, rounds=6):
     return out
 
 
+def measure_attention(gpu, A, ctxs=(1024, 4096, 16384), Hq=32, Hkv=8, d=128):
+    """GQA decode attention (scores + softmax.V issued as the decode loop does, inside a batch) over an fp16
+    KV cache: microseconds per attention and KV bytes per second.  Several distinct KV instances
+    (> 256 MB together where they fit 600 MB) are cycled so the last-level cache cannot serve them."""
+    up = lambda v: gpu.upload_dev(np.asarray(v, np.uint32))[0]
+    out = {}
+    for ctx in ctxs:
+        n_inst = max(2, min(32, (600 << 20) // (2 * Hkv * ctx * d * 2)))
+        step, sc_sz = ctx * d, Hq * ctx
+        q_pos, out_pos = sc_sz + 1, sc_sz + 1 + Hq * d          # odd: query rows need no alignment
+        kv_start = (out_pos + Hq * d + d - 1) // d * d
+        gpu.set_dtype(A.DTYPE_F32)
+        gpu.map_create(0, 1, kv_start + n_inst * 2 * Hkv * step)
+        gpu.kv_cache_fp16(0, kv_start, n_inst * 2 * Hkv * step)
+        rng = np.random.default_rng(ctx)
+        gpu.scatter_contiguous(0, q_pos, rng.standard_normal(Hq * d).astype(np.float32))
+        blk = rng.standard_normal(2 * Hkv * step).astype(np.float32)
+        for i in range(n_inst):
+            gpu.scatter_contiguous(0, kv_start + i * 2 * Hkv * step, blk)
+        heads = np.arange(Hq) // (Hq // Hkv)
+        q_rows, s_rows, o_rows = up(q_pos + np.arange(Hq) * d), up(np.arange(Hq) * ctx), up(out_pos + np.arange(Hq) * d)
+        ops = []
+        for i in range(n_inst):
+            base = kv_start + i * 2 * Hkv * step
+            ops.append(A.DecodePlanOp(kind=A.DECODE_OP_MATMUL_T, map_id=0, h0=q_rows, h1=up(base + heads * step),
+                                      h2=s_rows, u0=1, u1=d, u2=ctx, u3=Hq))
+            ops.append(A.DecodePlanOp(kind=A.DECODE_OP_ATTN_SOFTMAX_VALUE, map_id=0, h0=s_rows,
+                                      h1=up(base + (Hkv + heads) * step), h2=o_rows, u0=Hq, u1=ctx, u2=d,
+                                      f0=float(1 / np.sqrt(d)), f1=0.0))
+            ops.append(A.DecodePlanOp(kind=A.DECODE_OP_FUSION_FLUSH))
+        gpu.register_decode_plan(7, ops)
+        gpu.decode_step(7, 0, 0)
+        gpu.sync()
+        rounds = 4
+        gpu.timer_begin()
+        for _ in range(rounds):
+            gpu.decode_step(7, 0, 0)
+        us = gpu.timer_end() * 1e3 / (rounds * n_inst)
+        kvb = 2 * Hkv * ctx * d * 2
+        out[str(ctx)] = {"us": round(us, 2), "kv_MB": round(kvb / 1e6, 2), "GB/s": round(kvb / us / 1e3, 1),
+                         "frac": round(kvb / us / 1e3 / HBM_PEAK_GBPS, 4), "instances": n_inst}
+        log(f"attention {Hq}q/{Hkv}kv x{d} ctx {ctx}: {us:.2f} us, {kvb / us / 1e3:.0f} GB/s of KV")
+        gpu.clear_decode_plan(7)
+        gpu.map_destroy(0)
+    return out
+
+
+def measure_gemm(gpu, A, Ms=(16, 512), shapes=((28672, 4096), (4096, 4096), (4096, 14336))):
+    """Batched Q4_0 matmul C[M, N] = X[M, K] . W[N, K]^T (prefill chunk M = 512, batched decode M = 16) on
+    the fp16 matrix cores: microseconds per call, dense TFLOP/s and the rate at which weights stream."""
+    total = 4 * 28672 * 4096
+    rng = np.random.default_rng(5)
+    gpu.map_create_typed(3, A.DTYPE_Q4, 1, total, 32)
+    s = rng.uniform(0.001, 0.01, total // 32).astype(np.float16).astype(np.float32)
+    gpu.set_qparams(3, s, np.float32(-8.0) * s)
+    chunk = 1 << 26
+    for b in range(0, total // 2, chunk):
+        n = min(chunk, total // 2 - b)
+        gpu.scatter_q4_packed_contiguous(3, 2 * b, rng.integers(0, 256, n, dtype=np.uint8), n_locs=2 * n)
+    out = {}
+    for M in Ms:
+        for N, K in shapes:
+            gpu.set_dtype(A.DTYPE_F32)
+            gpu.map_create(5, 1, M * (K + N))
+            gpu.scatter_contiguous(5, 0, rng.standard_normal(M * K).astype(np.float32))
+            a = gpu.upload_dev(np.array([0], np.uint32))[0]
+            c = gpu.upload_dev(np.array([M * K], np.uint32))[0]
+            n_mats = total // (N * K)
+            bs = [gpu.upload_dev(np.array([i * N * K], np.uint32))[0] for i in range(n_mats)]
+            for b in bs:
+                gpu.map_matmul_t_xq4_dev(5, 3, a, b, c, M, K, N, 1)
+            gpu.sync()
+            rounds = 3
+            gpu.timer_begin()
+            for _ in range(rounds):
+                for b in bs:
+                    gpu.map_matmul_t_xq4_dev(5, 3, a, b, c, M, K, N, 1)
+            us = gpu.timer_end() * 1e3 / (rounds * n_mats)
+            out[f"M{M}_{N}x{K}"] = {"us": round(us, 2), "TFLOP/s": round(2 * M * N * K / us / 1e6, 1),
+                                   "frac_fp16_mfma_peak": round(2 * M * N * K / us / 1e6 / 2500.0, 4),
+                                   "weights_GB/s": round(N * K * 18 / 32 / us / 1e3, 1)}
+            log(f"gemm M={M} {N}x{K}: {us:.1f} us, {2 * M * N * K / us / 1e6:.1f} TFLOP/s")
+            gpu.map_destroy(5)
+    gpu.map_destroy(3)
+    return out
+
+
 def cpu_baseline(cfg, tensors, prompt, n_prompt=8, n_steps=48):
     """The oracle's NumPy forward pass (reference forward_cpu restated) on this host's cores."""
     from oracle.forward_cpu import CpuModel
@@ -126,10 +214,12 @@ def main():
     ap.add_argument("--workload", default="gemma3-1b", choices=["gemma3-1b", "llama3-8b"])
     ap.add_argument("--prompt", type=int, default=None, help="prompt length (default 512 / 3840)")
     ap.add_argument("--scheduler", default="level_batched", choices=["legacy", "level_batched"])
-    ap.add_argument("--only", default=None, choices=["roofline", "gemv", "probe"],
+    ap.add_argument("--only", default=None, choices=["roofline", "gemv", "probe", "attention", "gemm"],
                     help="roofline: just the 28672x4096 GEMV (one kernel row in a rocprofv3 --stats table); "
                          "gemv: that shape, 4096x4096 and 4096x14336; probe: plain read/copy kernels of known "
-                         "size (reference points for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
+                         "size (reference points for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE); attention: GQA "
+                         "decode attention 32q/8kv x128 at ctx 1024/4096/16384; gemm: batched Q4_0 matmul at "
+                         "M = 16 and 512 on the Llama-3-8B shapes")
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -145,6 +235,10 @@ def main():
             out = {"gemv_shapes": measure_gemv(gpu, A, LLAMA_GEMV_SHAPES[:1], rounds=8)}
         elif args.only == "gemv":
             out = {"gemv_shapes": measure_gemv(gpu, A, LLAMA_GEMV_SHAPES[:1] + LLAMA_GEMV_SHAPES[3:], rounds=3)}
+        elif args.only == "attention":
+            out = {"attention": measure_attention(gpu, A)}
+        elif args.only == "gemm":
+            out = {"gemm": measure_gemm(gpu, A)}
         else:
             nbytes = gemv_bytes(28672, 4096) // 4096 * 4096
             pool = nbytes * 16
@@ -229,6 +323,7 @@ def main():
                            "kernel": "k_gemv_mfma<Q4_0 block16, store> 28672x4096, "
                                      f"{gemv_bytes(28672, 4096)} algorithmic B/launch"}
         res["gemv_shapes"] = shapes
+        res["attention_32q8kv_d128"] = measure_attention(gpu, A)
     gpu.shutdown()
 
     if not args.no_cpu_baseline:
