@@ -127,7 +127,10 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
   };
 
   PreM A, B;   // A's first loads stay in flight while the activations are staged
-  if (PRO == PRO_NONE && first < seg_end) load(A, first, kpart, seg_end);
+  // Loads come back in order: the activation loads (cache hits) go out ahead of the first weights, so
+  // the conversion does not wait for the weights' trip to memory as well.
+  const bool x_first = fz.x_first != 0u;
+  if (PRO == PRO_NONE && !x_first && first < seg_end) load(A, first, kpart, seg_end);
 
   // ---- activations -> fixed-point digits; one 8-element word per thread and pass, four threads per
   // block.  stage() turns one word into digits; the prologues below decide what the word is. ------
@@ -195,6 +198,11 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       float x[4][8];
 #pragma unroll
       for (uint32_t u = 0; u < 4; u++) load8(act + a + (uint64_t)min(i0 + u * nthr + tid, nw - 1u) * 8u, x[u]);
+      if (i0 == 0u && x_first) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (first < seg_end) load(A, first, kpart, seg_end);
+        __builtin_amdgcn_sched_barrier(0);
+      }
 #pragma unroll
       for (uint32_t u = 0; u < 4; u++)
         if (i0 + u * nthr + (tid & ~63u) < nw)   // wave-uniform: waves without words skip the conversion
@@ -526,6 +534,8 @@ static int launch_mfma(int fmt, uint32_t grid, uint32_t threads, const Map* ma, 
                        uint32_t n_groups, uint32_t ks, const GemvFuse* fzp) {
   GemvFuse fz = {};
   if (fzp) fz = *fzp;
+  const int xf = tuning("ADAMAH_MFMA_XFIRST", -1);
+  fz.x_first = xf < 0 ? 1u : (uint32_t)(xf != 0);
 #define MP(P) launch_mfma_p<EPI, P>(fmt, grid, threads, ma, mw, a, b, c, lidx, lval, K, N, rpg, n_groups, ks, fz)
   switch (fz.pro) {
     case PRO_RMSNORM: MP(PRO_RMSNORM); break;
