@@ -5,12 +5,12 @@
 // dispatch adamah.c:8693-8803).  With more than one activation row the weights are reused, so this
 // is the one place on the path where the work is a dense contraction and belongs on MFMA.
 //
-// v_mfma_f32_16x16x16_f16:  D[i][j] += sum_k A[i][k] B[k][j];  lane l supplies A[l % 16][4g..4g+3] and
-// B[4g..4g+3][l % 16] with g = l / 16, and receives D[4g..4g+3][l % 16].  Here i runs over 16 weight
-// rows, j over 16 activation rows, and the sixteen k of one instruction are four weights out of each
-// of four consecutive 32-weight blocks: lane (row, g) loads block g of its row as one 16-byte word
+// v_mfma_f32_16x16x32_f16:  D[i][j] += sum_k A[i][k] B[k][j];  lane l supplies A[l % 16][8g..8g+7] and
+// B[8g..8g+7][l % 16] with g = l / 16, and receives D[4g..4g+3][l % 16].  Here i runs over 16 weight
+// rows, j over 16 activation rows, and the 32 k of one instruction are eight weights out of each of
+// four consecutive 32-weight blocks: lane (row, g) loads block g of its row as one 16-byte word
 // group, dequantises it in registers to fp16 (exactly (q - 8), then times the block's fp16 scale:
-// one rounding per weight) and feeds eight instructions from it.  The activations of the tile are
+// one rounding per weight) and feeds four instructions from it.  The activations of the tile are
 // converted once per step to fp16 in LDS, scaled per row by a power of two so that no row can
 // overflow fp16 (the scale is divided out of the fp32 result), in the element order the unpacking
 // produces.  Accumulation is fp32 in the matrix core.
@@ -29,6 +29,8 @@ typedef _Float16 h4q_t __attribute__((ext_vector_type(4)));
 typedef float f4q_t __attribute__((ext_vector_type(4)));
 typedef float f4qu_t __attribute__((ext_vector_type(4), aligned(4)));
 typedef uint32_t u2q_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u4q_t __attribute__((ext_vector_type(4)));
+typedef _Float16 h8q_t __attribute__((ext_vector_type(8)));
 
 // Per activation row: s = 2^e with max|x| * s in [2^13, 2^14) (1 when the row is zero, tiny or not
 // finite), and 1 / s.  One workgroup per row.
@@ -151,10 +153,11 @@ k_gemm_q4_f16(const float* act, float* out, const uint8_t* __restrict__ W, const
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const uint4 xv = *(const uint4*)(xp + j * 16);
-        const u2q_t a0 = {wq[2 * j][0], wq[2 * j][1]}, a1 = {wq[2 * j + 1][0], wq[2 * j + 1][1]};
-        const u2q_t b0 = {xv.x, xv.y}, b1 = {xv.z, xv.w};
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4q_t, a0), __builtin_bit_cast(h4q_t, b0), acc[t], 0, 0, 0);
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4q_t, a1), __builtin_bit_cast(h4q_t, b1), acc[t], 0, 0, 0);
+        // one K = 32 instruction over the two 4-element operand pairs (the sum over the 32 k is the same
+        // whichever lane group and slot a pair sits in, as long as A and B agree)
+        const u4q_t a = {wq[2 * j][0], wq[2 * j][1], wq[2 * j + 1][0], wq[2 * j + 1][1]};
+        const u4q_t b = {xv.x, xv.y, xv.z, xv.w};
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8q_t, a), __builtin_bit_cast(h8q_t, b), acc[t], 0, 0, 0);
       }
     }
     }

@@ -30,6 +30,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 LLAMA_GEMV_SHAPES = [(28672, 4096), (14336, 4096), (6144, 4096), (4096, 4096), (4096, 14336)]
+CONFIG1_GEMV_SHAPE = (6912, 1152)      # BASELINE config 1 (Gemma-3-1B FFN up): launch-bound, reported beside the others
 # HBM bytes per 28672x4096 Q4_0 GEMV launch from rocprofv3 --pmc (profiles/gemv_q4_0_llama_shapes_pmc_
 # fetch_write.txt): FETCH_SIZE 32,528.8 counts x 1.999 KiB (factor from a plain read kernel of known
 # size) + WRITE_SIZE 130.5 counts x 1.000 KiB (factor from a plain copy kernel).
@@ -201,9 +202,46 @@ def cpu_baseline(cfg, tensors, prompt, n_prompt=8, n_steps=48):
         nt = int(np.argmax(logits))
         logits = m.forward(nt, n_prompt + s)
     dt = time.perf_counter() - t0
-    return {"value": round(n_steps / dt, 3), "unit": "tok/s", "cores": int(threads), "kind": "port",
-            "sample": f"{n_steps} greedy decode steps after a {n_prompt}-token prompt, same model, NumPy "
-                      f"float32 BLAS on pre-dequantised weights ({os.cpu_count()} logical CPUs visible)"}
+    out = {"value": round(n_steps / dt, 3), "unit": "tok/s", "cores": int(threads), "kind": "port",
+           "sample": f"{n_steps} greedy decode steps after a {n_prompt}-token prompt, same model, NumPy "
+                     f"float32 BLAS on pre-dequantised weights ({os.cpu_count()} logical CPUs visible)"}
+    out.update(cpu_kernels())
+    return out
+
+
+def cpu_kernels():
+    """The two kernels of the path alone, restated in NumPy (oracle/blocks.py; the attention form of the
+    reference's engine.py:2428-2441): BASELINE config 1 GEMV and config 3 attention at context 4096."""
+    from oracle import blocks
+    rng = np.random.default_rng(0)
+    N, K = CONFIG1_GEMV_SHAPE
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    x = rng.standard_normal(K).astype(np.float32)
+    d, codes = blocks.quantize_q4_0(w)
+    wd = blocks.dequant_q4_0(d, codes).reshape(N, K)
+
+    def best(fn, secs=1.0):
+        fn(); t_end, b = time.perf_counter() + secs, 1e9
+        while time.perf_counter() < t_end:
+            t0 = time.perf_counter(); fn(); b = min(b, time.perf_counter() - t0)
+        return b
+    t_pre = best(lambda: wd @ x)
+    t_deq = best(lambda: blocks.dequant_q4_0(d, codes).reshape(N, K) @ x)
+    Hq, Hkv, dd, ctx = 32, 8, 128, 4096
+    q = rng.standard_normal((Hq, dd)).astype(np.float32)
+    Kc = rng.standard_normal((Hkv, ctx, dd)).astype(np.float16); Vc = rng.standard_normal((Hkv, ctx, dd)).astype(np.float16)
+
+    def attn():
+        o = np.empty((Hq, dd), np.float32)
+        for h in range(Hq):
+            kh, vh = Kc[h // (Hq // Hkv)].astype(np.float32), Vc[h // (Hq // Hkv)].astype(np.float32)
+            sc = kh @ q[h] * np.float32(1 / np.sqrt(dd))
+            p = np.exp(sc - sc.max()); p /= p.sum()
+            o[h] = p @ vh
+        return o
+    t_att = best(attn)
+    return {"gemv_6912x1152_us": {"pre_dequantised": round(t_pre * 1e6, 1), "dequant_and_gemv": round(t_deq * 1e6, 1)},
+            "attention_32q8kv_d128_ctx4096_us": round(t_att * 1e6, 1)}
 
 
 def main():
@@ -316,7 +354,7 @@ def main():
     del eng
 
     if not args.no_roofline:
-        shapes = measure_gemv(gpu, A, LLAMA_GEMV_SHAPES)
+        shapes = measure_gemv(gpu, A, LLAMA_GEMV_SHAPES + [CONFIG1_GEMV_SHAPE])
         top = shapes["28672x4096"]
         res["roofline"] = {"bound": "hbm", "achieved": top["GB/s"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                            "frac": top["frac"], "traffic": GEMV_TRAFFIC_BYTES,
