@@ -107,6 +107,8 @@ _SIGS = {
     "map_layernorm_dev": (i32, [_U] * 7 + [f32c]), "map_broadcast_dev": (i32, [_U] * 6),
     "map_reduce_dev": (i32, [_U] * 5), "map_argmax_dev": (i32, [_U] * 4),
     "map_topk_dev": (i32, [_U] * 6), "map_topp_dev": (i32, [_U] * 4 + [f32c, f32c]),
+    "map_resolve_idx_dev": (i32, [_U] * 5), "map_sample_categorical_dev": (i32, [_U] * 6),
+    "map_repeat_penalty_dev": (i32, [_U] * 4 + [f32c]),
     "map_rmsnorm_dev": (i32, [_U] * 6 + [f32c]), "map_rmsnorm_add_dev": (i32, [_U] * 7 + [f32c]),
     "map_rmsnorm_x_dev": (i32, [_U] * 7 + [f32c]), "map_rope_dev": (i32, [_U] * 7 + [f32c]),
     "map_qk_norm_rope_x_dev": (i32, [_U] * 12 + [f32c]),
@@ -136,13 +138,16 @@ _OPTIONAL_FLAGS = {
     "adamah_register_decode_plan": "_has_decode_plan",
     "adamah_set_dtype": "_has_dtype",
     "adamah_kv_cache_fp16": "_has_kv_cache_fp16",
+    "map_resolve_idx_dev": "_has_map_resolve_idx_dev",
+    "map_sample_categorical_dev": "_has_map_sample_categorical_dev",
+    "map_repeat_penalty_dev": "_has_map_repeat_penalty_dev",
 }
-# Present in the reference surface, deliberately absent here: sampling beyond argmax, the fused
-# qkv / gate-up entry points, and the monolithic full-decode / device-address API.
+# Present in the reference surface, deliberately absent here: the fused GEMV + top-k / rerank tail,
+# the fused qkv / gate-up entry points, and the monolithic full-decode / device-address API.
 _ABSENT_FLAGS = (
-    "_has_map_repeat_penalty_dev", "_has_map_matvec_topk_t_xq4_dev", "_has_map_matvec_topk_t_xq4_ex_dev",
+    "_has_map_matvec_topk_t_xq4_dev", "_has_map_matvec_topk_t_xq4_ex_dev",
     "_has_map_matvec_topk_t_xq8_dev", "_has_map_matvec_topk_t_xq8_ex_dev", "_has_map_matvec_rerank_t_xq8_dev",
-    "_has_map_resolve_idx_dev", "_has_map_sample_categorical_dev", "_has_map_fused_qkv_t_xq4_dev",
+    "_has_map_fused_qkv_t_xq4_dev",
     "_has_map_fused_gateup_t_xq4_dev", "_has_map_fused_qkv_t_xq8_dev", "_has_map_fused_gateup_t_xq8_dev",
     "_has_map_fused_gateup_act_t_xq8_dev", "_has_full_decode_step_api", "_has_full_decode_step",
     "_has_map_device_address", "_has_set_xq_matmul_wg",
@@ -455,6 +460,16 @@ class Adamah:
 
     def map_topp_dev(self, map_id, locs_src_handle, locs_dst_handle, n, temperature, top_p):
         self._op("map_topp_dev", map_id, locs_src_handle, locs_dst_handle, n, temperature, top_p)
+
+    def map_resolve_idx_dev(self, map_id, base_locs_handle, sel_locs_handle, dst_locs_handle, n):
+        self._op("map_resolve_idx_dev", map_id, base_locs_handle, sel_locs_handle, dst_locs_handle, n)
+
+    def map_sample_categorical_dev(self, map_id, locs_idx_handle, locs_prob_handle, rand_loc_handle, dst_loc_handle, n):
+        self._op("map_sample_categorical_dev", map_id, locs_idx_handle, locs_prob_handle, rand_loc_handle,
+                 dst_loc_handle, n)
+
+    def map_repeat_penalty_dev(self, map_id, locs_src_handle, token_ids_handle, n_ids, penalty):
+        self._op("map_repeat_penalty_dev", map_id, locs_src_handle, token_ids_handle, n_ids, penalty)
 
     def map_matvec_argmax_t_xq4_dev(self, map_act, map_wt, locs_a_handle, locs_b_handle, locs_idx_tmp_handle,
                                     locs_val_tmp_handle, locs_dst_handle, K, N, rows_per_group):

@@ -311,9 +311,6 @@ int map_argmax_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n) { ADAM
   count_launch();
   return check_launch();
 }
-// Sampling beyond argmax is not part of this build.
-int map_topk_dev(uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t) { ADAMAH_API(); return ADAMAH_ERR_INVALID; }
-int map_topp_dev(uint32_t, uint32_t, uint32_t, uint32_t, float, float) { ADAMAH_API(); return ADAMAH_ERR_INVALID; }
 
 int map_row_gather_xq8_dev(uint32_t map_act, uint32_t map_wt, uint32_t src_base, uint32_t dst_base, uint32_t row_idx,
                            uint32_t row_size, float scale) { ADAMAH_API();

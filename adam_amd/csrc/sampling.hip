@@ -1,0 +1,238 @@
+// Sampling tail on logits resident in a float32 map: top-k selection, temperature / top-p
+// renormalisation of a short candidate list, index resolution, categorical draw, repetition penalty.
+//
+// Reference: shaders/src/f32/map_topk.comp, map_topp.comp, map_resolve_idx.comp,
+// map_sample_categorical.comp, map_repeat_penalty.comp; dispatchers adamah.c:6787-6873 (repeat
+// penalty), 6978-7093 (top-k), 7095-7208 (top-p), 7210-7284 (resolve), 7286-7370 (categorical).
+// Limits as there: k, n <= 64 for top-p / categorical / repeat penalty ids, k <= 64 for top-k.
+// These are tiny latency-bound kernels; the serial parts run in one lane in the order the shaders
+// use, so the float32 results match a sequential evaluation.  Every location read from a handle is
+// checked against the map size before it is used.
+#include "common.h"
+#include "../../include/adamah_hip.h"
+
+namespace adamah {
+
+#define SMP_MAX 64u
+#define SMP_INVALID 0xffffffffu
+#define SMP_NEG_INF (-3.402823466e+38f)
+
+__device__ __forceinline__ bool smp_better(float cv, uint32_t ci, float bv, uint32_t bi) {
+  if (bi == SMP_INVALID) return true;
+  if (ci == SMP_INVALID) return false;
+  return cv > bv || (cv == bv && ci < bi);
+}
+
+// k rounds of "best not yet chosen" over n candidates (NaN counts as the lowest value, ties go to
+// the lower index); rounds past n store index 0 and the lowest value.
+__global__ void __launch_bounds__(256)
+k_topk(float* data, const uint32_t* __restrict__ ls, const uint32_t* __restrict__ li, const uint32_t* __restrict__ lv,
+       uint32_t n, uint32_t k, uint64_t n_elems) {
+  __shared__ float sv[256];
+  __shared__ uint32_t si[256];
+  __shared__ uint32_t top[SMP_MAX];
+  const uint32_t tid = threadIdx.x;
+  if (tid < SMP_MAX) top[tid] = SMP_INVALID;
+  __syncthreads();
+  for (uint32_t o = 0; o < k; o++) {
+    float bv = SMP_NEG_INF;
+    uint32_t bi = SMP_INVALID;
+    for (uint32_t i = tid; i < n; i += 256u) {
+      bool chosen = false;
+      for (uint32_t j = 0; j < o; j++) chosen = chosen || top[j] == i;
+      if (chosen) continue;
+      float v = ls[i] < n_elems ? data[ls[i]] : SMP_NEG_INF;
+      if (isnan(v)) v = SMP_NEG_INF;
+      if (smp_better(v, i, bv, bi)) { bv = v; bi = i; }
+    }
+    sv[tid] = bv; si[tid] = bi;
+    __syncthreads();
+    for (uint32_t s = 128; s > 0; s >>= 1) {
+      if (tid < s && smp_better(sv[tid + s], si[tid + s], sv[tid], si[tid])) { sv[tid] = sv[tid + s]; si[tid] = si[tid + s]; }
+      __syncthreads();
+    }
+    if (tid == 0) {
+      const uint32_t w = si[0];
+      top[o] = w;
+      if (li[o] < n_elems) data[li[o]] = (float)(w == SMP_INVALID ? 0u : w);
+      if (lv[o] < n_elems) data[lv[o]] = w == SMP_INVALID ? SMP_NEG_INF : sv[0];
+    }
+    __syncthreads();
+  }
+}
+
+// softmax(logits / temperature) over n <= 64 candidates in list order, cut after the first prefix
+// whose mass reaches top_p, renormalised over the kept prefix.
+__global__ void __launch_bounds__(64)
+k_topp(float* data, const uint32_t* __restrict__ ls, const uint32_t* __restrict__ ld, uint32_t n, float temperature,
+       float top_p, uint64_t n_elems) {
+  __shared__ float lg[SMP_MAX], pr[SMP_MAX];
+  const uint32_t tid = threadIdx.x;
+  lg[tid] = SMP_NEG_INF;
+  pr[tid] = 0.f;
+  if (tid < n) {
+    float v = ls[tid] < n_elems ? data[ls[tid]] : SMP_NEG_INF;
+    if (isnan(v) || isinf(v)) v = SMP_NEG_INF;
+    lg[tid] = v;
+  }
+  __syncthreads();
+  if (tid != 0) return;
+  auto put = [&](uint32_t i, float v) { if (ld[i] < n_elems) data[ld[i]] = v; };
+  const float temp = fmaxf(temperature, 1e-6f);
+  const float keep_p = fminf(fmaxf(top_p, 0.f), 1.f);
+  float mx = SMP_NEG_INF;
+  for (uint32_t i = 0; i < n; i++) if (lg[i] > mx) mx = lg[i];
+  if (mx == SMP_NEG_INF) { for (uint32_t i = 0; i < n; i++) put(i, 0.f); return; }
+  float sum = 0.f;
+  for (uint32_t i = 0; i < n; i++) {
+    if (lg[i] == SMP_NEG_INF) { pr[i] = 0.f; continue; }
+    const float p = expf((lg[i] - mx) / temp);
+    pr[i] = p;
+    sum += p;
+  }
+  if (sum <= 0.f) { for (uint32_t i = 0; i < n; i++) put(i, i == 0 ? 1.f : 0.f); return; }
+  for (uint32_t i = 0; i < n; i++) pr[i] /= sum;
+  uint32_t keep = 0;
+  float csum = 0.f;
+  for (uint32_t i = 0; i < n; i++) {
+    csum += pr[i];
+    keep = i + 1;
+    if (keep_p >= 0.999999f || csum >= keep_p) break;
+  }
+  if (keep == 0 && n > 0) keep = 1;
+  float ks = 0.f;
+  for (uint32_t i = 0; i < keep; i++) ks += pr[i];
+  if (ks <= 0.f) ks = 1.f;
+  for (uint32_t i = 0; i < n; i++) put(i, i < keep ? pr[i] / ks : 0.f);
+}
+
+// dst[i] = data[base + uint(data[sel[i]])]  (candidate position -> token id), negatives / non-finite -> 0
+__global__ void __launch_bounds__(64)
+k_resolve_idx(float* data, const uint32_t* __restrict__ lbase, const uint32_t* __restrict__ lsel,
+              const uint32_t* __restrict__ ldst, uint32_t n, uint64_t n_elems) {
+  const uint32_t i = blockIdx.x * 64u + threadIdx.x;
+  if (i >= n) return;
+  float s = lsel[i] < n_elems ? data[lsel[i]] : 0.f;
+  if (isnan(s) || isinf(s) || s < 0.f) s = 0.f;
+  const uint64_t src = (uint64_t)lbase[0] + (uint32_t)fminf(s, 4294967040.f);
+  float t = src < n_elems ? data[src] : 0.f;
+  if (isnan(t) || isinf(t) || t < 0.f) t = 0.f;
+  if (ldst[i] < n_elems) data[ldst[i]] = t;
+}
+
+// Inverse-CDF draw over n <= 64 probabilities with the uniform number stored in the map.
+__global__ void __launch_bounds__(64)
+k_sample_categorical(float* data, const uint32_t* __restrict__ lidx, const uint32_t* __restrict__ lprob,
+                     const uint32_t* __restrict__ lrand, const uint32_t* __restrict__ ldst, uint32_t n, uint64_t n_elems) {
+  if (threadIdx.x != 0 || n == 0) return;
+  auto prob = [&](uint32_t i) {
+    float p = lprob[i] < n_elems ? data[lprob[i]] : 0.f;
+    if (isnan(p) || isinf(p) || p < 0.f) p = 0.f;
+    return p;
+  };
+  auto idx = [&](uint32_t i) { return lidx[i] < n_elems ? data[lidx[i]] : 0.f; };
+  if (ldst[0] >= n_elems) return;
+  float total = 0.f;
+  for (uint32_t i = 0; i < n; i++) total += prob(i);
+  if (!(total > 0.f)) { data[ldst[0]] = idx(0); return; }
+  float r = lrand[0] < n_elems ? data[lrand[0]] : 0.f;
+  if (isnan(r) || isinf(r)) r = 0.f;
+  r = fminf(fmaxf(r, 0.f), 0.99999994f);
+  const float target = r * total;
+  float acc = 0.f;
+  uint32_t chosen = n - 1;
+  for (uint32_t i = 0; i < n; i++) {
+    acc += prob(i);
+    if (target < acc) { chosen = i; break; }
+  }
+  data[ldst[0]] = idx(chosen);
+}
+
+// logits[locs[tok]] /= penalty when positive, *= penalty otherwise, once per listed token id
+__global__ void __launch_bounds__(64)
+k_repeat_penalty(float* data, const uint32_t* __restrict__ llog, uint64_t n_logit_locs, const uint32_t* __restrict__ toks,
+                 uint32_t n_ids, float penalty, uint64_t n_elems) {
+  const uint32_t i = blockIdx.x * 64u + threadIdx.x;
+  if (i >= n_ids) return;
+  const uint32_t tok = toks[i];
+  if (tok >= n_logit_locs) return;
+  // The reference's callers pass distinct ids (adam/models/engine.py:2052); with a repeated id the
+  // shader's invocations race.  Here every distinct id is penalised exactly once.
+  for (uint32_t j = 0; j < i; j++) if (toks[j] == tok) return;
+  const uint32_t loc = llog[tok];
+  if (loc >= n_elems) return;
+  const float v = data[loc];
+  data[loc] = v > 0.f ? v / penalty : v * penalty;
+}
+
+}  // namespace adamah
+
+using namespace adamah;
+
+extern "C" {
+
+int map_topk_dev(uint32_t map_id, uint32_t hs, uint32_t hi, uint32_t hv, uint32_t n, uint32_t k) { ADAMAH_API();
+  Map* m = get_f32_map(map_id);
+  if (!m) return ADAMAH_ERR_INVALID;
+  if (n == 0 || k == 0) return ADAMAH_OK;
+  if (k > SMP_MAX) return ADAMAH_ERR_INVALID;
+  const uint32_t *ls = res_u32(hs, n), *li = res_u32(hi, k), *lv = res_u32(hv, k);
+  if (!ls || !li || !lv) return ADAMAH_ERR_INVALID;
+  k_topk<<<1, 256, 0, g.stream>>>((float*)m->buf, ls, li, lv, n, k, m->n_elems);
+  count_launch();
+  return check_launch();
+}
+
+int map_topp_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n, float temperature, float top_p) { ADAMAH_API();
+  Map* m = get_f32_map(map_id);
+  if (!m) return ADAMAH_ERR_INVALID;
+  if (n == 0) return ADAMAH_OK;
+  if (n > SMP_MAX) return ADAMAH_ERR_INVALID;
+  const uint32_t *ls = res_u32(hs, n), *ld = res_u32(hd, n);
+  if (!ls || !ld) return ADAMAH_ERR_INVALID;
+  k_topp<<<1, 64, 0, g.stream>>>((float*)m->buf, ls, ld, n, temperature, top_p, m->n_elems);
+  count_launch();
+  return check_launch();
+}
+
+int map_resolve_idx_dev(uint32_t map_id, uint32_t hbase, uint32_t hsel, uint32_t hdst, uint32_t n) { ADAMAH_API();
+  Map* m = get_f32_map(map_id);
+  if (!m) return ADAMAH_ERR_INVALID;
+  if (n == 0) return ADAMAH_OK;
+  const uint32_t *lb = res_u32(hbase, 1), *lsel = res_u32(hsel, n), *ld = res_u32(hdst, n);
+  if (!lb || !lsel || !ld) return ADAMAH_ERR_INVALID;
+  k_resolve_idx<<<cdiv(n, 64), 64, 0, g.stream>>>((float*)m->buf, lb, lsel, ld, n, m->n_elems);
+  count_launch();
+  return check_launch();
+}
+
+int map_sample_categorical_dev(uint32_t map_id, uint32_t hidx, uint32_t hprob, uint32_t hrand, uint32_t hdst, uint32_t n) {
+  ADAMAH_API();
+  Map* m = get_f32_map(map_id);
+  if (!m) return ADAMAH_ERR_INVALID;
+  if (n == 0) return ADAMAH_OK;
+  if (n > SMP_MAX) return ADAMAH_ERR_INVALID;
+  const uint32_t *li = res_u32(hidx, n), *lp = res_u32(hprob, n), *lr = res_u32(hrand, 1), *ld = res_u32(hdst, 1);
+  if (!li || !lp || !lr || !ld) return ADAMAH_ERR_INVALID;
+  k_sample_categorical<<<1, 64, 0, g.stream>>>((float*)m->buf, li, lp, lr, ld, n, m->n_elems);
+  count_launch();
+  return check_launch();
+}
+
+int map_repeat_penalty_dev(uint32_t map_id, uint32_t hlog, uint32_t htok, uint32_t n_ids, float penalty) { ADAMAH_API();
+  Map* m = get_f32_map(map_id);
+  if (!m) return ADAMAH_ERR_INVALID;
+  if (n_ids == 0) return ADAMAH_OK;
+  if (n_ids > SMP_MAX) return ADAMAH_ERR_INVALID;
+  Res* rl = get_res(hlog);
+  const uint32_t* toks = res_u32(htok, n_ids);
+  if (!rl || !toks || rl->size_bytes < 4) return ADAMAH_ERR_INVALID;
+  const uint32_t* llog = res_u32(hlog, 1);
+  if (!llog) return ADAMAH_ERR_INVALID;
+  k_repeat_penalty<<<cdiv(n_ids, 64), 64, 0, g.stream>>>((float*)m->buf, llog, rl->size_bytes / 4, toks, n_ids, penalty,
+                                                         m->n_elems);
+  count_launch();
+  return check_launch();
+}
+
+}  // extern "C"

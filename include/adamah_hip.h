@@ -117,9 +117,15 @@ int map_layernorm_dev(uint32_t map_id, uint32_t locs_src, uint32_t locs_dst, uin
                       uint32_t locs_beta, uint32_t n_rows, uint32_t dim, float eps); /* adamah.c:7503 */
 int map_argmax_dev(uint32_t map_id, uint32_t locs_src, uint32_t locs_dst, uint32_t n); /* adamah.c:6875 */
 int map_topk_dev(uint32_t map_id, uint32_t locs_src, uint32_t locs_idx_dst, uint32_t locs_val_dst,
-                 uint32_t n, uint32_t k);                     /* adamah.c:6978 (returns -3: sampling tail not built) */
+                 uint32_t n, uint32_t k);                     /* adamah.c:6978 (k <= 64) */
 int map_topp_dev(uint32_t map_id, uint32_t locs_src, uint32_t locs_dst, uint32_t n, float temperature,
-                 float top_p);                                /* adamah.c:7095 (returns -3) */
+                 float top_p);                                /* adamah.c:7095 (n <= 64) */
+int map_resolve_idx_dev(uint32_t map_id, uint32_t base_locs, uint32_t sel_locs, uint32_t dst_locs,
+                        uint32_t n);                          /* adamah.c:7210 */
+int map_sample_categorical_dev(uint32_t map_id, uint32_t locs_idx, uint32_t locs_prob, uint32_t rand_loc,
+                               uint32_t dst_loc, uint32_t n); /* adamah.c:7286 (n <= 64) */
+int map_repeat_penalty_dev(uint32_t map_id, uint32_t locs_src, uint32_t token_ids, uint32_t n_ids,
+                           float penalty);                    /* adamah.c:6787 (n_ids <= 64) */
 
 /* ---- decode hot path ----------------------------------------------------------------------- */
 int map_rmsnorm_dev(uint32_t map_id, uint32_t locs_src, uint32_t locs_wt, uint32_t locs_dst,

@@ -765,6 +765,139 @@ class NumpyAdamah:
         best = v.max()
         m.data[dst] = f32(int(np.flatnonzero(v == best)[0]))
 
+    # ---- sampling tail ----------------------------------------------------------------------
+    def map_topk_dev(self, map_id, locs_src_handle, locs_idx_dst_handle, locs_val_dst_handle, n, k):
+        """shaders/src/f32/map_topk.comp:38-90 (dispatch adamah.c:6978-7093): k rounds of the best value not
+        yet chosen; NaN -> -FLT_MAX, ties -> lower index; rounds past n store index 0 and -FLT_MAX."""
+        self.op_count += 1
+        fn = "map_topk_dev"
+        m = self._map(fn, map_id, DTYPE_F32)
+        if n == 0 or k == 0:
+            return
+        if k > 64:
+            self._fail(fn, ERR_INVALID)
+        v = m.data[self._locs(fn, locs_src_handle, n)].copy()
+        v[np.isnan(v)] = NEG_MAX
+        li = self._locs(fn, locs_idx_dst_handle, k); lv = self._locs(fn, locs_val_dst_handle, k)
+        taken = np.zeros(n, bool)
+        for o in range(k):
+            if taken.all():
+                m.data[li[o]] = 0.0; m.data[lv[o]] = NEG_MAX
+                continue
+            cand = np.where(taken, -np.inf, v.astype(np.float64))
+            w = int(np.flatnonzero(cand == cand.max())[0])
+            taken[w] = True
+            m.data[li[o]] = f32(w); m.data[lv[o]] = v[w]
+
+    def map_topp_dev(self, map_id, locs_src_handle, locs_dst_handle, n, temperature, top_p):
+        """shaders/src/f32/map_topp.comp:23-95 (dispatch adamah.c:7095-7208), float32 and sequential like
+        the shader's single lane: softmax(logit / max(T, 1e-6)) in list order, cut after the first prefix
+        whose mass reaches top_p, renormalised over the prefix."""
+        self.op_count += 1
+        fn = "map_topp_dev"
+        m = self._map(fn, map_id, DTYPE_F32)
+        if n == 0:
+            return
+        if n > 64:
+            self._fail(fn, ERR_INVALID)
+        lg = m.data[self._locs(fn, locs_src_handle, n)].copy()
+        ld = self._locs(fn, locs_dst_handle, n)
+        lg[~np.isfinite(lg)] = NEG_MAX
+        temp = max(f32(temperature), f32(1e-6)); keep_p = min(max(f32(top_p), f32(0.0)), f32(1.0))
+        mx = lg.max()
+        if mx == NEG_MAX:
+            m.data[ld] = 0.0; return
+        pr = np.zeros(n, np.float32); tot = f32(0.0)
+        for i in range(n):
+            if lg[i] == NEG_MAX:
+                continue
+            pr[i] = np.exp(f32(f32(lg[i] - mx) / temp), dtype=np.float32)
+            tot = f32(tot + pr[i])
+        if tot <= 0:
+            out = np.zeros(n, np.float32); out[0] = 1.0
+            m.data[ld] = out; return
+        pr = (pr / tot).astype(np.float32)
+        keep, cs = 0, f32(0.0)
+        for i in range(n):
+            cs = f32(cs + pr[i]); keep = i + 1
+            if keep_p >= f32(0.999999) or cs >= keep_p:
+                break
+        ks = f32(0.0)
+        for i in range(keep):
+            ks = f32(ks + pr[i])
+        if ks <= 0:
+            ks = f32(1.0)
+        out = np.zeros(n, np.float32)
+        out[:keep] = (pr[:keep] / ks).astype(np.float32)
+        m.data[ld] = out
+
+    def map_resolve_idx_dev(self, map_id, base_locs_handle, sel_locs_handle, dst_locs_handle, n):
+        """shaders/src/f32/map_resolve_idx.comp:13-26: dst[i] = data[base + uint(data[sel[i]])]; negative or
+        non-finite selectors and results count as 0."""
+        self.op_count += 1
+        fn = "map_resolve_idx_dev"
+        m = self._map(fn, map_id, DTYPE_F32)
+        if n == 0:
+            return
+        base = int(self._locs(fn, base_locs_handle, 1)[0])
+        sel = self._locs(fn, sel_locs_handle, n); dst = self._locs(fn, dst_locs_handle, n)
+        for i in range(n):
+            sv = m.data[sel[i]]
+            if not np.isfinite(sv) or sv < 0:
+                sv = f32(0.0)
+            t = m.data[base + int(sv)]
+            if not np.isfinite(t) or t < 0:
+                t = f32(0.0)
+            m.data[dst[i]] = t
+
+    def map_sample_categorical_dev(self, map_id, locs_idx_handle, locs_prob_handle, rand_loc_handle, dst_loc_handle, n):
+        """shaders/src/f32/map_sample_categorical.comp:14-50: inverse-CDF draw, float32 running sums in list
+        order, r clamped to [0, 0.99999994], zero total -> first index."""
+        self.op_count += 1
+        fn = "map_sample_categorical_dev"
+        m = self._map(fn, map_id, DTYPE_F32)
+        if n == 0:
+            return
+        if n > 64:
+            self._fail(fn, ERR_INVALID)
+        li = self._locs(fn, locs_idx_handle, n); lp = self._locs(fn, locs_prob_handle, n)
+        r_loc = int(self._locs(fn, rand_loc_handle, 1)[0]); d_loc = int(self._locs(fn, dst_loc_handle, 1)[0])
+        p = m.data[lp].copy()
+        p[~np.isfinite(p) | (p < 0)] = 0.0
+        tot = f32(0.0)
+        for x in p:
+            tot = f32(tot + x)
+        if not tot > 0:
+            m.data[d_loc] = m.data[li[0]]; return
+        r = m.data[r_loc]
+        if not np.isfinite(r):
+            r = f32(0.0)
+        r = min(max(r, f32(0.0)), f32(0.99999994))
+        target = f32(r * tot)
+        acc, chosen = f32(0.0), n - 1
+        for i in range(n):
+            acc = f32(acc + p[i])
+            if target < acc:
+                chosen = i; break
+        m.data[d_loc] = m.data[li[chosen]]
+
+    def map_repeat_penalty_dev(self, map_id, locs_src_handle, token_ids_handle, n_ids, penalty):
+        """shaders/src/f32/map_repeat_penalty.comp:13-21: logit / penalty when positive, * penalty otherwise.
+        The callers pass distinct ids (adam/models/engine.py:2052); with a repeated id the shader's
+        invocations race, so the definition used here is: every distinct id once."""
+        self.op_count += 1
+        fn = "map_repeat_penalty_dev"
+        m = self._map(fn, map_id, DTYPE_F32)
+        if n_ids == 0:
+            return
+        if n_ids > 64:
+            self._fail(fn, ERR_INVALID)
+        toks = self._locs(fn, token_ids_handle, n_ids)
+        for t in dict.fromkeys(int(x) for x in toks):
+            loc = int(self._locs(fn, locs_src_handle, int(t) + 1)[int(t)])
+            v = m.data[loc]
+            m.data[loc] = f32(v / f32(penalty)) if v > 0 else f32(v * f32(penalty))
+
     def _matvec_argmax(self, fn, dtype, map_act, map_wt, la_h, lb_h, idx_h, val_h, dst_h, K, N, rpg):
         """adamah.c:9558-9721; pass 1 shaders/src/f32/map_matvec_argmax_t_xq4.comp:66-158 (per group of
         rows_per_group rows: best (value,row)), pass 2 map_argmax_pairs.comp:34-67.  Row values are

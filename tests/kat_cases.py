@@ -244,8 +244,41 @@ def kat_decode_plan_runtime_args(g, A):
         d, p = _read(g, 6, probe), _read(g, 7, probe)
         assert np.allclose(d, p, atol=1e-6) and np.allclose(p, lit, atol=1e-6)
 
+def kat_topk(g, A):
+    """test_decode_primitives.py:32-45: top 3 of six logits, the tie at 5.5 resolved to the lower index."""
+    _f32map(g, A, 10, 20)
+    logits = np.array([-3.0, 5.5, 2.0, 5.5, 4.0, -1.0], np.float32)
+    g.scatter(10, np.arange(6, dtype=np.uint32), logits)
+    g.map_topk_dev(10, _h(g, np.arange(6)), _h(g, [8, 9, 10]), _h(g, [12, 13, 14]), 6, 3)
+    assert _read(g, 10, [8, 9, 10]).astype(np.int32).tolist() == [1, 3, 4]
+    assert np.allclose(_read(g, 10, [12, 13, 14]), [5.5, 5.5, 4.0], atol=1e-6)
 
-ALL = [kat_argmax, kat_softmax_abs, kat_attn_softmax_abs, kat_q8_gather_scatter, kat_row_gather_xq8,
+
+def kat_topp(g, A):
+    """:48-60: temperature 1, top_p 0.9 over [5, 4, 1, -1] keeps two candidates."""
+    _f32map(g, A, 11, 16)
+    g.scatter(11, np.arange(4, dtype=np.uint32), np.array([5.0, 4.0, 1.0, -1.0], np.float32))
+    g.map_topp_dev(11, _h(g, [0, 1, 2, 3]), _h(g, [8, 9, 10, 11]), 4, 1.0, 0.9)
+    assert np.allclose(_read(g, 11, [8, 9, 10, 11]), [0.7310586, 0.26894143, 0.0, 0.0], atol=1e-5)
+
+
+def kat_resolve_idx_and_categorical(g, A):
+    """:63-95: positions [2, 0] of the id list at 4.. resolve to [33, 11]; r = 0.6 over p = [0.25, 0.75]
+    picks the second candidate."""
+    _f32map(g, A, 12, 32)   # the reference's wrapper calls this array 16
+    vals = np.zeros(32, np.float32)
+    vals[4:8] = [11.0, 22.0, 33.0, 44.0]; vals[8:10] = [2.0, 0.0]; vals[16:18] = [0.25, 0.75]; vals[20] = 0.6
+    g.scatter(12, np.arange(32, dtype=np.uint32), vals)
+    resolved, dst = _h(g, [12, 13]), _h(g, [21])
+    g.batch_begin()
+    g.map_resolve_idx_dev(12, _h(g, [4]), _h(g, [8, 9]), resolved, 2)
+    g.map_sample_categorical_dev(12, resolved, _h(g, [16, 17]), _h(g, [20]), dst, 2)
+    g.batch_end()
+    assert _read(g, 12, [12, 13]).astype(np.int32).tolist() == [33, 11]
+    assert int(_read(g, 12, [21])[0]) == 11
+
+
+ALL = [kat_argmax, kat_topk, kat_topp, kat_resolve_idx_and_categorical, kat_softmax_abs, kat_attn_softmax_abs, kat_q8_gather_scatter, kat_row_gather_xq8,
        kat_matvec_t_xq8, kat_matvec_t_xq4, kat_q4_matmul_identity, kat_batch_gather_scatter,
        kat_row_copy_offset, kat_fusion_row_copy_then_matmul, kat_scalar_state, kat_fusion_batch_order,
        kat_decode_plan_runtime_args]

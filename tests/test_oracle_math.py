@@ -336,3 +336,79 @@ def test_error_codes():
         g.scatter_q4_packed_contiguous(1, 1, np.zeros(2, np.uint8))         # odd start
     h, _ = g.upload_dev(np.zeros(4, np.uint32))
     assert g.upload_dev(np.zeros(5, np.uint32), handle=h)[0] == 0           # size change on re-upload
+
+
+# ---- sampling tail: what the definitions fix, independent of the oracle's loops --------------------
+def _sampling_map(g, vals, n=256):
+    f32map(g, 2, n, np.zeros(n, np.float32))
+    g.scatter(2, np.arange(len(vals), dtype=np.uint32), np.asarray(vals, np.float32))
+
+
+def test_topk_equals_stable_sort_with_nan_lowest():
+    g = oracle.init()
+    rng = np.random.default_rng(3)
+    v = rng.integers(-5, 6, 100).astype(np.float32)          # many ties
+    v[[7, 50]] = np.nan
+    _sampling_map(g, v)
+    g.map_topk_dev(2, up(g, np.arange(100)), up(g, 128 + np.arange(64)), up(g, 192 + np.arange(64)), 100, 64)
+    clean = np.where(np.isnan(v), np.float32(-3.402823466e+38), v)
+    order = np.lexsort((np.arange(100), -clean.astype(np.float64)))[:64]   # value descending, then index ascending
+    assert read(g, 2, 128, 64).astype(np.int64).tolist() == order.tolist()
+    assert np.array_equal(read(g, 2, 192, 64), clean[order])
+    # more rounds than candidates: the surplus stores index 0 and the lowest float
+    _sampling_map(g, [1.0, 3.0])
+    g.map_topk_dev(2, up(g, [0, 1]), up(g, [8, 9, 10]), up(g, [12, 13, 14]), 2, 3)
+    assert read(g, 2, 8, 3).tolist() == [1.0, 0.0, 0.0]
+    assert read(g, 2, 12, 3).tolist() == [3.0, 1.0, np.float32(-3.402823466e+38)]
+
+
+def test_topp_closed_forms():
+    g = oracle.init()
+    logits = np.array([2.0, 1.0, 0.5, -1.0, -3.0], np.float32)
+    sm = lambda t: np.exp((logits.astype(np.float64) - 2.0) / t) / np.exp((logits.astype(np.float64) - 2.0) / t).sum()
+    for temp, top_p in [(1.0, 1.0), (0.7, 0.8), (2.0, 0.5), (1.0, 0.0)]:
+        _sampling_map(g, logits)
+        g.map_topp_dev(2, up(g, np.arange(5)), up(g, 16 + np.arange(5)), 5, temp, top_p)
+        p = sm(temp)
+        # map_topp.comp:77 leaves the prefix loop at once when top_p >= 0.999999: one candidate is kept
+        keep = 1 if top_p >= 0.999999 else int(np.searchsorted(np.cumsum(p), top_p - 1e-9) + 1)
+        want = np.zeros(5); want[:keep] = p[:keep] / p[:keep].sum()
+        assert np.allclose(read(g, 2, 16, 5), want, atol=2e-6), (temp, top_p)
+    # all candidates unusable -> zeros; a single usable one -> probability one on it
+    _sampling_map(g, [np.nan, np.inf, -np.inf])
+    g.map_topp_dev(2, up(g, [0, 1, 2]), up(g, [16, 17, 18]), 3, 1.0, 0.9)
+    assert read(g, 2, 16, 3).tolist() == [0.0, 0.0, 0.0]
+    _sampling_map(g, [np.nan, 4.0, np.nan])
+    g.map_topp_dev(2, up(g, [0, 1, 2]), up(g, [16, 17, 18]), 3, 1.0, 0.5)
+    assert read(g, 2, 16, 3).tolist() == [0.0, 1.0, 0.0]
+
+
+def test_categorical_is_the_inverse_cdf_and_repeat_penalty_is_its_own_inverse():
+    g = oracle.init()
+    p = np.array([0.1, 0.0, 0.4, 0.5], np.float32); ids = np.array([7.0, 8.0, 9.0, 10.0], np.float32)
+    edges = np.cumsum(p.astype(np.float64))
+    for r in [0.0, 0.05, 0.0999, 0.1001, 0.49, 0.51, 0.999, 1.0, 7.0, -2.0, np.nan]:
+        _sampling_map(g, np.concatenate([p, ids, [r]]))
+        g.map_sample_categorical_dev(2, up(g, [4, 5, 6, 7]), up(g, [0, 1, 2, 3]), up(g, [8]), up(g, [9]), 4)
+        rr = 0.0 if not np.isfinite(r) else min(max(r, 0.0), 0.99999994)
+        want = ids[int(np.searchsorted(edges, rr * edges[-1], side="right"))]
+        assert read(g, 2, 9, 1)[0] == want, r
+    _sampling_map(g, np.concatenate([np.zeros(4), ids, [0.3]]))       # zero mass -> first candidate
+    g.map_sample_categorical_dev(2, up(g, [4, 5, 6, 7]), up(g, [0, 1, 2, 3]), up(g, [8]), up(g, [9]), 4)
+    assert read(g, 2, 9, 1)[0] == 7.0
+    logits = np.array([2.0, -1.0, 0.0, 3.0, -4.0], np.float32)
+    _sampling_map(g, logits)
+    locs, toks = up(g, np.arange(5)), up(g, [3, 1, 4])
+    g.map_repeat_penalty_dev(2, locs, toks, 3, 2.0)
+    assert read(g, 2, 0, 5).tolist() == [2.0, -2.0, 0.0, 1.5, -8.0]
+    g.map_repeat_penalty_dev(2, locs, toks, 3, 0.5)
+    assert read(g, 2, 0, 5).tolist() == logits.tolist()
+
+
+def test_resolve_idx_guards():
+    g = oracle.init()
+    vals = np.zeros(32, np.float32)
+    vals[4:8] = [11.0, -5.0, np.nan, 44.0]; vals[8:13] = [3.0, 1.0, 2.0, -1.0, np.inf]
+    _sampling_map(g, vals)
+    g.map_resolve_idx_dev(2, up(g, [4]), up(g, [8, 9, 10, 11, 12]), up(g, 16 + np.arange(5)), 5)
+    assert read(g, 2, 16, 5).tolist() == [44.0, 0.0, 0.0, 11.0, 11.0]
