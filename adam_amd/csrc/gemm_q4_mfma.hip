@@ -195,7 +195,282 @@ k_gemm_q4_f16(const float* act, float* out, const uint8_t* __restrict__ W, const
   }
 }
 
+
+// Large M: the activations are converted once, by a kernel of their own, to the fp16 form the matrix
+// cores consume (scaled per row by its power of two, elements of every 8-word in the order the nibble
+// unpacking produces: (0,4)(1,5)(2,6)(3,7)), so the matmul workgroups copy 16-byte pieces into LDS
+// instead of each converting the whole tile again.  One workgroup per row; also stores (s, 1/s).
+__global__ void __launch_bounds__(256)
+k_act_f16(const float* act, const uint32_t* __restrict__ la, uint32_t M, uint32_t K, float* scale, uint4* xh) {
+  __shared__ float red[4];
+  const uint32_t row = blockIdx.x, op = blockIdx.y, tid = threadIdx.x;
+  const float* x = act + (uint64_t)la[op] + (uint64_t)row * K;
+  float m = 0.f;
+  for (uint32_t i = tid; i < K; i += 256u) m = fmaxf(m, fabsf(x[i]));
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  if ((tid & 63u) == 0) red[tid >> 6] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  const uint32_t e = (__float_as_uint(m) >> 23) & 0xFFu;
+  float s = 1.f, inv = 1.f;
+  if (e >= 14u && e <= 254u) { s = __uint_as_float((267u - e) << 23); inv = __uint_as_float((e - 13u) << 23); }
+  if (tid == 0) {
+    scale[2 * ((uint64_t)op * M + row)] = s;
+    scale[2 * ((uint64_t)op * M + row) + 1] = inv;
+  }
+  uint4* dst = xh + ((uint64_t)op * M + row) * (K >> 3);
+  for (uint32_t w = tid; w < (K >> 3); w += 256u) {
+    const f4qu_t v0 = *(const f4qu_t*)(x + w * 8u), v1 = *(const f4qu_t*)(x + w * 8u + 4u);
+    const h2q_t p0 = {(_Float16)(v0.x * s), (_Float16)(v1.x * s)}, p1 = {(_Float16)(v0.y * s), (_Float16)(v1.y * s)};
+    const h2q_t p2 = {(_Float16)(v0.z * s), (_Float16)(v1.z * s)}, p3 = {(_Float16)(v0.w * s), (_Float16)(v1.w * s)};
+    dst[w] = make_uint4(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1),
+                        __builtin_bit_cast(uint32_t, p2), __builtin_bit_cast(uint32_t, p3));
+  }
+}
+
+// Workgroup = 4 waves, each with R tiles of 16 weight rows = 64 R weight rows x 16 MT activation rows.
+// An activation fragment read from LDS feeds R matrix instructions, so the LDS traffic per
+// instruction falls with R; the weights of a wave's R tiles are dequantised in its registers as in
+// the kernel above.  One step = 128 weights of K; the next step's weight words and activation
+// pieces are loaded into registers while the matrix cores work on the current one.
+template <int MT, int R>
+__global__ void __launch_bounds__(256)
+k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh,
+                    const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc, const float* __restrict__ scale,
+                    uint32_t M, uint32_t K, uint32_t N) {
+  constexpr uint32_t BM = 16u * MT, ROWB = 272u;
+  __shared__ __attribute__((aligned(16))) uint8_t xs[BM * ROWB];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t r16 = lane & 15u, g = lane >> 4;
+  const uint32_t n0 = blockIdx.x * (64u * R) + wave * (16u * R), m0 = blockIdx.y * BM, op = blockIdx.z;
+  const uint64_t c_off = lc[op], gbase = (uint64_t)lb[op] >> 5;
+  const uint32_t nblk = K >> 5, kw = K >> 3;                   // blocks and 16-byte pieces per row
+  uint32_t nrow[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) nrow[r] = min(n0 + r * 16u + r16, N - 1u);   // rows past N: clamped, not stored
+
+  f4q_t acc[R][MT];
+#pragma unroll
+  for (int r = 0; r < R; r++)
+#pragma unroll
+    for (int t = 0; t < MT; t++) acc[r][t] = (f4q_t){0.f, 0.f, 0.f, 0.f};
+
+  uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u, nib_lo = 0x000F000Fu, nib_hi = 0x00F000F0u;
+  asm volatile("" : "+v"(magic_lo));   // opaque: lets instruction selection use the three-operand and-or
+  asm volatile("" : "+v"(magic_hi));
+  asm volatile("" : "+s"(nib_lo));
+  asm volatile("" : "+s"(nib_hi));
+  const h2q_t off_lo = {(_Float16)-1032.f, (_Float16)-1032.f}, off_hi = {(_Float16)-72.f, (_Float16)-72.f};
+
+  // staging: the tile's 16 pieces per row and step; thread -> (row, piece) pairs, MT per thread
+  const u4q_t* xrow[MT];
+#pragma unroll
+  for (uint32_t u = 0; u < MT; u++) {
+    const uint32_t w = tid + u * 256u, row = min(m0 + (w >> 4), M - 1u);   // rows past M: clamped, not stored
+    xrow[u] = xh + ((uint64_t)op * M + row) * kw + (w & 15u);
+  }
+  u4q_t xn[MT], qn[R];
+  _Float16 dn[R];
+  // always executed; the step past K re-reads the last one and is not used
+#define GEMM_FETCH(kb_raw)                                                        \
+  do {                                                                            \
+    const uint32_t kb_ = min((kb_raw), nblk - 4u);                                \
+    _Pragma("unroll") for (int r = 0; r < R; r++) {                               \
+      const uint64_t gi = gbase + (uint64_t)nrow[r] * nblk + kb_ + g;             \
+      qn[r] = *(const u4q_t*)(W + (gi << 4));                                     \
+      dn[r] = __builtin_bit_cast(_Float16, d16[gi]);                              \
+    }                                                                             \
+    _Pragma("unroll") for (uint32_t u = 0; u < MT; u++) xn[u] = xrow[u][kb_ * 4u]; \
+  } while (0)
+  GEMM_FETCH(0u);
+
+  for (uint32_t kb0 = 0; kb0 < nblk; kb0 += 4u) {
+#pragma unroll
+    for (uint32_t u = 0; u < MT; u++) {
+      const uint32_t w = tid + u * 256u;
+      *(u4q_t*)(xs + (w >> 4) * ROWB + (w & 15u) * 16u) = xn[u];
+    }
+    // dequantise: (1024 + n) - 1032 = n - 8 and (64 + n) - 72 = n - 8 exactly, then one rounding in d * (n - 8)
+    u4q_t a[R][4];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      const h2q_t d2 = {dn[r], dn[r]};
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const uint32_t w = j == 0 ? qn[r].x : j == 1 ? qn[r].y : j == 2 ? qn[r].z : qn[r].w, w8 = w >> 8;
+        const h2q_t t0 = __builtin_bit_cast(h2q_t, (w & nib_lo) | magic_lo), t1 = __builtin_bit_cast(h2q_t, (w & nib_hi) | magic_hi);
+        const h2q_t t2 = __builtin_bit_cast(h2q_t, (w8 & nib_lo) | magic_lo), t3 = __builtin_bit_cast(h2q_t, (w8 & nib_hi) | magic_hi);
+        a[r][j] = (u4q_t){__builtin_bit_cast(uint32_t, (h2q_t)((t0 + off_lo) * d2)), __builtin_bit_cast(uint32_t, (h2q_t)((t1 + off_hi) * d2)),
+                          __builtin_bit_cast(uint32_t, (h2q_t)((t2 + off_lo) * d2)), __builtin_bit_cast(uint32_t, (h2q_t)((t3 + off_hi) * d2))};
+      }
+    }
+    __syncthreads();
+    GEMM_FETCH(kb0 + 4u);
+#pragma unroll
+    for (int t = 0; t < MT; t++) {
+      const uint8_t* xp = xs + (t * 16u + r16) * ROWB + g * 64u;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const u4q_t b = *(const u4q_t*)(xp + j * 16);
+#pragma unroll
+        for (int r = 0; r < R; r++)
+          acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8q_t, a[r][j]), __builtin_bit_cast(h8q_t, b), acc[r][t], 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+  // lane (j = r16, g) holds D[4g + i][j]: weight rows n0 + 16 r + 4g + i, activation row m0 + 16 t + r16
+#pragma unroll
+  for (int t = 0; t < MT; t++) {
+    const uint32_t row = m0 + t * 16u + r16;
+    if (row >= M) continue;
+    const float inv = scale[2 * ((uint64_t)op * M + row) + 1];
+    float* c = out + c_off + (uint64_t)row * N;
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t n = n0 + r * 16u + 4u * g + i;
+        if (n < N) c[n] = acc[r][t][i] * inv;
+      }
+  }
+}
+
+#undef GEMM_FETCH
+
+// Few activation rows (M <= 32): the weights are read once and nothing is reused, so the work is
+// bound by how fast they stream.  The four waves of a workgroup share R tiles of 16 weight rows and
+// take every fourth step of K each (a matrix with few rows still spreads over the whole chip); every
+// wave stages its own activation tile from the fp16 copy into its own piece of LDS, so no
+// workgroup barrier sits in the K loop.  The four partial tiles are summed in wave order at the end.
+template <int MT, int R>
+__global__ void __launch_bounds__(256)
+k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh,
+                     const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc, const float* __restrict__ scale,
+                     uint32_t M, uint32_t K, uint32_t N) {
+  constexpr uint32_t BM = 16u * MT, ROWB = 272u, NP = 4u * MT;      // pieces per lane and step
+  constexpr uint32_t TILE = BM * ROWB, PART = 3u * R * MT * 4u * 64u * 4u;
+  __shared__ __attribute__((aligned(16))) uint8_t xs_all[(4u * TILE > PART) ? 4u * TILE : PART];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+  const uint32_t r16 = lane & 15u, g = lane >> 4;
+  uint8_t* xs = xs_all + wave * TILE;
+  const uint32_t n0 = blockIdx.x * (16u * R), m0 = blockIdx.y * BM, op = blockIdx.z;
+  const uint64_t c_off = lc[op], gbase = (uint64_t)lb[op] >> 5;
+  const uint32_t nblk = K >> 5, kw = K >> 3;
+  uint32_t nrow[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) nrow[r] = min(n0 + r * 16u + r16, N - 1u);
+
+  f4q_t acc[R][MT];
+#pragma unroll
+  for (int r = 0; r < R; r++)
+#pragma unroll
+    for (int t = 0; t < MT; t++) acc[r][t] = (f4q_t){0.f, 0.f, 0.f, 0.f};
+
+  uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u, nib_lo = 0x000F000Fu, nib_hi = 0x00F000F0u;
+  asm volatile("" : "+v"(magic_lo));
+  asm volatile("" : "+v"(magic_hi));
+  asm volatile("" : "+s"(nib_lo));
+  asm volatile("" : "+s"(nib_hi));
+  const h2q_t off_lo = {(_Float16)-1032.f, (_Float16)-1032.f}, off_hi = {(_Float16)-72.f, (_Float16)-72.f};
+
+  const u4q_t* xrow[NP];
+#pragma unroll
+  for (uint32_t u = 0; u < NP; u++) {
+    const uint32_t w = lane + u * 64u, row = min(m0 + (w >> 4), M - 1u);
+    xrow[u] = xh + ((uint64_t)op * M + row) * kw + (w & 15u);
+  }
+  u4q_t xn[NP], qn[R];
+  _Float16 dn[R];
+#define GEMM_FETCH(kb_raw)                                                        \
+  do {                                                                            \
+    const uint32_t kb_ = min((kb_raw), nblk - 4u);                                \
+    _Pragma("unroll") for (int r = 0; r < R; r++) {                               \
+      const uint64_t gi = gbase + (uint64_t)nrow[r] * nblk + kb_ + g;             \
+      qn[r] = *(const u4q_t*)(W + (gi << 4));                                     \
+      dn[r] = __builtin_bit_cast(_Float16, d16[gi]);                              \
+    }                                                                             \
+    _Pragma("unroll") for (uint32_t u = 0; u < NP; u++) xn[u] = xrow[u][kb_ * 4u]; \
+  } while (0)
+  GEMM_FETCH(wave * 4u);
+
+  for (uint32_t kb0 = wave * 4u; kb0 < nblk; kb0 += 16u) {
+#pragma unroll
+    for (uint32_t u = 0; u < NP; u++) {
+      const uint32_t w = lane + u * 64u;
+      *(u4q_t*)(xs + (w >> 4) * ROWB + (w & 15u) * 16u) = xn[u];
+    }
+    u4q_t a[R][4];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      const h2q_t d2 = {dn[r], dn[r]};
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const uint32_t w = j == 0 ? qn[r].x : j == 1 ? qn[r].y : j == 2 ? qn[r].z : qn[r].w, w8 = w >> 8;
+        const h2q_t t0 = __builtin_bit_cast(h2q_t, (w & nib_lo) | magic_lo), t1 = __builtin_bit_cast(h2q_t, (w & nib_hi) | magic_hi);
+        const h2q_t t2 = __builtin_bit_cast(h2q_t, (w8 & nib_lo) | magic_lo), t3 = __builtin_bit_cast(h2q_t, (w8 & nib_hi) | magic_hi);
+        a[r][j] = (u4q_t){__builtin_bit_cast(uint32_t, (h2q_t)((t0 + off_lo) * d2)), __builtin_bit_cast(uint32_t, (h2q_t)((t1 + off_hi) * d2)),
+                          __builtin_bit_cast(uint32_t, (h2q_t)((t2 + off_lo) * d2)), __builtin_bit_cast(uint32_t, (h2q_t)((t3 + off_hi) * d2))};
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    GEMM_FETCH(kb0 + 16u);
+#pragma unroll
+    for (int t = 0; t < MT; t++) {
+      const uint8_t* xp = xs + (t * 16u + r16) * ROWB + g * 64u;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const u4q_t b = *(const u4q_t*)(xp + j * 16);
+#pragma unroll
+        for (int r = 0; r < R; r++)
+          acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8q_t, a[r][j]), __builtin_bit_cast(h8q_t, b), acc[r][t], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  // sum the four waves' tiles in wave order; wave 0 stores
+  __syncthreads();
+  float* part = (float*)xs_all;
+  if (wave > 0) {
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+      for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) part[((((wave - 1u) * R + r) * MT + t) * 4u + i) * 64u + lane] = acc[r][t][i];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (uint32_t w = 0; w < 3; w++)
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+      for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[r][t][i] += part[(((w * R + r) * MT + t) * 4u + i) * 64u + lane];
+#pragma unroll
+  for (int t = 0; t < MT; t++) {
+    const uint32_t row = m0 + t * 16u + r16;
+    if (row >= M) continue;
+    const float inv = scale[2 * ((uint64_t)op * M + row) + 1];
+    float* c = out + c_off + (uint64_t)row * N;
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t n = n0 + r * 16u + 4u * g + i;
+        if (n < N) c[n] = acc[r][t][i] * inv;
+      }
+  }
+}
+#undef GEMM_FETCH
+
 static float* g_scale_buf = nullptr;
+static uint4* g_xh_buf = nullptr;     // fp16 activations of the tiled form
+static size_t g_xh_cap = 0;           // in bytes
 static size_t g_scale_cap = 0;
 
 // Preconditions (checked by the caller against the host copies of the handles): Q4 map whose blocks
@@ -210,14 +485,58 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
     if (hipMalloc((void**)&g_scale_buf, g_scale_cap * sizeof(float)) != hipSuccess) { g_scale_buf = nullptr; g_scale_cap = 0; return ADAMAH_ERR_MEMORY; }
   }
   float* act = (float*)ma->buf;
-  k_row_pow2_scale<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf);
-  count_launch();
-  const uint32_t mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8;
-  const bool ksplit = mt <= 2;    // few activation rows: bandwidth bound, spread K over the waves
-  dim3 grid(cdiv(N, ksplit ? 16 : 64), cdiv(M, 16 * mt), n_ops);
+  uint32_t mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8;
+  if (tuning("ADAMAH_GEMM_TILED", 1) == 0) {
+    // the first form: every workgroup converts its activation tile from float32 itself
+    k_row_pow2_scale<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf);
+    count_launch();
+    const bool ksplit = mt <= 2;
+    dim3 grid(cdiv(N, ksplit ? 16 : 64), cdiv(M, 16 * mt), n_ops);
 #define GQ(T, S) k_gemm_q4_f16<T, S><<<grid, 256, 0, g.stream>>>(act, act, mw->buf, mw->d16, la, lb, lc, g_scale_buf, M, K, N)
-  if (mt == 1) GQ(1, true); else if (mt == 2) GQ(2, true); else if (mt == 4) GQ(4, false); else GQ(8, false);
+    if (mt == 1) GQ(1, true); else if (mt == 2) GQ(2, true); else if (mt == 4) GQ(4, false); else GQ(8, false);
 #undef GQ
+    count_launch();
+    return check_launch();
+  }
+  const size_t xh_need = (size_t)n_ops * M * K * 2;
+  if (xh_need > g_xh_cap) {
+    if (g_xh_buf) { hipStreamSynchronize(g.stream); hipFree(g_xh_buf); }
+    g_xh_cap = xh_need;
+    if (hipMalloc((void**)&g_xh_buf, g_xh_cap) != hipSuccess) { g_xh_buf = nullptr; g_xh_cap = 0; return ADAMAH_ERR_MEMORY; }
+  }
+  k_act_f16<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf, g_xh_buf);
+  count_launch();
+  auto wgs = [&](uint32_t rows_per_wg, uint32_t t) { return (uint64_t)cdiv(N, rows_per_wg) * cdiv(M, 16 * t) * n_ops; };
+  const uint64_t want = 2ull * (uint64_t)g.n_cu;
+  if (mt <= 2) {
+    // few activation rows: the K-split form, as many weight-row tiles per workgroup as still fill the chip
+    uint32_t R = wgs(64, mt) >= want ? 4 : wgs(32, mt) >= want ? 2 : 1;
+    R = (uint32_t)tuning("ADAMAH_GEMM_R", (int)R);
+    R = R >= 4 ? 4 : R >= 2 ? 2 : 1;
+    dim3 grid(cdiv(N, 16 * R), cdiv(M, 16 * mt), n_ops);
+#define GK(T, RR) k_gemm_q4_f16_ksplit<T, RR><<<grid, 256, 0, g.stream>>>(act, mw->buf, mw->d16, (const u4q_t*)g_xh_buf, lb, lc, g_scale_buf, M, K, N)
+    if (mt == 1) { if (R == 4) GK(1, 4); else if (R == 2) GK(1, 2); else GK(1, 1); }
+    else { if (R == 4) GK(2, 4); else if (R == 2) GK(2, 2); else GK(2, 1); }
+#undef GK
+    count_launch();
+    return check_launch();
+  }
+  // Tile per workgroup: 64 R weight rows x 16 MT activation rows.  The largest of (8,2), (8,1), (4,1)
+  // that still gives every CU two workgroups; a larger tile reads the activations and LDS less often.
+  uint32_t R = 1;
+  if (mt == 8) {
+    if (wgs(128, 8) >= want) R = 2;
+    else if (wgs(64, 8) >= want) R = 1;
+    else mt = 4;
+  }
+  if (mt == 8 && tuning("ADAMAH_GEMM_MT", 8) == 4) mt = 4;
+  R = (uint32_t)tuning("ADAMAH_GEMM_R", (int)R);
+  R = R >= 4 && mt == 4 ? 4 : R >= 2 ? 2 : 1;
+  dim3 grid(cdiv(N, 64 * R), cdiv(M, 16 * mt), n_ops);
+#define GT(T, RR) k_gemm_q4_f16_tiled<T, RR><<<grid, 256, 0, g.stream>>>(act, mw->buf, mw->d16, (const u4q_t*)g_xh_buf, lb, lc, g_scale_buf, M, K, N)
+  if (mt == 4) { if (R == 4) GT(4, 4); else if (R == 2) GT(4, 2); else GT(4, 1); }
+  else { if (R == 2) GT(8, 2); else GT(8, 1); }
+#undef GT
   count_launch();
   return check_launch();
 }
@@ -226,6 +545,9 @@ void gemm_q4_mfma_release() {
   if (g_scale_buf) hipFree(g_scale_buf);
   g_scale_buf = nullptr;
   g_scale_cap = 0;
+  if (g_xh_buf) hipFree(g_xh_buf);
+  g_xh_buf = nullptr;
+  g_xh_cap = 0;
 }
 
 }  // namespace adamah
