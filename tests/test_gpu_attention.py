@@ -69,7 +69,11 @@ def test_config3_gqa_decode_attention_fp16_kv(hip, ctx):
 
 @pytest.mark.parametrize("ctx,kv16,softcap,Hq,Hkv,d", [
     (1, True, 50.0, 4, 1, 256), (640, True, 50.0, 4, 1, 256), (1023, False, 0.0, 8, 2, 64),
-    (1025, True, 0.0, 8, 2, 64), (2049, False, 30.0, 4, 4, 128), (300, True, 0.0, 6, 2, 96)])
+    (1025, True, 0.0, 8, 2, 64), (2049, False, 30.0, 4, 4, 128), (300, True, 0.0, 6, 2, 96),
+    # the grouped kernel's other shapes: one, two and eight query heads per KV head, tile edges, prefetching form
+    (17, True, 0.0, 8, 8, 128), (63, True, 20.0, 16, 2, 64), (64, True, 0.0, 4, 2, 256), (65, True, 0.0, 8, 1, 128),
+    (1000, True, 0.0, 16, 2, 128), (5000, True, 0.0, 8, 8, 64), (9000, True, 15.0, 16, 2, 64), (3001, True, 0.0, 6, 3, 128),
+    (700, True, 0.0, 68, 17, 64)])
 def test_attention_variants(hip, ctx, kv16, softcap, Hq, Hkv, d):
     rng = np.random.default_rng(ctx + d)
     q = rng.standard_normal((Hq, d)).astype(np.float32)
