@@ -94,3 +94,31 @@ def test_decode_plan_replay_equals_op_by_op(hip, arch):
         res.append((tok, eng.read_slot('hidden')))
     assert res[0][0] == res[1][0]
     assert np.array_equal(res[0][1], res[1][1])
+
+
+def _full_model_vs_cpu(hip, cfg, n_prompt, n_gen, seed):
+    """Full-size random-init model on the GPU against the reference NumPy forward pass (which never touches
+    the op surface): teacher-forced greedy tokens agree wherever the reference's top-two logit gap is
+    not at rounding level."""
+    tensors = synth.make_model(cfg, seed=seed, sigma=0.02)
+    prompt = [int(t) for t in np.random.default_rng(seed).integers(0, cfg.n_vocab, n_prompt)]
+    deq = {n: (v.dequant() if isinstance(v, QTensor) else v) for n, v in tensors.items()}
+    cpu = CpuModel(cfg, deq, kv_cap=n_prompt + n_gen + 2, kv_fp16=True, acc64=False)
+    cpu_tok, margins = cpu.generate(prompt, n_gen)
+    del deq, cpu
+    dev = DecodeEngine(hip, cfg, tensors, A=A, kv_cap=n_prompt + n_gen + 2, kv_fp16=True)
+    forced_tok, stats = dev.generate(prompt, GenerationConfig(max_tokens=n_gen), forced=cpu_tok)
+    assert stats['n_gen'] == n_gen
+    agree = [a == b or m < 1e-4 for a, b, m in zip(forced_tok, cpu_tok, margins)]
+    assert all(agree), (forced_tok, cpu_tok, margins)
+    assert sum(a == b for a, b in zip(forced_tok, cpu_tok)) >= n_gen - 1
+
+
+def test_gemma3_1b_full_model_tokens_match_reference_forward(hip):
+    note("engine gemma-3-1b shape, all 26 layers, vocabulary 262144")
+    _full_model_vs_cpu(hip, synth.gemma3_1b_config(), 12, 8, 0)
+
+
+def test_llama3_8b_full_model_tokens_match_reference_forward(hip):
+    note("engine llama-3-8b shape, all 32 layers, Q8_0 head")
+    _full_model_vs_cpu(hip, synth.llama3_8b_config(), 4, 3, 0)
