@@ -340,18 +340,20 @@ k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __r
 #undef GEMM_FETCH
 
 // Few activation rows (M <= 32): the weights are read once and nothing is reused, so the work is
-// bound by how fast they stream.  The four waves of a workgroup share R tiles of 16 weight rows and
-// take every fourth step of K each (a matrix with few rows still spreads over the whole chip); every
+// bound by how fast they stream.  The NWV waves of a workgroup share R tiles of 16 weight rows and
+// take every NWV-th step of K each (a matrix with few rows still spreads over the whole chip); every
 // wave stages its own activation tile from the fp16 copy into its own piece of LDS, so no
-// workgroup barrier sits in the K loop.  The four partial tiles are summed in wave order at the end.
-template <int MT, int R>
-__global__ void __launch_bounds__(256)
+// workgroup barrier sits in the K loop.  The partial tiles are summed in wave order at the end.
+// Eight waves (16 activation rows only: the wave-private tiles of 32 rows would not fit the static
+// LDS limit) keep twice as many loads in flight for matrices with few weight rows.
+template <int MT, int R, int NWV>
+__global__ void __launch_bounds__(64 * NWV)
 k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh,
                      const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc, const float* __restrict__ scale,
                      uint32_t M, uint32_t K, uint32_t N) {
   constexpr uint32_t BM = 16u * MT, ROWB = 272u, NP = 4u * MT;      // pieces per lane and step
-  constexpr uint32_t TILE = BM * ROWB, PART = 3u * R * MT * 4u * 64u * 4u;
-  __shared__ __attribute__((aligned(16))) uint8_t xs_all[(4u * TILE > PART) ? 4u * TILE : PART];
+  constexpr uint32_t TILE = BM * ROWB, PART = (NWV - 1u) * R * MT * 4u * 64u * 4u;
+  __shared__ __attribute__((aligned(16))) uint8_t xs_all[(NWV * TILE > PART) ? NWV * TILE : PART];
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
   const uint32_t r16 = lane & 15u, g = lane >> 4;
@@ -396,7 +398,7 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
   } while (0)
   GEMM_FETCH(wave * 4u);
 
-  for (uint32_t kb0 = wave * 4u; kb0 < nblk; kb0 += 16u) {
+  for (uint32_t kb0 = wave * 4u; kb0 < nblk; kb0 += 4u * NWV) {
 #pragma unroll
     for (uint32_t u = 0; u < NP; u++) {
       const uint32_t w = lane + u * 64u;
@@ -416,7 +418,7 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
       }
     }
     __builtin_amdgcn_wave_barrier();
-    GEMM_FETCH(kb0 + 16u);
+    GEMM_FETCH(kb0 + 4u * NWV);
 #pragma unroll
     for (int t = 0; t < MT; t++) {
       const uint8_t* xp = xs + (t * 16u + r16) * ROWB + g * 64u;
@@ -430,7 +432,7 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
     }
     __builtin_amdgcn_wave_barrier();
   }
-  // sum the four waves' tiles in wave order; wave 0 stores
+  // sum the waves' tiles in wave order; wave 0 stores
   __syncthreads();
   float* part = (float*)xs_all;
   if (wave > 0) {
@@ -444,7 +446,7 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
   __syncthreads();
   if (wave > 0) return;
 #pragma unroll
-  for (uint32_t w = 0; w < 3; w++)
+  for (uint32_t w = 0; w < NWV - 1u; w++)
 #pragma unroll
     for (int r = 0; r < R; r++)
 #pragma unroll
@@ -514,9 +516,12 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
     R = (uint32_t)tuning("ADAMAH_GEMM_R", (int)R);
     R = R >= 4 ? 4 : R >= 2 ? 2 : 1;
     dim3 grid(cdiv(N, 16 * R), cdiv(M, 16 * mt), n_ops);
-#define GK(T, RR) k_gemm_q4_f16_ksplit<T, RR><<<grid, 256, 0, g.stream>>>(act, mw->buf, mw->d16, (const u4q_t*)g_xh_buf, lb, lc, g_scale_buf, M, K, N)
-    if (mt == 1) { if (R == 4) GK(1, 4); else if (R == 2) GK(1, 2); else GK(1, 1); }
-    else { if (R == 4) GK(2, 4); else if (R == 2) GK(2, 2); else GK(2, 1); }
+    // eight waves where the matrix has too few weight rows for larger tiles (measured: no gain otherwise)
+    const uint32_t nwv = mt == 1 ? (uint32_t)tuning("ADAMAH_GEMM_NWV", R == 1 ? 8 : 4) : 4u;
+#define GK(T, RR, W) k_gemm_q4_f16_ksplit<T, RR, W><<<grid, 64 * W, 0, g.stream>>>(act, mw->buf, mw->d16, (const u4q_t*)g_xh_buf, lb, lc, g_scale_buf, M, K, N)
+    if (mt == 1 && nwv >= 8) { if (R == 4) GK(1, 4, 8); else if (R == 2) GK(1, 2, 8); else GK(1, 1, 8); }
+    else if (mt == 1) { if (R == 4) GK(1, 4, 4); else if (R == 2) GK(1, 2, 4); else GK(1, 1, 4); }
+    else { if (R == 4) GK(2, 4, 4); else if (R == 2) GK(2, 2, 4); else GK(2, 1, 4); }
 #undef GK
     count_launch();
     return check_launch();
