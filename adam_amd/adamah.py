@@ -119,6 +119,10 @@ _SIGS = {
     "map_matmul_t_xq8_dev": (i32, [_U] * 9), "map_matmul_xq8_dev": (i32, [_U] * 9),
     "map_row_gather_xq8_dev": (i32, [_U] * 6 + [f32c]),
     "map_matvec_argmax_t_xq4_dev": (i32, [_U] * 10), "map_matvec_argmax_t_xq8_dev": (i32, [_U] * 10),
+    "map_matvec_topk_t_xq4_dev": (i32, [_U] * 11 + [f32c]), "map_matvec_topk_t_xq8_dev": (i32, [_U] * 11 + [f32c]),
+    "map_matvec_topk_t_xq4_ex_dev": (i32, [_U] * 11 + [f32c, _U]),
+    "map_matvec_topk_t_xq8_ex_dev": (i32, [_U] * 11 + [f32c, _U]),
+    "map_matvec_rerank_t_xq8_dev": (i32, [_U] * 12 + [f32c]),
     # timing helpers for benchmarks (HIP events on the library's own stream)
     "adamah_hip_timer_begin": (i32, []), "adamah_hip_timer_end": (f32c, []),
     "adamah_hip_debug_dequant": (i32, [_U, u64, u64, pf32]),
@@ -141,12 +145,15 @@ _OPTIONAL_FLAGS = {
     "map_resolve_idx_dev": "_has_map_resolve_idx_dev",
     "map_sample_categorical_dev": "_has_map_sample_categorical_dev",
     "map_repeat_penalty_dev": "_has_map_repeat_penalty_dev",
+    "map_matvec_topk_t_xq4_dev": "_has_map_matvec_topk_t_xq4_dev",
+    "map_matvec_topk_t_xq4_ex_dev": "_has_map_matvec_topk_t_xq4_ex_dev",
+    "map_matvec_topk_t_xq8_dev": "_has_map_matvec_topk_t_xq8_dev",
+    "map_matvec_topk_t_xq8_ex_dev": "_has_map_matvec_topk_t_xq8_ex_dev",
+    "map_matvec_rerank_t_xq8_dev": "_has_map_matvec_rerank_t_xq8_dev",
 }
-# Present in the reference surface, deliberately absent here: the fused GEMV + top-k / rerank tail,
-# the fused qkv / gate-up entry points, and the monolithic full-decode / device-address API.
+# Present in the reference surface, deliberately absent here: the fused qkv / gate-up entry points
+# and the monolithic full-decode / device-address API.
 _ABSENT_FLAGS = (
-    "_has_map_matvec_topk_t_xq4_dev", "_has_map_matvec_topk_t_xq4_ex_dev",
-    "_has_map_matvec_topk_t_xq8_dev", "_has_map_matvec_topk_t_xq8_ex_dev", "_has_map_matvec_rerank_t_xq8_dev",
     "_has_map_fused_qkv_t_xq4_dev",
     "_has_map_fused_gateup_t_xq4_dev", "_has_map_fused_qkv_t_xq8_dev", "_has_map_fused_gateup_t_xq8_dev",
     "_has_map_fused_gateup_act_t_xq8_dev", "_has_full_decode_step_api", "_has_full_decode_step",
@@ -470,6 +477,35 @@ class Adamah:
 
     def map_repeat_penalty_dev(self, map_id, locs_src_handle, token_ids_handle, n_ids, penalty):
         self._op("map_repeat_penalty_dev", map_id, locs_src_handle, token_ids_handle, n_ids, penalty)
+
+    def map_matvec_topk_t_xq4_dev(self, map_act, map_wt, locs_a_handle, locs_b_handle, penalty_ids_handle,
+                                  locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty=0, repeat_penalty=1.0):
+        self._op("map_matvec_topk_t_xq4_dev", map_act, map_wt, locs_a_handle, locs_b_handle, penalty_ids_handle,
+                 locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty, repeat_penalty)
+
+    def map_matvec_topk_t_xq8_dev(self, map_act, map_wt, locs_a_handle, locs_b_handle, penalty_ids_handle,
+                                  locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty=0, repeat_penalty=1.0):
+        self._op("map_matvec_topk_t_xq8_dev", map_act, map_wt, locs_a_handle, locs_b_handle, penalty_ids_handle,
+                 locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty, repeat_penalty)
+
+    def map_matvec_topk_t_xq4_ex_dev(self, map_act, map_wt, locs_a_handle, locs_b_handle, penalty_ids_handle,
+                                     locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty=0,
+                                     repeat_penalty=1.0, rows_per_group=256):
+        self._op("map_matvec_topk_t_xq4_ex_dev", map_act, map_wt, locs_a_handle, locs_b_handle, penalty_ids_handle,
+                 locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty, repeat_penalty, rows_per_group)
+
+    def map_matvec_topk_t_xq8_ex_dev(self, map_act, map_wt, locs_a_handle, locs_b_handle, penalty_ids_handle,
+                                     locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty=0,
+                                     repeat_penalty=1.0, rows_per_group=256):
+        self._op("map_matvec_topk_t_xq8_ex_dev", map_act, map_wt, locs_a_handle, locs_b_handle, penalty_ids_handle,
+                 locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty, repeat_penalty, rows_per_group)
+
+    def map_matvec_rerank_t_xq8_dev(self, map_act, map_wt, locs_a_handle, locs_b_handle, partial_idx_base_handle,
+                                    sel_locs_handle, penalty_ids_handle, locs_idx_dst_handle, locs_val_dst_handle,
+                                    K, n_ids, n_penalty=0, repeat_penalty=1.0):
+        self._op("map_matvec_rerank_t_xq8_dev", map_act, map_wt, locs_a_handle, locs_b_handle,
+                 partial_idx_base_handle, sel_locs_handle, penalty_ids_handle, locs_idx_dst_handle,
+                 locs_val_dst_handle, K, n_ids, n_penalty, repeat_penalty)
 
     def map_matvec_argmax_t_xq4_dev(self, map_act, map_wt, locs_a_handle, locs_b_handle, locs_idx_tmp_handle,
                                     locs_val_tmp_handle, locs_dst_handle, K, N, rows_per_group):

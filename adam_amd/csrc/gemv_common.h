@@ -38,6 +38,13 @@ __device__ __forceinline__ float gelu_tanh(float a) {
   return 0.5f * a * (1.0f + tanhf(0.797884583f * (a + 0.0447149985f * a * a * a)));
 }
 
+// One quantised element of a map, affine form: code * scale + zero point of its group.
+__device__ __forceinline__ float deq_elem(const uint8_t* W, const float2* qp, uint64_t idx, uint32_t group, bool q4) {
+  uint32_t code = q4 ? ((W[idx >> 1] >> ((idx & 1u) * 4u)) & 0xFu) : W[idx];
+  float2 p = qp[idx / group];
+  return __fadd_rn(__fmul_rn((float)code, p.x), p.y);
+}
+
 #define DPP_ADD(v, ctrl, rmask)                                                                    \
   v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, rmask, 0xF, false))
 
@@ -90,8 +97,9 @@ struct GemvFuse {
 };
 // Threads per workgroup the launchers will use for a matrix with N rows (store variant).
 uint32_t mfma_store_threads(uint32_t K, uint32_t N);
+// `out` (optional): the result rows go to out[c + row] instead of the activation map.
 int launch_mfma_store(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32_t b, uint32_t c, uint32_t K,
-                      uint32_t N, const GemvFuse* fz = nullptr);
+                      uint32_t N, const GemvFuse* fz = nullptr, float* out = nullptr);
 int launch_mfma_argmax(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32_t b, const uint32_t* lidx,
                        const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rows_per_group,
                        const GemvFuse* fz = nullptr);
@@ -103,5 +111,11 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
 int launch_argmax_pairs(const Map* ma, const uint32_t* lidx, const uint32_t* lval, const uint32_t* ldst,
                         uint32_t n_groups);
 int tuning(const char* name, int dflt);
+// Preconditions of the block kernels, checked against the host copies of the handles: group size 32,
+// K a multiple of 32, weight base block aligned, operands in range.  Returns the two element offsets.
+bool block_path_ok(const Map* ma, const Map* mw, uint32_t ha, uint32_t hb, uint32_t K, uint32_t N, uint64_t* a_out,
+                   uint64_t* b_out);
+// Storage format (FMT_*) of the weights [b, b + n_w) of a quantised map.
+int fmt_of(const Map* mw, uint64_t b, uint64_t n_w);
 
 }  // namespace adamah

@@ -516,12 +516,13 @@ bool mfma_path_ok(const Map* mw, uint32_t K) {
 template <int EPI, int PRO>
 static void launch_mfma_p(int fmt, uint32_t grid, uint32_t threads, const Map* ma, const Map* mw, uint32_t a, uint32_t b,
                           uint32_t c, const uint32_t* lidx, const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rpg,
-                          uint32_t n_groups, uint32_t ks, const GemvFuse& fz) {
+                          uint32_t n_groups, uint32_t ks, const GemvFuse& fz, float* out) {
   float* act = (float*)ma->buf;
+  float* act_out = out ? out : act;
   const size_t smem = mfma_smem(K);
   const bool ragged = (K & 2047u) != 0;
 #define MK(F, R)                                                                                                  \
-  k_gemv_mfma<F, EPI, R, PRO><<<grid, threads, smem, g.stream>>>(act, act, mw->buf, mw->qp, mw->d16, a, b, c, lidx, \
+  k_gemv_mfma<F, EPI, R, PRO><<<grid, threads, smem, g.stream>>>(act, act_out, mw->buf, mw->qp, mw->d16, a, b, c, lidx, \
                                                                  lval, K, N, rpg, n_groups, ks, fz)
   if (fmt == FMT_Q4_B16) { if (ragged) MK(FMT_Q4_B16, true); else MK(FMT_Q4_B16, false); }
   else { if (ragged) MK(FMT_Q4_AFF, true); else MK(FMT_Q4_AFF, false); }
@@ -531,12 +532,12 @@ static void launch_mfma_p(int fmt, uint32_t grid, uint32_t threads, const Map* m
 template <int EPI>
 static int launch_mfma(int fmt, uint32_t grid, uint32_t threads, const Map* ma, const Map* mw, uint32_t a, uint32_t b,
                        uint32_t c, const uint32_t* lidx, const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rpg,
-                       uint32_t n_groups, uint32_t ks, const GemvFuse* fzp) {
+                       uint32_t n_groups, uint32_t ks, const GemvFuse* fzp, float* out = nullptr) {
   GemvFuse fz = {};
   if (fzp) fz = *fzp;
   const int xf = tuning("ADAMAH_MFMA_XFIRST", -1);
   fz.x_first = xf < 0 ? 1u : (uint32_t)(xf != 0);
-#define MP(P) launch_mfma_p<EPI, P>(fmt, grid, threads, ma, mw, a, b, c, lidx, lval, K, N, rpg, n_groups, ks, fz)
+#define MP(P) launch_mfma_p<EPI, P>(fmt, grid, threads, ma, mw, a, b, c, lidx, lval, K, N, rpg, n_groups, ks, fz, out)
   switch (fz.pro) {
     case PRO_RMSNORM: MP(PRO_RMSNORM); break;
     case PRO_NORM2: MP(PRO_NORM2); break;
@@ -591,12 +592,12 @@ uint32_t mfma_store_threads(uint32_t K, uint32_t N) {
 }
 
 int launch_mfma_store(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32_t b, uint32_t c, uint32_t K,
-                      uint32_t N, const GemvFuse* fz) {
+                      uint32_t N, const GemvFuse* fz, float* out) {
   uint32_t grid, threads;
   const bool paired = fz && (fz->e_mode == EPIX_GEGLU || fz->e_mode == EPIX_SWIGLU);
   const uint32_t ks = mfma_ksplit(K, N, paired);
   mfma_store_shape(K, N, ks, &grid, &threads);
-  return launch_mfma<EPI_STORE>(fmt, grid, threads, ma, mw, a, b, c, nullptr, nullptr, K, N, 0, 0, ks, fz);
+  return launch_mfma<EPI_STORE>(fmt, grid, threads, ma, mw, a, b, c, nullptr, nullptr, K, N, 0, 0, ks, fz, out);
 }
 
 int launch_mfma_argmax(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32_t b, const uint32_t* lidx,

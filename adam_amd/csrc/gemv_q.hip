@@ -301,12 +301,6 @@ k_gemv_regx(const float* act, float* act_out, const uint8_t* __restrict__ W, con
 }
 
 // ---- generic path: any K, N, M, n_ops, base offset, group size; one wave per output ------------
-__device__ __forceinline__ float deq_elem(const uint8_t* W, const float2* qp, uint64_t idx, uint32_t group, bool q4) {
-  uint32_t code = q4 ? ((W[idx >> 1] >> ((idx & 1u) * 4u)) & 0xFu) : W[idx];
-  float2 p = qp[idx / group];
-  return __fadd_rn(__fmul_rn((float)code, p.x), p.y);
-}
-
 template <bool Q4, bool TRANSPOSED>
 __global__ void __launch_bounds__(256)
 k_matmul_xq_generic(const float* act, float* out, const uint8_t* __restrict__ W,
@@ -425,7 +419,7 @@ struct XqArgs {
 };
 
 // Block-kernel preconditions, checked against the host copies of the handles.
-static bool block_path_ok(const Map* ma, const Map* mw, uint32_t ha, uint32_t hb, uint32_t K, uint32_t N,
+bool block_path_ok(const Map* ma, const Map* mw, uint32_t ha, uint32_t hb, uint32_t K, uint32_t N,
                           uint64_t* a_out, uint64_t* b_out) {
   if (mw->group_size != 32 || mw->pack_size != 1 || ma->pack_size != 1) return false;
   if (K == 0 || (K & 31u) || K > 16384) return false;
@@ -438,7 +432,7 @@ static bool block_path_ok(const Map* ma, const Map* mw, uint32_t ha, uint32_t hb
   return true;
 }
 
-static int fmt_of(const Map* mw, uint64_t b, uint64_t n_w) {
+int fmt_of(const Map* mw, uint64_t b, uint64_t n_w) {
   const bool q4 = mw->dtype == DTYPE_Q4;
   const bool b16 = (b + n_w + 31) / 32 <= mw->block16_groups;
   return q4 ? (b16 ? FMT_Q4_B16 : FMT_Q4_AFF) : (b16 ? FMT_Q8_B16 : FMT_Q8_AFF);

@@ -368,6 +368,7 @@ void adamah_shutdown(void) { ADAMAH_API();
   if (g.sync_ctr) hipFree(g.sync_ctr);
   g.sync_ctr = nullptr;
   gemm_q4_mfma_release();
+  topk_fused_release();
   g.pend.clear();
   for (int i = 0; i < MAX_PLANS; i++) { g.plans[i].clear(); g.plan_active[i] = false; }
   hipStreamDestroy(g.stream);

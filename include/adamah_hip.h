@@ -126,6 +126,29 @@ int map_sample_categorical_dev(uint32_t map_id, uint32_t locs_idx, uint32_t locs
                                uint32_t dst_loc, uint32_t n); /* adamah.c:7286 (n <= 64) */
 int map_repeat_penalty_dev(uint32_t map_id, uint32_t locs_src, uint32_t token_ids, uint32_t n_ids,
                            float penalty);                    /* adamah.c:6787 (n_ids <= 64) */
+/* Logits of a quantised [N, K] matrix reduced to a sorted partial top-k list per group of
+ * rows_per_group rows (256 in the forms without _ex); rows listed in penalty_ids get the repeat
+ * penalty before ranking.  locs_idx_dst / locs_val_dst hold ceil(N / rows_per_group) * k entries.
+ * k <= 64, n_penalty <= 64. */
+int map_matvec_topk_t_xq4_dev(uint32_t map_act, uint32_t map_wt, uint32_t locs_a, uint32_t locs_b,
+                              uint32_t penalty_ids, uint32_t locs_idx_dst, uint32_t locs_val_dst, uint32_t K,
+                              uint32_t N, uint32_t k, uint32_t n_penalty, float repeat_penalty); /* adamah.c:9816 */
+int map_matvec_topk_t_xq4_ex_dev(uint32_t map_act, uint32_t map_wt, uint32_t locs_a, uint32_t locs_b,
+                                 uint32_t penalty_ids, uint32_t locs_idx_dst, uint32_t locs_val_dst, uint32_t K,
+                                 uint32_t N, uint32_t k, uint32_t n_penalty, float repeat_penalty,
+                                 uint32_t rows_per_group);    /* adamah.c:9727 */
+int map_matvec_topk_t_xq8_dev(uint32_t map_act, uint32_t map_wt, uint32_t locs_a, uint32_t locs_b,
+                              uint32_t penalty_ids, uint32_t locs_idx_dst, uint32_t locs_val_dst, uint32_t K,
+                              uint32_t N, uint32_t k, uint32_t n_penalty, float repeat_penalty); /* adamah.c:10000 */
+int map_matvec_topk_t_xq8_ex_dev(uint32_t map_act, uint32_t map_wt, uint32_t locs_a, uint32_t locs_b,
+                                 uint32_t penalty_ids, uint32_t locs_idx_dst, uint32_t locs_val_dst, uint32_t K,
+                                 uint32_t N, uint32_t k, uint32_t n_penalty, float repeat_penalty,
+                                 uint32_t rows_per_group);    /* adamah.c:9911 */
+/* Exact logits of n_ids <= 64 shortlisted rows: row = act[partial_idx_base[0] + uint(act[sel_locs[i]])]. */
+int map_matvec_rerank_t_xq8_dev(uint32_t map_act, uint32_t map_wt, uint32_t locs_a, uint32_t locs_b,
+                                uint32_t partial_idx_base, uint32_t sel_locs, uint32_t penalty_ids,
+                                uint32_t locs_idx_dst, uint32_t locs_val_dst, uint32_t K, uint32_t n_ids,
+                                uint32_t n_penalty, float repeat_penalty); /* adamah.c:10018 */
 
 /* ---- decode hot path ----------------------------------------------------------------------- */
 int map_rmsnorm_dev(uint32_t map_id, uint32_t locs_src, uint32_t locs_wt, uint32_t locs_dst,

@@ -934,6 +934,96 @@ class NumpyAdamah:
         self._matvec_argmax("map_matvec_argmax_t_xq8_dev", DTYPE_Q8, map_act, map_wt, locs_a_handle, locs_b_handle,
                             locs_idx_tmp_handle, locs_val_tmp_handle, locs_dst_handle, K, N, rows_per_group)
 
+    # ---- fused GEMV + partial top-k, shortlist rerank -----------------------------------------
+    def _matvec_topk(self, fn, dtype, map_act, map_wt, la_h, lb_h, pen_h, idx_h, val_h, K, N, k, n_pen, rp, rpg):
+        """shaders/src/f32/map_matvec_topk_t_xq4.comp:108-208 (Q8 twin map_matvec_topk_t_xq8.comp), dispatch
+        adamah.c:9727-9830 / :9911-10016: per group of rows_per_group rows, logits -> repeat penalty on the
+        rows listed in penalty_ids (value > 0 ? value / p : value * p, membership test, so once per row) ->
+        list of k = min(k, 64) entries sorted by (value descending, row ascending); slots the group cannot
+        fill hold index 0 and -FLT_MAX."""
+        self.op_count += 1
+        ma = self._map(fn, map_act, DTYPE_F32); mw = self._map(fn, map_wt, dtype)
+        if N == 0 or k == 0:
+            return
+        if k > 64 or n_pen > 64 or rpg == 0 or mw.scale is None:
+            self._fail(fn, ERR_INVALID)
+        ng = (N + rpg - 1) // rpg
+        il = self._locs(fn, idx_h, ng * k); vl = self._locs(fn, val_h, ng * k)
+        self._h(fn, pen_h)
+        pen = set(int(t) for t in self._locs(fn, pen_h, n_pen)) if n_pen else set()
+        a = int(self._locs(fn, la_h, 1)[0]); b = int(self._locs(fn, lb_h, 1)[0])
+        self._chk(fn, ma, a, a + K); self._chk(fn, mw, b, b + N * K)
+        y = (mw.deq_range(b, N * K).reshape(N, K).astype(np.float64) @ ma.data[a:a + K].astype(np.float64)).astype(np.float32)
+        rp = f32(rp)
+        for r in pen:
+            if r < N:
+                y[r] = y[r] / rp if y[r] > 0 else y[r] * rp
+        for g in range(ng):
+            rows = np.arange(g * rpg, min(N, (g + 1) * rpg))
+            order = sorted(rows.tolist(), key=lambda r: (-float(y[r]), r))[:k]
+            for t in range(k):
+                if t < len(order):
+                    ma.data[il[g * k + t]] = f32(order[t]); ma.data[vl[g * k + t]] = y[order[t]]
+                else:
+                    ma.data[il[g * k + t]] = 0.0; ma.data[vl[g * k + t]] = NEG_MAX
+        self.last_logits = y
+
+    def map_matvec_topk_t_xq4_dev(self, map_act, map_wt, locs_a_handle, locs_b_handle, penalty_ids_handle,
+                                  locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty=0, repeat_penalty=1.0):
+        self._matvec_topk("map_matvec_topk_t_xq4_dev", DTYPE_Q4, map_act, map_wt, locs_a_handle, locs_b_handle,
+                          penalty_ids_handle, locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty,
+                          repeat_penalty, 256)
+
+    def map_matvec_topk_t_xq8_dev(self, map_act, map_wt, locs_a_handle, locs_b_handle, penalty_ids_handle,
+                                  locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty=0, repeat_penalty=1.0):
+        self._matvec_topk("map_matvec_topk_t_xq8_dev", DTYPE_Q8, map_act, map_wt, locs_a_handle, locs_b_handle,
+                          penalty_ids_handle, locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty,
+                          repeat_penalty, 256)
+
+    def map_matvec_topk_t_xq4_ex_dev(self, map_act, map_wt, locs_a_handle, locs_b_handle, penalty_ids_handle,
+                                     locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty=0,
+                                     repeat_penalty=1.0, rows_per_group=256):
+        self._matvec_topk("map_matvec_topk_t_xq4_ex_dev", DTYPE_Q4, map_act, map_wt, locs_a_handle, locs_b_handle,
+                          penalty_ids_handle, locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty,
+                          repeat_penalty, rows_per_group)
+
+    def map_matvec_topk_t_xq8_ex_dev(self, map_act, map_wt, locs_a_handle, locs_b_handle, penalty_ids_handle,
+                                     locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty=0,
+                                     repeat_penalty=1.0, rows_per_group=256):
+        self._matvec_topk("map_matvec_topk_t_xq8_ex_dev", DTYPE_Q8, map_act, map_wt, locs_a_handle, locs_b_handle,
+                          penalty_ids_handle, locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty,
+                          repeat_penalty, rows_per_group)
+
+    def map_matvec_rerank_t_xq8_dev(self, map_act, map_wt, locs_a_handle, locs_b_handle, partial_idx_base_handle,
+                                    sel_locs_handle, penalty_ids_handle, locs_idx_dst_handle, locs_val_dst_handle,
+                                    K, n_ids, n_penalty=0, repeat_penalty=1.0):
+        """shaders/src/f32/map_matvec_rerank_t_xq8.comp:43-82 (dispatch adamah.c:10018-10110): for each of the
+        n_ids <= 64 shortlist slots, token = uint(act[partial_base + uint(act[sel_locs[i]])]), value = exact
+        logit of that row (with the repeat penalty when the token is listed); stores float(token), value."""
+        self.op_count += 1
+        fn = "map_matvec_rerank_t_xq8_dev"
+        ma = self._map(fn, map_act, DTYPE_F32); mw = self._map(fn, map_wt, DTYPE_Q8)
+        if n_ids == 0:
+            return
+        if n_ids > 64 or n_penalty > 64 or mw.scale is None:
+            self._fail(fn, ERR_INVALID)
+        a = int(self._locs(fn, locs_a_handle, 1)[0]); b = int(self._locs(fn, locs_b_handle, 1)[0])
+        pb = int(self._locs(fn, partial_idx_base_handle, 1)[0])
+        sel = self._locs(fn, sel_locs_handle, n_ids)
+        il = self._locs(fn, locs_idx_dst_handle, n_ids); vl = self._locs(fn, locs_val_dst_handle, n_ids)
+        self._h(fn, penalty_ids_handle)
+        pen = set(int(t) for t in self._locs(fn, penalty_ids_handle, n_penalty)) if n_penalty else set()
+        self._chk(fn, ma, a, a + K)
+        x = ma.data[a:a + K].astype(np.float64)
+        rp = f32(repeat_penalty)
+        for i in range(n_ids):
+            tok = int(ma.data[pb + int(ma.data[sel[i]])])
+            self._chk(fn, mw, b + tok * K, b + (tok + 1) * K)
+            v = f32(mw.deq_range(b + tok * K, K).astype(np.float64) @ x)
+            if tok in pen:
+                v = v / rp if v > 0 else v * rp
+            ma.data[il[i]] = f32(tok); ma.data[vl[i]] = v
+
 
 def init(cache_mb=None, cold_cache_mb=None):
     return NumpyAdamah()

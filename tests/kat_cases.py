@@ -278,7 +278,64 @@ def kat_resolve_idx_and_categorical(g, A):
     assert int(_read(g, 12, [21])[0]) == 11
 
 
+def _diag_q8(g, A, map_id):
+    """Q8 rows [1,0,0,0], [0,2,0,0], [0,0,3,0], [0,0,0,4]: codes 128 + value, scale 1, zero point -128."""
+    g.map_create_typed(map_id, A.DTYPE_Q8, 1, 16, 4)
+    g.set_qparams(map_id, np.ones(4, np.float32), np.full(4, -128.0, np.float32))
+    raw = np.full(16, 128, np.uint8)
+    raw[[0, 5, 10, 15]] = [129, 130, 131, 132]
+    g.scatter(map_id, np.arange(16, dtype=np.uint32), raw)
+
+
+def kat_matvec_topk_t_xq8(g, A):
+    """:217-257: logits [1, 2, 3, 4] of a ones vector, repeat penalty 2 on row 3 (4 -> 2), k = 2:
+    [2, 1] with values [3, 2] (the tie at 2.0 goes to the lower row)."""
+    _diag_q8(g, A, 7)
+    _f32map(g, A, 8, 16)
+    g.scatter(8, np.arange(4, dtype=np.uint32), np.ones(4, np.float32))
+    idx_h, val_h = _h(g, [4, 5]), _h(g, [8, 9])
+    g.batch_begin()
+    g.map_matvec_topk_t_xq8_dev(8, 7, _h(g, [0, 1, 2, 3]), _h(g, [0]), _h(g, [3]), idx_h, val_h, 4, 4, 2, 1, 2.0)
+    g.batch_end()
+    assert _read(g, 8, [4, 5]).astype(np.int32).tolist() == [2, 1]
+    assert np.allclose(_read(g, 8, [8, 9]), [3.0, 2.0], atol=1e-5)
+
+
+def kat_matvec_topk_t_xq4(g, A):
+    """:260-301: the same through Q4 weights quantised on the device (scale 4/15): first index 2, second
+    1 or 3, values [3, 2] within 0.15."""
+    g.map_create_typed(13, A.DTYPE_Q4, 1, 16, 32)
+    g.set_qparams(13, np.array([4.0 / 15.0], np.float32), np.array([0.0], np.float32))
+    g.scatter(13, np.arange(16, dtype=np.uint32), np.diag([1.0, 2.0, 3.0, 4.0]).astype(np.float32).reshape(-1))
+    _f32map(g, A, 14, 16)
+    g.scatter(14, np.arange(4, dtype=np.uint32), np.ones(4, np.float32))
+    idx_h, val_h = _h(g, [4, 5]), _h(g, [8, 9])
+    g.batch_begin()
+    g.map_matvec_topk_t_xq4_dev(14, 13, _h(g, [0, 1, 2, 3]), _h(g, [0]), _h(g, [3]), idx_h, val_h, 4, 4, 2, 1, 2.0)
+    g.batch_end()
+    idx = _read(g, 14, [4, 5]).astype(np.int32)
+    assert idx[0] == 2 and idx[1] in (1, 3)
+    assert np.allclose(_read(g, 14, [8, 9]), [3.0, 2.0], atol=0.15)
+
+
+def kat_matvec_rerank_t_xq8(g, A):
+    """:304-352: partial id list [0, 1, 2, 3] at 8.., shortlist positions [3, 1]; exact logits 4 and 2, the
+    penalty 2 on token 3 -> ids [3, 1], values [2, 2]."""
+    _diag_q8(g, A, 13)
+    _f32map(g, A, 14, 32)
+    vals = np.zeros(32, np.float32)
+    vals[0:4] = 1.0; vals[8:12] = [0.0, 1.0, 2.0, 3.0]; vals[12:14] = [3.0, 1.0]
+    g.scatter(14, np.arange(32, dtype=np.uint32), vals)
+    idx_h, val_h = _h(g, [16, 17]), _h(g, [20, 21])
+    g.batch_begin()
+    g.map_matvec_rerank_t_xq8_dev(14, 13, _h(g, [0, 1, 2, 3]), _h(g, [0]), _h(g, [8]), _h(g, [12, 13]), _h(g, [3]),
+                                  idx_h, val_h, 4, 2, 1, 2.0)
+    g.batch_end()
+    assert _read(g, 14, [16, 17]).astype(np.int32).tolist() == [3, 1]
+    assert np.allclose(_read(g, 14, [20, 21]), [2.0, 2.0], atol=1e-5)
+
+
 ALL = [kat_argmax, kat_topk, kat_topp, kat_resolve_idx_and_categorical, kat_softmax_abs, kat_attn_softmax_abs, kat_q8_gather_scatter, kat_row_gather_xq8,
        kat_matvec_t_xq8, kat_matvec_t_xq4, kat_q4_matmul_identity, kat_batch_gather_scatter,
        kat_row_copy_offset, kat_fusion_row_copy_then_matmul, kat_scalar_state, kat_fusion_batch_order,
-       kat_decode_plan_runtime_args]
+       kat_decode_plan_runtime_args, kat_matvec_topk_t_xq8, kat_matvec_topk_t_xq4, kat_matvec_rerank_t_xq8]

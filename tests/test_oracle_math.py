@@ -412,3 +412,72 @@ def test_resolve_idx_guards():
     _sampling_map(g, vals)
     g.map_resolve_idx_dev(2, up(g, [4]), up(g, [8, 9, 10, 11, 12]), up(g, 16 + np.arange(5)), 5)
     assert read(g, 2, 16, 5).tolist() == [44.0, 0.0, 0.0, 11.0, 11.0]
+
+
+# ---------------------------------------------------------------- GEMV + partial top-k, rerank
+def _load_q(g, mid, qt):
+    dt = A.DTYPE_Q4 if qt.kind == "q4_0" else A.DTYPE_Q8
+    g.map_create_typed(mid, dt, 1, qt.size, 32)
+    g.set_qparams(mid, *qt.qparams())
+    if qt.kind == "q4_0":
+        g.scatter_q4_packed_contiguous(mid, 0, qt.codes)
+    else:
+        g.scatter_contiguous(mid, 0, qt.codes)
+
+
+@pytest.mark.parametrize("dtype", ["q4", "q8"])
+def test_matvec_topk_equals_insertion_into_a_sorted_list(dtype):
+    """Independent statement of the list the shader builds: rows visited in order, each inserted before
+    the first entry it beats (value greater, or equal with a smaller row), list cut at k."""
+    rng = np.random.default_rng(12)
+    N, K, k, rpg = 50, 64, 6, 16                               # last group has 2 rows < k
+    w = rng.standard_normal((N, K)).astype(np.float32)
+    w[21] = w[18]                                              # exact tie inside group 1
+    qt = quant.quantize_q4_0(w) if dtype == "q4" else quant.quantize_q8_0(w)
+    x = rng.standard_normal(K).astype(np.float32)
+    y = (qt.dequant().astype(np.float64) @ x.astype(np.float64)).astype(np.float32)
+    pen, rp = [18, 3, 3, 49, 77], np.float32(1.5)              # a duplicate and an id past N
+    for r in set(pen):
+        if r < N:
+            y[r] = y[r] / rp if y[r] > 0 else y[r] * rp
+    g = oracle.init()
+    _load_q(g, 1, qt)
+    ng = (N + rpg - 1) // rpg
+    f32map(g, 0, K + 2 * ng * k + 8, x)
+    fn = g.map_matvec_topk_t_xq4_ex_dev if dtype == "q4" else g.map_matvec_topk_t_xq8_ex_dev
+    fn(0, 1, up(g, [0]), up(g, [0]), up(g, pen), up(g, K + np.arange(ng * k)), up(g, K + ng * k + np.arange(ng * k)),
+       K, N, k, len(pen), float(rp), rpg)
+    idx = read(g, 0, K, ng * k).reshape(ng, k); val = read(g, 0, K + ng * k, ng * k).reshape(ng, k)
+    for gi in range(ng):
+        lst = []
+        for r in range(gi * rpg, min(N, (gi + 1) * rpg)):
+            pos = len(lst)
+            for i, (v, j) in enumerate(lst):
+                if y[r] > v or (y[r] == v and r < j):
+                    pos = i
+                    break
+            lst.insert(pos, (y[r], r))
+            lst = lst[:k]
+        for t in range(k):
+            if t < len(lst):
+                assert idx[gi, t] == lst[t][1] and val[gi, t] == lst[t][0]
+            else:
+                assert idx[gi, t] == 0 and val[gi, t] == np.float32(-3.402823466e+38)
+
+
+def test_rerank_equals_row_dot_products():
+    rng = np.random.default_rng(13)
+    N, K = 40, 64
+    qt = quant.quantize_q8_0(rng.standard_normal((N, K)).astype(np.float32))
+    x = rng.standard_normal(K).astype(np.float32)
+    y = qt.dequant().astype(np.float64) @ x.astype(np.float64)
+    partial = np.array([7, 39, 0, 12, 12, 5], np.float32); sel = np.array([4, 1, 0, 5], np.float32)
+    g = oracle.init()
+    _load_q(g, 2, qt)
+    f32map(g, 0, K + 64, np.concatenate([x, partial, sel]))
+    g.map_matvec_rerank_t_xq8_dev(0, 2, up(g, [0]), up(g, [0]), up(g, [K]), up(g, K + 6 + np.arange(4)), up(g, [39, 5]),
+                                  up(g, K + 20 + np.arange(4)), up(g, K + 30 + np.arange(4)), K, 4, 2, 2.0)
+    toks = read(g, 0, K + 20, 4).astype(int).tolist(); vals = read(g, 0, K + 30, 4)
+    assert toks == [12, 39, 7, 5]
+    exp = [y[12], y[39] / 2 if y[39] > 0 else y[39] * 2, y[7], y[5] / 2 if y[5] > 0 else y[5] * 2]
+    assert np.allclose(vals, np.array(exp, np.float32), rtol=1e-6)
