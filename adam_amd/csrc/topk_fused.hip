@@ -11,7 +11,10 @@
 // Here the dot products run on the ordinary GEMV kernels into a scratch vector owned by the library
 // (the int8 matrix-instruction kernel for Q4 block matrices, one wave per row otherwise); a second
 // launch ranks every group.  The ranking order is the reference's: larger value first, equal values
-// by smaller row index; slots a group cannot fill hold index 0 and the most negative float.
+// by smaller row index; slots a group cannot fill hold index 0 and the most negative float.  A NaN
+// logit ranks as the most negative float (the reference's insertion leaves a NaN wherever it was
+// first put, which no caller relies on).  Groups of up to 1024 rows are ranked by counting, for every
+// row, the rows that beat it; larger groups by k rounds of a workgroup-wide best-of.
 #include "gemv_common.h"
 #include "../../include/adamah_hip.h"
 
@@ -74,7 +77,8 @@ k_group_topk(float* act, float* logits, const uint32_t* __restrict__ pen, const 
     float bv = NEG_FLT_MAX;
     uint32_t bi = INVALID_IDX;
     for (uint32_t r = row0 + tid; r < row1; r += 256u) {
-      const float v = logits[r];
+      float v = logits[r];
+      if (v != v) v = NEG_FLT_MAX;
       const bool after = t == 0u || (pi != INVALID_IDX && ((pv > v) || (pv == v && pi < r)));
       if (after && better(v, r, bv, bi)) { bv = v; bi = r; }
     }
@@ -106,6 +110,55 @@ k_group_topk(float* act, float* logits, const uint32_t* __restrict__ pen, const 
         }
       break;
     }
+  }
+}
+
+// Groups of at most 1024 rows: the group's (penalised) logits sit in LDS, every thread counts the rows
+// that rank before its own and stores those with fewer than k of them straight into their slot.
+#define RANK_MAX 1024u
+__global__ void __launch_bounds__(256)
+k_group_topk_rank(float* act, const float* __restrict__ logits, const uint32_t* __restrict__ pen,
+                  const uint32_t* __restrict__ lidx, const uint32_t* __restrict__ lval, uint32_t N, uint32_t k,
+                  uint32_t n_pen, float rp, uint32_t rows_per_group, uint64_t act_elems) {
+  __shared__ float vs[RANK_MAX];
+  __shared__ uint32_t pen_s[TOPK_MAX];
+  const uint32_t tid = threadIdx.x, grp = blockIdx.x;
+  const uint32_t row0 = grp * rows_per_group, rows = min(N, row0 + rows_per_group) - row0;
+  for (uint32_t i = tid; i < rows; i += 256u) {
+    const float v = logits[row0 + i];
+    vs[i] = v != v ? NEG_FLT_MAX : v;
+  }
+  // padding of the last quad: NaN compares false both ways, so it is never counted
+  for (uint32_t i = rows + tid; i < ((rows + 3u) & ~3u); i += 256u) vs[i] = __uint_as_float(0x7FC00000u);
+  if (tid < n_pen) pen_s[tid] = pen[tid];
+  __syncthreads();
+  if (tid < n_pen) {
+    const uint32_t id = pen_s[tid];
+    bool first = id >= row0 && id - row0 < rows;
+    for (uint32_t j = 0; j < tid; j++) first = first && pen_s[j] != id;
+    if (first) vs[id - row0] = penalised(vs[id - row0], rp);
+  }
+  __syncthreads();
+  for (uint32_t i = tid; i < rows; i += 256u) {
+    const float v = vs[i];
+    uint32_t cnt = 0;
+    for (uint32_t j = 0; j < rows; j += 4u) {   // branch-free: rows before i win ties
+      const float4 w = *(const float4*)&vs[j];
+      cnt += (uint32_t)(w.x > v) | ((uint32_t)(w.x == v) & (uint32_t)(j < i));
+      cnt += (uint32_t)(w.y > v) | ((uint32_t)(w.y == v) & (uint32_t)(j + 1u < i));
+      cnt += (uint32_t)(w.z > v) | ((uint32_t)(w.z == v) & (uint32_t)(j + 2u < i));
+      cnt += (uint32_t)(w.w > v) | ((uint32_t)(w.w == v) & (uint32_t)(j + 3u < i));
+    }
+    if (cnt < k) {
+      const uint64_t di = lidx[(uint64_t)grp * k + cnt], dv = lval[(uint64_t)grp * k + cnt];
+      if (di < act_elems) act[di] = (float)(row0 + i);
+      if (dv < act_elems) act[dv] = v;
+    }
+  }
+  for (uint32_t t = rows + tid; t < k; t += 256u) {   // slots the group cannot fill
+    const uint64_t di = lidx[(uint64_t)grp * k + t], dv = lval[(uint64_t)grp * k + t];
+    if (di < act_elems) act[di] = 0.f;
+    if (dv < act_elems) act[dv] = NEG_FLT_MAX;
   }
 }
 
@@ -180,8 +233,15 @@ static int op_matvec_topk(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uin
     r = check_launch();
   }
   if (r) return r;
-  k_group_topk<<<n_groups, 256, 0, g.stream>>>(act, g_logit_buf, pen, lidx, lval, N, k, n_pen, rp, rows_per_group,
-                                               ma->n_elems);
+  // counting costs rows^2 / 256 comparisons per thread, the rounds k * (rows / 256 + a reduction)
+  const uint64_t rws = std::min(rows_per_group, N);
+  const bool by_rank = rows_per_group <= RANK_MAX && rws * rws / 256u <= (uint64_t)k * (rws / 256u + 40u);
+  if (tuning("ADAMAH_TOPK_RANK", by_rank ? 1 : 0) != 0 && rows_per_group <= RANK_MAX)
+    k_group_topk_rank<<<n_groups, 256, 0, g.stream>>>(act, g_logit_buf, pen, lidx, lval, N, k, n_pen, rp,
+                                                      rows_per_group, ma->n_elems);
+  else
+    k_group_topk<<<n_groups, 256, 0, g.stream>>>(act, g_logit_buf, pen, lidx, lval, N, k, n_pen, rp, rows_per_group,
+                                                 ma->n_elems);
   count_launch();
   return check_launch();
 }

@@ -940,7 +940,8 @@ class NumpyAdamah:
         adamah.c:9727-9830 / :9911-10016: per group of rows_per_group rows, logits -> repeat penalty on the
         rows listed in penalty_ids (value > 0 ? value / p : value * p, membership test, so once per row) ->
         list of k = min(k, 64) entries sorted by (value descending, row ascending); slots the group cannot
-        fill hold index 0 and -FLT_MAX."""
+        fill hold index 0 and -FLT_MAX.  A NaN logit ranks as -FLT_MAX (the shader's insertion would leave it
+        wherever it was first put)."""
         self.op_count += 1
         ma = self._map(fn, map_act, DTYPE_F32); mw = self._map(fn, map_wt, dtype)
         if N == 0 or k == 0:
@@ -955,6 +956,7 @@ class NumpyAdamah:
         self._chk(fn, ma, a, a + K); self._chk(fn, mw, b, b + N * K)
         y = (mw.deq_range(b, N * K).reshape(N, K).astype(np.float64) @ ma.data[a:a + K].astype(np.float64)).astype(np.float32)
         rp = f32(rp)
+        y[np.isnan(y)] = NEG_MAX
         for r in pen:
             if r < N:
                 y[r] = y[r] / rp if y[r] > 0 else y[r] * rp

@@ -59,6 +59,8 @@ def check(hip_out, ora, N, k, rpg):
     ("q4", 4096, 4096, 64, 1000, 64),    # rows_per_group that does not divide N, full penalty list
     ("q4", 300, 4096, 8, 512, 0),        # one group
     ("q4", 70, 256, 64, 32, 3),          # groups shorter than k: empty slots
+    ("q4", 4100, 256, 12, 2048, 4),      # groups above 1024 rows: ranked in rounds
+    ("q8", 3000, 128, 64, 1500, 0),
     ("q8", 777, 256, 16, 100, 7),
     ("q8", 2048, 1152, 1, 256, 2),
 ])
