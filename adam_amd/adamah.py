@@ -123,6 +123,9 @@ _SIGS = {
     "map_matvec_topk_t_xq4_ex_dev": (i32, [_U] * 11 + [f32c, _U]),
     "map_matvec_topk_t_xq8_ex_dev": (i32, [_U] * 11 + [f32c, _U]),
     "map_matvec_rerank_t_xq8_dev": (i32, [_U] * 12 + [f32c]),
+    "map_fused_qkv_t_xq4_dev": (i32, [_U] * 13), "map_fused_qkv_t_xq8_dev": (i32, [_U] * 13),
+    "map_fused_gateup_t_xq4_dev": (i32, [_U] * 10), "map_fused_gateup_t_xq8_dev": (i32, [_U] * 10),
+    "map_fused_gateup_act_t_xq8_dev": (i32, [_U] * 8),
     # timing helpers for benchmarks (HIP events on the library's own stream)
     "adamah_hip_timer_begin": (i32, []), "adamah_hip_timer_end": (f32c, []),
     "adamah_hip_debug_dequant": (i32, [_U, u64, u64, pf32]),
@@ -150,14 +153,16 @@ _OPTIONAL_FLAGS = {
     "map_matvec_topk_t_xq8_dev": "_has_map_matvec_topk_t_xq8_dev",
     "map_matvec_topk_t_xq8_ex_dev": "_has_map_matvec_topk_t_xq8_ex_dev",
     "map_matvec_rerank_t_xq8_dev": "_has_map_matvec_rerank_t_xq8_dev",
+    "map_fused_qkv_t_xq4_dev": "_has_map_fused_qkv_t_xq4_dev",
+    "map_fused_qkv_t_xq8_dev": "_has_map_fused_qkv_t_xq8_dev",
+    "map_fused_gateup_t_xq4_dev": "_has_map_fused_gateup_t_xq4_dev",
+    "map_fused_gateup_t_xq8_dev": "_has_map_fused_gateup_t_xq8_dev",
+    "map_fused_gateup_act_t_xq8_dev": "_has_map_fused_gateup_act_t_xq8_dev",
 }
-# Present in the reference surface, deliberately absent here: the fused qkv / gate-up entry points
-# and the monolithic full-decode / device-address API.
+# Present in the reference surface, deliberately absent here: the monolithic full-decode /
+# device-address API and the workgroup-size knob of the Vulkan matmul shaders.
 _ABSENT_FLAGS = (
-    "_has_map_fused_qkv_t_xq4_dev",
-    "_has_map_fused_gateup_t_xq4_dev", "_has_map_fused_qkv_t_xq8_dev", "_has_map_fused_gateup_t_xq8_dev",
-    "_has_map_fused_gateup_act_t_xq8_dev", "_has_full_decode_step_api", "_has_full_decode_step",
-    "_has_map_device_address", "_has_set_xq_matmul_wg",
+    "_has_full_decode_step_api", "_has_full_decode_step", "_has_map_device_address", "_has_set_xq_matmul_wg",
 )
 
 
@@ -477,6 +482,31 @@ class Adamah:
 
     def map_repeat_penalty_dev(self, map_id, locs_src_handle, token_ids_handle, n_ids, penalty):
         self._op("map_repeat_penalty_dev", map_id, locs_src_handle, token_ids_handle, n_ids, penalty)
+
+    def map_fused_qkv_t_xq4_dev(self, map_act, map_wt, locs_a_handle, locs_bq_handle, locs_bk_handle, locs_bv_handle,
+                                locs_cq_handle, locs_ck_handle, locs_cv_handle, K, N_q, N_k, N_v):
+        self._op("map_fused_qkv_t_xq4_dev", map_act, map_wt, locs_a_handle, locs_bq_handle, locs_bk_handle,
+                 locs_bv_handle, locs_cq_handle, locs_ck_handle, locs_cv_handle, K, N_q, N_k, N_v)
+
+    def map_fused_qkv_t_xq8_dev(self, map_act, map_wt, locs_a_handle, locs_bq_handle, locs_bk_handle, locs_bv_handle,
+                                locs_cq_handle, locs_ck_handle, locs_cv_handle, K, N_q, N_k, N_v):
+        self._op("map_fused_qkv_t_xq8_dev", map_act, map_wt, locs_a_handle, locs_bq_handle, locs_bk_handle,
+                 locs_bv_handle, locs_cq_handle, locs_ck_handle, locs_cv_handle, K, N_q, N_k, N_v)
+
+    def map_fused_gateup_t_xq4_dev(self, map_act, map_wt, locs_a_handle, locs_b_gate_handle, locs_b_up_handle,
+                                   locs_c_gate_handle, locs_c_up_handle, K, N_gate, N_up):
+        self._op("map_fused_gateup_t_xq4_dev", map_act, map_wt, locs_a_handle, locs_b_gate_handle, locs_b_up_handle,
+                 locs_c_gate_handle, locs_c_up_handle, K, N_gate, N_up)
+
+    def map_fused_gateup_t_xq8_dev(self, map_act, map_wt, locs_a_handle, locs_b_gate_handle, locs_b_up_handle,
+                                   locs_c_gate_handle, locs_c_up_handle, K, N_gate, N_up):
+        self._op("map_fused_gateup_t_xq8_dev", map_act, map_wt, locs_a_handle, locs_b_gate_handle, locs_b_up_handle,
+                 locs_c_gate_handle, locs_c_up_handle, K, N_gate, N_up)
+
+    def map_fused_gateup_act_t_xq8_dev(self, map_act, map_wt, locs_a_handle, locs_b_gate_handle, locs_b_up_handle,
+                                       locs_c_out_handle, K, N_ff):
+        self._op("map_fused_gateup_act_t_xq8_dev", map_act, map_wt, locs_a_handle, locs_b_gate_handle,
+                 locs_b_up_handle, locs_c_out_handle, K, N_ff)
 
     def map_matvec_topk_t_xq4_dev(self, map_act, map_wt, locs_a_handle, locs_b_handle, penalty_ids_handle,
                                   locs_idx_dst_handle, locs_val_dst_handle, K, N, k, n_penalty=0, repeat_penalty=1.0):

@@ -12,6 +12,7 @@
 //   RMSNorm+residual(o, r -> r); RMSNorm(r -> n); GEMV(n)  -> GEMV that does both norms while staging
 //   GEMV(-> y); ADD(r, y -> d)                            -> GEMV that also stores r + y
 //   GEMV(-> [g; u]); GEGLU/SWIGLU(g, u -> t)              -> GEMV over paired rows that also stores t
+//   GEMV(x, W1 -> y1); GEMV(x, W2 -> y2), W2 after W1, y2 after y1 -> one GEMV over the stacked rows
 //   RoPE(q); RoPE(k) | QK-norm+RoPE; row copy (KV append)  -> one launch of row tasks (rowprep.hip)
 //
 // Every folded op still stores its own result where it would have stored it alone, so the contents
@@ -191,7 +192,25 @@ void flush_pending() {
       i++;
       continue;
     }
-    const PendOp& gp = q[gi];
+    // GEMVs over the same activation vector whose matrices and results lie back to back (Q, K, V or
+    // gate, up issued one after the other): one launch over the stacked rows.  All of them read the
+    // activations as they were before the first, so no result may overlap what the launch reads.
+    PendOp gp = q[gi];
+    if (gp.kind == PK_GEMV) {
+      while (gi + 1 < n && q[gi + 1].kind == PK_GEMV) {
+        const PendOp& nx = q[gi + 1];
+        if (nx.map_act != gp.map_act || nx.map_wt != gp.map_wt || nx.a != gp.a || nx.k != gp.k || nx.op != gp.op ||
+            (uint64_t)nx.b != (uint64_t)gp.b + (uint64_t)gp.n * gp.k || (uint64_t)nx.c != (uint64_t)gp.c + gp.n)
+          break;
+        const uint64_t nn = (uint64_t)gp.n + nx.n;
+        bool clear = nn <= 0xFFFFFFFFull && disjoint(gp.c, nn, gp.a, gp.k);
+        if (fz.pro == PRO_RMSNORM || fz.pro == PRO_NORM2) clear = clear && disjoint(gp.c, nn, fz.p_src, gp.k);
+        if (fz.pro == PRO_NORM2) clear = clear && disjoint(gp.c, nn, fz.p_res, gp.k) && disjoint(gp.c, nn, fz.p_tdst, gp.k);
+        if (!clear) break;
+        gp.n = (uint32_t)nn;
+        gi++;
+      }
+    }
     size_t last = gi;
     if (gp.kind == PK_GEMV && gi + 1 < n && q[gi + 1].kind == PK_OP2 && q[gi + 1].map_act == gp.map_act) {
       const PendOp& e = q[gi + 1];

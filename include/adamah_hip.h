@@ -150,6 +150,24 @@ int map_matvec_rerank_t_xq8_dev(uint32_t map_act, uint32_t map_wt, uint32_t locs
                                 uint32_t locs_idx_dst, uint32_t locs_val_dst, uint32_t K, uint32_t n_ids,
                                 uint32_t n_penalty, float repeat_penalty); /* adamah.c:10018 */
 
+/* Projections that share one activation vector, in one call.  Every handle holds one element offset.
+ * Matrices and results that lie back to back are computed by one launch. */
+int map_fused_qkv_t_xq4_dev(uint32_t map_act, uint32_t map_wt, uint32_t locs_a, uint32_t locs_bq, uint32_t locs_bk,
+                            uint32_t locs_bv, uint32_t locs_cq, uint32_t locs_ck, uint32_t locs_cv, uint32_t K,
+                            uint32_t N_q, uint32_t N_k, uint32_t N_v);  /* adamah.c:8809 */
+int map_fused_qkv_t_xq8_dev(uint32_t map_act, uint32_t map_wt, uint32_t locs_a, uint32_t locs_bq, uint32_t locs_bk,
+                            uint32_t locs_bv, uint32_t locs_cq, uint32_t locs_ck, uint32_t locs_cv, uint32_t K,
+                            uint32_t N_q, uint32_t N_k, uint32_t N_v);  /* adamah.c:9081 */
+int map_fused_gateup_t_xq4_dev(uint32_t map_act, uint32_t map_wt, uint32_t locs_a, uint32_t locs_b_gate,
+                               uint32_t locs_b_up, uint32_t locs_c_gate, uint32_t locs_c_up, uint32_t K,
+                               uint32_t N_gate, uint32_t N_up);        /* adamah.c:8953 */
+int map_fused_gateup_t_xq8_dev(uint32_t map_act, uint32_t map_wt, uint32_t locs_a, uint32_t locs_b_gate,
+                               uint32_t locs_b_up, uint32_t locs_c_gate, uint32_t locs_c_up, uint32_t K,
+                               uint32_t N_gate, uint32_t N_up);        /* adamah.c:9225 */
+/* out[i] = silu(x . Wgate[i]) * (x . Wup[i]), i < N_ff */
+int map_fused_gateup_act_t_xq8_dev(uint32_t map_act, uint32_t map_wt, uint32_t locs_a, uint32_t locs_b_gate,
+                                   uint32_t locs_b_up, uint32_t locs_c_out, uint32_t K, uint32_t N_ff); /* adamah.c:9353 */
+
 /* ---- decode hot path ----------------------------------------------------------------------- */
 int map_rmsnorm_dev(uint32_t map_id, uint32_t locs_src, uint32_t locs_wt, uint32_t locs_dst,
                     uint32_t n_rows, uint32_t dim, float eps); /* adamah.c:7687 */

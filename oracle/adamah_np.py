@@ -1026,6 +1026,68 @@ class NumpyAdamah:
                 v = v / rp if v > 0 else v * rp
             ma.data[il[i]] = f32(tok); ma.data[vl[i]] = v
 
+    # ---- projections that share one activation vector -----------------------------------------
+    def _fused_proj(self, fn, dtype, map_act, map_wt, la_h, parts, K):
+        """adamah.c:8826-8951 (and the Q8 / gate-up twins): every handle must exist, nothing to do when all
+        row counts are zero; each projection is the M = 1 transposed matmul of its own matrix
+        (shaders/src/f32/map_fused_qkv_t_xq4.comp, map_fused_gateup_t_xq4.comp)."""
+        self.op_count += 1
+        self._map(fn, map_act, DTYPE_F32); mw = self._map(fn, map_wt)
+        if not any(n for _, _, n in parts):
+            return
+        if mw.scale is None:
+            self._fail(fn, ERR_INVALID)
+        self._h(fn, la_h)
+        for hb, hc, _ in parts:
+            self._h(fn, hb); self._h(fn, hc)
+        for hb, hc, n in parts:
+            if n:
+                self.op_count -= 1
+                self._xq(fn, map_act, map_wt, dtype, la_h, hb, hc, 1, K, n, 1, True)
+
+    def map_fused_qkv_t_xq4_dev(self, map_act, map_wt, locs_a_handle, locs_bq_handle, locs_bk_handle, locs_bv_handle,
+                                locs_cq_handle, locs_ck_handle, locs_cv_handle, K, N_q, N_k, N_v):
+        self._fused_proj("map_fused_qkv_t_xq4_dev", DTYPE_Q4, map_act, map_wt, locs_a_handle,
+                         [(locs_bq_handle, locs_cq_handle, N_q), (locs_bk_handle, locs_ck_handle, N_k),
+                          (locs_bv_handle, locs_cv_handle, N_v)], K)
+
+    def map_fused_qkv_t_xq8_dev(self, map_act, map_wt, locs_a_handle, locs_bq_handle, locs_bk_handle, locs_bv_handle,
+                                locs_cq_handle, locs_ck_handle, locs_cv_handle, K, N_q, N_k, N_v):
+        self._fused_proj("map_fused_qkv_t_xq8_dev", DTYPE_Q8, map_act, map_wt, locs_a_handle,
+                         [(locs_bq_handle, locs_cq_handle, N_q), (locs_bk_handle, locs_ck_handle, N_k),
+                          (locs_bv_handle, locs_cv_handle, N_v)], K)
+
+    def map_fused_gateup_t_xq4_dev(self, map_act, map_wt, locs_a_handle, locs_b_gate_handle, locs_b_up_handle,
+                                   locs_c_gate_handle, locs_c_up_handle, K, N_gate, N_up):
+        self._fused_proj("map_fused_gateup_t_xq4_dev", DTYPE_Q4, map_act, map_wt, locs_a_handle,
+                         [(locs_b_gate_handle, locs_c_gate_handle, N_gate), (locs_b_up_handle, locs_c_up_handle, N_up)], K)
+
+    def map_fused_gateup_t_xq8_dev(self, map_act, map_wt, locs_a_handle, locs_b_gate_handle, locs_b_up_handle,
+                                   locs_c_gate_handle, locs_c_up_handle, K, N_gate, N_up):
+        self._fused_proj("map_fused_gateup_t_xq8_dev", DTYPE_Q8, map_act, map_wt, locs_a_handle,
+                         [(locs_b_gate_handle, locs_c_gate_handle, N_gate), (locs_b_up_handle, locs_c_up_handle, N_up)], K)
+
+    def map_fused_gateup_act_t_xq8_dev(self, map_act, map_wt, locs_a_handle, locs_b_gate_handle, locs_b_up_handle,
+                                       locs_c_out_handle, K, N_ff):
+        """shaders/src/f32/map_fused_gateup_act_t_xq8.comp:62-160 (dispatch adamah.c:9353-9466):
+        out[i] = silu(x . Wgate[i]) * (x . Wup[i]) with silu(v) = v / (1 + exp(-v)), float32."""
+        self.op_count += 1
+        fn = "map_fused_gateup_act_t_xq8_dev"
+        ma = self._map(fn, map_act, DTYPE_F32); mw = self._map(fn, map_wt, DTYPE_Q8)
+        if N_ff == 0:
+            return
+        if mw.scale is None:
+            self._fail(fn, ERR_INVALID)
+        a = int(self._locs(fn, locs_a_handle, 1)[0]); bg = int(self._locs(fn, locs_b_gate_handle, 1)[0])
+        bu = int(self._locs(fn, locs_b_up_handle, 1)[0]); co = int(self._locs(fn, locs_c_out_handle, 1)[0])
+        self._chk(fn, ma, a, a + K); self._chk(fn, mw, bg, bg + N_ff * K); self._chk(fn, mw, bu, bu + N_ff * K)
+        self._chk(fn, ma, co, co + N_ff)
+        x = ma.data[a:a + K].astype(np.float64)
+        gate = (mw.deq_range(bg, N_ff * K).reshape(N_ff, K).astype(np.float64) @ x).astype(np.float32)
+        upv = (mw.deq_range(bu, N_ff * K).reshape(N_ff, K).astype(np.float64) @ x).astype(np.float32)
+        with np.errstate(over="ignore"):
+            ma.data[co:co + N_ff] = (gate / (f32(1.0) + np.exp(-gate))) * upv
+
 
 def init(cache_mb=None, cold_cache_mb=None):
     return NumpyAdamah()

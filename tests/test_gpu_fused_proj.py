@@ -1,0 +1,124 @@
+"""Projections that share an activation vector (Q/K/V, gate/up, gate/up + SiLU) in one call: HIP vs the
+oracle through the C ABI, 1e-3 relative L2 per projection (the bar of the GEMV they are made of).
+
+Also checked: matrices and results that lie back to back cost ONE launch (two when a gated activation
+follows: it folds into the same launch), matrices apart cost one launch each, results are the same
+either way, and the calls work outside a batch."""
+import numpy as np
+import pytest
+
+import oracle
+from adam_amd import adamah as A
+from adam_amd import quant
+from gpu_util import note, up, f32map, read, rel_l2, load_qtensor
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+def stacked(kind, rows, K, seed, gap=0):
+    """One QTensor holding the matrices one after the other (`gap` unused rows between them)."""
+    rng = np.random.default_rng(seed)
+    tot = sum(rows) + gap * (len(rows) - 1)
+    w = rng.standard_normal((tot, K), dtype=np.float32) * np.float32(0.05)
+    qt = (quant.quantize_q4_0 if kind == "q4" else quant.quantize_q8_0)(w)
+    bases, r = [], 0
+    for n in rows:
+        bases.append(r * K)
+        r += n + gap
+    return qt, bases
+
+
+@pytest.mark.parametrize("kind,K,rows,gap,batch", [
+    ("q4", 1152, (1024, 256, 256), 0, True),      # Gemma-3-1B QKV, adjacent: one launch
+    ("q4", 4096, (4096, 1024, 1024), 0, False),   # Llama-3-8B QKV outside a batch
+    ("q4", 1152, (1024, 256, 256), 36, True),     # matrices apart: three launches
+    ("q4", 4096, (512, 0, 256), 0, True),         # a projection without rows
+    ("q8", 1152, (1024, 256, 256), 0, True),
+])
+def test_fused_qkv(hip, kind, K, rows, gap, batch):
+    qt, bases = stacked(kind, rows, K, K + sum(rows), gap=gap)
+    x = np.random.default_rng(1).standard_normal(K).astype(np.float32)
+    outs, launches = [], None
+    for g in (hip, oracle.init()):
+        note(f"fused_qkv {kind} K={K} rows={rows} gap={gap} batch={batch}")
+        load_qtensor(g, 1, qt)
+        f32map(g, 0, K + sum(rows) + 64, x)
+        cs = [K, K + rows[0], K + rows[0] + rows[1]]
+        fn = g.map_fused_qkv_t_xq4_dev if kind == "q4" else g.map_fused_qkv_t_xq8_dev
+        hs = [up(g, [0])] + [up(g, [b]) for b in bases] + [up(g, [c]) for c in cs]
+        if batch:
+            g.batch_begin()
+        fn(0, 1, *hs, K, *rows)
+        if batch:
+            g.batch_end()
+        if g is hip and batch:
+            launches = g.get_last_barrier_count()
+        outs.append(read(g, 0, K, sum(rows)))
+    lo = 0
+    for n in rows:
+        if n:
+            assert rel_l2(outs[0][lo:lo + n], outs[1][lo:lo + n]) < TOL
+        lo += n
+    if launches is not None and kind == "q4":
+        n_proj = sum(1 for n in rows if n)
+        assert launches == (1 if gap == 0 else n_proj), launches
+
+
+@pytest.mark.parametrize("kind,K,ff,act", [("q4", 1152, 6912, "geglu"), ("q4", 4096, 14336, "swiglu"), ("q4", 4096, 1024, None),
+                                           ("q8", 1152, 512, None)])
+def test_fused_gateup_and_folded_activation(hip, kind, K, ff, act):
+    qt, bases = stacked(kind, (ff, ff), K, ff)
+    x = np.random.default_rng(2).standard_normal(K).astype(np.float32)
+    outs, launches = [], None
+    for g in (hip, oracle.init()):
+        note(f"fused_gateup {kind} K={K} ff={ff} act={act}")
+        load_qtensor(g, 1, qt)
+        f32map(g, 0, K + 3 * ff + 64, x)
+        fn = g.map_fused_gateup_t_xq4_dev if kind == "q4" else g.map_fused_gateup_t_xq8_dev
+        g.batch_begin()
+        fn(0, 1, up(g, [0]), up(g, [bases[0]]), up(g, [bases[1]]), up(g, [K]), up(g, [K + ff]), K, ff, ff)
+        if act:
+            g.map_op2_dev(0, A.OP_GEGLU if act == "geglu" else A.OP_SWIGLU, up(g, K + np.arange(ff)), up(g, K + ff + np.arange(ff)),
+                          up(g, K + 2 * ff + np.arange(ff)), ff)
+        g.batch_end()
+        if g is hip:
+            launches = g.get_last_barrier_count()
+        outs.append(read(g, 0, K, 3 * ff))
+    assert rel_l2(outs[0][:ff], outs[1][:ff]) < TOL and rel_l2(outs[0][ff:2 * ff], outs[1][ff:2 * ff]) < TOL
+    if act:
+        assert rel_l2(outs[0][2 * ff:], outs[1][2 * ff:]) < TOL
+    if kind == "q4":
+        assert launches == 1, launches
+
+
+def test_fused_gateup_act_q8(hip):
+    rng = np.random.default_rng(4)
+    K, ff = 1152, 700
+    qt, bases = stacked("q8", (ff, ff), K, 9)
+    x = rng.standard_normal(K).astype(np.float32)
+    outs = []
+    for g in (hip, oracle.init()):
+        note("fused_gateup_act q8")
+        load_qtensor(g, 1, qt)
+        f32map(g, 0, K + ff + 64, x)
+        g.map_fused_gateup_act_t_xq8_dev(0, 1, up(g, [0]), up(g, [bases[0]]), up(g, [bases[1]]), up(g, [K]), K, ff)
+        outs.append(read(g, 0, K, ff))
+    assert rel_l2(outs[0], outs[1]) < TOL
+
+
+def test_errors(hip):
+    note("fused projections: errors")
+    qt = quant.quantize_q4_0(np.ones((8, 32), np.float32))
+    load_qtensor(hip, 1, qt)
+    f32map(hip, 0, 256, np.ones(32, np.float32))
+    a, b, c = up(hip, [0]), up(hip, [0]), up(hip, [64])
+    hip.map_fused_qkv_t_xq4_dev(0, 1, a, b, b, b, c, c, c, 32, 0, 0, 0)                # no rows: nothing to do
+    with pytest.raises(RuntimeError):
+        hip.map_fused_qkv_t_xq4_dev(0, 1, a, b, b, 987654, c, c, c, 32, 4, 0, 0)       # a missing handle, even unused
+    with pytest.raises(RuntimeError):
+        hip.map_fused_qkv_t_xq8_dev(0, 1, a, b, b, b, c, c, c, 32, 4, 0, 0)            # Q8 entry on a Q4 map
+    with pytest.raises(RuntimeError):
+        hip.map_fused_gateup_t_xq4_dev(0, 1, a, b, b, c, up(hip, [250]), 32, 4, 8)     # result past the map
+    with pytest.raises(RuntimeError):
+        hip.map_fused_gateup_act_t_xq8_dev(0, 1, a, b, b, c, 32, 4)                    # Q8 only

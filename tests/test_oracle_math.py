@@ -481,3 +481,27 @@ def test_rerank_equals_row_dot_products():
     assert toks == [12, 39, 7, 5]
     exp = [y[12], y[39] / 2 if y[39] > 0 else y[39] * 2, y[7], y[5] / 2 if y[5] > 0 else y[5] * 2]
     assert np.allclose(vals, np.array(exp, np.float32), rtol=1e-6)
+
+
+def test_fused_projections_equal_their_separate_dot_products():
+    rng = np.random.default_rng(14)
+    K, rows = 64, (6, 2, 3)
+    qt = quant.quantize_q4_0(rng.standard_normal((sum(rows), K)).astype(np.float32))
+    x = rng.standard_normal(K).astype(np.float32)
+    y = (qt.dequant().astype(np.float64) @ x.astype(np.float64)).astype(np.float32)
+    g = oracle.init()
+    _load_q(g, 1, qt)
+    f32map(g, 0, K + 32, x)
+    # results deliberately out of order: K first, then V, then Q
+    g.map_fused_qkv_t_xq4_dev(0, 1, up(g, [0]), up(g, [0]), up(g, [6 * K]), up(g, [8 * K]), up(g, [K + 5]), up(g, [K]),
+                              up(g, [K + 2]), K, *rows)
+    assert np.array_equal(read(g, 0, K, 2), y[6:8]) and np.array_equal(read(g, 0, K + 2, 3), y[8:11])
+    assert np.array_equal(read(g, 0, K + 5, 6), y[0:6])
+    q8 = quant.quantize_q8_0(rng.standard_normal((8, K)).astype(np.float32))
+    _load_q(g, 2, q8)
+    g.map_fused_gateup_act_t_xq8_dev(0, 2, up(g, [0]), up(g, [0]), up(g, [4 * K]), up(g, [K + 16]), K, 4)
+    z = q8.dequant().astype(np.float64) @ x.astype(np.float64)
+    exp = z[:4] / (1 + np.exp(-z[:4])) * z[4:]
+    assert np.allclose(read(g, 0, K + 16, 4), exp, rtol=1e-5)
+    with pytest.raises(RuntimeError):
+        g.map_fused_qkv_t_xq4_dev(0, 1, up(g, [0]), up(g, [0]), 424242, up(g, [0]), up(g, [K]), up(g, [K]), up(g, [K]), K, 1, 0, 0)
