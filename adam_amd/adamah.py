@@ -160,7 +160,7 @@ _OPTIONAL_FLAGS = {
     "map_fused_gateup_act_t_xq8_dev": "_has_map_fused_gateup_act_t_xq8_dev",
 }
 # Present in the reference surface, deliberately absent here: the monolithic full-decode /
-# device-address API and the workgroup-size knob of the Vulkan matmul shaders.
+# device-address API (the wg-size flag is tied to a Vulkan shader knob that has no effect here).
 _ABSENT_FLAGS = (
     "_has_full_decode_step_api", "_has_full_decode_step", "_has_map_device_address", "_has_set_xq_matmul_wg",
 )
