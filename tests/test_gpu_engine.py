@@ -122,3 +122,25 @@ def test_gemma3_1b_full_model_tokens_match_reference_forward(hip):
 def test_llama3_8b_full_model_tokens_match_reference_forward(hip):
     note("engine llama-3-8b shape, all 32 layers, Q8_0 head")
     _full_model_vs_cpu(hip, synth.llama3_8b_config(), 4, 3, 0)
+
+
+@pytest.mark.parametrize("arch", ["llama", "gemma3"])
+def test_model_read_from_a_gguf_file(hip, arch, tmp_path):
+    """Q4_K, Q4_0 and Q8_0 blocks of a file uploaded in map form (nothing re-quantised): the harness on the
+    HIP library follows the harness on the oracle, and the restated reference forward over the
+    dequantised blocks."""
+    from adam_amd import gguf
+    from test_gguf_loader import _model_file
+    p = tmp_path / f"{arch}.gguf"
+    _model_file(str(p), arch, np.random.default_rng(11))
+    cfg, tensors = gguf.load_model(str(p))
+    note(f"engine from gguf {arch}")
+    prompt = [5, 17, 3, 90, 44]
+    ref, dev, ref_tok, free_tok, forced_tok, _ = run_pair(hip, cfg, tensors, prompt, 8, 32, True, "legacy", rpg=32)
+    assert rel_l2(dev.read_slot('hidden'), ref.read_slot('hidden')) < 1e-3
+    assert forced_tok == ref_tok
+    deq = {n: (v.dequant() if isinstance(v, QTensor) else v) for n, v in tensors.items()}
+    cpu = CpuModel(cfg, deq, kv_cap=32, kv_fp16=True)
+    cpu_tok, margins = cpu.generate(prompt, 8, forced=ref_tok)
+    for i in range(8):
+        assert cpu_tok[i] == forced_tok[i] or margins[i] < 1e-5
