@@ -154,6 +154,7 @@ bool res_scalar(uint32_t h, uint32_t* out);
 // First element of a handle whose host copy is a run of n consecutive indices; false otherwise.
 bool res_run(uint32_t h, uint64_t n, uint32_t* start);
 void gemm_q4_mfma_release();   // frees the GEMM's scratch (shutdown)
+void sampling_release();       // frees the scratch lists of the chunked top-k (shutdown)
 void topk_fused_release();     // frees the scratch logits of the GEMV + top-k ops (shutdown)
 int launch_rmsnorm_v(const PendOp& p);
 bool row_op_deferrable(const PendOp& p);                                  // rowprep.hip

@@ -369,6 +369,7 @@ void adamah_shutdown(void) { ADAMAH_API();
   g.sync_ctr = nullptr;
   gemm_q4_mfma_release();
   topk_fused_release();
+  sampling_release();
   g.pend.clear();
   for (int i = 0; i < MAX_PLANS; i++) { g.plans[i].clear(); g.plan_active[i] = false; }
   hipStreamDestroy(g.stream);

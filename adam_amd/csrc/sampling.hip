@@ -9,6 +9,7 @@
 // use, so the float32 results match a sequential evaluation.  Every location read from a handle is
 // checked against the map size before it is used.
 #include "common.h"
+#include <algorithm>
 #include "../../include/adamah_hip.h"
 
 namespace adamah {
@@ -23,42 +24,116 @@ __device__ __forceinline__ bool smp_better(float cv, uint32_t ci, float bv, uint
   return cv > bv || (cv == bv && ci < bi);
 }
 
-// k rounds of "best not yet chosen" over n candidates (NaN counts as the lowest value, ties go to
-// the lower index); rounds past n store index 0 and the lowest value.
-__global__ void __launch_bounds__(256)
-k_topk(float* data, const uint32_t* __restrict__ ls, const uint32_t* __restrict__ li, const uint32_t* __restrict__ lv,
-       uint32_t n, uint32_t k, uint64_t n_elems) {
-  __shared__ float sv[256];
-  __shared__ uint32_t si[256];
-  __shared__ uint32_t top[SMP_MAX];
-  const uint32_t tid = threadIdx.x;
-  if (tid < SMP_MAX) top[tid] = SMP_INVALID;
+// Top-k over n candidates: the k best in the order (value descending, candidate index ascending); NaN
+// counts as the lowest value; rounds past n store index 0 and the lowest value.  The order is strict,
+// so round t takes the best candidate that ranks after the pick of round t - 1 and no list of taken
+// candidates is needed.  A workgroup keeps a chunk of 4096 candidates in registers (16 per thread,
+// one coalesced pass over the handle and the map); one chunk writes the result itself, several chunks
+// leave their own k best in a scratch list that a second launch merges the same way.
+#define TOPK_CHUNK 4096u
+#define TOPK_PER_THREAD 16u
+
+struct TopkPick { float v; uint32_t i; };
+
+// best (value, index) over the workgroup, the same in every thread
+__device__ __forceinline__ TopkPick topk_block_best(float bv, uint32_t bi, float* sv, uint32_t* si) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, 64);
+    const uint32_t oi = __shfl_xor(bi, o, 64);
+    if (smp_better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+  }
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  __syncthreads();                       // sv / si may still be read from the previous round
+  if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
   __syncthreads();
-  for (uint32_t o = 0; o < k; o++) {
+  bv = sv[0]; bi = si[0];
+#pragma unroll
+  for (int w = 1; w < 4; w++)
+    if (smp_better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
+  return {bv, bi};
+}
+
+__device__ __forceinline__ bool topk_after(float pv, uint32_t pi, float v, uint32_t i) {
+  return pv > v || (pv == v && pi < i);
+}
+
+__global__ void __launch_bounds__(256)
+k_topk_chunk(float* data, const uint32_t* __restrict__ ls, const uint32_t* __restrict__ li, const uint32_t* __restrict__ lv,
+             uint32_t n, uint32_t k, uint64_t n_elems, float* part_v, uint32_t* part_i) {
+  __shared__ float sv[4];
+  __shared__ uint32_t si[4];
+  const uint32_t tid = threadIdx.x, c0 = blockIdx.x * TOPK_CHUNK;
+  const bool single = gridDim.x == 1u;
+  float v[TOPK_PER_THREAD];
+#pragma unroll
+  for (uint32_t u = 0; u < TOPK_PER_THREAD; u++) {
+    const uint32_t i = c0 + u * 256u + tid;
+    float x = SMP_NEG_INF;
+    if (i < n) { const uint32_t l = ls[i]; if (l < n_elems) x = data[l]; }
+    v[u] = x != x ? SMP_NEG_INF : x;
+  }
+  float pv = 0.f;
+  uint32_t pi = SMP_INVALID;
+  for (uint32_t t = 0; t < k; t++) {
     float bv = SMP_NEG_INF;
     uint32_t bi = SMP_INVALID;
-    for (uint32_t i = tid; i < n; i += 256u) {
-      bool chosen = false;
-      for (uint32_t j = 0; j < o; j++) chosen = chosen || top[j] == i;
-      if (chosen) continue;
-      float v = ls[i] < n_elems ? data[ls[i]] : SMP_NEG_INF;
-      if (isnan(v)) v = SMP_NEG_INF;
-      if (smp_better(v, i, bv, bi)) { bv = v; bi = i; }
+    if (t == 0u || pi != SMP_INVALID) {
+#pragma unroll
+      for (uint32_t u = 0; u < TOPK_PER_THREAD; u++) {
+        const uint32_t i = c0 + u * 256u + tid;
+        if (i < n && (t == 0u || topk_after(pv, pi, v[u], i)) && smp_better(v[u], i, bv, bi)) { bv = v[u]; bi = i; }
+      }
     }
-    sv[tid] = bv; si[tid] = bi;
-    __syncthreads();
-    for (uint32_t s = 128; s > 0; s >>= 1) {
-      if (tid < s && smp_better(sv[tid + s], si[tid + s], sv[tid], si[tid])) { sv[tid] = sv[tid + s]; si[tid] = si[tid + s]; }
-      __syncthreads();
-    }
+    const TopkPick b = topk_block_best(bv, bi, sv, si);
+    pv = b.v; pi = b.i;
     if (tid == 0) {
-      const uint32_t w = si[0];
-      top[o] = w;
-      if (li[o] < n_elems) data[li[o]] = (float)(w == SMP_INVALID ? 0u : w);
-      if (lv[o] < n_elems) data[lv[o]] = w == SMP_INVALID ? SMP_NEG_INF : sv[0];
+      if (single) {
+        if (li[t] < n_elems) data[li[t]] = (float)(b.i == SMP_INVALID ? 0u : b.i);
+        if (lv[t] < n_elems) data[lv[t]] = b.i == SMP_INVALID ? SMP_NEG_INF : b.v;
+      } else {
+        part_v[blockIdx.x * k + t] = b.v;
+        part_i[blockIdx.x * k + t] = b.i;
+      }
     }
-    __syncthreads();
   }
+}
+
+// merge of the chunks' lists: n2 = chunks * k (value, candidate index) pairs, invalid entries skipped
+__global__ void __launch_bounds__(256)
+k_topk_merge(float* data, const float* __restrict__ part_v, const uint32_t* __restrict__ part_i,
+             const uint32_t* __restrict__ li, const uint32_t* __restrict__ lv, uint32_t n2, uint32_t k, uint64_t n_elems) {
+  __shared__ float sv[4];
+  __shared__ uint32_t si[4];
+  const uint32_t tid = threadIdx.x;
+  float pv = 0.f;
+  uint32_t pi = SMP_INVALID;
+  for (uint32_t t = 0; t < k; t++) {
+    float bv = SMP_NEG_INF;
+    uint32_t bi = SMP_INVALID;
+    if (t == 0u || pi != SMP_INVALID) {
+      for (uint32_t j = tid; j < n2; j += 256u) {
+        const uint32_t i = part_i[j];
+        const float x = part_v[j];
+        if (i != SMP_INVALID && (t == 0u || topk_after(pv, pi, x, i)) && smp_better(x, i, bv, bi)) { bv = x; bi = i; }
+      }
+    }
+    const TopkPick b = topk_block_best(bv, bi, sv, si);
+    pv = b.v; pi = b.i;
+    if (tid == 0) {
+      if (li[t] < n_elems) data[li[t]] = (float)(b.i == SMP_INVALID ? 0u : b.i);
+      if (lv[t] < n_elems) data[lv[t]] = b.i == SMP_INVALID ? SMP_NEG_INF : b.v;
+    }
+  }
+}
+
+static float* g_topk_part = nullptr;   // chunks * k values, then chunks * k candidate indices
+static size_t g_topk_part_cap = 0;     // entries
+
+void sampling_release() {
+  if (g_topk_part) hipFree(g_topk_part);
+  g_topk_part = nullptr;
+  g_topk_part_cap = 0;
 }
 
 // softmax(logits / temperature) over n <= 64 candidates in list order, cut after the first prefix
@@ -178,8 +253,28 @@ int map_topk_dev(uint32_t map_id, uint32_t hs, uint32_t hi, uint32_t hv, uint32_
   if (k > SMP_MAX) return ADAMAH_ERR_INVALID;
   const uint32_t *ls = res_u32(hs, n), *li = res_u32(hi, k), *lv = res_u32(hv, k);
   if (!ls || !li || !lv) return ADAMAH_ERR_INVALID;
-  k_topk<<<1, 256, 0, g.stream>>>((float*)m->buf, ls, li, lv, n, k, m->n_elems);
+  const uint32_t chunks = cdiv(n, TOPK_CHUNK);
+  float* pv = nullptr;
+  uint32_t* pi = nullptr;
+  if (chunks > 1) {
+    const size_t need = (size_t)chunks * k;
+    if (need > g_topk_part_cap) {
+      if (g_topk_part) { hipStreamSynchronize(g.stream); hipFree(g_topk_part); }
+      g_topk_part_cap = std::max<size_t>(need, 4096);
+      if (hipMalloc((void**)&g_topk_part, g_topk_part_cap * 8) != hipSuccess) {
+        g_topk_part = nullptr; g_topk_part_cap = 0;
+        return ADAMAH_ERR_MEMORY;
+      }
+    }
+    pv = g_topk_part;
+    pi = (uint32_t*)(g_topk_part + g_topk_part_cap);
+  }
+  k_topk_chunk<<<chunks, 256, 0, g.stream>>>((float*)m->buf, ls, li, lv, n, k, m->n_elems, pv, pi);
   count_launch();
+  if (chunks > 1) {
+    k_topk_merge<<<1, 256, 0, g.stream>>>((float*)m->buf, pv, pi, li, lv, chunks * k, k, m->n_elems);
+    count_launch();
+  }
   return check_launch();
 }
 

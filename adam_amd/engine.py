@@ -69,6 +69,8 @@ class DecodeEngine:
     WS_MAP = 0
     Q8_MAP = 2
     Q4_GROUP = 32
+    SAMPLE_TOPK_MAX = 64       # reference engine.py:118
+    SAMPLE_REPEAT_MAX = 64     # reference engine.py:120
     SAMPLE_TOPK_MAX = 64
     SAMPLE_APPROX_SHORTLIST_MAX = 256
 
@@ -172,13 +174,19 @@ class DecodeEngine:
         if c.attn_softcap > 0:
             self._pos_attn_cap = pos; pos += 1
         if c.final_softcap > 0:
-            self._pos_final_cap = pos; pos += 1
+            self._pos_final_cap = pos
+            self._final_cap_h = self._up(np.full(self.SAMPLE_TOPK_MAX, pos))
+            g.register_loc_span(self._final_cap_h, 0, pos, 1)
+            pos += 1
 
         slots = [('hidden', c.n_embd), ('normed', c.n_embd), ('q', q_dim), ('k', k_dim), ('v', k_dim),
                  ('attn_out', c.n_head * c.head_dim_kv), ('o_proj', c.n_embd), ('gate', c.n_ff),
                  ('up', c.n_ff), ('act', c.n_ff), ('ffn_out', c.n_embd), ('logits', c.n_vocab),
                  ('sample_token', 1), ('sample_rand', 1),
-                 ('sample_fused_idx', self._fused_groups), ('sample_fused_val', self._fused_groups),
+                 ('sample_fused_idx', self._fused_groups * self.SAMPLE_TOPK_MAX),
+                 ('sample_fused_val', self._fused_groups * self.SAMPLE_TOPK_MAX),
+                 ('sample_topk_idx', self.SAMPLE_TOPK_MAX), ('sample_topk_val', self.SAMPLE_TOPK_MAX),
+                 ('sample_topk_prob', self.SAMPLE_TOPK_MAX), ('sample_short_sel', self.SAMPLE_TOPK_MAX),
                  ('normed2', c.n_embd)]
         for name, sz in slots:
             span(name, sz, pos); pos += sz
@@ -237,6 +245,10 @@ class DecodeEngine:
 
         self._hid_locs = np.arange(self._ws['hidden'][2], self._ws['hidden'][2] + c.n_embd, dtype=np.uint32)
         self._sample_locs = np.array([self._ws['sample_token'][2]], dtype=np.uint32)
+        self._rand_locs = np.array([self._ws['sample_rand'][2]], dtype=np.uint32)
+        self._sample_fused_base_h = self._up([self._ws['sample_fused_idx'][2]])
+        self._sample_repeat_ids = np.zeros(self.SAMPLE_REPEAT_MAX, np.uint32)
+        self._sample_repeat_ids_h = self._up(self._sample_repeat_ids)
         self._ws_total = pos
 
     # ------------------------------------------------------------------ upload
@@ -424,7 +436,7 @@ class DecodeEngine:
         return ops
 
     # ------------------------------------------------------------------ forward
-    def _forward(self, tok, pos, sample=True):
+    def _forward(self, tok, pos, sample=True, sample_cfg=None, sample_prev=()):
         """One decode step; op order of reference engine.py:2971-3402 (default discrete-GPU path)."""
         c, g, A, ws = self.cfg, self.gpu, self.A, self.WS_MAP
         q_dim, k_dim = c.n_head * c.head_dim, c.n_head_kv * c.head_dim_kv
@@ -506,7 +518,9 @@ class DecodeEngine:
             self._rms(hid_h, 'output_norm.weight', normed_h, 1, c.n_embd)
         else:
             g.decode_step(self._plan_id, pos, seq_len)
-        if sample:
+        if sample and sample_cfg is not None and sample_cfg.temperature > 0.0 and sample_cfg.top_k > 1:
+            self._sample_fused_topk(sample_cfg, sample_prev, normed_h)
+        elif sample:
             fn = (g.map_matvec_argmax_t_xq8_dev if self._kind[self._lm_name] == 'q8'
                   else g.map_matvec_argmax_t_xq4_dev)
             fn(ws, self._map_of[self._lm_name], normed_h, self._wh[self._lm_name],
@@ -514,6 +528,38 @@ class DecodeEngine:
                c.n_embd, c.n_vocab, self._rows_per_group)
             self._sample_token_ready = True
         g.batch_end()
+
+    def _sample_fused_topk(self, cfg, prev, normed_h):
+        """Sampled LM head inside the forward batch, the reference's 'gpu_fused_topk' mode
+        (engine.py:3404-3508): partial top-k per group of rows with the repeat penalty, top-k of the
+        partial values, final soft-cap on the k survivors, temperature / top-p, token ids resolved
+        through the partial list, one categorical draw with a uniform number from the host."""
+        c, g, A, ws, W = self.cfg, self.gpu, self.A, self.WS_MAP, self._ws
+        top_k = max(1, min(int(cfg.top_k), self.SAMPLE_TOPK_MAX, c.n_vocab))
+        n_pen = 0
+        if cfg.repeat_penalty != 1.0 and len(prev):
+            ids = list(dict.fromkeys(int(t) for t in reversed(list(prev))))[:self.SAMPLE_REPEAT_MAX]
+            n_pen = len(ids)
+            self._sample_repeat_ids[:] = 0
+            self._sample_repeat_ids[:n_pen] = ids
+            g.upload_dev(self._sample_repeat_ids, handle=self._sample_repeat_ids_h)
+        g.scatter(ws, self._rand_locs, np.array([self._rng.random()], np.float32))
+        pidx_h, pval_h = W['sample_fused_idx'][0], W['sample_fused_val'][0]
+        fn = (g.map_matvec_topk_t_xq8_ex_dev if self._kind[self._lm_name] == 'q8' else g.map_matvec_topk_t_xq4_ex_dev)
+        fn(ws, self._map_of[self._lm_name], normed_h, self._wh[self._lm_name], self._sample_repeat_ids_h, pidx_h, pval_h,
+           c.n_embd, c.n_vocab, top_k, n_pen, float(cfg.repeat_penalty), self._rows_per_group)
+        idx_h, val_h, prob_h = W['sample_topk_idx'][0], W['sample_topk_val'][0], W['sample_topk_prob'][0]
+        g.map_topk_dev(ws, pval_h, idx_h, val_h, self._fused_groups * top_k, top_k)
+        if c.final_softcap > 0:
+            cap_h = self._final_cap_h
+            g.map_broadcast_dev(ws, A.OP_DIV, val_h, cap_h, val_h, top_k)
+            g.map_op1_dev(ws, A.OP_TANH, val_h, val_h, top_k)
+            g.map_broadcast_dev(ws, A.OP_MUL, val_h, cap_h, val_h, top_k)
+        g.map_topp_dev(ws, val_h, prob_h, top_k, float(cfg.temperature), float(cfg.top_p))
+        sel_h = W['sample_short_sel'][0]
+        g.map_resolve_idx_dev(ws, self._sample_fused_base_h, idx_h, sel_h, top_k)
+        g.map_sample_categorical_dev(ws, sel_h, prob_h, W['sample_rand'][0], W['sample_token'][0], top_k)
+        self._sample_token_ready = True
 
     def read_token(self):
         # reference engine.py:1979-1981: token id crosses the boundary as float32
@@ -532,7 +578,9 @@ class DecodeEngine:
 
     # ------------------------------------------------------------------ generate
     def generate(self, token_ids, config=None, forced=None):
-        """Greedy generation.  Prefill is the same `_forward` once per prompt token, LM head only
+        """Greedy generation, or sampled generation when `config.temperature > 0` and `config.top_k > 1`
+        (top-k, top-p and repeat penalty on the device, one uniform number per token from a host
+        generator seeded with `config.seed`).  Prefill is the same `_forward` once per prompt token, LM head only
         on the last one; `decode_tps = n_gen / wall(decode loop)` including the per-token
         read-back (reference engine.py:3838-3931).  `forced`, when given, is a token list fed
         back instead of the model's own choices (teacher forcing) while the choices are still
@@ -543,10 +591,13 @@ class DecodeEngine:
                 f"KV cache too small: need {len(token_ids) + config.max_tokens} tokens but "
                 f"kv_cap={self._kv_cap}. Reinitialize with kv_cap>={len(token_ids) + config.max_tokens}.")
         self.reset()
+        sampled = config.temperature > 0.0 and config.top_k > 1
+        self._rng = np.random.default_rng(config.seed)
+        hist = [int(t) for t in token_ids]
         tp = time.perf_counter()
         last = len(token_ids) - 1
         for i, t in enumerate(token_ids):
-            self._forward(int(t), i, sample=(i == last))
+            self._forward(int(t), i, sample=(i == last), sample_cfg=config, sample_prev=hist)
         self.gpu.sync()
         t_pre = time.perf_counter() - tp
         out, ttimes = [], []
@@ -558,7 +609,8 @@ class DecodeEngine:
                 break
             out.append(nt)
             feed = nt if forced is None else int(forced[step])
-            self._forward(feed, len(token_ids) + step, sample=True)
+            hist.append(feed)
+            self._forward(feed, len(token_ids) + step, sample=True, sample_cfg=config, sample_prev=hist)
             ttimes.append(time.perf_counter() - t0)
         self.gpu.sync()
         t_dec = time.perf_counter() - td
@@ -568,5 +620,5 @@ class DecodeEngine:
             'prefill_tps': n_p / t_pre if t_pre > 0 else 0.0,
             'decode_tps': n_g / t_dec if t_dec > 0 else 0.0,
             'avg_ms': float(np.mean(ttimes) * 1000) if ttimes else 0.0,
-            'sampling_mode': 'gpu_matvec_argmax',
+            'sampling_mode': 'gpu_fused_topk' if sampled else 'gpu_matvec_argmax',
         }

@@ -58,3 +58,35 @@ def test_kv_cap_guard():
     eng = DecodeEngine(oracle.init(), cfg, synth.make_model(cfg, seed=1, sigma=0.3), A=A, kv_cap=8)
     with pytest.raises(RuntimeError, match="KV cache too small"):
         eng.generate([1, 2, 3, 4, 5], GenerationConfig(max_tokens=4))
+
+
+@pytest.mark.parametrize("arch", ["gemma3", "llama"])
+def test_sampled_generation_draws_from_the_top_k_of_the_reference_logits(arch):
+    """temperature / top-k / top-p / repeat penalty on the op surface: every drawn token lies in the top k
+    of the restated reference forward's logits (after the same penalty), the run is reproducible from
+    its seed, and a different seed gives a different continuation."""
+    cfg = synth.tiny_config(arch, n_layer=2, n_embd=64, n_head=4, n_head_kv=2, head_dim=32, n_ff=96, n_vocab=160)
+    tensors = synth.make_model(cfg, seed=6, sigma=0.3)
+    gc = GenerationConfig(max_tokens=10, temperature=4.0, top_k=8, top_p=0.98, repeat_penalty=1.2, seed=123)
+    prompt = [5, 17, 3, 101]
+    runs = []
+    for seed in (123, 123, 7):
+        gc.seed = seed
+        eng = DecodeEngine(oracle.init(), cfg, tensors, A=A, kv_cap=32, gpu_fused_rows_per_group=32)
+        out, stats = eng.generate(prompt, gc)
+        assert stats['sampling_mode'] == 'gpu_fused_topk' and len(out) == 10
+        runs.append(out)
+    assert runs[0] == runs[1] and runs[0] != runs[2]
+    ref = CpuModel(cfg, dequant_tensors(tensors), kv_cap=32)
+    hist = list(prompt)
+    logits = None
+    for i, t in enumerate(prompt):
+        logits = ref.forward(int(t), i)
+    for step, tok in enumerate(runs[0]):
+        lg = np.array(logits, np.float32)
+        for r in set(hist):
+            lg[r] = lg[r] / np.float32(1.2) if lg[r] > 0 else lg[r] * np.float32(1.2)
+        top = np.argsort(-lg, kind="stable")[:8]
+        assert tok in top, (step, tok, top)
+        hist.append(tok)
+        logits = ref.forward(tok, len(prompt) + step)
