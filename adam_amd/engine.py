@@ -76,7 +76,8 @@ class DecodeEngine:
 
     def __init__(self, gpu, cfg, tensors, A=None, kv_cap=1024, kv_fp16=False,
                  fusion_scheduler_mode='legacy', gpu_fused_rows_per_group=256,
-                 q4_map_elem_limit=(1 << 32) - 64, verbose=False, decode_plan=True, plan_id=0):
+                 q4_map_elem_limit=(1 << 32) - 64, verbose=False, decode_plan=True, plan_id=0,
+                 prefill_chunk=0):
         if A is None:
             from . import adamah as A
         self.gpu, self.cfg, self.tensors, self.A = gpu, cfg, tensors, A
@@ -85,6 +86,7 @@ class DecodeEngine:
         self._kv_fp16 = bool(kv_fp16)
         self._rows_per_group = max(1, int(gpu_fused_rows_per_group))
         self._q4_limit = int(q4_map_elem_limit)
+        self._chunk = max(0, int(prefill_chunk))
         self._build_layout()
         self._alloc_workspace()
         self._upload_all()
@@ -195,6 +197,9 @@ class DecodeEngine:
             self._off[name] = pos; self._map_of[name] = 0
             pos += self.tensors[name].size
 
+        if self._chunk:
+            pos = self._alloc_chunk_slots(pos)
+
         pos_q, pos_k, pos_v = self._ws['q'][2], self._ws['k'][2], self._ws['v'][2]
         self._q_rows_h = self._up(pos_q + np.arange(c.n_head) * c.head_dim)
         g.register_row_base_span(self._q_rows_h, 0, pos_q, c.n_head, c.head_dim, c.head_dim)
@@ -239,6 +244,8 @@ class DecodeEngine:
                 spec[4 * gi:4 * gi + 4] = (gi, kb // c.head_dim_kv + gi * kv_cap,
                                            gi + c.n_head_kv, vb // c.head_dim_kv + gi * kv_cap)
             self._kv_copy_h.append(self._up(spec))
+            if self._chunk:
+                self._chunk_kv_spec(L, kb, vb)
         pos_ao = self._ws['attn_out'][2]
         self._ao_rows_h = self._up(pos_ao + np.arange(c.n_head) * c.head_dim_kv)
         g.register_row_base_span(self._ao_rows_h, 0, pos_ao, c.n_head, c.head_dim_kv, c.head_dim_kv)
@@ -250,6 +257,77 @@ class DecodeEngine:
         self._sample_repeat_ids = np.zeros(self.SAMPLE_REPEAT_MAX, np.uint32)
         self._sample_repeat_ids_h = self._up(self._sample_repeat_ids)
         self._ws_total = pos
+
+    # ------------------------------------------------------------------ chunked prefill: workspace
+    def _alloc_chunk_slots(self, pos):
+        """Row-major [M, width] slots for a prefill chunk of M tokens and the handles its ops take: one
+        element offset per matrix operand, one row base per token for the row-wise ops, contiguous
+        spans for the element-wise ones, per-token head-row lists for attention."""
+        c, g, M = self.cfg, self.gpu, self._chunk
+        q_dim, k_dim = c.n_head * c.head_dim, c.n_head_kv * c.head_dim_kv
+        d = c.head_dim_kv
+        pos += (-pos) % max(c.head_dim, d)                    # K / V rows are addressed in units of the head size
+        gemma = c.head_dim == c.head_dim_kv and any('attn_q_norm' in n for n in self._norm_names)
+        widths = [('hidden', c.n_embd), ('normed', c.n_embd), ('q', q_dim), ('k', k_dim), ('v', k_dim),
+                  ('attn_out', c.n_head * c.head_dim_kv), ('o_proj', c.n_embd),
+                  ('gate', c.n_ff), ('up', c.n_ff), ('act', c.n_ff), ('ffn_out', c.n_embd), ('normed2', c.n_embd)]
+        if gemma:                                             # rotated [q heads | k heads] of every token
+            widths.append(('qk', q_dim + k_dim))
+        self._cp, self._cw = {}, dict(widths)
+        for name, w in widths:
+            if name in ('k', 'v', 'qk'):
+                pos += (-pos) % d
+            self._cp[name] = pos
+            pos += M * w
+        t = np.arange(M)
+        self._c1 = {n: self._up([p]) for n, p in self._cp.items()}                        # matrix operands
+        self._crow = {n: self._up(self._cp[n] + t * self._cw[n]) for n in ('hidden', 'normed', 'normed2', 'o_proj', 'ffn_out', 'q', 'k')}
+        self._cspan = {n: self._up(np.arange(self._cp[n], self._cp[n] + M * self._cw[n]))
+                       for n in ('hidden', 'o_proj', 'ffn_out', 'gate', 'up', 'act')}
+        self._chunk_qk = gemma
+        qsrc, qw = ('qk', q_dim + k_dim) if gemma else ('q', q_dim)
+        heads = np.arange(c.n_head)
+        self._c_qrows = [self._up(self._cp[qsrc] + i * qw + heads * c.head_dim) for i in range(M)]
+        self._c_aorows = [self._up(self._cp['attn_out'] + i * c.n_head * c.head_dim_kv + heads * c.head_dim_kv) for i in range(M)]
+        if gemma:
+            kh = np.arange(c.n_head_kv)
+            self._c_lq = [self._up(self._cp['q'] + i * q_dim + heads * c.head_dim) for i in range(M)]
+            self._c_lk = [self._up(self._cp['k'] + i * k_dim + kh * d) for i in range(M)]
+            self._c_qkdst = [self._up([self._cp['qk'] + i * (q_dim + k_dim)]) for i in range(M)]
+        self._c_last = self._up(np.zeros(c.n_embd, np.uint32))
+        self._c_zero = self._up([0])
+        self._c_emb_hs = {}
+        self._c_wrows = {}
+        self._c_kvspec = {}
+        if c.emb_scale != 1.0:
+            self._c_embscale_h = self._up(np.full(M * c.n_embd, self._pos_emb_scale))
+        return pos
+
+    def _chunk_kv_spec(self, L, kb, vb):
+        """(source row, cache row) pairs of a whole chunk, token-major, so that a prefix serves a shorter
+        chunk; rows are counted in head-size units from element 0 of the workspace."""
+        c, M, d = self.cfg, self._chunk, self.cfg.head_dim_kv
+        k_dim = c.n_head_kv * d
+        if self._chunk_qk:
+            ksrc, kstride = self._cp['qk'] + c.n_head * c.head_dim, c.n_head * c.head_dim + k_dim
+        else:
+            ksrc, kstride = self._cp['k'], k_dim
+        spec = np.empty((M, 2 * c.n_head_kv, 2), np.uint32)
+        for gi in range(c.n_head_kv):
+            t = np.arange(M)
+            spec[:, 2 * gi, 0] = (ksrc + t * kstride + gi * d) // d
+            spec[:, 2 * gi, 1] = kb // d + gi * self._kv_cap + t
+            spec[:, 2 * gi + 1, 0] = (self._cp['v'] + t * k_dim + gi * d) // d
+            spec[:, 2 * gi + 1, 1] = vb // d + gi * self._kv_cap + t
+        assert ksrc % d == 0 and kstride % d == 0 and self._cp['v'] % d == 0
+        self._c_kvspec[L] = self._up(spec.reshape(-1))
+
+    def _wrows(self, name):
+        """Norm weight handle with one (identical) base per chunk row."""
+        h = self._c_wrows.get(name)
+        if h is None:
+            h = self._c_wrows[name] = self._up(np.full(self._chunk, self._off[name]))
+        return h
 
     # ------------------------------------------------------------------ upload
     def _upload_all(self):
@@ -561,6 +639,107 @@ class DecodeEngine:
         g.map_sample_categorical_dev(ws, sel_h, prob_h, W['sample_rand'][0], W['sample_token'][0], top_k)
         self._sample_token_ready = True
 
+    # ------------------------------------------------------------------ chunked prefill: forward
+    def _forward_chunk(self, toks, pos0, sample=True):
+        """m <= prefill_chunk prompt tokens at positions pos0 .. pos0 + m - 1 in one pass: the row-wise ops
+        over m rows, the projections as [m, K] x [N, K]^T matmuls (the fp16 matrix-core kernel for Q4
+        blocks), RoPE and the KV append for all tokens at once, attention token by token over the growing
+        cache.  Same ops, operands and order per token as `_forward`; the last token's hidden state
+        lands in the decode slots, so decoding continues from there."""
+        c, g, A, ws = self.cfg, self.gpu, self.A, self.WS_MAP
+        m = len(toks)
+        if not self._chunk or m == 0 or m > self._chunk:
+            raise RuntimeError(f"chunk of {m} tokens does not fit prefill_chunk={self._chunk}")
+        E, FF = c.n_embd, c.n_ff
+        q_dim, k_dim = c.n_head * c.head_dim, c.n_head_kv * c.head_dim_kv
+        C1, CR, CS, W = self._c1, self._crow, self._cspan, self._ws
+        toks = np.asarray(toks, np.int64)
+        if self._tied:
+            locs = (np.uint32(self._off[self._lm_name]) + (toks[:, None] * E + np.arange(E)[None, :])).astype(np.uint32)
+            if m in self._c_emb_hs:                   # a handle can be re-uploaded at its own size only
+                g.upload_dev(np.ascontiguousarray(locs.reshape(-1)), handle=self._c_emb_hs[m])
+            else:
+                self._c_emb_hs[m] = self._up(locs.reshape(-1))
+            emb_h = self._c_emb_hs[m]
+        else:
+            rows = np.stack([self.tensors['token_embd.weight'].row(int(t)) for t in toks]).astype(np.float32)
+            if c.emb_scale != 1.0:
+                rows = rows * np.float32(c.emb_scale)
+            g.scatter(ws, np.arange(self._cp['hidden'], self._cp['hidden'] + m * E, dtype=np.uint32), rows.reshape(-1))
+        last = self._cp['hidden'] + (m - 1) * E
+        g.upload_dev(np.arange(last, last + E, dtype=np.uint32), handle=self._c_last)
+
+        def mm(src, name, dst, K, N):
+            fn = g.map_matmul_t_xq8_dev if self._kind[name] == 'q8' else g.map_matmul_t_xq4_dev
+            fn(ws, self._map_of[name], C1[src], self._wh[name], C1[dst], m, K, N)
+
+        g.batch_begin()
+        if self._tied:
+            src_h, _, _, _ = g.map_gather_dev(self._map_of[self._lm_name], emb_h, m * E)
+            g.map_scatter_dev(ws, CS['hidden'], m * E, src_h)
+            if c.emb_scale != 1.0:
+                g.map_broadcast_dev(ws, A.OP_MUL, CS['hidden'], self._c_embscale_h, CS['hidden'], m * E)
+        scale = float(1.0 / np.sqrt(c.head_dim))
+        for L in range(c.n_layer):
+            p = f'blk.{L}'
+            freq = c.rope_base_global if c.is_global(L) else c.rope_base_local
+            g.map_rmsnorm_dev(ws, CR['hidden'], self._wrows(f'{p}.attn_norm.weight'), CR['normed'], m, E, c.norm_eps)
+            mm('normed', f'{p}.attn_q.weight', 'q', E, q_dim)
+            mm('normed', f'{p}.attn_k.weight', 'k', E, k_dim)
+            mm('normed', f'{p}.attn_v.weight', 'v', E, k_dim)
+            if self._chunk_qk:
+                qn, kn = self._wh[f'{p}.attn_q_norm.weight'], self._wh[f'{p}.attn_k_norm.weight']
+                for t in range(m):
+                    g.map_qk_norm_rope_x_dev(ws, ws, self._c_lq[t], qn, self._c_lk[t], kn, self._c_qkdst[t],
+                                             c.n_head, c.head_dim, c.n_head_kv, c.head_dim_kv, pos0 + t, freq)
+            else:
+                g.map_rope_dev(ws, CR['q'], CR['q'], m, c.n_head, c.head_dim, pos0, freq)
+                g.map_rope_dev(ws, CR['k'], CR['k'], m, c.n_head_kv, c.head_dim_kv, pos0, freq)
+            g.map_row_copy_offset_dev(ws, self._c_kvspec[L], self._c_zero, pos0, 2 * c.n_head_kv * m, c.head_dim_kv)
+            for t in range(m):
+                seq = pos0 + t + 1
+                g.map_matmul_t_dev(ws, self._c_qrows[t], self._k_locs_h[L], self._scores_row_h, 1, c.head_dim, seq, c.n_head)
+                g.map_attn_softmax_value_dev(ws, self._scores_row_h, self._v_locs_h[L], self._c_aorows[t], c.n_head, seq,
+                                             c.head_dim_kv, scale, float(c.attn_softcap))
+            mm('attn_out', f'{p}.attn_output.weight', 'o_proj', c.n_head * c.head_dim_kv, E)
+            pan = f'{p}.post_attention_norm.weight'
+            if pan in self._wh:
+                g.map_rmsnorm_add_dev(ws, CR['o_proj'], self._wrows(pan), CR['hidden'], CR['hidden'], m, E, c.norm_eps)
+            else:
+                g.map_op2_dev(ws, A.OP_ADD, CS['hidden'], CS['o_proj'], CS['hidden'], m * E)
+            g.map_rmsnorm_dev(ws, CR['hidden'], self._wrows(f'{p}.ffn_norm.weight'), CR['normed2'], m, E, c.norm_eps)
+            mm('normed2', f'{p}.ffn_gate.weight', 'gate', E, FF)
+            mm('normed2', f'{p}.ffn_up.weight', 'up', E, FF)
+            g.map_op2_dev(ws, A.OP_GEGLU if c.ffn_act == 'gelu' else A.OP_SWIGLU, CS['gate'], CS['up'], CS['act'], m * FF)
+            mm('act', f'{p}.ffn_down.weight', 'ffn_out', FF, E)
+            pfn = f'{p}.post_ffw_norm.weight'
+            if pfn in self._wh:
+                g.map_rmsnorm_add_dev(ws, CR['ffn_out'], self._wrows(pfn), CR['hidden'], CR['hidden'], m, E, c.norm_eps)
+            else:
+                g.map_op2_dev(ws, A.OP_ADD, CS['hidden'], CS['ffn_out'], CS['hidden'], m * E)
+        # the last token's hidden state -> the decode slots; output norm and LM head as in a decode step
+        src_h, _, _, _ = g.map_gather_dev(ws, self._c_last, E)
+        g.map_scatter_dev(ws, W['hidden'][0], E, src_h)
+        if sample:
+            self._rms(W['hidden'][0], 'output_norm.weight', W['normed'][0], 1, E)
+            fn = (g.map_matvec_argmax_t_xq8_dev if self._kind[self._lm_name] == 'q8' else g.map_matvec_argmax_t_xq4_dev)
+            fn(ws, self._map_of[self._lm_name], W['normed'][0], self._wh[self._lm_name], W['sample_fused_idx'][0],
+               W['sample_fused_val'][0], W['sample_token'][0], E, c.n_vocab, self._rows_per_group)
+            self._sample_token_ready = True
+        g.batch_end()
+
+    def prefill(self, token_ids, pos0=0, sample=True):
+        """The prompt in chunks of `prefill_chunk` tokens (token by token when the engine was built
+        without one); the LM head runs after the last token only."""
+        n = len(token_ids)
+        if not self._chunk:
+            for i, t in enumerate(token_ids):
+                self._forward(int(t), pos0 + i, sample=sample and i == n - 1)
+            return
+        for lo in range(0, n, self._chunk):
+            hi = min(n, lo + self._chunk)
+            self._forward_chunk(token_ids[lo:hi], pos0 + lo, sample=sample and hi == n)
+
     def read_token(self):
         # reference engine.py:1979-1981: token id crosses the boundary as float32
         tok = self.gpu.gather(self.WS_MAP, self._sample_locs).view(np.float32)
@@ -596,8 +775,11 @@ class DecodeEngine:
         hist = [int(t) for t in token_ids]
         tp = time.perf_counter()
         last = len(token_ids) - 1
-        for i, t in enumerate(token_ids):
-            self._forward(int(t), i, sample=(i == last), sample_cfg=config, sample_prev=hist)
+        if self._chunk and not sampled:
+            self.prefill([int(t) for t in token_ids])
+        else:
+            for i, t in enumerate(token_ids):
+                self._forward(int(t), i, sample=(i == last), sample_cfg=config, sample_prev=hist)
         self.gpu.sync()
         t_pre = time.perf_counter() - tp
         out, ttimes = [], []

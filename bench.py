@@ -252,6 +252,9 @@ def main():
     ap.add_argument("--workload", default="gemma3-1b", choices=["gemma3-1b", "llama3-8b"])
     ap.add_argument("--prompt", type=int, default=None, help="prompt length (default 512 / 3840)")
     ap.add_argument("--scheduler", default="level_batched", choices=["legacy", "level_batched"])
+    ap.add_argument("--prefill-chunk", type=int, default=0,
+                    help="prompt in chunks of this many tokens on the matrix-core matmul (0: token by token, as the "
+                         "reference does; the timed region is the decode loop either way)")
     ap.add_argument("--only", default=None, choices=["roofline", "gemv", "probe", "attention", "gemm"],
                     help="roofline: just the 28672x4096 GEMV (one kernel row in a rocprofv3 --stats table); "
                          "gemv: that shape, 4096x4096 and 4096x14336; probe: plain read/copy kernels of known "
@@ -300,7 +303,7 @@ def main():
     gpu = A.init()
     t0 = time.perf_counter()
     eng = DecodeEngine(gpu, cfg, tensors, A=A, kv_cap=kv_cap, kv_fp16=True,
-                       fusion_scheduler_mode=args.scheduler)
+                       fusion_scheduler_mode=args.scheduler, prefill_chunk=args.prefill_chunk)
     gpu.sync()
     log(f"uploaded in {time.perf_counter() - t0:.1f}s; maps {sorted(eng._q4_sizes)}")
 
@@ -308,11 +311,10 @@ def main():
     prompt = [int(t) for t in rng.integers(0, cfg.n_vocab, n_prompt)]
     eng.reset()
     t0 = time.perf_counter()
-    for i, t in enumerate(prompt):
-        eng._forward(t, i, sample=(i == n_prompt - 1))
+    eng.prefill(prompt)
     gpu.sync()
     prefill_s = time.perf_counter() - t0
-    log(f"prefill {n_prompt} tokens (token by token): {prefill_s:.2f}s")
+    log(f"prefill {n_prompt} tokens ({'chunks of ' + str(args.prefill_chunk) if args.prefill_chunk else 'token by token'}): {prefill_s:.2f}s")
 
     tokens, pos = [], n_prompt
     for _ in range(args.warmup):

@@ -90,3 +90,22 @@ def test_sampled_generation_draws_from_the_top_k_of_the_reference_logits(arch):
         assert tok in top, (step, tok, top)
         hist.append(tok)
         logits = ref.forward(tok, len(prompt) + step)
+
+
+@pytest.mark.parametrize("arch", ["gemma3", "llama"])
+@pytest.mark.parametrize("chunk", [3, 7, 16])
+def test_chunked_prefill_equals_token_by_token(arch, chunk):
+    """The prompt run as [m, K] matmuls and m-row norms with attention token by token leaves the same
+    KV cache and hidden state as m single-token steps (exactly, on the oracle), also when the last chunk
+    is short and when the chunk is longer than the prompt."""
+    cfg = synth.tiny_config(arch, n_layer=2, n_embd=64, n_head=4, n_head_kv=2, head_dim=32, n_ff=96, n_vocab=160)
+    tensors = synth.make_model(cfg, seed=3, sigma=0.3)
+    prompt = [5, 17, 3, 101, 64, 9, 33]
+    outs = []
+    for m in (0, chunk):
+        eng = DecodeEngine(oracle.init(), cfg, tensors, A=A, kv_cap=32, kv_fp16=True, prefill_chunk=m)
+        out, _ = eng.generate(prompt, GenerationConfig(max_tokens=6))
+        kv = eng.gpu.gather(0, np.arange(eng._kv_start, eng._kv_start + cfg.n_layer * eng._kv_per_layer, dtype=np.uint32))
+        outs.append((out, eng.read_slot('hidden'), kv))
+    assert outs[0][0] == outs[1][0]
+    assert np.array_equal(outs[0][1], outs[1][1]) and np.array_equal(outs[0][2], outs[1][2])
