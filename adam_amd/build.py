@@ -7,7 +7,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libadamah_hip.so")
-SOURCES = ["runtime.hip", "gemv_q.hip", "gemv_mfma.hip", "gemm_q4_mfma.hip", "fuse.hip", "norm_rope.hip", "rowprep.hip", "attention.hip", "attn_decode.hip", "elementwise.hip", "sampling.hip", "topk_fused.hip", "fused_proj.hip", "probe.hip"]
+SOURCES = ["runtime.hip", "gemv_q.hip", "gemv_mfma.hip", "gemm_q4_mfma.hip", "fuse.hip", "norm_rope.hip", "rowprep.hip", "attention.hip", "attn_decode.hip", "attn_prefill.hip", "elementwise.hip", "sampling.hip", "topk_fused.hip", "fused_proj.hip", "probe.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", "-ffp-contract=off",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result", "-Wno-unused-value"]
 # gemv_mfma.hip draws a ticket with one atomic per workgroup and looks at it much later; the

@@ -168,6 +168,7 @@ int launch_scores(const PendOp& sc);
 int launch_attn(const PendOp* sc, const PendOp& at, bool leave_partials, AttnPartials* ap);
 int launch_attn_combine(const PendOp& at, const AttnPartials& ap);
 bool attn_foldable(const PendOp& sc, const PendOp& at);
+size_t launch_attn_chunk(const std::vector<PendOp>& q, size_t i, int* rc);   // attn_prefill.hip
 
 inline void count_launch(int n = 1) { g.stats.dispatch += n; g.stats.barrier += n; g.stats.last_batch_dispatch += n; }
 int check_launch();                              // hipGetLastError -> ADAMAH code

@@ -13,6 +13,7 @@
 //   GEMV(-> y); ADD(r, y -> d)                            -> GEMV that also stores r + y
 //   GEMV(-> [g; u]); GEGLU/SWIGLU(g, u -> t)              -> GEMV over paired rows that also stores t
 //   GEMV(x, W1 -> y1); GEMV(x, W2 -> y2), W2 after W1, y2 after y1 -> one GEMV over the stacked rows
+//   (scores; softmax . V) of tokens t, t+1, ... over one cache      -> one causal launch (attn_prefill.hip)
 //   RoPE(q); RoPE(k) | QK-norm+RoPE; row copy (KV append)  -> one launch of row tasks (rowprep.hip)
 //
 // Every folded op still stores its own result where it would have stored it alone, so the contents
@@ -131,6 +132,12 @@ void flush_pending() {
       int rc = 0;
       i += launch_row_run(q, i, &rc);
       continue;
+    }
+    if (p.kind == PK_SCORES) {
+      // a prefill chunk: the attention of consecutive tokens over one growing cache, one launch
+      int rc = 0;
+      const size_t used = launch_attn_chunk(q, i, &rc);
+      if (used) { i += used; continue; }
     }
     if (p.kind == PK_SCORES || p.kind == PK_ATTN) {
       // decode attention: scores computed inside the softmax . V launch; the merge of the sequence

@@ -102,3 +102,105 @@ def test_gqa_heads_with_equal_queries_agree(hip):
     for g0 in range(Hkv):
         for j in range(1, Hq // Hkv):
             assert np.array_equal(out[g0 * 4], out[g0 * 4 + j])
+
+
+def chunk_case(g, q, K, V, seq0, cap_len, scale, softcap, gap=0):
+    """m tokens' (scores, softmax.V) pairs in one batch: q [m, Hq, d]; token t sees seq0 + t cache rows.
+    Layout: score rows, q [m][Hq][d], out [m][Hq][d] (+ gap floats between tokens), fp16 KV region."""
+    m, Hq, d = q.shape
+    Hkv = K.shape[0]
+    gs = Hq // Hkv
+    sc_sz = Hq * cap_len
+    q_pos = sc_sz
+    out_pos = q_pos + m * Hq * d
+    o_stride = Hq * d + gap
+    kv_start = (out_pos + m * o_stride + d - 1) // d * d
+    step = cap_len * d
+    f32map(g, 0, kv_start + 2 * Hkv * step, None)
+    g.kv_cache_fp16(0, kv_start, 2 * Hkv * step)
+    put(g, 0, q_pos, q)
+    for h in range(Hkv):
+        put(g, 0, kv_start + h * step, K[h])
+        put(g, 0, kv_start + (Hkv + h) * step, V[h])
+    heads = np.arange(Hq) // gs
+    k_locs, v_locs = up(g, kv_start + heads * step), up(g, kv_start + (Hkv + heads) * step)
+    s_rows = up(g, np.arange(Hq) * cap_len)
+    qh = [up(g, q_pos + t * Hq * d + np.arange(Hq) * d) for t in range(m)]
+    oh = [up(g, out_pos + t * o_stride + np.arange(Hq) * d) for t in range(m)]
+    g.batch_begin()
+    for t in range(m):
+        g.map_matmul_t_dev(0, qh[t], k_locs, s_rows, 1, d, seq0 + t, Hq)
+        g.map_attn_softmax_value_dev(0, s_rows, v_locs, oh[t], Hq, seq0 + t, d, scale, softcap)
+    g.batch_end()
+    launches = g.get_last_barrier_count() if hasattr(g, "get_last_barrier_count") else None
+    out = np.stack([read(g, 0, out_pos + t * o_stride, Hq * d).reshape(Hq, d) for t in range(m)])
+    scores = np.stack([read(g, 0, h * cap_len, seq0 + m - 1) for h in range(Hq)])
+    return out, scores, launches
+
+
+@pytest.mark.parametrize("m,seq0,Hq,Hkv,d,softcap,gap", [
+    (40, 1, 4, 1, 256, 50.0, 0),        # Gemma-3-1B heads, a prompt from position 0, last tile short
+    (64, 200, 32, 8, 128, 0.0, 0),      # Llama-3-8B heads, second chunk of a prompt
+    (17, 3, 8, 2, 64, 0.0, 8),          # head size 64, padded output rows
+    (2, 5, 4, 4, 128, 30.0, 0),         # the shortest run
+])
+def test_prefill_chunk_is_one_causal_launch(hip, m, seq0, Hq, Hkv, d, softcap, gap):
+    """The per-token pairs of a prompt chunk, issued in one batch, run as one launch and give what the
+    oracle gives token by token: outputs per token and head within 1e-3 relative L2, and the score rows
+    hold the last token's raw scores."""
+    rng = np.random.default_rng(m * 1000 + seq0)
+    cap_len = seq0 + m + 7
+    q = rng.standard_normal((m, Hq, d)).astype(np.float32)
+    K = rng.standard_normal((Hkv, cap_len, d)).astype(np.float32)
+    V = rng.standard_normal((Hkv, cap_len, d)).astype(np.float32)
+    scale = float(1.0 / np.sqrt(d))
+    note(f"attention chunk m={m} seq0={seq0} {Hq}q/{Hkv}kv d={d}")
+    out, scores, launches = chunk_case(hip, q, K, V, seq0, cap_len, scale, softcap, gap)
+    ref, ref_scores, _ = chunk_case(oracle.init(), q, K, V, seq0, cap_len, scale, softcap, gap)
+    assert launches == 1, launches
+    for t in range(m):
+        for h in range(Hq):
+            assert rel_l2(out[t, h], ref[t, h]) < TOL, (t, h)
+    assert rel_l2(scores, ref_scores) < 1e-5
+
+
+@pytest.mark.parametrize("layout,expect", [("hole", 2), ("irregular", 3)])
+def test_prefill_chunk_splits_or_falls_back_when_tokens_do_not_line_up(hip, layout, expect):
+    """A hole in the query rows after the third token: two chunk launches.  No common stride at all: the
+    tokens pair up (any two tokens have a stride), three launches.  Same results either way."""
+    rng = np.random.default_rng(9)
+    m, Hq, Hkv, d, seq0 = 6, 4, 2, 128, 4
+    cap_len = 32
+    q = rng.standard_normal((m, Hq, d)).astype(np.float32)
+    K = rng.standard_normal((Hkv, cap_len, d)).astype(np.float32)
+    V = rng.standard_normal((Hkv, cap_len, d)).astype(np.float32)
+    outs = []
+    for g in (hip, oracle.init()):
+        note("attention chunk fallback")
+        sc_sz = Hq * cap_len
+        q_pos = sc_sz
+        out_pos = q_pos + (3 * m) * Hq * d
+        kv_start = (out_pos + m * Hq * d + d - 1) // d * d
+        step = cap_len * d
+        f32map(g, 0, kv_start + 2 * Hkv * step, None)
+        g.kv_cache_fp16(0, kv_start, 2 * Hkv * step)
+        if layout == "hole":
+            qoff = [t * Hq * d + (Hq * d if t >= 3 else 0) for t in range(m)]
+        else:
+            qoff = [2 * t * Hq * d + 8 * t * t for t in range(m)]
+        for t in range(m):
+            put(g, 0, q_pos + qoff[t], q[t])
+        for h in range(Hkv):
+            put(g, 0, kv_start + h * step, K[h]); put(g, 0, kv_start + (Hkv + h) * step, V[h])
+        heads = np.arange(Hq) // (Hq // Hkv)
+        k_locs, v_locs, s_rows = up(g, kv_start + heads * step), up(g, kv_start + (Hkv + heads) * step), up(g, np.arange(Hq) * cap_len)
+        g.batch_begin()
+        for t in range(m):
+            g.map_matmul_t_dev(0, up(g, q_pos + qoff[t] + np.arange(Hq) * d), k_locs, s_rows, 1, d, seq0 + t, Hq)
+            g.map_attn_softmax_value_dev(0, s_rows, v_locs, up(g, out_pos + t * Hq * d + np.arange(Hq) * d), Hq, seq0 + t, d,
+                                         0.1, 0.0)
+        g.batch_end()
+        if g is hip:
+            assert g.get_last_barrier_count() == expect
+        outs.append(read(g, 0, out_pos, m * Hq * d))
+    assert rel_l2(outs[0], outs[1]) < TOL
