@@ -661,6 +661,15 @@ int launch_attn_combine(const PendOp& at, const AttnPartials& ap) {
   return check_launch();
 }
 
+// Merge of the sequence slices for output rows listed in device memory.
+int launch_attn_combine_dev(Map* m, const float* partial, const uint32_t* lo_dev, uint32_t n_ops, uint32_t value_dim,
+                            uint32_t n_splits) {
+  k_attn_combine<<<dim3(n_ops, cdiv(value_dim, 32)), 256, 0, g.stream>>>((float*)m->buf, partial, lo_dev, value_dim, n_splits,
+                                                                        m->n_elems);
+  count_launch();
+  return check_launch();
+}
+
 }  // namespace adamah
 
 #ifdef ADAMAH_TRACE

@@ -25,6 +25,8 @@
 // each of those writes back and invalidates the L2 of its XCD and the kernel got 4x slower.)
 #include "attn_common.h"
 #include <algorithm>
+#include <utility>
+#include <vector>
 
 namespace adamah {
 
@@ -62,7 +64,8 @@ __device__ __forceinline__ float row16_sum(float v) {
 template <int D, int G, int NW, bool PF>
 __global__ void __launch_bounds__(NW * 64)
 k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift, const AttdBases bs,
-              uint32_t row_size, float scale, float cap, uint32_t n_splits, uint32_t chunk, float* partial) {
+              uint32_t row_size, float scale, float cap, uint32_t n_splits, uint32_t chunk, float* partial,
+              const uint32_t* __restrict__ ext) {
   constexpr int NI = D / 32;           // 16-byte K loads per lane and tile
   constexpr int DPL = D / 64;          // V dims per lane (every lane sees all 16 rows of the tile)
   constexpr int DW = DPL > 2 ? DPL / 2 : 1;
@@ -82,8 +85,13 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
   const uint32_t split = blockIdx.x, group = blockIdx.y, op0 = group * G;
   const uint32_t t0 = split * chunk, t1 = min(row_size, t0 + chunk);
   // wave-uniform bases plus 32-bit byte offsets: the V row of a load is the same for all lanes
-  const char* kbase = (const char*)(kv + ((uint64_t)bs.kb[group] - kv_shift));
-  const char* vbase = (const char*)(kv + ((uint64_t)bs.vb[group] - kv_shift));
+  // `ext` (several sets of heads in one launch, too many for the argument block): the bases come from
+  // device memory as [q | score rows | out rows] per head, then [K | V] per group; a score row of
+  // 0xFFFFFFFF is not stored.
+  const uint32_t n_all = gridDim.y * (uint32_t)G;
+  const uint32_t *e_q = ext, *e_sc = ext + n_all, *e_o = ext + 2u * n_all, *e_kb = ext + 3u * n_all, *e_vb = e_kb + gridDim.y;
+  const char* kbase = (const char*)(kv + ((uint64_t)(ext ? e_kb[group] : bs.kb[group]) - kv_shift));
+  const char* vbase = (const char*)(kv + ((uint64_t)(ext ? e_vb[group] : bs.vb[group]) - kv_shift));
   const uint32_t klane = 16u * kc, vlane = 2u * (uint32_t)DPL * lane;
 
   auto fetch = [&](uint4 (&kr)[NI], uint32_t (&vr)[16][DW], uint32_t rb) {
@@ -113,7 +121,7 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
     __syncthreads();
     for (uint32_t i = tid; i < (uint32_t)(G * D); i += NT) {   // a wave's 64 elements belong to one head
       const uint32_t hq = (uint32_t)__builtin_amdgcn_readfirstlane((int)(i / D));   // scalar: read from the arguments
-      const float x = data[(uint64_t)bs.q[op0 + hq] + i % D];
+      const float x = data[(uint64_t)(ext ? e_q[op0 + hq] : bs.q[op0 + hq]) + i % D];
       qs[i] = x;
       float m = fabsf(x);
 #pragma unroll
@@ -154,8 +162,8 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
     inv_s[r] = hval[r] ? qinv[4u * kc + r] : 0.f;
     // scalar reads of the arguments, then a per-lane choice
     crow[r] = 0u;
-    if (r < G) crow[r] = bs.sc[op0 + r];
-    if (G > 4 && kc == 1u) crow[r] = bs.sc[op0 + (4 + r) % G];
+    if (r < G) crow[r] = ext ? e_sc[op0 + r] : bs.sc[op0 + r];
+    if (G > 4 && kc == 1u) crow[r] = ext ? e_sc[op0 + (4 + r) % G] : bs.sc[op0 + (4 + r) % G];
     m_run[r] = ATTD_NEG;
     l_run[r] = 0.f;
   }
@@ -184,7 +192,7 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
 #pragma unroll
     for (int r = 0; r < 4; r++) {
       const float raw = ((s0[r] + s2[r]) + (s1[r] + s3[r])) * inv_s[r];
-      if (rok && hval[r]) out[(uint64_t)crow[r] + row] = raw;
+      if (rok && hval[r] && crow[r] != 0xFFFFFFFFu) out[(uint64_t)crow[r] + row] = raw;
       v[r] = rok && hval[r] ? prep(raw, scale, cap) : ATTD_NEG;
       mt[r] = row16_max(v[r]);
     }
@@ -283,7 +291,7 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
       L = fmaf(mlbuf[w][h][1], e, L);
     }
     if (n_splits == 1u) {
-      out[(uint64_t)bs.o[op0 + h] + d] = o * (1.0f / L);
+      out[(uint64_t)(ext ? e_o[op0 + h] : bs.o[op0 + h]) + d] = o * (1.0f / L);
     } else {
       float* pp = partial + ((uint64_t)(op0 + h) * n_splits + split) * (D + 2);
       pp[2 + d] = o;
@@ -295,20 +303,20 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
 
 template <int D, int NW, bool PF>
 static void launch_dg(uint32_t G, dim3 grid, const AttnDecodeArgs& a, const AttdBases& bs, uint32_t n_splits,
-                      uint32_t chunk) {
+                      uint32_t chunk, const uint32_t* ext) {
 #define ADL(GG)                                                                                       \
   k_attn_decode<D, GG, NW, PF><<<grid, NW * 64, 0, g.stream>>>(a.data, a.data, a.kv, a.kv_shift, bs, a.row_size, \
-                                                               a.scale, a.cap, n_splits, chunk, g.attn_scratch)
+                                                               a.scale, a.cap, n_splits, chunk, g.attn_scratch, ext)
   if (G == 1) ADL(1); else if (G == 2) ADL(2); else if (G == 4) ADL(4); else ADL(8);
 #undef ADL
 }
 
 template <int D>
 static void launch_d(uint32_t G, uint32_t nw, bool pf, dim3 grid, const AttnDecodeArgs& a, const AttdBases& bs,
-                     uint32_t n_splits, uint32_t chunk) {
-  if (nw == 8) launch_dg<D, 8, false>(G, grid, a, bs, n_splits, chunk);
-  else if (pf) launch_dg<D, 4, true>(G, grid, a, bs, n_splits, chunk);
-  else launch_dg<D, 4, false>(G, grid, a, bs, n_splits, chunk);
+                     uint32_t n_splits, uint32_t chunk, const uint32_t* ext = nullptr) {
+  if (nw == 8) launch_dg<D, 8, false>(G, grid, a, bs, n_splits, chunk, ext);
+  else if (pf) launch_dg<D, 4, true>(G, grid, a, bs, n_splits, chunk, ext);
+  else launch_dg<D, 4, false>(G, grid, a, bs, n_splits, chunk, ext);
 }
 
 bool launch_attn_decode(const AttnDecodeArgs& a, AttnPartials* ap, bool* left, int* rc) {
@@ -361,6 +369,127 @@ bool launch_attn_decode(const AttnDecodeArgs& a, AttnPartials* ap, bool* left, i
   *ap = AttnPartials{g.attn_scratch, *rc == 0 ? n_splits : 1u, D, n_ops, 0};
   *left = leave;
   return true;
+}
+
+
+// ---- several sequences in lockstep ----------------------------------------------------------------
+// A batched decode step issues one (scores, softmax . V) pair per sequence: same length, head count and
+// parameters, the same score rows, but queries, outputs and KV cache of its own.  A run of such pairs
+// becomes one launch of the kernel above over all their heads (bases in device memory); only the
+// last pair stores raw scores, which is what the shared score rows hold after the pairs ran one by one.
+static uint32_t* g_ext_buf = nullptr;
+static size_t g_ext_cap = 0;   // words
+
+void attn_decode_release() {
+  if (g_ext_buf) hipFree(g_ext_buf);
+  g_ext_buf = nullptr;
+  g_ext_cap = 0;
+}
+
+size_t launch_attn_batch(const std::vector<PendOp>& q, size_t i, int* rc) {
+  *rc = ADAMAH_OK;
+  if (tuning("ADAMAH_ATTN_BATCH", 1) == 0) return 0;
+  const size_t n = q.size();
+  if (i + 3 >= n || !attn_foldable(q[i], q[i + 1])) return 0;
+  const PendOp &s0 = q[i], &a0 = q[i + 1];
+  Map* mp = get_f32_map(a0.map_act);
+  const uint32_t H = a0.rpg, D = a0.k, rows = a0.n;
+  if (!mp || !mp->kv16 || H == 0 || s0.k != D || (D != 64 && D != 128 && D != 256) || rows == 0) return 0;
+  const uint32_t* sc0 = res_host(s0.h[2], H);
+  if (!sc0) return 0;
+  std::vector<const uint32_t*> hq, hk, hv, ho;
+  size_t B = 0;
+  while (i + 2 * B + 1 < n) {
+    const PendOp &st = q[i + 2 * B], &at = q[i + 2 * B + 1];
+    if (!attn_foldable(st, at) || st.map_act != s0.map_act || st.rpg != H || st.k != D || at.k != D || st.n != rows ||
+        at.eps != a0.eps || at.f2 != a0.f2)
+      break;
+    const uint32_t *qt = res_host(st.h[0], H), *kt = res_host(st.h[1], H), *ct = res_host(st.h[2], H);
+    const uint32_t *vt = res_host(at.h[1], H), *ot = res_host(at.h[2], H);
+    if (!qt || !kt || !ct || !vt || !ot) break;
+    bool same = true;
+    for (uint32_t h = 0; same && h < H; h++) same = ct[h] == sc0[h];
+    if (!same) break;
+    hq.push_back(qt); hk.push_back(kt); hv.push_back(vt); ho.push_back(ot);
+    B++;
+  }
+  if (B < 2) return 0;
+  // group structure of the first pair, required of all
+  uint32_t G = 1;
+  while (G < H && G < 8 && hk[0][G] == hk[0][0] && hv[0][G] == hv[0][0]) G++;
+  if (G != 1 && G != 2 && G != 4 && G != 8) G = G > 4 ? 4 : G == 3 ? 2 : 1;
+  while (G > 1 && H % G) G >>= 1;
+  const uint64_t need_rows = (uint64_t)rows * D;
+  for (size_t b = 0; b < B; b++)
+    for (uint32_t op = 0; op < H; op++) {
+      const uint32_t o0 = op - op % G;
+      if (hk[b][op] != hk[b][o0] || hv[b][op] != hv[b][o0]) return 0;
+      if (hk[b][op] < mp->kv_start || hv[b][op] < mp->kv_start || (hk[b][op] - mp->kv_start) % 8u || (hv[b][op] - mp->kv_start) % 8u) return 0;
+      if (hk[b][op] - mp->kv_start + need_rows > mp->kv_count || hv[b][op] - mp->kv_start + need_rows > mp->kv_count) return 0;
+      if (!in_range(hq[b][op], D, mp->n_elems) || !in_range(ho[b][op], D, mp->n_elems)) return 0;
+    }
+  // no pair may write what another reads: outputs apart from all queries and from each other
+  {
+    std::vector<std::pair<uint64_t, uint64_t>> qs, os;
+    for (size_t b = 0; b < B; b++)
+      for (uint32_t op = 0; op < H; op++) { qs.push_back({hq[b][op], (uint64_t)hq[b][op] + D}); os.push_back({ho[b][op], (uint64_t)ho[b][op] + D}); }
+    std::sort(os.begin(), os.end());
+    for (size_t k = 1; k < os.size(); k++) if (os[k].first < os[k - 1].second) return 0;
+    std::sort(qs.begin(), qs.end());
+    size_t j = 0;
+    for (const auto& o : os) {
+      while (j < qs.size() && qs[j].second <= o.first) j++;
+      if (j < qs.size() && qs[j].first < o.second) return 0;
+    }
+    const uint64_t kv0 = mp->kv_start, kv1 = mp->kv_start + mp->kv_count;
+    for (const auto& o : os) if (!(o.second <= kv0 || kv1 <= o.first)) return 0;
+    for (uint32_t h = 0; h < H; h++) {
+      const uint64_t s_lo = sc0[h], s_hi = (uint64_t)sc0[h] + rows;
+      if (!in_range(sc0[h], rows, mp->n_elems) || !(s_hi <= kv0 || kv1 <= s_lo)) return 0;
+      for (const auto& o : os) if (!(o.second <= s_lo || s_hi <= o.first)) return 0;
+      for (const auto& qq : qs) if (!(qq.second <= s_lo || s_hi <= qq.first)) return 0;
+    }
+  }
+  const uint32_t n_all = (uint32_t)(B * H), n_groups = n_all / G;
+  // slices as for a single pair, sized for all the groups
+  const uint32_t target = (uint32_t)std::max(1, tuning("ADAMAH_ATTN_WAVES", 4 * g.n_cu));
+  const uint64_t tiles = (uint64_t)n_groups * cdiv(rows, 16u);
+  uint32_t nw = (tiles <= target && G * D <= 1024u) ? 8u : 4u;
+  const uint32_t step = nw * 16u;
+  uint32_t chunk = step * std::max<uint32_t>(1u, cdiv(tiles, target));
+  while (cdiv(rows, chunk) > ATTD_MAX_SPLITS) chunk += step;
+  if (nw == 8u && chunk > step) nw = 4u;
+  const bool pf = chunk > nw * 16u;
+  const uint32_t n_splits = cdiv(rows, chunk);
+  if (n_groups > 65535u || (uint64_t)n_all * n_splits * (D + 2) > g.attn_scratch_floats) return 0;
+  const size_t words = 3 * (size_t)n_all + 2 * (size_t)n_groups;
+  if (words > g_ext_cap) {
+    if (g_ext_buf) { hipStreamSynchronize(g.stream); hipFree(g_ext_buf); }
+    g_ext_cap = std::max<size_t>(words, 4096);
+    if (hipMalloc((void**)&g_ext_buf, g_ext_cap * 4) != hipSuccess) { g_ext_buf = nullptr; g_ext_cap = 0; *rc = ADAMAH_ERR_MEMORY; return 2 * B; }
+  }
+  std::vector<uint32_t> ext(words);
+  for (size_t b = 0; b < B; b++)
+    for (uint32_t op = 0; op < H; op++) {
+      const size_t k = b * H + op;
+      ext[k] = hq[b][op];
+      ext[n_all + k] = b + 1 == B ? sc0[op] : 0xFFFFFFFFu;
+      ext[2 * (size_t)n_all + k] = ho[b][op];
+      if (op % G == 0) { ext[3 * (size_t)n_all + k / G] = hk[b][op]; ext[3 * (size_t)n_all + n_groups + k / G] = hv[b][op]; }
+    }
+  if ((*rc = h2d(g_ext_buf, ext.data(), words * 4)) != ADAMAH_OK) return 2 * B;
+  AttnDecodeArgs da = {(float*)mp->buf, mp->kv16, mp->kv_start, nullptr, nullptr, nullptr, nullptr, nullptr,
+                       nullptr, nullptr, nullptr, nullptr, nullptr, n_all, D, rows, a0.eps, a0.f2, false, 0};
+  AttdBases bs = {};
+  dim3 grid(n_splits, n_groups);
+  if (D == 64) launch_d<64>(G, nw, pf, grid, da, bs, n_splits, chunk, g_ext_buf);
+  else if (D == 128) launch_d<128>(G, nw, pf, grid, da, bs, n_splits, chunk, g_ext_buf);
+  else launch_d<256>(G, nw, pf, grid, da, bs, n_splits, chunk, g_ext_buf);
+  count_launch();
+  *rc = check_launch();
+  if (*rc == ADAMAH_OK && n_splits > 1)
+    *rc = launch_attn_combine_dev(mp, g.attn_scratch, g_ext_buf + 2 * (size_t)n_all, n_all, D, n_splits);
+  return 2 * B;
 }
 
 }  // namespace adamah

@@ -169,6 +169,10 @@ int launch_attn(const PendOp* sc, const PendOp& at, bool leave_partials, AttnPar
 int launch_attn_combine(const PendOp& at, const AttnPartials& ap);
 bool attn_foldable(const PendOp& sc, const PendOp& at);
 size_t launch_attn_chunk(const std::vector<PendOp>& q, size_t i, int* rc);   // attn_prefill.hip
+size_t launch_attn_batch(const std::vector<PendOp>& q, size_t i, int* rc);   // attn_decode.hip
+int launch_attn_combine_dev(Map* m, const float* partial, const uint32_t* lo_dev, uint32_t n_ops, uint32_t value_dim,
+                            uint32_t n_splits);
+void attn_decode_release();
 
 inline void count_launch(int n = 1) { g.stats.dispatch += n; g.stats.barrier += n; g.stats.last_batch_dispatch += n; }
 int check_launch();                              // hipGetLastError -> ADAMAH code

@@ -136,7 +136,8 @@ void flush_pending() {
     if (p.kind == PK_SCORES) {
       // a prefill chunk: the attention of consecutive tokens over one growing cache, one launch
       int rc = 0;
-      const size_t used = launch_attn_chunk(q, i, &rc);
+      size_t used = launch_attn_chunk(q, i, &rc);
+      if (!used) used = launch_attn_batch(q, i, &rc);   // or one token of several sequences in lockstep
       if (used) { i += used; continue; }
     }
     if (p.kind == PK_SCORES || p.kind == PK_ATTN) {

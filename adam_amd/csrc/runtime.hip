@@ -370,6 +370,7 @@ void adamah_shutdown(void) { ADAMAH_API();
   gemm_q4_mfma_release();
   topk_fused_release();
   sampling_release();
+  attn_decode_release();
   g.pend.clear();
   for (int i = 0; i < MAX_PLANS; i++) { g.plans[i].clear(); g.plan_active[i] = false; }
   hipStreamDestroy(g.stream);

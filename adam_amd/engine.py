@@ -77,7 +77,7 @@ class DecodeEngine:
     def __init__(self, gpu, cfg, tensors, A=None, kv_cap=1024, kv_fp16=False,
                  fusion_scheduler_mode='legacy', gpu_fused_rows_per_group=256,
                  q4_map_elem_limit=(1 << 32) - 64, verbose=False, decode_plan=True, plan_id=0,
-                 prefill_chunk=0):
+                 prefill_chunk=0, batch=1):
         if A is None:
             from . import adamah as A
         self.gpu, self.cfg, self.tensors, self.A = gpu, cfg, tensors, A
@@ -86,7 +86,10 @@ class DecodeEngine:
         self._kv_fp16 = bool(kv_fp16)
         self._rows_per_group = max(1, int(gpu_fused_rows_per_group))
         self._q4_limit = int(q4_map_elem_limit)
+        self._batch = max(1, int(batch))
         self._chunk = max(0, int(prefill_chunk))
+        if self._batch > 1:                       # the rows of a batched decode step use the chunk slots
+            self._chunk = max(self._chunk, self._batch)
         self._build_layout()
         self._alloc_workspace()
         self._upload_all()
@@ -228,24 +231,34 @@ class DecodeEngine:
         if pos % c.head_dim_kv:
             pos += c.head_dim_kv - pos % c.head_dim_kv
         self._kv_start, self._kv_step, self._kv_per_layer = pos, kv_step, kv_per_layer
-        self._k_base = [pos + L * kv_per_layer for L in range(c.n_layer)]
-        self._v_base = [kb + c.n_head_kv * kv_step for kb in self._k_base]
-        pos += c.n_layer * kv_per_layer
-        self._k_locs_h, self._v_locs_h, self._kv_copy_h = [], [], []
+        self._kv_per_seq = c.n_layer * kv_per_layer
+        # one cache per sequence of the batch (sequence 0 is the one single-sequence decoding uses)
+        self._k_base_s = [[pos + sq * self._kv_per_seq + L * kv_per_layer for L in range(c.n_layer)] for sq in range(self._batch)]
+        self._v_base_s = [[kb + c.n_head_kv * kv_step for kb in row] for row in self._k_base_s]
+        self._k_base, self._v_base = self._k_base_s[0], self._v_base_s[0]
+        pos += self._batch * self._kv_per_seq
+        self._k_locs_hs, self._v_locs_hs, self._kv_copy_h = [], [], []
         heads = np.arange(c.n_head) // gs
-        for L in range(c.n_layer):
-            kb, vb = self._k_base[L], self._v_base[L]
-            hk = self._up(kb + heads * kv_step); hv = self._up(vb + heads * kv_step)
-            g.register_row_base_span(hk, 0, kb, c.n_head_kv, kv_step, kv_step)
-            g.register_row_base_span(hv, 0, vb, c.n_head_kv, kv_step, kv_step)
-            self._k_locs_h.append(hk); self._v_locs_h.append(hv)
-            spec = np.empty(4 * c.n_head_kv, np.uint32)
-            for gi in range(c.n_head_kv):
-                spec[4 * gi:4 * gi + 4] = (gi, kb // c.head_dim_kv + gi * kv_cap,
-                                           gi + c.n_head_kv, vb // c.head_dim_kv + gi * kv_cap)
-            self._kv_copy_h.append(self._up(spec))
-            if self._chunk:
-                self._chunk_kv_spec(L, kb, vb)
+        for sq in range(self._batch):
+            hks, hvs = [], []
+            for L in range(c.n_layer):
+                kb, vb = self._k_base_s[sq][L], self._v_base_s[sq][L]
+                hk = self._up(kb + heads * kv_step); hv = self._up(vb + heads * kv_step)
+                g.register_row_base_span(hk, 0, kb, c.n_head_kv, kv_step, kv_step)
+                g.register_row_base_span(hv, 0, vb, c.n_head_kv, kv_step, kv_step)
+                hks.append(hk); hvs.append(hv)
+                if sq == 0:
+                    spec = np.empty(4 * c.n_head_kv, np.uint32)
+                    for gi in range(c.n_head_kv):
+                        spec[4 * gi:4 * gi + 4] = (gi, kb // c.head_dim_kv + gi * kv_cap,
+                                                   gi + c.n_head_kv, vb // c.head_dim_kv + gi * kv_cap)
+                    self._kv_copy_h.append(self._up(spec))
+                if self._chunk:
+                    self._chunk_kv_spec(sq, L, kb, vb)
+            self._k_locs_hs.append(hks); self._v_locs_hs.append(hvs)
+        self._k_locs_h, self._v_locs_h = self._k_locs_hs[0], self._v_locs_hs[0]
+        if self._batch > 1:
+            self._batch_kv_spec()
         pos_ao = self._ws['attn_out'][2]
         self._ao_rows_h = self._up(pos_ao + np.arange(c.n_head) * c.head_dim_kv)
         g.register_row_base_span(self._ao_rows_h, 0, pos_ao, c.n_head, c.head_dim_kv, c.head_dim_kv)
@@ -294,6 +307,13 @@ class DecodeEngine:
             self._c_lq = [self._up(self._cp['q'] + i * q_dim + heads * c.head_dim) for i in range(M)]
             self._c_lk = [self._up(self._cp['k'] + i * k_dim + kh * d) for i in range(M)]
             self._c_qkdst = [self._up([self._cp['qk'] + i * (q_dim + k_dim)]) for i in range(M)]
+        self._c_q1 = [self._up([self._cp['q'] + i * q_dim]) for i in range(M)]             # one row of the chunk each
+        self._c_k1 = [self._up([self._cp['k'] + i * k_dim]) for i in range(M)]
+        self._c_n1 = [self._up([self._cp['normed'] + i * c.n_embd]) for i in range(M)]
+        self._c_tok_pos = pos
+        self._c_tok1 = [self._up([pos + i]) for i in range(M)]                               # sampled token of row i
+        self._c_tok_locs = np.arange(pos, pos + M, dtype=np.uint32)
+        pos += M
         self._c_last = self._up(np.zeros(c.n_embd, np.uint32))
         self._c_zero = self._up([0])
         self._c_emb_hs = {}
@@ -303,7 +323,7 @@ class DecodeEngine:
             self._c_embscale_h = self._up(np.full(M * c.n_embd, self._pos_emb_scale))
         return pos
 
-    def _chunk_kv_spec(self, L, kb, vb):
+    def _chunk_kv_spec(self, sq, L, kb, vb):
         """(source row, cache row) pairs of a whole chunk, token-major, so that a prefix serves a shorter
         chunk; rows are counted in head-size units from element 0 of the workspace."""
         c, M, d = self.cfg, self._chunk, self.cfg.head_dim_kv
@@ -320,7 +340,25 @@ class DecodeEngine:
             spec[:, 2 * gi + 1, 0] = (self._cp['v'] + t * k_dim + gi * d) // d
             spec[:, 2 * gi + 1, 1] = vb // d + gi * self._kv_cap + t
         assert ksrc % d == 0 and kstride % d == 0 and self._cp['v'] % d == 0
-        self._c_kvspec[L] = self._up(spec.reshape(-1))
+        self._c_kvspec[(sq, L)] = self._up(spec.reshape(-1))
+
+    def _batch_kv_spec(self):
+        """Per layer: (source row, cache row) pairs of one decode step of the whole batch -- row s of the
+        chunk slots goes to the cache of sequence s."""
+        c, B, d = self.cfg, self._batch, self.cfg.head_dim_kv
+        k_dim = c.n_head_kv * d
+        if self._chunk_qk:
+            ksrc, kstride = self._cp['qk'] + c.n_head * c.head_dim, c.n_head * c.head_dim + k_dim
+        else:
+            ksrc, kstride = self._cp['k'], k_dim
+        self._b_kvspec = []
+        for L in range(c.n_layer):
+            spec = np.empty((B, 2 * c.n_head_kv, 2), np.uint32)
+            for sq in range(B):
+                for gi in range(c.n_head_kv):
+                    spec[sq, 2 * gi] = ((ksrc + sq * kstride + gi * d) // d, self._k_base_s[sq][L] // d + gi * self._kv_cap)
+                    spec[sq, 2 * gi + 1] = ((self._cp['v'] + sq * k_dim + gi * d) // d, self._v_base_s[sq][L] // d + gi * self._kv_cap)
+            self._b_kvspec.append(self._up(spec.reshape(-1)))
 
     def _wrows(self, name):
         """Norm weight handle with one (identical) base per chunk row."""
@@ -335,7 +373,7 @@ class DecodeEngine:
         g.set_dtype(A.DTYPE_F32)
         g.map_create(self.WS_MAP, 1, self._ws_total)
         if self._kv_fp16:
-            g.kv_cache_fp16(self.WS_MAP, self._kv_start, self.cfg.n_layer * self._kv_per_layer)
+            g.kv_cache_fp16(self.WS_MAP, self._kv_start, self._batch * self.cfg.n_layer * self._kv_per_layer)
         chunk = 1 << 25
         for mid, total in self._q4_sizes.items():
             g.map_create_typed(mid, A.DTYPE_Q4, 1, total, self.Q4_GROUP)
@@ -640,12 +678,16 @@ class DecodeEngine:
         self._sample_token_ready = True
 
     # ------------------------------------------------------------------ chunked prefill: forward
-    def _forward_chunk(self, toks, pos0, sample=True):
+    def _forward_chunk(self, toks, pos0, sample=True, seq=0, lockstep=False):
         """m <= prefill_chunk prompt tokens at positions pos0 .. pos0 + m - 1 in one pass: the row-wise ops
         over m rows, the projections as [m, K] x [N, K]^T matmuls (the fp16 matrix-core kernel for Q4
         blocks), RoPE and the KV append for all tokens at once, attention token by token over the growing
-        cache.  Same ops, operands and order per token as `_forward`; the last token's hidden state
-        lands in the decode slots, so decoding continues from there."""
+        cache (sequence `seq` of the batch).  Same ops, operands and order per token as `_forward`; the
+        last token's hidden state lands in the decode slots, so decoding continues from there.
+
+        `lockstep`: the rows are one token of each of the first m sequences of the batch instead, all at
+        position pos0 -- a batched decode step: every row is rotated for pos0, appended to and attended
+        over its own sequence's cache, and gets its own LM head pass (tokens in `read_tokens`)."""
         c, g, A, ws = self.cfg, self.gpu, self.A, self.WS_MAP
         m = len(toks)
         if not self._chunk or m == 0 or m > self._chunk:
@@ -691,16 +733,24 @@ class DecodeEngine:
                 qn, kn = self._wh[f'{p}.attn_q_norm.weight'], self._wh[f'{p}.attn_k_norm.weight']
                 for t in range(m):
                     g.map_qk_norm_rope_x_dev(ws, ws, self._c_lq[t], qn, self._c_lk[t], kn, self._c_qkdst[t],
-                                             c.n_head, c.head_dim, c.n_head_kv, c.head_dim_kv, pos0 + t, freq)
+                                             c.n_head, c.head_dim, c.n_head_kv, c.head_dim_kv,
+                                             pos0 if lockstep else pos0 + t, freq)
+            elif lockstep:
+                for t in range(m):
+                    g.map_rope_dev(ws, self._c_q1[t], self._c_q1[t], 1, c.n_head, c.head_dim, pos0, freq)
+                    g.map_rope_dev(ws, self._c_k1[t], self._c_k1[t], 1, c.n_head_kv, c.head_dim_kv, pos0, freq)
             else:
                 g.map_rope_dev(ws, CR['q'], CR['q'], m, c.n_head, c.head_dim, pos0, freq)
                 g.map_rope_dev(ws, CR['k'], CR['k'], m, c.n_head_kv, c.head_dim_kv, pos0, freq)
-            g.map_row_copy_offset_dev(ws, self._c_kvspec[L], self._c_zero, pos0, 2 * c.n_head_kv * m, c.head_dim_kv)
+            g.map_row_copy_offset_dev(ws, self._b_kvspec[L] if lockstep else self._c_kvspec[(seq, L)], self._c_zero, pos0,
+                                      2 * c.n_head_kv * m, c.head_dim_kv)
             for t in range(m):
-                seq = pos0 + t + 1
-                g.map_matmul_t_dev(ws, self._c_qrows[t], self._k_locs_h[L], self._scores_row_h, 1, c.head_dim, seq, c.n_head)
-                g.map_attn_softmax_value_dev(ws, self._scores_row_h, self._v_locs_h[L], self._c_aorows[t], c.n_head, seq,
-                                             c.head_dim_kv, scale, float(c.attn_softcap))
+                n_keys = pos0 + 1 if lockstep else pos0 + t + 1
+                sq = t if lockstep else seq
+                g.map_matmul_t_dev(ws, self._c_qrows[t], self._k_locs_hs[sq][L], self._scores_row_h, 1, c.head_dim, n_keys,
+                                   c.n_head)
+                g.map_attn_softmax_value_dev(ws, self._scores_row_h, self._v_locs_hs[sq][L], self._c_aorows[t], c.n_head,
+                                             n_keys, c.head_dim_kv, scale, float(c.attn_softcap))
             mm('attn_out', f'{p}.attn_output.weight', 'o_proj', c.n_head * c.head_dim_kv, E)
             pan = f'{p}.post_attention_norm.weight'
             if pan in self._wh:
@@ -717,6 +767,15 @@ class DecodeEngine:
                 g.map_rmsnorm_add_dev(ws, CR['ffn_out'], self._wrows(pfn), CR['hidden'], CR['hidden'], m, E, c.norm_eps)
             else:
                 g.map_op2_dev(ws, A.OP_ADD, CS['hidden'], CS['ffn_out'], CS['hidden'], m * E)
+        if lockstep:
+            # every row is the newest token of its sequence: output norm over the rows, one LM head pass per row
+            fn = (g.map_matvec_argmax_t_xq8_dev if self._kind[self._lm_name] == 'q8' else g.map_matvec_argmax_t_xq4_dev)
+            g.map_rmsnorm_dev(ws, CR['hidden'], self._wrows('output_norm.weight'), CR['normed'], m, E, c.norm_eps)
+            for t in range(m):
+                fn(ws, self._map_of[self._lm_name], self._c_n1[t], self._wh[self._lm_name], W['sample_fused_idx'][0],
+                   W['sample_fused_val'][0], self._c_tok1[t], E, c.n_vocab, self._rows_per_group)
+            g.batch_end()
+            return
         # the last token's hidden state -> the decode slots; output norm and LM head as in a decode step
         src_h, _, _, _ = g.map_gather_dev(ws, self._c_last, E)
         g.map_scatter_dev(ws, W['hidden'][0], E, src_h)
@@ -728,9 +787,9 @@ class DecodeEngine:
             self._sample_token_ready = True
         g.batch_end()
 
-    def prefill(self, token_ids, pos0=0, sample=True):
+    def prefill(self, token_ids, pos0=0, sample=True, seq=0):
         """The prompt in chunks of `prefill_chunk` tokens (token by token when the engine was built
-        without one); the LM head runs after the last token only."""
+        without one); the LM head runs after the last token only.  `seq`: which sequence of the batch."""
         n = len(token_ids)
         if not self._chunk:
             for i, t in enumerate(token_ids):
@@ -738,12 +797,47 @@ class DecodeEngine:
             return
         for lo in range(0, n, self._chunk):
             hi = min(n, lo + self._chunk)
-            self._forward_chunk(token_ids[lo:hi], pos0 + lo, sample=sample and hi == n)
+            self._forward_chunk(token_ids[lo:hi], pos0 + lo, sample=sample and hi == n, seq=seq)
 
     def read_token(self):
         # reference engine.py:1979-1981: token id crosses the boundary as float32
         tok = self.gpu.gather(self.WS_MAP, self._sample_locs).view(np.float32)
         return int(tok[0]) if tok.size else 0
+
+    def read_tokens(self, m):
+        """Tokens of the first m rows after a batched decode step."""
+        return [int(t) for t in self.gpu.gather(self.WS_MAP, self._c_tok_locs[:m]).view(np.float32)]
+
+    def generate_batch(self, prompts, max_tokens, forced=None):
+        """Greedy decoding of len(prompts) <= batch sequences in lockstep (prompts of equal length): each
+        prompt is prefilled into its own cache, then every step runs the row-wise ops and projections
+        once over all sequences ([B, K] x [N, K]^T matmuls) and attention per sequence.  `forced[s]`:
+        tokens fed back for sequence s instead of its own choices.  Returns (tokens per sequence, stats)."""
+        B, P = len(prompts), len(prompts[0])
+        if B > self._batch or any(len(p) != P for p in prompts):
+            raise RuntimeError(f"need at most {self._batch} prompts of equal length")
+        if P + max_tokens > self._kv_cap:
+            raise RuntimeError(f"KV cache too small: need {P + max_tokens} tokens but kv_cap={self._kv_cap}.")
+        self.reset()
+        t0 = time.perf_counter()
+        cur = []
+        for sq, pr in enumerate(prompts):
+            self.prefill([int(t) for t in pr], seq=sq)
+            cur.append(self.read_token())
+        self.gpu.sync()
+        t_pre = time.perf_counter() - t0
+        out = [[] for _ in range(B)]
+        t0 = time.perf_counter()
+        for step in range(max_tokens):
+            for sq in range(B):
+                out[sq].append(cur[sq])
+            feed = cur if forced is None else [int(forced[sq][step]) for sq in range(B)]
+            self._forward_chunk(feed, P + step, lockstep=True)
+            cur = self.read_tokens(B)
+        self.gpu.sync()
+        t_dec = time.perf_counter() - t0
+        return out, {'n_seq': B, 'n_prompt': P, 'n_gen': max_tokens, 'prefill_s': t_pre, 'decode_s': t_dec,
+                     'decode_tps': B * max_tokens / t_dec if t_dec > 0 else 0.0}
 
     def read_slot(self, name):
         _, sz, pos = self._ws[name]

@@ -109,3 +109,23 @@ def test_chunked_prefill_equals_token_by_token(arch, chunk):
         outs.append((out, eng.read_slot('hidden'), kv))
     assert outs[0][0] == outs[1][0]
     assert np.array_equal(outs[0][1], outs[1][1]) and np.array_equal(outs[0][2], outs[1][2])
+
+
+@pytest.mark.parametrize("arch", ["gemma3", "llama"])
+def test_batched_lockstep_decode_equals_independent_sequences(arch):
+    """Several sequences decoded in lockstep (rows of one [B, K] matmul, own KV cache each) give, on the
+    oracle, exactly the tokens of the same prompts decoded one sequence at a time; a batch engine still
+    decodes a single sequence."""
+    cfg = synth.tiny_config(arch, n_layer=2, n_embd=64, n_head=4, n_head_kv=2, head_dim=32, n_ff=96, n_vocab=160)
+    tensors = synth.make_model(cfg, seed=3, sigma=0.3)
+    prompts = [[5, 17, 3, 101, 64], [9, 33, 2, 8, 150], [1, 1, 1, 1, 1]]
+    singles = []
+    for pr in prompts:
+        eng = DecodeEngine(oracle.init(), cfg, tensors, A=A, kv_cap=32, kv_fp16=True)
+        singles.append(eng.generate(pr, GenerationConfig(max_tokens=6))[0])
+    eng = DecodeEngine(oracle.init(), cfg, tensors, A=A, kv_cap=32, kv_fp16=True, batch=4, prefill_chunk=3)
+    out, stats = eng.generate_batch(prompts, 6)
+    assert out == singles and stats['n_seq'] == 3
+    assert eng.generate(prompts[1], GenerationConfig(max_tokens=6))[0] == singles[1]
+    with pytest.raises(RuntimeError):
+        eng.generate_batch([[1, 2], [3]], 2)

@@ -204,3 +204,45 @@ def test_prefill_chunk_splits_or_falls_back_when_tokens_do_not_line_up(hip, layo
             assert g.get_last_barrier_count() == expect
         outs.append(read(g, 0, out_pos, m * Hq * d))
     assert rel_l2(outs[0], outs[1]) < TOL
+
+
+@pytest.mark.parametrize("B,ctx,Hq,Hkv,d,softcap", [(16, 300, 8, 2, 128, 0.0), (3, 40, 4, 1, 256, 50.0), (5, 2000, 32, 8, 128, 0.0)])
+def test_lockstep_sequences_are_one_launch(hip, B, ctx, Hq, Hkv, d, softcap):
+    """One (scores, softmax.V) pair per sequence of a batch, own queries / outputs / KV cache each, shared
+    score rows: on the HIP library one attention launch (plus the merge of the slices when the context
+    is long) with the oracle's per-sequence results; the score rows end up holding the last sequence's."""
+    rng = np.random.default_rng(B * 100 + ctx)
+    gs = Hq // Hkv
+    scale = float(1.0 / np.sqrt(d))
+    q = rng.standard_normal((B, Hq, d)).astype(np.float32)
+    K = rng.standard_normal((B, Hkv, ctx, d)).astype(np.float32)
+    V = rng.standard_normal((B, Hkv, ctx, d)).astype(np.float32)
+    res = []
+    for g in (hip, oracle.init()):
+        note(f"attention lockstep B={B} ctx={ctx} {Hq}q/{Hkv}kv d={d}")
+        sc_sz = Hq * ctx
+        q_pos, out_pos = sc_sz, sc_sz + B * Hq * d
+        kv_start = (out_pos + B * Hq * d + d - 1) // d * d
+        step = ctx * d
+        per_seq = 2 * Hkv * step
+        f32map(g, 0, kv_start + B * per_seq, None)
+        g.kv_cache_fp16(0, kv_start, B * per_seq)
+        put(g, 0, q_pos, q)
+        for b in range(B):
+            put(g, 0, kv_start + b * per_seq, K[b]); put(g, 0, kv_start + b * per_seq + Hkv * step, V[b])
+        heads = np.arange(Hq) // gs
+        s_rows = up(g, np.arange(Hq) * ctx)
+        g.batch_begin()
+        for b in range(B):
+            kb = kv_start + b * per_seq
+            g.map_matmul_t_dev(0, up(g, q_pos + b * Hq * d + np.arange(Hq) * d), up(g, kb + heads * step), s_rows, 1, d, ctx, Hq)
+            g.map_attn_softmax_value_dev(0, s_rows, up(g, kb + (Hkv + heads) * step), up(g, out_pos + b * Hq * d + np.arange(Hq) * d),
+                                         Hq, ctx, d, scale, softcap)
+        g.batch_end()
+        launches = g.get_last_barrier_count() if g is hip else None
+        res.append((read(g, 0, out_pos, B * Hq * d).reshape(B, Hq, d), read(g, 0, 0, sc_sz), launches))
+    assert res[0][2] in (1, 2), res[0][2]
+    for b in range(B):
+        for h in range(Hq):
+            assert rel_l2(res[0][0][b, h], res[1][0][b, h]) < TOL, (b, h)
+    assert rel_l2(res[0][1], res[1][1]) < 1e-5

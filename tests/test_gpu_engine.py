@@ -188,3 +188,23 @@ def test_chunked_prefill_on_the_matrix_cores(hip, arch, chunk):
     dev_tok, _ = dev.generate(prompt, GenerationConfig(max_tokens=8), forced=ref_tok)
     for i in range(8):
         assert dev_tok[i] == ref_tok[i] or margins[i] < 5e-2, (i, dev_tok[i], ref_tok[i], margins[i])
+
+
+@pytest.mark.parametrize("arch", ["gemma3", "llama"])
+def test_batched_lockstep_decode(hip, arch):
+    """Four sequences in lockstep on the HIP library (projections as [4, K] matmuls on the matrix cores,
+    attention per sequence): teacher-forced on the reference forward's tokens, every sequence agrees at
+    every step unless the reference's own top-2 margin is at the matmul's rounding level."""
+    cfg = synth.tiny_config(arch, n_layer=3, n_embd=256, n_head=4, n_head_kv=2, head_dim=64, n_ff=512, n_vocab=1000)
+    tensors = synth.make_model(cfg, seed=5, sigma=0.1)
+    rng = np.random.default_rng(3)
+    prompts = [[int(t) for t in rng.integers(0, 1000, 20)] for _ in range(4)]
+    deq = {n: (v.dequant() if isinstance(v, QTensor) else v) for n, v in tensors.items()}
+    refs = [CpuModel(cfg, deq, kv_cap=64, kv_fp16=True).generate(p, 10) for p in prompts]
+    note(f"engine batched decode {arch}")
+    dev = DecodeEngine(hip, cfg, tensors, A=A, kv_cap=64, kv_fp16=True, batch=4, prefill_chunk=16)
+    out, stats = dev.generate_batch(prompts, 10, forced=[r[0] for r in refs])
+    assert stats['n_seq'] == 4
+    for sq in range(4):
+        for i in range(10):
+            assert out[sq][i] == refs[sq][0][i] or refs[sq][1][i] < 5e-2, (sq, i, out[sq][i], refs[sq][0][i], refs[sq][1][i])
