@@ -61,7 +61,7 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
-template <int D, int G, int NW, bool PF>
+template <int D, int G, int NW, bool PF, bool EXT>
 __global__ void __launch_bounds__(NW * 64)
 k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift, const AttdBases bs,
               uint32_t row_size, float scale, float cap, uint32_t n_splits, uint32_t chunk, float* partial,
@@ -85,13 +85,13 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
   const uint32_t split = blockIdx.x, group = blockIdx.y, op0 = group * G;
   const uint32_t t0 = split * chunk, t1 = min(row_size, t0 + chunk);
   // wave-uniform bases plus 32-bit byte offsets: the V row of a load is the same for all lanes
-  // `ext` (several sets of heads in one launch, too many for the argument block): the bases come from
+  // EXT (several sets of heads in one launch, too many for the argument block): the bases come from
   // device memory as [q | score rows | out rows] per head, then [K | V] per group; a score row of
   // 0xFFFFFFFF is not stored.
   const uint32_t n_all = gridDim.y * (uint32_t)G;
   const uint32_t *e_q = ext, *e_sc = ext + n_all, *e_o = ext + 2u * n_all, *e_kb = ext + 3u * n_all, *e_vb = e_kb + gridDim.y;
-  const char* kbase = (const char*)(kv + ((uint64_t)(ext ? e_kb[group] : bs.kb[group]) - kv_shift));
-  const char* vbase = (const char*)(kv + ((uint64_t)(ext ? e_vb[group] : bs.vb[group]) - kv_shift));
+  const char* kbase = (const char*)(kv + ((uint64_t)(EXT ? e_kb[group] : bs.kb[group]) - kv_shift));
+  const char* vbase = (const char*)(kv + ((uint64_t)(EXT ? e_vb[group] : bs.vb[group]) - kv_shift));
   const uint32_t klane = 16u * kc, vlane = 2u * (uint32_t)DPL * lane;
 
   auto fetch = [&](uint4 (&kr)[NI], uint32_t (&vr)[16][DW], uint32_t rb) {
@@ -121,7 +121,7 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
     __syncthreads();
     for (uint32_t i = tid; i < (uint32_t)(G * D); i += NT) {   // a wave's 64 elements belong to one head
       const uint32_t hq = (uint32_t)__builtin_amdgcn_readfirstlane((int)(i / D));   // scalar: read from the arguments
-      const float x = data[(uint64_t)(ext ? e_q[op0 + hq] : bs.q[op0 + hq]) + i % D];
+      const float x = data[(uint64_t)(EXT ? e_q[op0 + hq] : bs.q[op0 + hq]) + i % D];
       qs[i] = x;
       float m = fabsf(x);
 #pragma unroll
@@ -162,8 +162,8 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
     inv_s[r] = hval[r] ? qinv[4u * kc + r] : 0.f;
     // scalar reads of the arguments, then a per-lane choice
     crow[r] = 0u;
-    if (r < G) crow[r] = ext ? e_sc[op0 + r] : bs.sc[op0 + r];
-    if (G > 4 && kc == 1u) crow[r] = ext ? e_sc[op0 + (4 + r) % G] : bs.sc[op0 + (4 + r) % G];
+    if (r < G) crow[r] = EXT ? e_sc[op0 + r] : bs.sc[op0 + r];
+    if (G > 4 && kc == 1u) crow[r] = EXT ? e_sc[op0 + (4 + r) % G] : bs.sc[op0 + (4 + r) % G];
     m_run[r] = ATTD_NEG;
     l_run[r] = 0.f;
   }
@@ -192,7 +192,7 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
 #pragma unroll
     for (int r = 0; r < 4; r++) {
       const float raw = ((s0[r] + s2[r]) + (s1[r] + s3[r])) * inv_s[r];
-      if (rok && hval[r] && crow[r] != 0xFFFFFFFFu) out[(uint64_t)crow[r] + row] = raw;
+      if (rok && hval[r] && (!EXT || crow[r] != 0xFFFFFFFFu)) out[(uint64_t)crow[r] + row] = raw;
       v[r] = rok && hval[r] ? prep(raw, scale, cap) : ATTD_NEG;
       mt[r] = row16_max(v[r]);
     }
@@ -291,7 +291,7 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
       L = fmaf(mlbuf[w][h][1], e, L);
     }
     if (n_splits == 1u) {
-      out[(uint64_t)(ext ? e_o[op0 + h] : bs.o[op0 + h]) + d] = o * (1.0f / L);
+      out[(uint64_t)(EXT ? e_o[op0 + h] : bs.o[op0 + h]) + d] = o * (1.0f / L);
     } else {
       float* pp = partial + ((uint64_t)(op0 + h) * n_splits + split) * (D + 2);
       pp[2 + d] = o;
@@ -304,10 +304,11 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
 template <int D, int NW, bool PF>
 static void launch_dg(uint32_t G, dim3 grid, const AttnDecodeArgs& a, const AttdBases& bs, uint32_t n_splits,
                       uint32_t chunk, const uint32_t* ext) {
-#define ADL(GG)                                                                                       \
-  k_attn_decode<D, GG, NW, PF><<<grid, NW * 64, 0, g.stream>>>(a.data, a.data, a.kv, a.kv_shift, bs, a.row_size, \
-                                                               a.scale, a.cap, n_splits, chunk, g.attn_scratch, ext)
-  if (G == 1) ADL(1); else if (G == 2) ADL(2); else if (G == 4) ADL(4); else ADL(8);
+#define ADL(GG, EE)                                                                                       \
+  k_attn_decode<D, GG, NW, PF, EE><<<grid, NW * 64, 0, g.stream>>>(a.data, a.data, a.kv, a.kv_shift, bs, a.row_size, \
+                                                                   a.scale, a.cap, n_splits, chunk, g.attn_scratch, ext)
+  if (ext) { if (G == 1) ADL(1, true); else if (G == 2) ADL(2, true); else if (G == 4) ADL(4, true); else ADL(8, true); }
+  else { if (G == 1) ADL(1, false); else if (G == 2) ADL(2, false); else if (G == 4) ADL(4, false); else ADL(8, false); }
 #undef ADL
 }
 
@@ -392,6 +393,10 @@ size_t launch_attn_batch(const std::vector<PendOp>& q, size_t i, int* rc) {
   const size_t n = q.size();
   if (i + 3 >= n || !attn_foldable(q[i], q[i + 1])) return 0;
   const PendOp &s0 = q[i], &a0 = q[i + 1];
+  // cheap way out first: the next pair has to bring its own query, output and cache handles
+  if (q[i + 2].kind != PK_SCORES || q[i + 3].kind != PK_ATTN || q[i + 2].h[0] == s0.h[0] || q[i + 3].h[2] == a0.h[2] ||
+      q[i + 2].h[1] == s0.h[1] || q[i + 2].n != s0.n)
+    return 0;
   Map* mp = get_f32_map(a0.map_act);
   const uint32_t H = a0.rpg, D = a0.k, rows = a0.n;
   if (!mp || !mp->kv16 || H == 0 || s0.k != D || (D != 64 && D != 128 && D != 256) || rows == 0) return 0;

@@ -244,6 +244,8 @@ size_t launch_attn_chunk(const std::vector<PendOp>& q, size_t i, int* rc) {
   const size_t n = q.size();
   if (i + 3 >= n || !attn_foldable(q[i], q[i + 1])) return 0;
   const PendOp &s0 = q[i], &a0 = q[i + 1];
+  // cheap way out first: the next token sees one more row of the same cache
+  if (q[i + 2].kind != PK_SCORES || q[i + 3].kind != PK_ATTN || q[i + 2].n != s0.n + 1 || q[i + 2].h[0] == s0.h[0]) return 0;
   Map* mp = get_f32_map(a0.map_act);
   const uint32_t H = a0.rpg, D = a0.k;
   if (!mp || !mp->kv16 || H == 0 || H > ATTP_MAX_HEADS || s0.k != D || (D != 64 && D != 128 && D != 256)) return 0;

@@ -244,6 +244,44 @@ def cpu_kernels():
             "attention_32q8kv_d128_ctx4096_us": round(t_att * 1e6, 1)}
 
 
+def measure_model_batched(args, A, synth, DecodeEngine):
+    """Whole-model legs beyond bs = 1 decode: the prompt as one chunk, and lockstep decoding of a batch."""
+    cfg = synth.gemma3_1b_config() if args.workload == "gemma3-1b" else synth.llama3_8b_config()
+    tensors = synth.make_model(cfg, seed=0, sigma=0.02)
+    gpu = A.init()
+    rng = np.random.default_rng(0)
+    out = {"workload": args.workload}
+    if args.only == "prefill":
+        n_prompt = args.prompt or 512
+        prompt = [int(t) for t in rng.integers(0, cfg.n_vocab, n_prompt)]
+        ref = None
+        for chunk in (0, n_prompt):
+            eng = DecodeEngine(gpu, cfg, tensors, A=A, kv_cap=n_prompt + 16, kv_fp16=True, fusion_scheduler_mode=args.scheduler,
+                               prefill_chunk=chunk)
+            eng.reset()
+            eng.prefill(prompt); gpu.sync()                                  # warm-up (allocations, code objects)
+            gpu.reset_native_stats()
+            t0 = time.perf_counter(); eng.prefill(prompt); gpu.sync(); dt = time.perf_counter() - t0
+            hid, tok = eng.read_slot('hidden'), eng.read_token()
+            ref = ref if ref is not None else (hid, tok)
+            key = "token_by_token" if chunk == 0 else f"chunk_{chunk}"
+            out[key] = {"ms": round(dt * 1e3, 2), "tok/s": round(n_prompt / dt, 1),
+                        "launches": gpu.get_native_stats()["dispatch_count"],
+                        "hidden_rel_l2_vs_token_by_token": float(np.linalg.norm(hid - ref[0]) / np.linalg.norm(ref[0])),
+                        "first_token_same": bool(tok == ref[1])}
+            log(f"prefill {n_prompt} tokens {key}: {dt * 1e3:.1f} ms")
+    else:
+        B, P = args.batch, args.prompt or 1024
+        eng = DecodeEngine(gpu, cfg, tensors, A=A, kv_cap=P + args.steps + 8, kv_fp16=True,
+                           fusion_scheduler_mode=args.scheduler, prefill_chunk=512, batch=B)
+        prompts = [[int(t) for t in rng.integers(0, cfg.n_vocab, P)] for _ in range(B)]
+        _, st = eng.generate_batch(prompts, args.steps)
+        out.update({"batch": B, "prompt": P, "steps": args.steps, "prefill_tok/s": round(B * P / st["prefill_s"], 1),
+                    "decode_tok/s_aggregate": round(st["decode_tps"], 1), "ms_per_step": round(st["decode_s"] / args.steps * 1e3, 3)})
+    gpu.shutdown()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -255,12 +293,16 @@ def main():
     ap.add_argument("--prefill-chunk", type=int, default=0,
                     help="prompt in chunks of this many tokens on the matrix-core matmul (0: token by token, as the "
                          "reference does; the timed region is the decode loop either way)")
-    ap.add_argument("--only", default=None, choices=["roofline", "gemv", "probe", "attention", "gemm"],
+    ap.add_argument("--batch", type=int, default=16, help="--only batch: sequences decoded in lockstep")
+    ap.add_argument("--only", default=None, choices=["roofline", "gemv", "probe", "attention", "gemm", "prefill", "batch"],
                     help="roofline: just the 28672x4096 GEMV (one kernel row in a rocprofv3 --stats table); "
                          "gemv: that shape, 4096x4096 and 4096x14336; probe: plain read/copy kernels of known "
                          "size (reference points for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE); attention: GQA "
                          "decode attention 32q/8kv x128 at ctx 1024/4096/16384; gemm: batched Q4_0 matmul at "
-                         "M = 16 and 512 on the Llama-3-8B shapes")
+                         "M = 16 and 512 on the Llama-3-8B shapes; prefill: a 512-token prompt of --workload token "
+                         "by token and in one chunk (matrix-core matmuls, causal attention in one launch per "
+                         "layer); batch: --batch random prompts of --prompt (default 1024) tokens prefilled in "
+                         "chunks of 512, then --steps lockstep decode steps of --workload")
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -270,6 +312,9 @@ def main():
     from adam_amd import adamah as A, synth
     from adam_amd.engine import DecodeEngine
 
+    if args.only in ("prefill", "batch"):
+        print(json.dumps(measure_model_batched(args, A, synth, DecodeEngine)), flush=True)
+        return
     if args.only:
         gpu = A.init()
         if args.only == "roofline":
