@@ -73,7 +73,7 @@ struct PendOp {
   uint32_t a = 0, b = 0, c = 0, d = 0;   // RMSNORM: src, weight, dst, residual.  GEMV: x, W, y.  OP2: a, b, dst.
   uint32_t n = 0, k = 0;                 // RMSNORM: n = dim.  GEMV/ARGMAX: k = K, n = N.  OP2: n elements.
   uint32_t op = 0;                       // RMSNORM: 1 = with residual.  GEMV/ARGMAX: weight format.  OP2: op code.
-  uint32_t h[5] = {0, 0, 0, 0, 0};       // ARGMAX: idx, val, dst handles.  SCORES: q, K, score rows.  ATTN: scores, V, out
+  uint32_t h[5] = {0, 0, 0, 0, 0};       // ARGMAX: idx, val, dst, x, W handles.  SCORES: q, K, score rows.  ATTN: scores, V, out
   uint32_t rpg = 0;                      // ARGMAX: rows per group.  SCORES / ATTN: number of heads (ops)
   float eps = 0.f;                       // RMSNORM: eps.  ATTN: score scale
   float f2 = 0.f;                        // ATTN: soft cap
@@ -125,6 +125,7 @@ struct Ctx {
   // deferred row-wise ops of the open batch
   std::vector<PendOp> pend;
   int no_defer = 0;              // > 0 while an entry point runs on library-owned scratch handles
+  uint64_t mem_gen = 0;          // counts host-to-device copies (with stats.dispatch: "has device memory changed?")
   uint32_t* sync_ctr = nullptr;  // device counters for last-workgroup epilogues, zero between launches
 };
 
@@ -156,6 +157,8 @@ bool res_run(uint32_t h, uint64_t n, uint32_t* start);
 void gemm_q4_mfma_release();   // frees the GEMM's scratch (shutdown)
 void sampling_release();       // frees the scratch lists of the chunked top-k (shutdown)
 void topk_fused_release();     // frees the scratch logits of the GEMV + top-k ops (shutdown)
+size_t launch_argmax_run(const std::vector<PendOp>& q, size_t i, int* rc);   // topk_fused.hip
+int launch_argmax_direct(const PendOp& p);   // gemv_q.hip: one queued Q8 GEMV + argmax
 int launch_rmsnorm_v(const PendOp& p);
 bool row_op_deferrable(const PendOp& p);                                  // rowprep.hip
 size_t launch_row_run(const std::vector<PendOp>& q, size_t i, int* rc);   // rowprep.hip

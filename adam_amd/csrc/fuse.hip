@@ -124,7 +124,9 @@ void flush_pending() {
   size_t i = 0;
   while (i < n) {
     const PendOp& p = q[i];
-    auto is_gemv = [&](size_t j) { return j < n && (q[j].kind == PK_GEMV || q[j].kind == PK_ARGMAX); };
+    auto is_gemv = [&](size_t j) {   // a launch of the int8 matrix-instruction kernel (Q8 argmax ops are not)
+      return j < n && (q[j].kind == PK_GEMV || (q[j].kind == PK_ARGMAX && q[j].op != (uint32_t)FMT_Q8_B16));
+    };
     size_t gi = n;    // the GEMV this group is built around, if any
     GemvFuse fz = {};
     if (p.kind == PK_ROPE || p.kind == PK_QKNR || p.kind == PK_ROWCOPY) {
@@ -132,6 +134,13 @@ void flush_pending() {
       int rc = 0;
       i += launch_row_run(q, i, &rc);
       continue;
+    }
+    if (p.kind == PK_ARGMAX) {
+      // the LM head of several sequences in lockstep: one pass over the matrix for all their rows
+      int rc = 0;
+      const size_t used = launch_argmax_run(q, i, &rc);
+      if (used) { i += used; continue; }
+      if (p.op == (uint32_t)FMT_Q8_B16) { launch_argmax_direct(p); i++; continue; }
     }
     if (p.kind == PK_SCORES) {
       // a prefill chunk: the attention of consecutive tokens over one growing cache, one launch

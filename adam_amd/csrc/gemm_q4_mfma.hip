@@ -346,7 +346,11 @@ k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __r
 // workgroup barrier sits in the K loop.  The partial tiles are summed in wave order at the end.
 // Eight waves (16 activation rows only: the wave-private tiles of 32 rows would not fit the static
 // LDS limit) keep twice as many loads in flight for matrices with few weight rows.
-template <int MT, int R, int NWV>
+//
+// Q8: the weights are Q8_0 blocks in the same block16 layout (32 code bytes, w = d (code - 128)): two 16-byte
+// loads per block, bytes widened with a byte permute into the fp16 pairs (1024 + code), then -1152 and d
+// as for the nibbles.  `lc` null: the result rows go to out[row * N + n] (a scratch buffer of the caller).
+template <int MT, int R, int NWV, bool Q8>
 __global__ void __launch_bounds__(64 * NWV)
 k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh,
                      const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc, const float* __restrict__ scale,
@@ -359,7 +363,7 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
   const uint32_t r16 = lane & 15u, g = lane >> 4;
   uint8_t* xs = xs_all + wave * TILE;
   const uint32_t n0 = blockIdx.x * (16u * R), m0 = blockIdx.y * BM, op = blockIdx.z;
-  const uint64_t c_off = lc[op], gbase = (uint64_t)lb[op] >> 5;
+  const uint64_t c_off = lc ? (uint64_t)lc[op] : 0ull, gbase = (uint64_t)lb[op] >> 5;
   const uint32_t nblk = K >> 5, kw = K >> 3;
   uint32_t nrow[R];
 #pragma unroll
@@ -377,6 +381,7 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
   asm volatile("" : "+s"(nib_lo));
   asm volatile("" : "+s"(nib_hi));
   const h2q_t off_lo = {(_Float16)-1032.f, (_Float16)-1032.f}, off_hi = {(_Float16)-72.f, (_Float16)-72.f};
+  const h2q_t off_q8 = {(_Float16)-1152.f, (_Float16)-1152.f};
 
   const u4q_t* xrow[NP];
 #pragma unroll
@@ -384,14 +389,17 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
     const uint32_t w = lane + u * 64u, row = min(m0 + (w >> 4), M - 1u);
     xrow[u] = xh + ((uint64_t)op * M + row) * kw + (w & 15u);
   }
-  u4q_t xn[NP], qn[R];
+  u4q_t xn[NP], qn[R], qn2[Q8 ? R : 1];
   _Float16 dn[R];
 #define GEMM_FETCH(kb_raw)                                                        \
   do {                                                                            \
     const uint32_t kb_ = min((kb_raw), nblk - 4u);                                \
     _Pragma("unroll") for (int r = 0; r < R; r++) {                               \
       const uint64_t gi = gbase + (uint64_t)nrow[r] * nblk + kb_ + g;             \
-      qn[r] = *(const u4q_t*)(W + (gi << 4));                                     \
+      if (Q8) {                                                                   \
+        qn[r] = *(const u4q_t*)(W + (gi << 5));                                   \
+        qn2[r] = *(const u4q_t*)(W + (gi << 5) + 16);                             \
+      } else qn[r] = *(const u4q_t*)(W + (gi << 4));                              \
       dn[r] = __builtin_bit_cast(_Float16, d16[gi]);                              \
     }                                                                             \
     _Pragma("unroll") for (uint32_t u = 0; u < NP; u++) xn[u] = xrow[u][kb_ * 4u]; \
@@ -410,6 +418,19 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
       const h2q_t d2 = {dn[r], dn[r]};
 #pragma unroll
       for (int j = 0; j < 4; j++) {
+        if (Q8) {
+          // piece j = code bytes 8j .. 8j+7 in two words; pair p = (byte p of the first, byte p of the second)
+          const uint32_t w0 = j == 0 ? qn[r].x : j == 1 ? qn[r].z : j == 2 ? qn2[r].x : qn2[r].z;
+          const uint32_t w1 = j == 0 ? qn[r].y : j == 1 ? qn[r].w : j == 2 ? qn2[r].y : qn2[r].w;
+          uint32_t o[4];
+#pragma unroll
+          for (uint32_t p = 0; p < 4; p++) {
+            const uint32_t t = __builtin_amdgcn_perm(w1, w0, 0x0C000C00u | ((4u + p) << 16) | p) | magic_lo;
+            o[p] = __builtin_bit_cast(uint32_t, (h2q_t)((__builtin_bit_cast(h2q_t, t) + off_q8) * d2));
+          }
+          a[r][j] = (u4q_t){o[0], o[1], o[2], o[3]};
+          continue;
+        }
         const uint32_t w = j == 0 ? qn[r].x : j == 1 ? qn[r].y : j == 2 ? qn[r].z : qn[r].w, w8 = w >> 8;
         const h2q_t t0 = __builtin_bit_cast(h2q_t, (w & nib_lo) | magic_lo), t1 = __builtin_bit_cast(h2q_t, (w & nib_hi) | magic_hi);
         const h2q_t t2 = __builtin_bit_cast(h2q_t, (w8 & nib_lo) | magic_lo), t3 = __builtin_bit_cast(h2q_t, (w8 & nib_hi) | magic_hi);
@@ -474,13 +495,30 @@ static float* g_scale_buf = nullptr;
 static uint4* g_xh_buf = nullptr;     // fp16 activations of the tiled form
 static size_t g_xh_cap = 0;           // in bytes
 static size_t g_scale_cap = 0;
+// The rows last converted into g_xh_buf / g_scale_buf, and the launch and upload counts right after the
+// matmul that used them: while both counts stand still nothing has written device memory since, so a
+// matmul over the same rows (K and V after Q, up after gate) skips the conversion launch.
+static struct { const void* buf; uint64_t a; uint32_t M, K; uint64_t dispatch, mem_gen; bool valid; } g_xh_key = {};
 
 // Preconditions (checked by the caller against the host copies of the handles): Q4 map whose blocks
 // in range are in the block16 layout, K a multiple of 128, weight bases block aligned, all operands
 // in range.
 int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb, const uint32_t* lc,
-                        uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops) {
+                        uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops, bool q8, float* out, int64_t a_host,
+                        int64_t c_host) {
+  if (((q8 || out) && M > 32) || (out && n_ops != 1)) return ADAMAH_ERR_INVALID;
   const size_t need = (size_t)2 * M * n_ops;
+  const bool reuse = g_xh_key.valid && n_ops == 1 && a_host >= 0 && g_xh_key.buf == ma->buf && g_xh_key.a == (uint64_t)a_host &&
+                     g_xh_key.M == M && g_xh_key.K == K && g_xh_key.dispatch == g.stats.dispatch &&
+                     g_xh_key.mem_gen == g.mem_gen && tuning("ADAMAH_GEMM_REUSE", 1) != 0;
+  g_xh_key.valid = false;
+  // after the matmul: the converted rows stay usable if the result did not land on them
+  auto keep = [&]() {
+    if (n_ops != 1 || a_host < 0 || (c_host < 0 && !out)) return;
+    const uint64_t a0 = (uint64_t)a_host, a1 = a0 + (uint64_t)M * K, c0 = (uint64_t)c_host, c1 = c0 + (uint64_t)M * N;
+    if (!out && c0 < a1 && a0 < c1) return;
+    g_xh_key = {ma->buf, a0, M, K, g.stats.dispatch, g.mem_gen, true};
+  };
   if (need > g_scale_cap) {
     if (g_scale_buf) { hipStreamSynchronize(g.stream); hipFree(g_scale_buf); }
     g_scale_cap = std::max<size_t>(need, 8192);
@@ -488,7 +526,7 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
   }
   float* act = (float*)ma->buf;
   uint32_t mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8;
-  if (tuning("ADAMAH_GEMM_TILED", 1) == 0) {
+  if (!q8 && !out && tuning("ADAMAH_GEMM_TILED", 1) == 0) {
     // the first form: every workgroup converts its activation tile from float32 itself
     k_row_pow2_scale<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf);
     count_launch();
@@ -506,8 +544,10 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
     g_xh_cap = xh_need;
     if (hipMalloc((void**)&g_xh_buf, g_xh_cap) != hipSuccess) { g_xh_buf = nullptr; g_xh_cap = 0; return ADAMAH_ERR_MEMORY; }
   }
-  k_act_f16<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf, g_xh_buf);
-  count_launch();
+  if (!reuse) {
+    k_act_f16<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf, g_xh_buf);
+    count_launch();
+  }
   auto wgs = [&](uint32_t rows_per_wg, uint32_t t) { return (uint64_t)cdiv(N, rows_per_wg) * cdiv(M, 16 * t) * n_ops; };
   const uint64_t want = 2ull * (uint64_t)g.n_cu;
   if (mt <= 2) {
@@ -515,15 +555,23 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
     uint32_t R = wgs(64, mt) >= want ? 4 : wgs(32, mt) >= want ? 2 : 1;
     R = (uint32_t)tuning("ADAMAH_GEMM_R", (int)R);
     R = R >= 4 ? 4 : R >= 2 ? 2 : 1;
+    if (q8 && R > 2) R = 2;   // a Q8 tile holds twice the registers
     dim3 grid(cdiv(N, 16 * R), cdiv(M, 16 * mt), n_ops);
+    float* dst = out ? out : act;
+    const uint32_t* lcd = out ? nullptr : lc;
     // eight waves where the matrix has too few weight rows for larger tiles (measured: no gain otherwise)
-    const uint32_t nwv = mt == 1 ? (uint32_t)tuning("ADAMAH_GEMM_NWV", R == 1 ? 8 : 4) : 4u;
-#define GK(T, RR, W) k_gemm_q4_f16_ksplit<T, RR, W><<<grid, 64 * W, 0, g.stream>>>(act, mw->buf, mw->d16, (const u4q_t*)g_xh_buf, lb, lc, g_scale_buf, M, K, N)
-    if (mt == 1 && nwv >= 8) { if (R == 4) GK(1, 4, 8); else if (R == 2) GK(1, 2, 8); else GK(1, 1, 8); }
-    else if (mt == 1) { if (R == 4) GK(1, 4, 4); else if (R == 2) GK(1, 2, 4); else GK(1, 1, 4); }
-    else { if (R == 4) GK(2, 4, 4); else if (R == 2) GK(2, 2, 4); else GK(2, 1, 4); }
+    const uint32_t nwv = mt == 1 && !q8 ? (uint32_t)tuning("ADAMAH_GEMM_NWV", R == 1 ? 8 : 4) : 4u;
+#define GK(T, RR, W, Q) k_gemm_q4_f16_ksplit<T, RR, W, Q><<<grid, 64 * W, 0, g.stream>>>(dst, mw->buf, mw->d16, (const u4q_t*)g_xh_buf, lb, lcd, g_scale_buf, M, K, N)
+    if (q8) {
+      if (mt == 1) { if (R == 2) GK(1, 2, 4, true); else GK(1, 1, 4, true); }
+      else { if (R == 2) GK(2, 2, 4, true); else GK(2, 1, 4, true); }
+    }
+    else if (mt == 1 && nwv >= 8) { if (R == 4) GK(1, 4, 8, false); else if (R == 2) GK(1, 2, 8, false); else GK(1, 1, 8, false); }
+    else if (mt == 1) { if (R == 4) GK(1, 4, 4, false); else if (R == 2) GK(1, 2, 4, false); else GK(1, 1, 4, false); }
+    else { if (R == 4) GK(2, 4, 4, false); else if (R == 2) GK(2, 2, 4, false); else GK(2, 1, 4, false); }
 #undef GK
     count_launch();
+    keep();
     return check_launch();
   }
   // Tile per workgroup: 64 R weight rows x 16 MT activation rows.  The largest of (8,2), (8,1), (4,1)
@@ -543,6 +591,7 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
   else { if (R == 2) GT(8, 2); else GT(8, 1); }
 #undef GT
   count_launch();
+  keep();
   return check_launch();
 }
 
@@ -553,6 +602,7 @@ void gemm_q4_mfma_release() {
   if (g_xh_buf) hipFree(g_xh_buf);
   g_xh_buf = nullptr;
   g_xh_cap = 0;
+  g_xh_key.valid = false;
 }
 
 }  // namespace adamah

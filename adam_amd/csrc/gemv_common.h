@@ -105,8 +105,12 @@ int launch_mfma_argmax(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32
                        const GemvFuse* fz = nullptr);
 bool mfma_path_ok(const Map* mw, uint32_t K);
 // M > 1: fp16 matrix-core GEMM over Q4 block16 weights (gemm_q4_mfma.hip); operands already validated.
+// q8: Q8 block16 weights instead (M <= 32).  out: the [M, N] result goes to this buffer instead of the
+// activation map (one op).  a_host / c_host: element offsets of op 0's activations and result when the
+// host knows them (n_ops == 1): lets consecutive matmuls over the same rows share one conversion.
 int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb, const uint32_t* lc,
-                        uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops);
+                        uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops, bool q8 = false, float* out = nullptr,
+                        int64_t a_host = -1, int64_t c_host = -1);
 // Second pass of the fused GEMV + argmax: best of the per-group partials, token id stored as float.
 int launch_argmax_pairs(const Map* ma, const uint32_t* lidx, const uint32_t* lval, const uint32_t* ldst,
                         uint32_t n_groups);

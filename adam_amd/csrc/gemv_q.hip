@@ -543,14 +543,17 @@ int op_matmul_t_xq(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t h
                                    (uint32_t)tuning("ADAMAH_GEMV_RPG", 16));
   }
   // several activation rows over Q4_0 blocks: fp16 matrix-core GEMM
-  if (transposed && M > 1 && dtype == DTYPE_Q4 && mw->group_size == 32 && K >= 128 && (K & 127u) == 0 && ah && bh && ch &&
-      mw->pack_size == 1 && ma->pack_size == 1 && tuning("ADAMAH_GEMM_IMPL", 1) == 1) {
+  // (Q8_0 blocks: up to 32 rows)
+  if (transposed && M > 1 && (dtype == DTYPE_Q4 || M <= 32) && mw->group_size == 32 && K >= 128 && (K & 127u) == 0 && ah && bh &&
+      ch && mw->pack_size == 1 && ma->pack_size == 1 && tuning("ADAMAH_GEMM_IMPL", 1) == 1) {
+    const int want = dtype == DTYPE_Q4 ? FMT_Q4_B16 : FMT_Q8_B16;
     bool ok = true;
     for (uint32_t op = 0; ok && op < n_ops; op++)
-      ok = (bh[op] & 31u) == 0 && fmt_of(mw, bh[op], (uint64_t)N * K) == FMT_Q4_B16;
+      ok = (bh[op] & 31u) == 0 && fmt_of(mw, bh[op], (uint64_t)N * K) == want;
     if (ok) {
       flush_pending();
-      return launch_gemm_q4_mfma(ma, mw, la, lb, lc, M, K, N, n_ops);
+      return launch_gemm_q4_mfma(ma, mw, la, lb, lc, M, K, N, n_ops, dtype == DTYPE_Q8, nullptr,
+                                 n_ops == 1 ? (int64_t)ah[0] : -1, n_ops == 1 ? (int64_t)ch[0] : -1);
     }
   }
 generic:
@@ -591,7 +594,17 @@ int op_matvec_argmax(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t
     if (impl == 3 && mfma_path_ok(mw, K) && can_defer()) {
       PendOp p;
       p.kind = PK_ARGMAX; p.map_act = map_act; p.map_wt = map_wt; p.a = (uint32_t)a0; p.b = (uint32_t)b0; p.k = K; p.n = N;
-      p.op = (uint32_t)fmt_of(mw, b0, (uint64_t)N * K); p.h[0] = hidx; p.h[1] = hval; p.h[2] = hdst; p.rpg = rows_per_group;
+      p.op = (uint32_t)fmt_of(mw, b0, (uint64_t)N * K); p.h[0] = hidx; p.h[1] = hval; p.h[2] = hdst; p.h[3] = ha; p.h[4] = hb;
+      p.rpg = rows_per_group;
+      g.pend.push_back(p);
+      return ADAMAH_OK;
+    }
+    if (impl != 3 && fmt_of(mw, b0, (uint64_t)N * K) == FMT_Q8_B16 && K >= 128 && (K & 127u) == 0 && can_defer() &&
+        tuning("ADAMAH_ARGMAX_RUN", 1) != 0) {
+      // queued so that the LM head passes of several sequences can share one read of the matrix
+      PendOp p;
+      p.kind = PK_ARGMAX; p.map_act = map_act; p.map_wt = map_wt; p.a = (uint32_t)a0; p.b = (uint32_t)b0; p.k = K; p.n = N;
+      p.op = FMT_Q8_B16; p.h[0] = hidx; p.h[1] = hval; p.h[2] = hdst; p.h[3] = ha; p.h[4] = hb; p.rpg = rows_per_group;
       g.pend.push_back(p);
       return ADAMAH_OK;
     }
@@ -622,6 +635,21 @@ int op_matvec_argmax(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t
     count_launch();
     r = check_launch();
   }
+  if (r) return r;
+  return launch_argmax_pairs(ma, lidx, lval, ldst, n_groups);
+}
+
+// A queued Q8 GEMV + argmax that did not join a run: the float32 block kernels, as when launched at once.
+int launch_argmax_direct(const PendOp& p) {
+  Map* ma = get_f32_map(p.map_act);
+  Map* mw = get_map(p.map_wt);
+  const uint32_t n_groups = cdiv(p.n, p.rpg);
+  const uint32_t *la = res_u32(p.h[3], 1), *lb = res_u32(p.h[4], 1), *lidx = res_u32(p.h[0], n_groups),
+                 *lval = res_u32(p.h[1], n_groups), *ldst = res_u32(p.h[2], 1);
+  if (!ma || !mw || !la || !lb || !lidx || !lval || !ldst) return ADAMAH_ERR_INVALID;
+  int r;
+  if (p.k > 8192) r = launch_regx<EPI_ARGMAX>((int)p.op, ma, mw, la, lb, nullptr, lidx, lval, p.k, p.n, p.rpg);
+  else r = launch_block<EPI_ARGMAX>((int)p.op, ma, mw, la, lb, nullptr, lidx, lval, p.k, p.n, p.rpg);
   if (r) return r;
   return launch_argmax_pairs(ma, lidx, lval, ldst, n_groups);
 }

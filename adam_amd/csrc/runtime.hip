@@ -133,6 +133,7 @@ void* stage_alloc(size_t n) {
 }
 
 int h2d(void* dst, const void* src, size_t n) {
+  g.mem_gen++;
   const uint8_t* s = (const uint8_t*)src;
   uint8_t* d = (uint8_t*)dst;
   while (n) {
@@ -452,6 +453,7 @@ int map_init_dtype(uint32_t id, uint32_t dtype, uint32_t pack_size, uint32_t n_p
   if (!g.initialized || id >= MAX_MAPS || dtype >= DTYPE_COUNT) return ADAMAH_ERR_INVALID;
   if (dtype == DTYPE_BF16 || dtype == DTYPE_Q6) return ADAMAH_ERR_INVALID;
   Map* m = &g.maps[id];
+  g.mem_gen++;   // the fills below rewrite device memory without counting as launches
   if (m->active) destroy_map(m);
   bool quant = dtype == DTYPE_Q8 || dtype == DTYPE_Q4;
   m->dtype = dtype; m->pack_size = pack_size; m->n_packs = n_packs;
@@ -488,6 +490,7 @@ int map_init(uint32_t id, uint32_t word_size, uint32_t pack_size, uint32_t n_pac
 int map_destroy(uint32_t id) { ADAMAH_API();
   Map* m = get_map(id);
   if (!m) return ADAMAH_ERR_INVALID;
+  g.mem_gen++;
   destroy_map(m);
   return ADAMAH_OK;
 }

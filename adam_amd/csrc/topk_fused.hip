@@ -246,6 +246,128 @@ static int op_matvec_topk(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uin
   return check_launch();
 }
 
+// ---- several GEMV + argmax ops over one matrix: one pass over the weights -------------------------
+// Lockstep decoding asks for the LM head once per sequence, over consecutive activation rows.  The rows
+// go through the matrix-core GEMM together (weights read once instead of once per row), the logits
+// [m, N] into the scratch buffer; the two kernels below then produce what every op would have: the
+// per-group (index, value) partials -- all ops name the same lists, so the last op's remain -- and
+// each op's token.
+
+// best row of group blockIdx.x for activation row blockIdx.y; pairs[row][group] = (value, index bits)
+__global__ void __launch_bounds__(256)
+k_rows_group_argmax(float* __restrict__ act, const float* __restrict__ logits, const uint32_t* __restrict__ lidx,
+                    const uint32_t* __restrict__ lval, float2* __restrict__ pairs, uint32_t N, uint32_t rows_per_group,
+                    uint32_t n_groups, uint32_t last, uint64_t act_elems) {
+  __shared__ float sv[256];
+  __shared__ uint32_t si[256];
+  const uint32_t tid = threadIdx.x, grp = blockIdx.x, j = blockIdx.y;
+  const uint32_t row0 = grp * rows_per_group, row1 = min(N, row0 + rows_per_group);
+  const float* y = logits + (uint64_t)j * N;
+  float bv = NEG_FLT_MAX; uint32_t bi = INVALID_IDX;
+  for (uint32_t r = row0 + tid; r < row1; r += 256u)
+    if (better(y[r], r, bv, bi)) { bv = y[r]; bi = r; }
+  sv[tid] = bv; si[tid] = bi;
+  __syncthreads();
+  for (uint32_t s = 128; s > 0; s >>= 1) {
+    if (tid < s && better(sv[tid + s], si[tid + s], sv[tid], si[tid])) { sv[tid] = sv[tid + s]; si[tid] = si[tid + s]; }
+    __syncthreads();
+  }
+  if (tid == 0) {
+    pairs[(uint64_t)j * n_groups + grp] = make_float2(sv[0], __uint_as_float(si[0]));
+    if (j == last) {
+      if (lidx[grp] < act_elems) act[lidx[grp]] = (float)(si[0] == INVALID_IDX ? 0u : si[0]);
+      if (lval[grp] < act_elems) act[lval[grp]] = sv[0];
+    }
+  }
+}
+
+struct RowDsts { const uint32_t* p[16]; };
+
+// best pair of activation row blockIdx.x -> its token slot
+__global__ void __launch_bounds__(256)
+k_rows_argmax_pairs(float* __restrict__ act, const float2* __restrict__ pairs, RowDsts dst, uint32_t n_groups,
+                    uint64_t act_elems) {
+  __shared__ float sv[256];
+  __shared__ uint32_t si[256];
+  const uint32_t tid = threadIdx.x, j = blockIdx.x;
+  float bv = NEG_FLT_MAX; uint32_t bi = INVALID_IDX;
+  for (uint32_t i = tid; i < n_groups; i += 256u) {
+    const float2 pr = pairs[(uint64_t)j * n_groups + i];
+    if (better(pr.x, __float_as_uint(pr.y), bv, bi)) { bv = pr.x; bi = __float_as_uint(pr.y); }
+  }
+  sv[tid] = bv; si[tid] = bi;
+  __syncthreads();
+  for (uint32_t s = 128; s > 0; s >>= 1) {
+    if (tid < s && better(sv[tid + s], si[tid + s], sv[tid], si[tid])) { sv[tid] = sv[tid + s]; si[tid] = si[tid + s]; }
+    __syncthreads();
+  }
+  const uint32_t d = dst.p[j][0];
+  if (tid == 0 && d < act_elems) act[d] = (float)(si[0] == INVALID_IDX ? 0u : si[0]);
+}
+
+// q[i] is a queued GEMV + argmax: when it starts a run of such ops over the same matrix, the same partial
+// lists and consecutive activation rows, launches the run and returns its length (0: not a run).
+size_t launch_argmax_run(const std::vector<PendOp>& q, size_t i, int* rc) {
+  const PendOp& p = q[i];
+  if (p.kind != PK_ARGMAX || (p.op != FMT_Q4_B16 && p.op != FMT_Q8_B16) || p.k < 128 || (p.k & 127u) || p.n == 0) return 0;
+  if (i + 1 >= q.size() || q[i + 1].kind != PK_ARGMAX || tuning("ADAMAH_ARGMAX_RUN", 1) == 0) return 0;
+  size_t m = 1;
+  while (i + m < q.size() && m < 16) {
+    const PendOp& x = q[i + m];
+    if (x.kind != PK_ARGMAX || x.map_act != p.map_act || x.map_wt != p.map_wt || x.b != p.b || x.k != p.k || x.n != p.n ||
+        x.rpg != p.rpg || x.op != p.op || x.h[0] != p.h[0] || x.h[1] != p.h[1] ||
+        (uint64_t)x.a != (uint64_t)p.a + (uint64_t)m * p.k)
+      break;
+    m++;
+  }
+  if (m < 2) return 0;
+  Map* ma = get_f32_map(p.map_act);
+  Map* mw = get_map(p.map_wt);
+  if (!ma || !mw) return 0;
+  const uint32_t N = p.n, K = p.k, n_groups = cdiv(N, p.rpg);
+  const uint32_t *ih = res_host(p.h[0], n_groups), *vh = res_host(p.h[1], n_groups);
+  const uint32_t *lidx = res_u32(p.h[0], n_groups), *lval = res_u32(p.h[1], n_groups);
+  const uint32_t *la = res_u32(p.h[3], 1), *lb = res_u32(p.h[4], 1);
+  if (!ih || !vh || !lidx || !lval || !la || !lb) return 0;
+  // Every op reads its row after the earlier ops have stored their partials and tokens: none of those
+  // may land on the rows, and no token slot inside the span of the partial lists (a later op's
+  // partials would overwrite it).
+  const uint64_t a0 = p.a, a1 = a0 + (uint64_t)m * K;
+  uint32_t lo = 0xFFFFFFFFu, hi = 0;
+  for (uint32_t gq = 0; gq < n_groups; gq++) {
+    lo = std::min(lo, std::min(ih[gq], vh[gq]));
+    hi = std::max(hi, std::max(ih[gq], vh[gq]));
+  }
+  if ((uint64_t)hi >= a0 && (uint64_t)lo < a1) return 0;
+  RowDsts dst;
+  for (size_t j = 0; j < m; j++) {
+    const uint32_t* dh = res_host(q[i + j].h[2], 1);
+    dst.p[j] = res_u32(q[i + j].h[2], 1);
+    if (!dh || !dst.p[j] || ((uint64_t)dh[0] >= a0 && (uint64_t)dh[0] < a1) || (dh[0] >= lo && dh[0] <= hi)) return 0;
+  }
+  const size_t need = (size_t)m * N + 2 * (size_t)m * n_groups + 2;
+  if (need > g_logit_cap) {
+    if (g_logit_buf) { hipStreamSynchronize(g.stream); hipFree(g_logit_buf); }
+    g_logit_cap = std::max<size_t>(need, 1u << 16);
+    if (hipMalloc((void**)&g_logit_buf, g_logit_cap * sizeof(float)) != hipSuccess) {
+      g_logit_buf = nullptr; g_logit_cap = 0;
+      *rc = ADAMAH_ERR_MEMORY;
+      return m;
+    }
+  }
+  float2* pairs = (float2*)(g_logit_buf + (((size_t)m * N + 1) & ~(size_t)1));
+  int r = launch_gemm_q4_mfma(ma, mw, la, lb, nullptr, (uint32_t)m, K, N, 1, p.op == FMT_Q8_B16, g_logit_buf, (int64_t)p.a);
+  if (r) { *rc = r; return m; }
+  k_rows_group_argmax<<<dim3(n_groups, (uint32_t)m), 256, 0, g.stream>>>((float*)ma->buf, g_logit_buf, lidx, lval, pairs, N,
+                                                                         p.rpg, n_groups, (uint32_t)m - 1, ma->n_elems);
+  count_launch();
+  k_rows_argmax_pairs<<<(uint32_t)m, 256, 0, g.stream>>>((float*)ma->buf, pairs, dst, n_groups, ma->n_elems);
+  count_launch();
+  *rc = check_launch();
+  return m;
+}
+
+
 }  // namespace adamah
 
 using namespace adamah;

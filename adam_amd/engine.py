@@ -307,8 +307,7 @@ class DecodeEngine:
             self._c_lq = [self._up(self._cp['q'] + i * q_dim + heads * c.head_dim) for i in range(M)]
             self._c_lk = [self._up(self._cp['k'] + i * k_dim + kh * d) for i in range(M)]
             self._c_qkdst = [self._up([self._cp['qk'] + i * (q_dim + k_dim)]) for i in range(M)]
-        self._c_q1 = [self._up([self._cp['q'] + i * q_dim]) for i in range(M)]             # one row of the chunk each
-        self._c_k1 = [self._up([self._cp['k'] + i * k_dim]) for i in range(M)]
+        self._c_qbase, self._c_kbase = self._up([self._cp['q']]), self._up([self._cp['k']])   # first row of the chunk
         self._c_n1 = [self._up([self._cp['normed'] + i * c.n_embd]) for i in range(M)]
         self._c_tok_pos = pos
         self._c_tok1 = [self._up([pos + i]) for i in range(M)]                               # sampled token of row i
@@ -736,9 +735,9 @@ class DecodeEngine:
                                              c.n_head, c.head_dim, c.n_head_kv, c.head_dim_kv,
                                              pos0 if lockstep else pos0 + t, freq)
             elif lockstep:
-                for t in range(m):
-                    g.map_rope_dev(ws, self._c_q1[t], self._c_q1[t], 1, c.n_head, c.head_dim, pos0, freq)
-                    g.map_rope_dev(ws, self._c_k1[t], self._c_k1[t], 1, c.n_head_kv, c.head_dim_kv, pos0, freq)
+                # every row sits at the same position: the m rows' heads rotate as the heads of one token
+                g.map_rope_dev(ws, self._c_qbase, self._c_qbase, 1, m * c.n_head, c.head_dim, pos0, freq)
+                g.map_rope_dev(ws, self._c_kbase, self._c_kbase, 1, m * c.n_head_kv, c.head_dim_kv, pos0, freq)
             else:
                 g.map_rope_dev(ws, CR['q'], CR['q'], m, c.n_head, c.head_dim, pos0, freq)
                 g.map_rope_dev(ws, CR['k'], CR['k'], m, c.n_head_kv, c.head_dim_kv, pos0, freq)

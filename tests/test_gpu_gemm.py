@@ -74,3 +74,70 @@ def test_batched_matmul_other_layouts_take_generic_path(hip):
         x = rng.standard_normal((1, 5, K)).astype(np.float32)
         note(f"gemm generic N={N} K={K} affine={affine}")
         assert rel_l2(run(hip, qt, x, scale=s, zp=z), run(oracle.init(), qt, x, scale=s, zp=z)) < TOL
+
+
+@pytest.mark.parametrize("M,N,K", [(16, 3000, 4096), (2, 64, 128), (23, 130, 256), (32, 1000, 1152)])
+def test_batched_q8_matmul_matches_oracle(hip, M, N, K):
+    """Up to 32 rows over Q8_0 blocks take the matrix cores as well (the LM head of a lockstep batch)."""
+    rng = np.random.default_rng(M + N + K)
+    qt = quant.quantize_q8_0((rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.02)))
+    x = rng.standard_normal((M, K), dtype=np.float32)
+    x[M - 1] *= 1e4
+    outs = []
+    for g in (hip, oracle.init()) if M * N * K <= 23 * 130 * 256 else (hip,):
+        note(f"gemm q8 M={M} N={N} K={K}")
+        load_qtensor(g, 2, qt)
+        f32map(g, 0, M * (K + N) + 8, x.reshape(-1))
+        g.batch_begin()
+        g.map_matmul_t_xq8_dev(0, 2, up(g, [0]), up(g, [0]), up(g, [M * K]), M, K, N, 1)
+        g.batch_end()
+        outs.append(read(g, 0, M * K, M * N).reshape(M, N))
+    want = x.astype(np.float64) @ qt.dequant().astype(np.float64).T
+    for m in range(M):
+        assert rel_l2(outs[0][m], want[m]) < TOL, m
+    if len(outs) > 1:
+        assert rel_l2(outs[0], outs[1]) < TOL
+
+
+def test_consecutive_matmuls_over_the_same_rows_convert_them_once(hip):
+    """Q, K and V projections of a chunk read the same rows: the second and third matmul skip the fp16
+    conversion launch.  A write to the rows in between (kernel or upload) brings it back, and so does a
+    result that lands on them."""
+    rng = np.random.default_rng(11)
+    M, K, N = 16, 256, 64
+    qt = quant.quantize_q4_0(rng.standard_normal((3 * N, K), dtype=np.float32) * np.float32(0.05))
+    x = rng.standard_normal((M, K), dtype=np.float32)
+    w = qt.dequant().astype(np.float64)
+    note("gemm conversion reuse")
+    load_qtensor(hip, 1, qt)
+    f32map(hip, 0, M * K + 3 * M * N + 64, x.reshape(-1))
+    a, cs = up(hip, [0]), [up(hip, [M * K + i * M * N]) for i in range(3)]
+    bs = [up(hip, [i * N * K]) for i in range(3)]
+    hip.batch_begin()
+    for i in range(3):
+        hip.map_matmul_t_xq4_dev(0, 1, a, bs[i], cs[i], M, K, N, 1)
+    hip.batch_end()
+    assert hip.get_last_barrier_count() == 4           # one conversion, three matmuls
+    y = read(hip, 0, M * K, 3 * M * N).reshape(3, M, N)
+    for i in range(3):
+        assert rel_l2(y[i], x.astype(np.float64) @ w[i * N:(i + 1) * N].T) < TOL
+    # rows rewritten between two matmuls: converted again, and the new values are the ones used
+    x2 = rng.standard_normal((M, K), dtype=np.float32)
+    hip.batch_begin()
+    hip.map_matmul_t_xq4_dev(0, 1, a, bs[0], cs[0], M, K, N, 1)
+    hip.scatter_contiguous(0, 0, x2.reshape(-1))
+    hip.map_matmul_t_xq4_dev(0, 1, a, bs[1], cs[1], M, K, N, 1)
+    hip.batch_end()
+    y = read(hip, 0, M * K, 2 * M * N).reshape(2, M, N)
+    assert rel_l2(y[0], x.astype(np.float64) @ w[:N].T) < TOL
+    assert rel_l2(y[1], x2.astype(np.float64) @ w[N:2 * N].T) < TOL
+    # a result stored over the rows themselves (M * N == M * K here): nothing is reused afterwards
+    qs = quant.quantize_q4_0(rng.standard_normal((K, K), dtype=np.float32) * np.float32(0.05))
+    load_qtensor(hip, 3, qs)
+    hip.batch_begin()
+    hip.map_matmul_t_xq4_dev(0, 3, a, up(hip, [0]), a, M, K, K, 1)
+    hip.map_matmul_t_xq4_dev(0, 1, a, bs[2], cs[2], M, K, N, 1)
+    hip.batch_end()
+    assert hip.get_last_barrier_count() == 4
+    x3 = (x2.astype(np.float64) @ qs.dequant().astype(np.float64).T)
+    assert rel_l2(read(hip, 0, M * K + 2 * M * N, M * N).reshape(M, N), x3 @ w[2 * N:].T) < 3 * TOL

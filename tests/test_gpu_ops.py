@@ -201,3 +201,43 @@ def test_argmax_plain_ties_nan(hip):
     f32map(hip, 0, 5008, vals)
     hip.map_argmax_dev(0, up(hip, np.arange(5000)), up(hip, [5004]), 5000)
     assert read(hip, 0, 5004, 1)[0] == 77.0
+
+
+@pytest.mark.parametrize("kind,N,K,rpg,m", [("q8", 3001, 4096, 256, 16), ("q4", 5000, 1152, 256, 5), ("q8", 700, 128, 64, 19),
+                                            ("q4", 4096, 256, 1000, 2)])
+def test_matvec_argmax_of_consecutive_rows_in_one_pass(hip, kind, N, K, rpg, m):
+    """The LM head of a lockstep batch: m GEMV + argmax ops over one matrix and consecutive activation
+    rows in one batch read the matrix once (fp16 matrix-core GEMM + two ranking launches per 16 rows).
+    Tokens equal the oracle's unless its own top two logits are closer than the fp16 operand rounding;
+    the partial lists left behind are the last op's, values within 1e-3 relative L2."""
+    rng = np.random.default_rng(N + m)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    qt = (quant.quantize_q4_0 if kind == "q4" else quant.quantize_q8_0)(w)
+    x = rng.standard_normal((m, K)).astype(np.float32)
+    x[m - 1] *= 100.0
+    ng = (N + rpg - 1) // rpg
+    mid = 1 if kind == "q4" else 2
+    base = m * K
+    res = []
+    for g in pair(hip):
+        note(f"matvec_argmax run {kind} {N}x{K} rpg={rpg} m={m}")
+        load_qtensor(g, mid, qt)
+        f32map(g, 0, base + 2 * ng + m + 8, x.reshape(-1))
+        fn = g.map_matvec_argmax_t_xq4_dev if kind == "q4" else g.map_matvec_argmax_t_xq8_dev
+        b, li, lv = up(g, [0]), up(g, np.arange(base, base + ng)), up(g, np.arange(base + ng, base + 2 * ng))
+        rows, dsts = [up(g, [j * K]) for j in range(m)], [up(g, [base + 2 * ng + j]) for j in range(m)]
+        g.batch_begin()
+        for j in range(m):
+            fn(0, mid, rows[j], b, li, lv, dsts[j], K, N, rpg)
+        g.batch_end()
+        if g is hip:
+            assert hip.get_last_barrier_count() == 4 * ((m + 15) // 16)   # conversion, GEMM, two ranking launches
+        res.append((read(g, 0, base + 2 * ng, m).astype(np.int64), read(g, 0, base, ng), read(g, 0, base + ng, ng)))
+    logits = x.astype(np.float64) @ qt.dequant().astype(np.float64).T
+    for j in range(m):
+        if res[0][0][j] != res[1][0][j]:
+            top2 = np.sort(logits[j])[-2:]
+            assert top2[1] - top2[0] <= 2e-3 * abs(top2[1]), (j, res[0][0][j], res[1][0][j])
+            assert logits[j, res[0][0][j]] >= top2[0] - 1e-9
+    assert rel_l2(res[0][2], res[1][2]) < 1e-3
+    assert (res[0][1] == res[1][1]).mean() > 0.95
