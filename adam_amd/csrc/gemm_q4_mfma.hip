@@ -500,6 +500,35 @@ static size_t g_scale_cap = 0;
 // matmul over the same rows (K and V after Q, up after gate) skips the conversion launch.
 static struct { const void* buf; uint64_t a; uint32_t M, K; uint64_t dispatch, mem_gen; bool valid; } g_xh_key = {};
 
+static bool ensure_act_bufs(size_t scale_floats, size_t xh_bytes) {
+  if (scale_floats > g_scale_cap) {
+    if (g_scale_buf) { hipStreamSynchronize(g.stream); hipFree(g_scale_buf); }
+    g_xh_key.valid = false;
+    g_scale_cap = std::max<size_t>(scale_floats, 8192);
+    if (hipMalloc((void**)&g_scale_buf, g_scale_cap * sizeof(float)) != hipSuccess) { g_scale_buf = nullptr; g_scale_cap = 0; return false; }
+  }
+  if (xh_bytes > g_xh_cap) {
+    if (g_xh_buf) { hipStreamSynchronize(g.stream); hipFree(g_xh_buf); }
+    g_xh_key.valid = false;
+    g_xh_cap = xh_bytes;
+    if (hipMalloc((void**)&g_xh_buf, g_xh_cap) != hipSuccess) { g_xh_buf = nullptr; g_xh_cap = 0; return false; }
+  }
+  return true;
+}
+
+bool gemm_act_slots(uint32_t M, uint32_t K, float** scale, __half** xh) {
+  if (tuning("ADAMAH_GEMM_TILED", 1) == 0 || tuning("ADAMAH_GEMM_REUSE", 1) == 0) return false;
+  if (!ensure_act_bufs((size_t)2 * M, (size_t)M * K * 2)) return false;
+  g_xh_key.valid = false;   // the buffers are about to be rewritten
+  *scale = g_scale_buf;
+  *xh = (__half*)g_xh_buf;
+  return true;
+}
+
+void gemm_act_mark(const void* buf, uint64_t a, uint32_t M, uint32_t K) {
+  g_xh_key = {buf, a, M, K, g.stats.dispatch, g.mem_gen, true};
+}
+
 // Preconditions (checked by the caller against the host copies of the handles): Q4 map whose blocks
 // in range are in the block16 layout, K a multiple of 128, weight bases block aligned, all operands
 // in range.
@@ -519,11 +548,7 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
     if (!out && c0 < a1 && a0 < c1) return;
     g_xh_key = {ma->buf, a0, M, K, g.stats.dispatch, g.mem_gen, true};
   };
-  if (need > g_scale_cap) {
-    if (g_scale_buf) { hipStreamSynchronize(g.stream); hipFree(g_scale_buf); }
-    g_scale_cap = std::max<size_t>(need, 8192);
-    if (hipMalloc((void**)&g_scale_buf, g_scale_cap * sizeof(float)) != hipSuccess) { g_scale_buf = nullptr; g_scale_cap = 0; return ADAMAH_ERR_MEMORY; }
-  }
+  if (!ensure_act_bufs(need, 0)) return ADAMAH_ERR_MEMORY;
   float* act = (float*)ma->buf;
   uint32_t mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8;
   if (!q8 && !out && tuning("ADAMAH_GEMM_TILED", 1) == 0) {
@@ -539,11 +564,7 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
     return check_launch();
   }
   const size_t xh_need = (size_t)n_ops * M * K * 2;
-  if (xh_need > g_xh_cap) {
-    if (g_xh_buf) { hipStreamSynchronize(g.stream); hipFree(g_xh_buf); }
-    g_xh_cap = xh_need;
-    if (hipMalloc((void**)&g_xh_buf, g_xh_cap) != hipSuccess) { g_xh_buf = nullptr; g_xh_cap = 0; return ADAMAH_ERR_MEMORY; }
-  }
+  if (!ensure_act_bufs(0, xh_need)) return ADAMAH_ERR_MEMORY;
   if (!reuse) {
     k_act_f16<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf, g_xh_buf);
     count_launch();

@@ -5,6 +5,7 @@
 // map_row_copy.comp:13-24; dispatchers adamah.c:7610-7878, 8476-8604, 8061-8085.
 // Row bases come from device-resident loc arrays, one entry per row, as in the reference.
 #include "common.h"
+#include "gemv_common.h"
 #include "../../include/adamah_hip.h"
 
 namespace adamah {
@@ -37,6 +38,62 @@ k_rmsnorm(const float* act, const float* wt, float* out, const uint32_t* __restr
     float y = act[sb + i] * inv * wt[wb + i];
     if (ADD) y += act[rb + i];
     out[db + i] = y;
+  }
+}
+
+// The same row op with the row held in registers (dim <= 256 NU): one trip to memory instead of two
+// dependent passes.  Thread t owns elements t, t + 256, ... and sums their squares in that order, as the
+// kernel above does, so the results are the same bits.  EMIT: the rows are [n_rows, dim] back to back and a
+// batched matmul follows; its fp16 operand form (row scaled by a power of two, 8-element words in the
+// order (0,4)(1,5)(2,6)(3,7), plus (s, 1/s) per row) is written here as well, which spares that
+// matmul its conversion launch.
+template <bool ADD, bool EMIT, int NU>
+__global__ void __launch_bounds__(256)
+k_rmsnorm_rows(const float* act, const float* wt, float* out, const uint32_t* __restrict__ ls,
+               const uint32_t* __restrict__ lw, const uint32_t* __restrict__ lr, const uint32_t* __restrict__ ld,
+               uint32_t dim, float eps, uint64_t act_elems, uint64_t wt_elems, float* scale, __half* xh) {
+  __shared__ float sh[4];
+  const uint32_t ri = blockIdx.x, tid = threadIdx.x;
+  const uint64_t sb = ls[ri], wb = lw[ri], db = ld[ri], rb = ADD ? (uint64_t)lr[ri] : 0;
+  if (sb + dim > act_elems || db + dim > act_elems || wb + dim > wt_elems || (ADD && rb + dim > act_elems)) return;
+  float x[NU], w[NU], r[NU];
+#pragma unroll
+  for (int u = 0; u < NU; u++) {
+    const uint32_t i = tid + 256u * u;
+    const bool in = i < dim;
+    x[u] = in ? act[sb + i] : 0.f;
+    w[u] = in ? wt[wb + i] : 0.f;
+    r[u] = (ADD && in) ? act[rb + i] : 0.f;
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < NU; u++)
+    if (tid + 256u * u < dim) ss = fmaf(x[u], x[u], ss);
+  ss = block_sum_256(ss, sh);
+  const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
+  float m = 0.f;
+#pragma unroll
+  for (int u = 0; u < NU; u++) {
+    float y = x[u] * inv * w[u];
+    if (ADD) y += r[u];
+    x[u] = y;
+    if (tid + 256u * u < dim) { out[db + tid + 256u * u] = y; m = fmaxf(m, fabsf(y)); }
+  }
+  if (!EMIT) return;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  if ((tid & 63u) == 0) sh[tid >> 6] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+  const uint32_t e = (__float_as_uint(m) >> 23) & 0xFFu;
+  float s = 1.f, si = 1.f;
+  if (e >= 14u && e <= 254u) { s = __uint_as_float((267u - e) << 23); si = __uint_as_float((e - 13u) << 23); }
+  if (tid == 0) { scale[2 * ri] = s; scale[2 * ri + 1] = si; }
+  __half* dst = xh + (uint64_t)ri * dim;
+#pragma unroll
+  for (int u = 0; u < NU; u++) {
+    const uint32_t i = tid + 256u * u, q = i & 7u;
+    if (i < dim) dst[(i & ~7u) + (q < 4u ? 2u * q : 2u * (q - 4u) + 1u)] = __float2half(x[u] * s);
   }
 }
 
@@ -142,6 +199,32 @@ static int rmsnorm_impl(uint32_t map_act, uint32_t map_wt, uint32_t hs, uint32_t
   const uint32_t* lr = add ? res_u32(hr, n_rows) : ls;
   if (!ls || !lw || !ld || !lr) return ADAMAH_ERR_INVALID;
   float* a = (float*)ma->buf;
+  if (n_rows > 1 && dim <= 8192 && tuning("ADAMAH_RMSNORM_ROWS", 1) != 0) {
+    // rows in registers; when the results are the rows of a matrix [n_rows, dim], also in the form the
+    // batched matmul reads
+    const uint32_t* dh = res_host(hd, n_rows);
+    bool emit = dh && dim >= 128 && (dim & 127u) == 0 && n_rows <= 4096 && tuning("ADAMAH_RMSNORM_EMIT", 1) != 0;
+    for (uint32_t i = 1; emit && i < n_rows; i++) emit = (uint64_t)dh[i] == (uint64_t)dh[0] + (uint64_t)i * dim;
+    // the kernel skips a row whose operands are out of range: only rows the host can vouch for are marked
+    const uint32_t *sh = res_host(hs, n_rows), *wh = res_host(hw, n_rows), *rh = add ? res_host(hr, n_rows) : nullptr;
+    emit = emit && sh && wh && (!add || rh);
+    for (uint32_t i = 0; emit && i < n_rows; i++)
+      emit = in_range(sh[i], dim, ma->n_elems) && in_range(dh[i], dim, ma->n_elems) && in_range(wh[i], dim, mw->n_elems) &&
+             (!add || in_range(rh[i], dim, ma->n_elems));
+    float* scale = nullptr;
+    __half* xh = nullptr;
+    if (emit) emit = gemm_act_slots(n_rows, dim, &scale, &xh);
+    const float* w = (const float*)mw->buf;
+#define RR(A, E, NU) k_rmsnorm_rows<A, E, NU><<<n_rows, 256, 0, g.stream>>>(a, w, a, ls, lw, lr, ld, dim, eps, ma->n_elems, mw->n_elems, scale, xh)
+#define RN(A, E) do { if (dim <= 2048) RR(A, E, 8); else if (dim <= 4096) RR(A, E, 16); else RR(A, E, 32); } while (0)
+    if (add) { if (emit) RN(true, true); else RN(true, false); }
+    else { if (emit) RN(false, true); else RN(false, false); }
+#undef RN
+#undef RR
+    count_launch();
+    if (emit) gemm_act_mark(ma->buf, dh[0], n_rows, dim);
+    return check_launch();
+  }
   if (add)
     k_rmsnorm<true><<<n_rows, 256, 0, g.stream>>>(a, (const float*)mw->buf, a, ls, lw, lr, ld, dim, eps, ma->n_elems,
                                                   mw->n_elems);

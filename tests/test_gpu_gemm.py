@@ -8,7 +8,7 @@ import pytest
 import oracle
 from adam_amd import adamah as A
 from adam_amd import quant
-from gpu_util import note, up, f32map, read, rel_l2, load_qtensor
+from gpu_util import note, up, f32map, put, read, rel_l2, load_qtensor
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
@@ -141,3 +141,50 @@ def test_consecutive_matmuls_over_the_same_rows_convert_them_once(hip):
     assert hip.get_last_barrier_count() == 4
     x3 = (x2.astype(np.float64) @ qs.dequant().astype(np.float64).T)
     assert rel_l2(read(hip, 0, M * K + 2 * M * N, M * N).reshape(M, N), x3 @ w[2 * N:].T) < 3 * TOL
+
+
+@pytest.mark.parametrize("dim,rows,add", [(4096, 16, False), (1152, 5, True), (8192, 3, False), (256, 40, True)])
+def test_rmsnorm_rows_feed_the_matmul_without_a_conversion_launch(hip, dim, rows, add):
+    """RMSNorm over the rows of a matrix followed by a batched matmul over those rows: the norm kernel also
+    writes the matmul's fp16 operand form, so the pair costs two launches, and every output word equals
+    the three-launch form's (ADAMAH_RMSNORM_EMIT=0).  Dims that are not a multiple of 128 take the
+    element-wise matmul and still match the oracle."""
+    import os
+    rng = np.random.default_rng(dim + rows)
+    N = 96
+    qt = quant.quantize_q4_0(rng.standard_normal((N, dim), dtype=np.float32) * np.float32(0.05))
+    x = rng.standard_normal((rows, dim), dtype=np.float32) * np.float32(3.0)
+    res = rng.standard_normal((rows, dim), dtype=np.float32)
+    wn = rng.uniform(0.5, 1.5, dim).astype(np.float32)
+
+    def go(g):
+        load_qtensor(g, 1, qt)
+        w0 = 3 * rows * dim + rows * N
+        f32map(g, 0, w0 + dim + 8, np.concatenate([x.reshape(-1), res.reshape(-1)]))
+        put(g, 0, w0, wn)
+        src, rs = up(g, np.arange(rows) * dim), up(g, rows * dim + np.arange(rows) * dim)
+        dst, wl = up(g, 2 * rows * dim + np.arange(rows) * dim), up(g, [w0] * rows)
+        a, b, c = up(g, [2 * rows * dim]), up(g, [0]), up(g, [3 * rows * dim])   # (an upload in between would void the note)
+        g.batch_begin()
+        if add:
+            g.map_rmsnorm_add_dev(0, src, wl, rs, dst, rows, dim, 1e-5)
+        else:
+            g.map_rmsnorm_dev(0, src, wl, dst, rows, dim, 1e-5)
+        g.map_matmul_t_xq4_dev(0, 1, a, b, c, rows, dim, N, 1)
+        g.batch_end()
+        n = g.get_last_barrier_count() if g is hip else None
+        return read(g, 0, 2 * rows * dim, rows * dim + rows * N), n
+
+    note(f"rmsnorm rows + matmul dim={dim} rows={rows} add={add}")
+    fused, n_fused = go(hip)
+    os.environ["ADAMAH_RMSNORM_EMIT"] = "0"
+    try:
+        apart, n_apart = go(hip)
+    finally:
+        del os.environ["ADAMAH_RMSNORM_EMIT"]
+    assert np.array_equal(fused.view(np.uint32), apart.view(np.uint32))
+    if dim % 128 == 0:
+        assert (n_fused, n_apart) == (2, 3)
+    want, _ = go(oracle.init())
+    assert rel_l2(fused[:rows * dim], want[:rows * dim]) < 1e-5
+    assert rel_l2(fused[rows * dim:], want[rows * dim:]) < TOL
