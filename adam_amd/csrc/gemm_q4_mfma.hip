@@ -491,6 +491,53 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
 }
 #undef GEMM_FETCH
 
+// The same conversion with the row held in registers: 1024 threads, thread t owns the 8-element words
+// t, t + 1024, ... (NW of them; K <= 8192 NW), so the row makes one trip from memory instead of two
+// dependent passes -- the rows of a decode batch are few and each workgroup's latency is the launch's.
+template <int NW>
+__global__ void __launch_bounds__(1024)
+k_act_f16_regs(const float* act, const uint32_t* __restrict__ la, uint32_t M, uint32_t K, float* scale, uint4* xh) {
+  __shared__ float red[16];
+  const uint32_t row = blockIdx.x, op = blockIdx.y, tid = threadIdx.x, kw = K >> 3;
+  const float* x = act + (uint64_t)la[op] + (uint64_t)row * K;
+  f4qu_t v0[NW], v1[NW];
+  float m = 0.f;
+#pragma unroll
+  for (int u = 0; u < NW; u++) {
+    const uint32_t w = tid + 1024u * u;
+    if (w < kw) {
+      v0[u] = *(const f4qu_t*)(x + w * 8u);
+      v1[u] = *(const f4qu_t*)(x + w * 8u + 4u);
+      m = fmaxf(m, fmaxf(fmaxf(fmaxf(fabsf(v0[u].x), fabsf(v0[u].y)), fmaxf(fabsf(v0[u].z), fabsf(v0[u].w))),
+                         fmaxf(fmaxf(fabsf(v1[u].x), fabsf(v1[u].y)), fmaxf(fabsf(v1[u].z), fabsf(v1[u].w)))));
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  if ((tid & 63u) == 0) red[tid >> 6] = m;
+  __syncthreads();
+  m = red[0];
+#pragma unroll
+  for (int i = 1; i < 16; i++) m = fmaxf(m, red[i]);
+  const uint32_t e = (__float_as_uint(m) >> 23) & 0xFFu;
+  float s = 1.f, inv = 1.f;
+  if (e >= 14u && e <= 254u) { s = __uint_as_float((267u - e) << 23); inv = __uint_as_float((e - 13u) << 23); }
+  if (tid == 0) {
+    scale[2 * ((uint64_t)op * M + row)] = s;
+    scale[2 * ((uint64_t)op * M + row) + 1] = inv;
+  }
+  uint4* dst = xh + ((uint64_t)op * M + row) * kw;
+#pragma unroll
+  for (int u = 0; u < NW; u++) {
+    const uint32_t w = tid + 1024u * u;
+    if (w >= kw) continue;
+    const h2q_t p0 = {(_Float16)(v0[u].x * s), (_Float16)(v1[u].x * s)}, p1 = {(_Float16)(v0[u].y * s), (_Float16)(v1[u].y * s)};
+    const h2q_t p2 = {(_Float16)(v0[u].z * s), (_Float16)(v1[u].z * s)}, p3 = {(_Float16)(v0[u].w * s), (_Float16)(v1[u].w * s)};
+    dst[w] = make_uint4(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1),
+                        __builtin_bit_cast(uint32_t, p2), __builtin_bit_cast(uint32_t, p3));
+  }
+}
+
 static float* g_scale_buf = nullptr;
 static uint4* g_xh_buf = nullptr;     // fp16 activations of the tiled form
 static size_t g_xh_cap = 0;           // in bytes
@@ -566,7 +613,11 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
   const size_t xh_need = (size_t)n_ops * M * K * 2;
   if (!ensure_act_bufs(0, xh_need)) return ADAMAH_ERR_MEMORY;
   if (!reuse) {
-    k_act_f16<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf, g_xh_buf);
+    if (K <= 16384 && tuning("ADAMAH_ACT_REGS", 1) != 0) {
+      if (K <= 8192) k_act_f16_regs<1><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, la, M, K, g_scale_buf, g_xh_buf);
+      else k_act_f16_regs<2><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, la, M, K, g_scale_buf, g_xh_buf);
+    } else
+      k_act_f16<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf, g_xh_buf);
     count_launch();
   }
   auto wgs = [&](uint32_t rows_per_wg, uint32_t t) { return (uint64_t)cdiv(N, rows_per_wg) * cdiv(M, 16 * t) * n_ops; };

@@ -159,22 +159,29 @@ def measure_gemm(gpu, A, Ms=(16, 512), shapes=((28672, 4096), (4096, 4096), (409
     for M in Ms:
         for N, K in shapes:
             gpu.set_dtype(A.DTYPE_F32)
-            gpu.map_create(5, 1, M * (K + N))
-            gpu.scatter_contiguous(5, 0, rng.standard_normal(M * K).astype(np.float32))
-            a = gpu.upload_dev(np.array([0], np.uint32))[0]
-            c = gpu.upload_dev(np.array([M * K], np.uint32))[0]
+            gpu.map_create(5, 1, M * (2 * K + N))
+            gpu.scatter_contiguous(5, 0, rng.standard_normal(2 * M * K).astype(np.float32))
+            # two copies of the rows, alternated: every call converts its rows to fp16 (a lone matmul's cost);
+            # with one copy the calls after the first find them converted (K and V after Q, up after gate)
+            a2 = [gpu.upload_dev(np.array([i * M * K], np.uint32))[0] for i in range(2)]
+            c = gpu.upload_dev(np.array([2 * M * K], np.uint32))[0]
             n_mats = total // (N * K)
             bs = [gpu.upload_dev(np.array([i * N * K], np.uint32))[0] for i in range(n_mats)]
-            for b in bs:
-                gpu.map_matmul_t_xq4_dev(5, 3, a, b, c, M, K, N, 1)
-            gpu.sync()
             rounds = 3
-            gpu.timer_begin()
-            for _ in range(rounds):
-                for b in bs:
-                    gpu.map_matmul_t_xq4_dev(5, 3, a, b, c, M, K, N, 1)
-            us = gpu.timer_end() * 1e3 / (rounds * n_mats)
-            out[f"M{M}_{N}x{K}"] = {"us": round(us, 2), "TFLOP/s": round(2 * M * N * K / us / 1e6, 1),
+            t = {}
+            for mode in ("alone", "shared"):
+                pick = (lambda i: a2[i & 1]) if mode == "alone" else (lambda i: a2[0])
+                for i, b in enumerate(bs):
+                    gpu.map_matmul_t_xq4_dev(5, 3, pick(i), b, c, M, K, N, 1)
+                gpu.sync()
+                gpu.timer_begin()
+                for r in range(rounds):
+                    for i, b in enumerate(bs):
+                        gpu.map_matmul_t_xq4_dev(5, 3, pick(i + r * n_mats), b, c, M, K, N, 1)
+                t[mode] = gpu.timer_end() * 1e3 / (rounds * n_mats)
+            us = t["alone"]
+            out[f"M{M}_{N}x{K}"] = {"us": round(us, 2), "us_rows_already_converted": round(t["shared"], 2),
+                                   "TFLOP/s": round(2 * M * N * K / us / 1e6, 1),
                                    "frac_fp16_mfma_peak": round(2 * M * N * K / us / 1e6 / 2500.0, 4),
                                    "weights_GB/s": round(N * K * 18 / 32 / us / 1e3, 1)}
             log(f"gemm M={M} {N}x{K}: {us:.1f} us, {2 * M * N * K / us / 1e6:.1f} TFLOP/s")
