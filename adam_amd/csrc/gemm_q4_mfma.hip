@@ -365,9 +365,15 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
   const uint32_t n0 = blockIdx.x * (16u * R), m0 = blockIdx.y * BM, op = blockIdx.z;
   const uint64_t c_off = lc ? (uint64_t)lc[op] : 0ull, gbase = (uint64_t)lb[op] >> 5;
   const uint32_t nblk = K >> 5, kw = K >> 3;
+  // Weight loads: lane -> (row lane / 4, block lane % 4 of the step), so the four lanes of a quad read 64
+  // contiguous bytes of one row -- one request to the L1 instead of one per lane, which is what the
+  // matrix-instruction layout (lane -> row lane % 16, block lane / 16) costs when loaded directly.
+  // A cross-lane permute brings each 16-byte block (and its scale) to the lane that consumes it.
+  const uint32_t lrow = lane >> 2, lblk = lane & 3u;
+  const int perm_addr = (int)((4u * r16 + g) << 2);
   uint32_t nrow[R];
 #pragma unroll
-  for (int r = 0; r < R; r++) nrow[r] = min(n0 + r * 16u + r16, N - 1u);
+  for (int r = 0; r < R; r++) nrow[r] = min(n0 + r * 16u + lrow, N - 1u);
 
   f4q_t acc[R][MT];
 #pragma unroll
@@ -395,7 +401,7 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
   do {                                                                            \
     const uint32_t kb_ = min((kb_raw), nblk - 4u);                                \
     _Pragma("unroll") for (int r = 0; r < R; r++) {                               \
-      const uint64_t gi = gbase + (uint64_t)nrow[r] * nblk + kb_ + g;             \
+      const uint64_t gi = gbase + (uint64_t)nrow[r] * nblk + kb_ + lblk;          \
       if (Q8) {                                                                   \
         qn[r] = *(const u4q_t*)(W + (gi << 5));                                   \
         qn2[r] = *(const u4q_t*)(W + (gi << 5) + 16);                             \
@@ -415,7 +421,14 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
     u4q_t a[R][4];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-      const h2q_t d2 = {dn[r], dn[r]};
+#define PERM_U4(v) (v) = (u4q_t){(uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)(v).x), (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)(v).y), \
+                                 (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)(v).z), (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)(v).w)}
+      PERM_U4(qn[r]);
+      if (Q8) PERM_U4(qn2[r]);
+#undef PERM_U4
+      const uint32_t dbits = (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)__builtin_bit_cast(uint16_t, dn[r]));
+      const _Float16 dl = __builtin_bit_cast(_Float16, (uint16_t)dbits);
+      const h2q_t d2 = {dl, dl};
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         if (Q8) {
