@@ -111,15 +111,20 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
     if (glu) return (row0 >> 1) + (l & 1u) + (l >> 1) * (N >> 1);
     return min(row0 + l, end - 1u);
   };
+  // Loads use their own lane mapping, lane -> (bundle row lane / 16, block column lane % 16): sixteen
+  // consecutive lanes read 256 contiguous bytes of one row, so a quad's 64 bytes are one request to the
+  // L1 (with the compute mapping a quad is four rows, i.e. four requests per quad, 64 per instruction).
+  // compute() moves every block and its scale to the lane that owns it with a cross-lane permute.
+  const uint32_t ll = lane >> 4, lbcol = lane & 15u;
   auto load = [&](PreM& R, uint32_t row0, uint32_t chunk, uint32_t end) {
-    const uint32_t row = row_of(row0, end);
-    const uint64_t g0 = gbase + (uint64_t)row * nblk + chunk * 64u + bcol;
+    const uint32_t row = glu ? (row0 >> 1) + (ll & 1u) + (ll >> 1) * (N >> 1) : min(row0 + ll, end - 1u);
+    const uint64_t g0 = gbase + (uint64_t)row * nblk + chunk * 64u + lbcol;
 #pragma unroll
     for (uint32_t u = 0; u < MF_U; u++) {
       uint64_t gi = g0 + u * 16u;
       // blocks past the end of the row are clamped, not skipped: the number of loads per step has to be
       // fixed for the prefetch to stay ahead (see the step loop)
-      if (RAGGED) gi = gbase + (uint64_t)row * nblk + min(chunk * 64u + u * 16u + bcol, nblk - 1u);
+      if (RAGGED) gi = gbase + (uint64_t)row * nblk + min(chunk * 64u + u * 16u + lbcol, nblk - 1u);
       R.q[u] = *(const uint4*)(W + (gi << 4));
       if (B16) R.h[u] = d16[gi];
       else R.p[u] = qp[gi];
@@ -338,7 +343,23 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
   float best_v = NEG_FLT_MAX;
   uint32_t best_i = INVALID_IDX;
 
-  auto compute = [&](const PreM& R, uint32_t row0, uint32_t chunk, uint32_t end) {
+  const int perm_addr = (int)((16u * l + bcol) << 2);   // the lane that loaded this lane's (row, block column)
+  auto compute = [&](const PreM& Rl, uint32_t row0, uint32_t chunk, uint32_t end) {
+    PreM R;
+#pragma unroll
+    for (uint32_t u = 0; u < MF_U; u++) {
+      R.q[u] = make_uint4((uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)Rl.q[u].x),
+                          (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)Rl.q[u].y),
+                          (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)Rl.q[u].z),
+                          (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)Rl.q[u].w));
+      if (B16) {
+        const uint32_t hb = (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)__half_as_ushort(Rl.h[u]));
+        R.h[u] = __ushort_as_half((unsigned short)hb);
+      } else {
+        R.p[u].x = __int_as_float(__builtin_amdgcn_ds_bpermute(perm_addr, __float_as_int(Rl.p[u].x)));
+        R.p[u].y = __int_as_float(__builtin_amdgcn_ds_bpermute(perm_addr, __float_as_int(Rl.p[u].y)));
+      }
+    }
     const uint8_t* base = xs + (size_t)(chunk * 64u + bcol) * 128u;
     uint4 xa[MF_U], xb[MF_U], prm[MF_U];
     bool valid[MF_U];
