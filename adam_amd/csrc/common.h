@@ -66,7 +66,7 @@ struct Res {
 // folded into one kernel when the batch is flushed.  All offsets are element offsets resolved from
 // the host copies of the handles at record time (any later handle upload flushes the queue first).
 enum PendKind : uint32_t { PK_RMSNORM = 1, PK_GEMV = 2, PK_OP2 = 3, PK_ARGMAX = 4, PK_SCORES = 5, PK_ATTN = 6,
-                           PK_ROPE = 7, PK_QKNR = 8, PK_ROWCOPY = 9 };
+                           PK_ROPE = 7, PK_QKNR = 8, PK_ROWCOPY = 9, PK_GEMM = 10 };
 struct PendOp {
   uint32_t kind = 0;
   uint32_t map_act = 0, map_wt = 0;
@@ -81,6 +81,8 @@ struct PendOp {
   // ROPE (one token): a = src, c = dst, rpg = heads, k = head dim, n = position, eps = frequency base.
   // QKNR: h = q rows, q weights, k rows, k weights, dst; rpg/k = q rows/dim, op/d = k rows/dim, n, eps as ROPE.
   // ROWCOPY: h = spec, source base; rpg = copies, k = row size, n = destination row offset.
+  // GEMM (2..32 activation rows, block16 weights): a, b, c = X, W, Y; rpg = M; k, n = K, N; op = weight format;
+  //   h = X, W, Y handles.
 };
 
 struct Stats {

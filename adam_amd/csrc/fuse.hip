@@ -135,6 +135,38 @@ void flush_pending() {
       i += launch_row_run(q, i, &rc);
       continue;
     }
+    if (p.kind == PK_GEMM) {
+      // Matmuls over the same few rows whose weight matrices lie back to back: one launch over the stacked
+      // rows, every result where its own op puts it.  All of them read the rows as they were before the
+      // first, so no result may touch the rows (or another result).
+      Map* ma = get_f32_map(p.map_act);
+      Map* mw = get_map(p.map_wt);
+      const uint64_t M = p.rpg, an = M * p.k;
+      GemmSegs sg = {};
+      sg.count = 1; sg.begin[0] = 0; sg.begin[1] = p.n; sg.n[0] = p.n; sg.c[0] = p.c;
+      size_t m = 1;
+      uint64_t next_b = (uint64_t)p.b + (uint64_t)p.n * p.k;
+      bool clear = disjoint(p.c, M * p.n, p.a, an);
+      while (clear && i + m < n && m < 4) {
+        const PendOp& x = q[i + m];
+        if (x.kind != PK_GEMM || x.map_act != p.map_act || x.map_wt != p.map_wt || x.a != p.a || x.rpg != p.rpg || x.k != p.k ||
+            x.op != p.op || (uint64_t)x.b != next_b || (uint64_t)sg.begin[m] + x.n > 0xFFFFFFFFull)
+          break;
+        bool ok = disjoint(x.c, M * x.n, p.a, an);
+        for (size_t j = 0; ok && j < m; j++) ok = disjoint(x.c, M * x.n, sg.c[j], M * sg.n[j]);
+        if (!ok) break;
+        sg.n[m] = x.n; sg.c[m] = x.c; sg.begin[m + 1] = sg.begin[m] + x.n;
+        next_b += (uint64_t)x.n * x.k;
+        m++;
+      }
+      sg.count = (uint32_t)m;
+      const uint32_t *la = res_u32(p.h[0], 1), *lb = res_u32(p.h[1], 1), *lc = res_u32(p.h[2], 1);
+      if (ma && mw && la && lb && lc)
+        launch_gemm_q4_mfma(ma, mw, la, lb, lc, p.rpg, p.k, sg.begin[m], 1, p.op == (uint32_t)FMT_Q8_B16, nullptr, (int64_t)p.a,
+                            m == 1 ? (int64_t)p.c : -1, m == 1 ? nullptr : &sg);
+      i += m;
+      continue;
+    }
     if (p.kind == PK_ARGMAX) {
       // the LM head of several sequences in lockstep: one pass over the matrix for all their rows
       int rc = 0;

@@ -354,7 +354,7 @@ template <int MT, int R, int NWV, bool Q8>
 __global__ void __launch_bounds__(64 * NWV)
 k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh,
                      const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc, const float* __restrict__ scale,
-                     uint32_t M, uint32_t K, uint32_t N) {
+                     uint32_t M, uint32_t K, uint32_t N, GemmSegs segs) {
   constexpr uint32_t BM = 16u * MT, ROWB = 272u, NP = 4u * MT;      // pieces per lane and step
   constexpr uint32_t TILE = BM * ROWB, PART = (NWV - 1u) * R * MT * 4u * 64u * 4u;
   __shared__ __attribute__((aligned(16))) uint8_t xs_all[(NWV * TILE > PART) ? NWV * TILE : PART];
@@ -498,7 +498,13 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const uint32_t n = n0 + r * 16u + 4u * g + i;
-        if (n < N) c[n] = acc[r][t][i] * inv;
+        if (n >= N) continue;
+        if (segs.count) {   // stacked matrices: the row's own matrix and its result base
+          uint32_t sgi = 0;
+#pragma unroll
+          for (uint32_t q = 1; q < 4; q++) sgi += (q < segs.count && n >= segs.begin[q]) ? 1u : 0u;
+          out[segs.c[sgi] + (uint64_t)row * segs.n[sgi] + (n - segs.begin[sgi])] = acc[r][t][i] * inv;
+        } else c[n] = acc[r][t][i] * inv;
       }
   }
 }
@@ -594,8 +600,10 @@ void gemm_act_mark(const void* buf, uint64_t a, uint32_t M, uint32_t K) {
 // in range.
 int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb, const uint32_t* lc,
                         uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops, bool q8, float* out, int64_t a_host,
-                        int64_t c_host) {
-  if (((q8 || out) && M > 32) || (out && n_ops != 1)) return ADAMAH_ERR_INVALID;
+                        int64_t c_host, const GemmSegs* segs) {
+  if (((q8 || out || segs) && M > 32) || ((out || segs) && n_ops != 1) || (out && segs)) return ADAMAH_ERR_INVALID;
+  GemmSegs sg = {};
+  if (segs) sg = *segs;
   const size_t need = (size_t)2 * M * n_ops;
   const bool reuse = g_xh_key.valid && n_ops == 1 && a_host >= 0 && g_xh_key.buf == ma->buf && g_xh_key.a == (uint64_t)a_host &&
                      g_xh_key.M == M && g_xh_key.K == K && g_xh_key.dispatch == g.stats.dispatch &&
@@ -611,7 +619,7 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
   if (!ensure_act_bufs(need, 0)) return ADAMAH_ERR_MEMORY;
   float* act = (float*)ma->buf;
   uint32_t mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8;
-  if (!q8 && !out && tuning("ADAMAH_GEMM_TILED", 1) == 0) {
+  if (!q8 && !out && !segs && tuning("ADAMAH_GEMM_TILED", 1) == 0) {
     // the first form: every workgroup converts its activation tile from float32 itself
     k_row_pow2_scale<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf);
     count_launch();
@@ -646,7 +654,7 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
     const uint32_t* lcd = out ? nullptr : lc;
     // eight waves where the matrix has too few weight rows for larger tiles (measured: no gain otherwise)
     const uint32_t nwv = mt == 1 && !q8 ? (uint32_t)tuning("ADAMAH_GEMM_NWV", R == 1 ? 8 : 4) : 4u;
-#define GK(T, RR, W, Q) k_gemm_q4_f16_ksplit<T, RR, W, Q><<<grid, 64 * W, 0, g.stream>>>(dst, mw->buf, mw->d16, (const u4q_t*)g_xh_buf, lb, lcd, g_scale_buf, M, K, N)
+#define GK(T, RR, W, Q) k_gemm_q4_f16_ksplit<T, RR, W, Q><<<grid, 64 * W, 0, g.stream>>>(dst, mw->buf, mw->d16, (const u4q_t*)g_xh_buf, lb, lcd, g_scale_buf, M, K, N, sg)
     if (q8) {
       if (mt == 1) { if (R == 2) GK(1, 2, 4, true); else GK(1, 1, 4, true); }
       else { if (R == 2) GK(2, 2, 4, true); else GK(2, 1, 4, true); }

@@ -104,13 +104,23 @@ int launch_mfma_argmax(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32
                        const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rows_per_group,
                        const GemvFuse* fz = nullptr);
 bool mfma_path_ok(const Map* mw, uint32_t K);
+// Result placement of a matmul over several weight matrices stacked row-wise (Q, K, V or gate, up in one
+// launch): rows [begin[s], begin[s + 1]) of the stack belong to matrix s, whose [M, n[s]] result starts
+// at element c[s] of the activation map.
+struct GemmSegs {
+  uint32_t count;
+  uint32_t begin[5];
+  uint32_t n[4];
+  uint64_t c[4];
+};
 // M > 1: fp16 matrix-core GEMM over Q4 block16 weights (gemm_q4_mfma.hip); operands already validated.
 // q8: Q8 block16 weights instead (M <= 32).  out: the [M, N] result goes to this buffer instead of the
 // activation map (one op).  a_host / c_host: element offsets of op 0's activations and result when the
 // host knows them (n_ops == 1): lets consecutive matmuls over the same rows share one conversion.
+// segs (M <= 32, one op): the weights are several matrices back to back, results placed per segment.
 int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb, const uint32_t* lc,
                         uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops, bool q8 = false, float* out = nullptr,
-                        int64_t a_host = -1, int64_t c_host = -1);
+                        int64_t a_host = -1, int64_t c_host = -1, const GemmSegs* segs = nullptr);
 // For a kernel that produces the rows [M, K] of a coming batched matmul: the buffers of their fp16 form
 // ((s, 1/s) per row; K halves per row), grown as needed, and -- after that kernel's launch has been
 // counted -- the note that rows [a, a + M K) of `buf` are converted, so the matmul skips its conversion.

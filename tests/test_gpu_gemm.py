@@ -99,7 +99,7 @@ def test_batched_q8_matmul_matches_oracle(hip, M, N, K):
         assert rel_l2(outs[0], outs[1]) < TOL
 
 
-def test_consecutive_matmuls_over_the_same_rows_convert_them_once(hip):
+def test_consecutive_matmuls_over_the_same_rows_share_conversion_and_launch(hip):
     """Q, K and V projections of a chunk read the same rows: the second and third matmul skip the fp16
     conversion launch.  A write to the rows in between (kernel or upload) brings it back, and so does a
     result that lands on them."""
@@ -113,14 +113,22 @@ def test_consecutive_matmuls_over_the_same_rows_convert_them_once(hip):
     f32map(hip, 0, M * K + 3 * M * N + 64, x.reshape(-1))
     a, cs = up(hip, [0]), [up(hip, [M * K + i * M * N]) for i in range(3)]
     bs = [up(hip, [i * N * K]) for i in range(3)]
-    hip.batch_begin()
-    for i in range(3):
-        hip.map_matmul_t_xq4_dev(0, 1, a, bs[i], cs[i], M, K, N, 1)
-    hip.batch_end()
-    assert hip.get_last_barrier_count() == 4           # one conversion, three matmuls
-    y = read(hip, 0, M * K, 3 * M * N).reshape(3, M, N)
-    for i in range(3):
-        assert rel_l2(y[i], x.astype(np.float64) @ w[i * N:(i + 1) * N].T) < TOL
+    for order, launches in (((2, 1, 0), 4), ((0, 1, 2), 2)):
+        # matrices not in storage order: one conversion, three matmuls; in storage order (W_k right after
+        # W_q, W_v right after W_k): one conversion and ONE matmul over the stacked rows
+        put(hip, 0, M * K, np.zeros(3 * M * N, np.float32))
+        hip.batch_begin()
+        for i in order:
+            hip.map_matmul_t_xq4_dev(0, 1, a, bs[i], cs[i], M, K, N, 1)
+        hip.batch_end()
+        assert hip.get_last_barrier_count() == launches
+        y = read(hip, 0, M * K, 3 * M * N).reshape(3, M, N)
+        for i in range(3):
+            assert rel_l2(y[i], x.astype(np.float64) @ w[i * N:(i + 1) * N].T) < TOL
+        if launches == 4:
+            apart = y.copy()
+        else:
+            assert np.array_equal(y.view(np.uint32), apart.view(np.uint32))   # merged == one by one, bit for bit
     # rows rewritten between two matmuls: converted again, and the new values are the ones used
     x2 = rng.standard_normal((M, K), dtype=np.float32)
     hip.batch_begin()
@@ -188,3 +196,54 @@ def test_rmsnorm_rows_feed_the_matmul_without_a_conversion_launch(hip, dim, rows
     want, _ = go(oracle.init())
     assert rel_l2(fused[:rows * dim], want[:rows * dim]) < 1e-5
     assert rel_l2(fused[rows * dim:], want[rows * dim:]) < TOL
+
+
+@pytest.mark.parametrize("kind,M,K,Ns", [("q4", 16, 4096, (4096, 1024, 1024)), ("q4", 5, 256, (40, 24)), ("q8", 16, 512, (100, 60, 33, 7)),
+                                         ("q4", 32, 1152, (1024, 256, 256))])
+def test_stacked_matmuls_place_every_result_where_its_op_asked(hip, kind, M, K, Ns):
+    """Matmuls over the same rows with weight matrices back to back but results at unrelated places and of
+    different widths (not multiples of 16 either): one launch, each [M, N_i] result at its own base, equal
+    bit for bit to the ops run one by one (ADAMAH_GEMM_MERGE=0)."""
+    import os
+    rng = np.random.default_rng(sum(Ns) + M)
+    Nt = sum(Ns)
+    w = rng.standard_normal((Nt, K), dtype=np.float32) * np.float32(0.05)
+    qt = (quant.quantize_q4_0 if kind == "q4" else quant.quantize_q8_0)(w)
+    x = rng.standard_normal((M, K), dtype=np.float32)
+    fn_name = "map_matmul_t_xq4_dev" if kind == "q4" else "map_matmul_t_xq8_dev"
+    mid = 1 if kind == "q4" else 2
+    gap = 24
+    c0, offs = [], M * K + 8
+    for n_i in reversed(Ns):                       # results in reverse order, with gaps between them
+        c0.insert(0, offs); offs += M * n_i + gap
+    total = offs
+
+    def go(g):
+        load_qtensor(g, mid, qt)
+        f32map(g, 0, total, x.reshape(-1))
+        a = up(g, [0])
+        bs, cs, b = [], [], 0
+        for n_i, c in zip(Ns, c0):
+            bs.append(up(g, [b])); cs.append(up(g, [c])); b += n_i * K
+        g.batch_begin()
+        for n_i, bh, ch in zip(Ns, bs, cs):
+            getattr(g, fn_name)(0, mid, a, bh, ch, M, K, n_i, 1)
+        g.batch_end()
+        return read(g, 0, 0, total), (g.get_last_barrier_count() if g is hip else None)
+
+    note(f"stacked matmuls {kind} M={M} K={K} Ns={Ns}")
+    merged, n_merged = go(hip)
+    os.environ["ADAMAH_GEMM_MERGE"] = "0"
+    try:
+        apart, n_apart = go(hip)
+    finally:
+        del os.environ["ADAMAH_GEMM_MERGE"]
+    assert (n_merged, n_apart) == (2, 1 + len(Ns))
+    assert np.array_equal(merged.view(np.uint32), apart.view(np.uint32))
+    wd = qt.dequant().astype(np.float64)
+    r0 = 0
+    for n_i, c in zip(Ns, c0):
+        want = x.astype(np.float64) @ wd[r0:r0 + n_i].T
+        assert rel_l2(merged[c:c + M * n_i].reshape(M, n_i), want) < TOL
+        r0 += n_i
+    assert not merged[M * K:M * K + 8].any()       # nothing outside the results was written
