@@ -160,11 +160,25 @@ void flush_pending() {
         m++;
       }
       sg.count = (uint32_t)m;
+      // one matrix followed by the add that consumes its result (hidden += projection): stored by the matmul.
+      // The matmul reads its fp16 copy of the rows, so only the result and the residual have to lie clear.
+      size_t used = m;
+      if (m == 1 && i + 1 < n && q[i + 1].kind == PK_OP2 && q[i + 1].op == 0 && q[i + 1].map_act == p.map_act &&
+          q[i + 1].n == M * p.n && tuning("ADAMAH_GEMM_EPI", 1) != 0) {
+        const PendOp& e = q[i + 1];
+        if ((e.a == p.c) != (e.b == p.c)) {
+          const uint32_t r = e.a == p.c ? e.b : e.a;
+          if (disjoint(e.c, e.n, p.c, e.n) && (r == e.c || disjoint(r, e.n, e.c, e.n)) && disjoint(r, e.n, p.c, e.n)) {
+            sg.count = 0; sg.add = 1; sg.res = r; sg.dst = e.c;
+            used = 2;
+          }
+        }
+      }
       const uint32_t *la = res_u32(p.h[0], 1), *lb = res_u32(p.h[1], 1), *lc = res_u32(p.h[2], 1);
       if (ma && mw && la && lb && lc)
         launch_gemm_q4_mfma(ma, mw, la, lb, lc, p.rpg, p.k, sg.begin[m], 1, p.op == (uint32_t)FMT_Q8_B16, nullptr, (int64_t)p.a,
-                            m == 1 ? (int64_t)p.c : -1, m == 1 ? nullptr : &sg);
-      i += m;
+                            (m == 1 && !sg.add) ? (int64_t)p.c : -1, (m == 1 && !sg.add) ? nullptr : &sg);
+      i += used;
       continue;
     }
     if (p.kind == PK_ARGMAX) {

@@ -504,7 +504,11 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
 #pragma unroll
           for (uint32_t q = 1; q < 4; q++) sgi += (q < segs.count && n >= segs.begin[q]) ? 1u : 0u;
           out[segs.c[sgi] + (uint64_t)row * segs.n[sgi] + (n - segs.begin[sgi])] = acc[r][t][i] * inv;
-        } else c[n] = acc[r][t][i] * inv;
+        } else {
+          const float y = acc[r][t][i] * inv;
+          c[n] = y;
+          if (segs.add) out[segs.dst + (uint64_t)row * N + n] = out[segs.res + (uint64_t)row * N + n] + y;
+        }
       }
   }
 }

@@ -107,11 +107,15 @@ bool mfma_path_ok(const Map* mw, uint32_t K);
 // Result placement of a matmul over several weight matrices stacked row-wise (Q, K, V or gate, up in one
 // launch): rows [begin[s], begin[s + 1]) of the stack belong to matrix s, whose [M, n[s]] result starts
 // at element c[s] of the activation map.
+// add (count == 0, one matrix): a queued element-wise add that consumes the result, r + y, is stored as
+// well: y goes to its own place, r[row * N + n] + y to dst[row * N + n] (element offsets res, dst).
 struct GemmSegs {
   uint32_t count;
   uint32_t begin[5];
   uint32_t n[4];
   uint64_t c[4];
+  uint32_t add;
+  uint64_t res, dst;
 };
 // M > 1: fp16 matrix-core GEMM over Q4 block16 weights (gemm_q4_mfma.hip); operands already validated.
 // q8: Q8 block16 weights instead (M <= 32).  out: the [M, N] result goes to this buffer instead of the

@@ -108,6 +108,14 @@ class DecodeEngine:
             if len(ops) <= 4096:
                 gpu.register_decode_plan(plan_id, ops)
                 self._plan_id = plan_id
+        # A lockstep step of the full batch is also the same op list every step: a second plan (one native
+        # call per step instead of ~47 Python calls per layer, which would otherwise bound the step).
+        self._ls_plan_id = None
+        if decode_plan and self._batch > 1 and getattr(gpu, '_has_decode_plan', False):
+            ops = self._lockstep_plan_ops(self._batch)
+            if len(ops) <= 4096:
+                gpu.register_decode_plan(plan_id + 1, ops)
+                self._ls_plan_id = plan_id + 1
 
     # ------------------------------------------------------------------ layout
     @staticmethod
@@ -677,6 +685,72 @@ class DecodeEngine:
         self._sample_token_ready = True
 
     # ------------------------------------------------------------------ chunked prefill: forward
+    def _lockstep_plan_ops(self, m):
+        """The layer loop of a lockstep step over m sequences (`_forward_chunk(..., lockstep=True)`) as
+        DecodePlanOp records, position and context length as runtime sentinels."""
+        c, A, ws = self.cfg, self.A, self.WS_MAP
+        P, S = A.DECODE_RUNTIME_POS, A.DECODE_RUNTIME_SEQ_LEN
+        E, FF = c.n_embd, c.n_ff
+        q_dim, k_dim = c.n_head * c.head_dim, c.n_head_kv * c.head_dim_kv
+        C1, CR, CS = self._c1, self._crow, self._cspan
+        Op = A.DecodePlanOp
+        ops = []
+        scale = float(1.0 / np.sqrt(c.head_dim))
+
+        def mm(src, name, dst, K, N):
+            kind = A.DECODE_OP_MATMUL_T_XQ8 if self._kind[name] == 'q8' else A.DECODE_OP_MATMUL_T_XQ4
+            ops.append(Op(kind=kind, map_id=ws, map_id2=self._map_of[name], h0=C1[src], h1=self._wh[name], h2=C1[dst],
+                          u0=m, u1=K, u2=N, u3=1))
+
+        def rms(src, name, dst):
+            ops.append(Op(kind=A.DECODE_OP_RMSNORM, map_id=ws, h0=CR[src], h1=self._wrows(name), h2=CR[dst], u0=m, u1=E,
+                          f0=c.norm_eps))
+
+        def residual(src, name):
+            if name in self._wh:
+                ops.append(Op(kind=A.DECODE_OP_RMSNORM_ADD, map_id=ws, h0=CR[src], h1=self._wrows(name), h2=CR['hidden'],
+                              h3=CR['hidden'], u0=m, u1=E, f0=c.norm_eps))
+            else:
+                ops.append(Op(kind=A.DECODE_OP_OP2, map_id=ws, op_code=A.OP_ADD, h0=CS['hidden'], h1=CS[src], h2=CS['hidden'],
+                              u0=m * E))
+
+        for L in range(c.n_layer):
+            p = f'blk.{L}'
+            freq = c.rope_base_global if c.is_global(L) else c.rope_base_local
+            rms('hidden', f'{p}.attn_norm.weight', 'normed')
+            mm('normed', f'{p}.attn_q.weight', 'q', E, q_dim)
+            mm('normed', f'{p}.attn_k.weight', 'k', E, k_dim)
+            mm('normed', f'{p}.attn_v.weight', 'v', E, k_dim)
+            if self._chunk_qk:
+                qn, kn = self._wh[f'{p}.attn_q_norm.weight'], self._wh[f'{p}.attn_k_norm.weight']
+                for t in range(m):
+                    ops.append(Op(kind=A.DECODE_OP_QK_NORM_ROPE_X, map_id=ws, map_id2=ws, h0=self._c_lq[t], h1=qn,
+                                  h2=self._c_lk[t], h3=kn, h4=self._c_qkdst[t], u0=c.n_head, u1=c.head_dim,
+                                  u2=c.n_head_kv, u3=c.head_dim_kv, u4=P, f0=freq))
+            else:
+                ops.append(Op(kind=A.DECODE_OP_ROPE, map_id=ws, h0=self._c_qbase, h1=self._c_qbase, u0=1, u1=m * c.n_head,
+                              u2=c.head_dim, u3=P, f0=freq))
+                ops.append(Op(kind=A.DECODE_OP_ROPE, map_id=ws, h0=self._c_kbase, h1=self._c_kbase, u0=1,
+                              u1=m * c.n_head_kv, u2=c.head_dim_kv, u3=P, f0=freq))
+            ops.append(Op(kind=A.DECODE_OP_ROW_COPY_OFFSET, map_id=ws, h0=self._b_kvspec[L], h1=self._c_zero, u0=P,
+                          u1=2 * c.n_head_kv * m, u2=c.head_dim_kv))
+            for t in range(m):
+                ops.append(Op(kind=A.DECODE_OP_MATMUL_T, map_id=ws, h0=self._c_qrows[t], h1=self._k_locs_hs[t][L],
+                              h2=self._scores_row_h, u0=1, u1=c.head_dim, u2=S, u3=c.n_head))
+                ops.append(Op(kind=A.DECODE_OP_ATTN_SOFTMAX_VALUE, map_id=ws, h0=self._scores_row_h,
+                              h1=self._v_locs_hs[t][L], h2=self._c_aorows[t], u0=c.n_head, u1=S, u2=c.head_dim_kv,
+                              f0=scale, f1=float(c.attn_softcap)))
+            mm('attn_out', f'{p}.attn_output.weight', 'o_proj', c.n_head * c.head_dim_kv, E)
+            residual('o_proj', f'{p}.post_attention_norm.weight')
+            rms('hidden', f'{p}.ffn_norm.weight', 'normed2')
+            mm('normed2', f'{p}.ffn_gate.weight', 'gate', E, FF)
+            mm('normed2', f'{p}.ffn_up.weight', 'up', E, FF)
+            ops.append(Op(kind=A.DECODE_OP_OP2, map_id=ws, op_code=A.OP_GEGLU if c.ffn_act == 'gelu' else A.OP_SWIGLU,
+                          h0=CS['gate'], h1=CS['up'], h2=CS['act'], u0=m * FF))
+            mm('act', f'{p}.ffn_down.weight', 'ffn_out', FF, E)
+            residual('ffn_out', f'{p}.post_ffw_norm.weight')
+        return ops
+
     def _forward_chunk(self, toks, pos0, sample=True, seq=0, lockstep=False):
         """m <= prefill_chunk prompt tokens at positions pos0 .. pos0 + m - 1 in one pass: the row-wise ops
         over m rows, the projections as [m, K] x [N, K]^T matmuls (the fp16 matrix-core kernel for Q4
@@ -721,7 +795,10 @@ class DecodeEngine:
             if c.emb_scale != 1.0:
                 g.map_broadcast_dev(ws, A.OP_MUL, CS['hidden'], self._c_embscale_h, CS['hidden'], m * E)
         scale = float(1.0 / np.sqrt(c.head_dim))
-        for L in range(c.n_layer):
+        planned = lockstep and self._ls_plan_id is not None and m == self._batch
+        if planned:
+            g.decode_step(self._ls_plan_id, pos0, pos0 + 1)
+        for L in range(0 if planned else c.n_layer):
             p = f'blk.{L}'
             freq = c.rope_base_global if c.is_global(L) else c.rope_base_local
             g.map_rmsnorm_dev(ws, CR['hidden'], self._wrows(f'{p}.attn_norm.weight'), CR['normed'], m, E, c.norm_eps)

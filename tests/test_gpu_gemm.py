@@ -247,3 +247,41 @@ def test_stacked_matmuls_place_every_result_where_its_op_asked(hip, kind, M, K, 
         assert rel_l2(merged[c:c + M * n_i].reshape(M, n_i), want) < TOL
         r0 += n_i
     assert not merged[M * K:M * K + 8].any()       # nothing outside the results was written
+
+
+@pytest.mark.parametrize("M,K,N,in_place", [(16, 4096, 4096, True), (7, 256, 50, False), (32, 1152, 72, True)])
+def test_residual_add_stored_by_the_matmul(hip, M, K, N, in_place):
+    """hidden += X W^T issued as matmul then add: the matmul's store also writes residual + result (two launches
+    with the conversion instead of three); the projection itself still lands in its own rows.  All words equal
+    the unfused sequence's (ADAMAH_GEMM_EPI=0)."""
+    import os
+    rng = np.random.default_rng(M + N)
+    qt = quant.quantize_q4_0(rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.05))
+    x = rng.standard_normal((M, K), dtype=np.float32)
+    hid = rng.standard_normal((M, N), dtype=np.float32)
+    y0, h0 = M * K, M * K + M * N
+    d0 = h0 if in_place else h0 + M * N
+    total = h0 + 2 * M * N
+
+    def go(g):
+        load_qtensor(g, 1, qt)
+        f32map(g, 0, total, np.concatenate([x.reshape(-1), np.zeros(M * N, np.float32), hid.reshape(-1)]))
+        a, b, c = up(g, [0]), up(g, [0]), up(g, [y0])
+        hy, hh, hd = up(g, y0 + np.arange(M * N)), up(g, h0 + np.arange(M * N)), up(g, d0 + np.arange(M * N))
+        g.batch_begin()
+        g.map_matmul_t_xq4_dev(0, 1, a, b, c, M, K, N, 1)
+        g.map_op2_dev(0, A.OP_ADD, hh, hy, hd, M * N)
+        g.batch_end()
+        return read(g, 0, 0, total), (g.get_last_barrier_count() if g is hip else None)
+
+    note(f"matmul + residual add M={M} K={K} N={N} in_place={in_place}")
+    fused, n_fused = go(hip)
+    os.environ["ADAMAH_GEMM_EPI"] = "0"
+    try:
+        apart, n_apart = go(hip)
+    finally:
+        del os.environ["ADAMAH_GEMM_EPI"]
+    assert (n_fused, n_apart) == (2, 3)
+    assert np.array_equal(fused.view(np.uint32), apart.view(np.uint32))
+    want, _ = go(oracle.init())
+    assert rel_l2(fused[y0:], want[y0:]) < TOL
