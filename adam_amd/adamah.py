@@ -87,6 +87,7 @@ _SIGS = {
     "adamah_register_decode_plan": (i32, [_U, ctypes.POINTER(DecodePlanOp), _U]),
     "adamah_clear_decode_plan": (None, [_U]), "adamah_decode_step": (i32, [_U] * 3),
     "adamah_kv_cache_fp16": (i32, [_U] * 3),
+    "adamah_attn_causal_rows_dev": (i32, [_U, pu32, _U, _U, _U, pu32, _U, _U, _U, _U, _U, f32c, f32c]),
     "batch_begin": (None, []), "batch_end": (None, []),
     "map_init": (i32, [_U] * 4), "map_init_dtype": (i32, [_U] * 5), "map_destroy": (i32, [_U]),
     "map_size": (u64, [_U]), "map_get_dtype": (u32, [_U]),
@@ -145,6 +146,7 @@ _OPTIONAL_FLAGS = {
     "adamah_register_decode_plan": "_has_decode_plan",
     "adamah_set_dtype": "_has_dtype",
     "adamah_kv_cache_fp16": "_has_kv_cache_fp16",
+    "adamah_attn_causal_rows_dev": "_has_attn_causal_rows_dev",
     "map_resolve_idx_dev": "_has_map_resolve_idx_dev",
     "map_sample_categorical_dev": "_has_map_sample_categorical_dev",
     "map_repeat_penalty_dev": "_has_map_repeat_penalty_dev",
@@ -407,6 +409,16 @@ class Adamah:
                             locs_dst_handle, n_rows, dim, eps=1e-5):
         self._op("map_rmsnorm_add_dev", map_id, locs_src_handle, locs_wt_handle, locs_resid_handle,
                  locs_dst_handle, n_rows, dim, eps)
+
+    def attn_causal_rows_dev(self, map_id, q_handles, locs_k_handle, locs_scores_handle, locs_v_handle, out_handles,
+                             head_dim, n_keys0, n_heads, value_dim, scale, softcap=0.0):
+        """Extension: for t in range(len(q_handles)) the pair map_matmul_t_dev(q_handles[t] -> scores over
+        n_keys0 + t keys) / map_attn_softmax_value_dev(-> out_handles[t]) in one native call."""
+        m = len(q_handles)
+        qa = (ctypes.c_uint32 * m)(*q_handles)
+        oa = (ctypes.c_uint32 * m)(*out_handles)
+        self._op("adamah_attn_causal_rows_dev", map_id, qa, locs_k_handle, locs_scores_handle, locs_v_handle, oa, m,
+                 head_dim, n_keys0, n_heads, value_dim, scale, softcap)
 
     def map_rope_dev(self, map_id, locs_src_handle, locs_dst_handle, n_tokens, n_heads, head_dim,
                      pos_offset=0, freq_base=10000.0):

@@ -809,4 +809,18 @@ int map_attn_softmax_abs_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t
   return softmax_rows(map_id, hs, hd, n_rows, row_size, scale, cap, false);
 }
 
+int adamah_attn_causal_rows_dev(uint32_t map_id, const uint32_t* q_handles, uint32_t locs_k, uint32_t locs_scores,
+                                uint32_t locs_v, const uint32_t* out_handles, uint32_t m, uint32_t head_dim,
+                                uint32_t n_keys0, uint32_t n_heads, uint32_t value_dim, float scale, float softcap) {
+  if (m == 0) return ADAMAH_OK;
+  if (!q_handles || !out_handles) return ADAMAH_ERR_INVALID;
+  for (uint32_t t = 0; t < m; t++) {
+    int r = map_matmul_t_dev(map_id, q_handles[t], locs_k, locs_scores, 1, head_dim, n_keys0 + t, n_heads);
+    if (r != ADAMAH_OK) return r;
+    r = map_attn_softmax_value_dev(map_id, locs_scores, locs_v, out_handles[t], n_heads, n_keys0 + t, value_dim, scale, softcap);
+    if (r != ADAMAH_OK) return r;
+  }
+  return ADAMAH_OK;
+}
+
 }  // extern "C"

@@ -820,7 +820,12 @@ class DecodeEngine:
                 g.map_rope_dev(ws, CR['k'], CR['k'], m, c.n_head_kv, c.head_dim_kv, pos0, freq)
             g.map_row_copy_offset_dev(ws, self._b_kvspec[L] if lockstep else self._c_kvspec[(seq, L)], self._c_zero, pos0,
                                       2 * c.n_head_kv * m, c.head_dim_kv)
-            for t in range(m):
+            if not lockstep and hasattr(g, 'attn_causal_rows_dev'):
+                # the m (scores, softmax . V) pairs of the chunk in one native call
+                g.attn_causal_rows_dev(ws, self._c_qrows[:m], self._k_locs_hs[seq][L], self._scores_row_h,
+                                       self._v_locs_hs[seq][L], self._c_aorows[:m], c.head_dim, pos0 + 1, c.n_head,
+                                       c.head_dim_kv, scale, float(c.attn_softcap))
+            for t in range(0 if not lockstep and hasattr(g, 'attn_causal_rows_dev') else m):
                 n_keys = pos0 + 1 if lockstep else pos0 + t + 1
                 sq = t if lockstep else seq
                 g.map_matmul_t_dev(ws, self._c_qrows[t], self._k_locs_hs[sq][L], self._scores_row_h, 1, c.head_dim, n_keys,

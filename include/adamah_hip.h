@@ -225,6 +225,15 @@ int adamah_decode_step(uint32_t plan_id, uint32_t pos, uint32_t seq_len); /* ada
  * copied into the range by map_row_copy(_offset)_dev are rounded to fp16, and the attention entry
  * points read the fp16 copy when their K/V operands lie inside it. */
 int adamah_kv_cache_fp16(uint32_t map_id, uint32_t start, uint32_t count);
+/* Causal attention of m consecutive tokens over one growing KV cache, as one call: for t = 0 .. m-1 exactly
+ * the pair  map_matmul_t_dev(map_id, q_handles[t], locs_k, locs_scores, 1, head_dim, n_keys0 + t, n_heads);
+ * map_attn_softmax_value_dev(map_id, locs_scores, locs_v, out_handles[t], n_heads, n_keys0 + t, value_dim,
+ * scale, softcap)  (adamah.c:7894, adamah.c:6768) -- same results, same queueing inside a batch; it exists because a
+ * prompt chunk of 512 tokens would otherwise cost the host 1024 calls per layer.  q_handles / out_handles:
+ * m handle ids each (host arrays). */
+int adamah_attn_causal_rows_dev(uint32_t map_id, const uint32_t* q_handles, uint32_t locs_k, uint32_t locs_scores,
+                                uint32_t locs_v, const uint32_t* out_handles, uint32_t m, uint32_t head_dim,
+                                uint32_t n_keys0, uint32_t n_heads, uint32_t value_dim, float scale, float softcap);
 /* HIP-event stopwatch on the library's stream (benchmarks). begin: 0 on success; end: ms or <0. */
 int adamah_hip_timer_begin(void);
 float adamah_hip_timer_end(void);

@@ -556,6 +556,15 @@ class NumpyAdamah:
     def map_row_copy_dev(self, map_id, copy_spec_handle, src_base_handle, n_copies, row_size):
         self.map_row_copy_offset_dev(map_id, copy_spec_handle, src_base_handle, 0, n_copies, row_size)
 
+    def attn_causal_rows_dev(self, map_id, q_handles, locs_k_handle, locs_scores_handle, locs_v_handle, out_handles,
+                             head_dim, n_keys0, n_heads, value_dim, scale, softcap=0.0):
+        """Extension shared with the HIP library (no counterpart in the reference): the (scores, softmax . V)
+        pair of m consecutive tokens over one growing cache, token t over n_keys0 + t keys."""
+        for t, (qh, oh) in enumerate(zip(q_handles, out_handles)):
+            self.map_matmul_t_dev(map_id, qh, locs_k_handle, locs_scores_handle, 1, head_dim, n_keys0 + t, n_heads)
+            self.map_attn_softmax_value_dev(map_id, locs_scores_handle, locs_v_handle, oh, n_heads, n_keys0 + t,
+                                            value_dim, scale, softcap)
+
     def kv_cache_fp16(self, map_id, start, count):
         """Extension shared with the HIP library: elements [start, start+count) of a float32
         map are a KV cache kept in fp16.  Values copied or scattered into that range are rounded

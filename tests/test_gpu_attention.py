@@ -104,7 +104,7 @@ def test_gqa_heads_with_equal_queries_agree(hip):
             assert np.array_equal(out[g0 * 4], out[g0 * 4 + j])
 
 
-def chunk_case(g, q, K, V, seq0, cap_len, scale, softcap, gap=0):
+def chunk_case(g, q, K, V, seq0, cap_len, scale, softcap, gap=0, one_call=False):
     """m tokens' (scores, softmax.V) pairs in one batch: q [m, Hq, d]; token t sees seq0 + t cache rows.
     Layout: score rows, q [m][Hq][d], out [m][Hq][d] (+ gap floats between tokens), fp16 KV region."""
     m, Hq, d = q.shape
@@ -128,7 +128,9 @@ def chunk_case(g, q, K, V, seq0, cap_len, scale, softcap, gap=0):
     qh = [up(g, q_pos + t * Hq * d + np.arange(Hq) * d) for t in range(m)]
     oh = [up(g, out_pos + t * o_stride + np.arange(Hq) * d) for t in range(m)]
     g.batch_begin()
-    for t in range(m):
+    if one_call:
+        g.attn_causal_rows_dev(0, qh, k_locs, s_rows, v_locs, oh, d, seq0, Hq, d, scale, softcap)
+    for t in range(0 if one_call else m):
         g.map_matmul_t_dev(0, qh[t], k_locs, s_rows, 1, d, seq0 + t, Hq)
         g.map_attn_softmax_value_dev(0, s_rows, v_locs, oh[t], Hq, seq0 + t, d, scale, softcap)
     g.batch_end()
@@ -162,6 +164,28 @@ def test_prefill_chunk_is_one_causal_launch(hip, m, seq0, Hq, Hkv, d, softcap, g
         for h in range(Hq):
             assert rel_l2(out[t, h], ref[t, h]) < TOL, (t, h)
     assert rel_l2(scores, ref_scores) < 1e-5
+
+
+def test_causal_rows_entry_point_equals_the_pairs_issued_one_by_one(hip):
+    """adamah_attn_causal_rows_dev (an extension: m pairs in one native call) leaves the words the 2 m calls
+    leave, in as many launches; the oracle's form of it agrees within the attention bar; bad arguments fail."""
+    rng = np.random.default_rng(77)
+    m, seq0, Hq, Hkv, d = 33, 10, 8, 2, 128
+    cap_len = seq0 + m + 3
+    q = rng.standard_normal((m, Hq, d)).astype(np.float32)
+    K = rng.standard_normal((Hkv, cap_len, d)).astype(np.float32)
+    V = rng.standard_normal((Hkv, cap_len, d)).astype(np.float32)
+    scale = float(1.0 / np.sqrt(d))
+    note("attention causal rows entry point")
+    a = chunk_case(hip, q, K, V, seq0, cap_len, scale, 20.0, one_call=True)
+    b = chunk_case(hip, q, K, V, seq0, cap_len, scale, 20.0)
+    assert a[2] == b[2] == 1
+    assert np.array_equal(a[0].view(np.uint32), b[0].view(np.uint32)) and np.array_equal(a[1].view(np.uint32), b[1].view(np.uint32))
+    ref = chunk_case(oracle.init(), q, K, V, seq0, cap_len, scale, 20.0, one_call=True)
+    assert rel_l2(a[0], ref[0]) < TOL and rel_l2(a[1], ref[1]) < 1e-5
+    hip.attn_causal_rows_dev(0, [], 1, 1, 1, [], d, seq0, Hq, d, scale)           # m = 0: nothing to do
+    with pytest.raises(RuntimeError):
+        hip.attn_causal_rows_dev(0, [987654], 1, 1, 1, [987655], d, seq0, Hq, d, scale)   # unknown handles
 
 
 @pytest.mark.parametrize("layout,expect", [("hole", 2), ("irregular", 3)])
