@@ -49,10 +49,17 @@ class SyntheticEmbedding:
     def __init__(self, n_vocab, n_embd, seed, sigma):
         self.shape = (n_vocab, n_embd)
         self.seed, self.sigma = seed, sigma
+        self._seen = {}          # rows already generated (a real model's lookup is a copy, not a generator run)
 
     def row(self, tok):
-        rng = np.random.default_rng([self.seed, 0x0E3B, int(tok)])
-        return (rng.standard_normal(self.shape[1], dtype=np.float32) * np.float32(self.sigma))
+        tok = int(tok)
+        r = self._seen.get(tok)
+        if r is None:
+            rng = np.random.default_rng([self.seed, 0x0E3B, tok])
+            r = rng.standard_normal(self.shape[1], dtype=np.float32) * np.float32(self.sigma)
+            if len(self._seen) < 8192:
+                self._seen[tok] = r
+        return r
 
 
 def _gen(name, shape, seed, sigma, quant, rows_per_chunk=8192):
