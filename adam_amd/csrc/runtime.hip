@@ -313,6 +313,8 @@ static void destroy_map(Map* m) {
 
 using namespace adamah;
 
+static void plan_graph_reset(uint32_t plan_id);   // drops the recorded graphs of a decode plan (defined with them)
+
 // =================================================================================================
 extern "C" {
 
@@ -373,7 +375,7 @@ void adamah_shutdown(void) { ADAMAH_API();
   sampling_release();
   attn_decode_release();
   g.pend.clear();
-  for (int i = 0; i < MAX_PLANS; i++) { g.plans[i].clear(); g.plan_active[i] = false; }
+  for (int i = 0; i < MAX_PLANS; i++) { g.plans[i].clear(); g.plan_active[i] = false; plan_graph_reset(i); }
   hipStreamDestroy(g.stream);
   g.stream = nullptr;
   g.initialized = false;
@@ -744,18 +746,17 @@ int adamah_register_decode_plan(uint32_t plan_id, const AdamahDecodePlanOp* ops,
   g.plans[plan_id].resize(n_ops);
   if (n_ops) memcpy(g.plans[plan_id].data(), ops, sizeof(PlanOp) * n_ops);
   g.plan_active[plan_id] = true;
+  plan_graph_reset(plan_id);
   return ADAMAH_OK;
 }
 void adamah_clear_decode_plan(uint32_t plan_id) { ADAMAH_API();
   if (plan_id >= MAX_PLANS) return;
   g.plans[plan_id].clear();
   g.plan_active[plan_id] = false;
+  plan_graph_reset(plan_id);
 }
-int adamah_decode_step(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
-  if (plan_id >= MAX_PLANS) return ADAMAH_ERR_INVALID;
-  if (!g.plan_active[plan_id]) return ADAMAH_ERR_NOT_FOUND;
-  bool opened = g.batch_depth == 0;
-  if (opened) batch_begin();
+// The op list of a plan with pos / seq_len substituted, through the ordinary entry points.
+static int replay_plan(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
   int ret = ADAMAH_OK;
   for (const PlanOp& op : g.plans[plan_id]) {
     auto rs = [&](uint32_t v) { return v == RT_POS ? pos : v == RT_SEQ ? seq_len : v; };
@@ -784,6 +785,114 @@ int adamah_decode_step(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
       default: ret = ADAMAH_ERR_INVALID; break;   // fused qkv / gate-up kinds are not built
     }
     if (ret != ADAMAH_OK) break;
+  }
+  return ret;
+}
+
+// Graph replay of a plan (ADAMAH_PLAN_GRAPH=1).  A decode loop calls the plan with pos, pos + 1, ...: after
+// serving step (pos, seq_len) the library records the launches of step (pos + 1, seq_len + 1) into a HIP graph
+// -- stream capture of the same entry points, nothing executes -- while the device is still busy with the
+// current step, and the next call launches that graph if it asks for exactly that step (anything else is
+// replayed the ordinary way).  Kernels of a graph start ~0.7 us sooner after their predecessor than
+// stream launches do.  Two executable graphs alternate, so the one being updated is never in flight.
+// A plan whose ops copy from the host (tables of operand bases) or fail to capture is left to the
+// ordinary replay for good.
+struct PlanGraph {
+  hipGraphExec_t exec[2] = {nullptr, nullptr};
+  int cur = 0;               // exec[cur] holds the recorded step when ready
+  bool ready = false, disabled = false;
+  uint32_t pos = 0, seq = 0, n_nodes = 0;
+  int eager_steps = 0;
+  uint32_t n_graph = 0, n_update = 0, n_inst = 0;   // steps served by a graph, in-place updates, instantiations
+};
+static PlanGraph g_pg[MAX_PLANS];
+
+static bool plan_graphs_on() {
+  static int on = -1;
+  if (on < 0) { const char* e = getenv("ADAMAH_PLAN_GRAPH"); on = (e && e[0] == '1') ? 1 : 0; }
+  return on == 1;
+}
+
+static void plan_graph_drop(PlanGraph& pg, bool for_good) {
+  for (int i = 0; i < 2; i++) { if (pg.exec[i]) hipGraphExecDestroy(pg.exec[i]); pg.exec[i] = nullptr; }
+  pg.ready = false;
+  if (for_good) pg.disabled = true;
+}
+
+static void plan_graph_record(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
+  PlanGraph& pg = g_pg[plan_id];
+  pg.ready = false;
+  const uint64_t gen0 = g.mem_gen;
+  const Stats saved = g.stats;
+  if (hipStreamBeginCapture(g.stream, hipStreamCaptureModeThreadLocal) != hipSuccess) { (void)hipGetLastError(); plan_graph_drop(pg, true); return; }
+  int r = replay_plan(plan_id, pos, seq_len);
+  flush_pending();
+  hipGraph_t graph = nullptr;
+  const hipError_t e = hipStreamEndCapture(g.stream, &graph);
+  const uint32_t n_nodes = (uint32_t)(g.stats.dispatch - saved.dispatch);
+  g.stats = saved;                                   // nothing ran: the launches are counted when the graph does
+  if (r != ADAMAH_OK || e != hipSuccess || !graph || g.mem_gen != gen0 || n_nodes == 0) {
+    if (graph) hipGraphDestroy(graph);
+    (void)hipGetLastError();
+    plan_graph_drop(pg, true);
+    return;
+  }
+  const int slot = pg.cur ^ 1;
+  if (pg.exec[slot]) {
+    hipGraphNode_t bad = nullptr;
+    hipGraphExecUpdateResult res;
+    if (hipGraphExecUpdate(pg.exec[slot], graph, &bad, &res) != hipSuccess) {   // another launch shape (e.g. one more slice)
+      (void)hipGetLastError();
+      hipGraphExecDestroy(pg.exec[slot]);
+      pg.exec[slot] = nullptr;
+    } else pg.n_update++;
+  }
+  const bool fresh = !pg.exec[slot];
+  if (fresh) pg.n_inst++;
+  if (!pg.exec[slot] && hipGraphInstantiate(&pg.exec[slot], graph, nullptr, nullptr, 0) != hipSuccess) {
+    (void)hipGetLastError();
+    pg.exec[slot] = nullptr;
+    hipGraphDestroy(graph);
+    plan_graph_drop(pg, true);
+    return;
+  }
+  hipGraphDestroy(graph);
+  pg.cur = slot; pg.ready = true; pg.pos = pos; pg.seq = seq_len; pg.n_nodes = n_nodes;
+}
+
+static void plan_graph_reset(uint32_t plan_id) {
+  const PlanGraph& o = g_pg[plan_id];
+  if (getenv("ADAMAH_DEBUG") && (o.n_graph || o.eager_steps))
+    fprintf(stderr, "[adamah] plan %u: %u steps from graphs, %d replayed, %u updates, %u instantiations, %u nodes%s\n", plan_id,
+            o.n_graph, o.eager_steps, o.n_update, o.n_inst, o.n_nodes, o.disabled ? ", graphs given up" : "");
+  hipStreamSynchronize(g.stream);
+  plan_graph_drop(g_pg[plan_id], false);
+  g_pg[plan_id] = PlanGraph();
+}
+
+int adamah_decode_step(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
+  if (plan_id >= MAX_PLANS) return ADAMAH_ERR_INVALID;
+  if (!g.plan_active[plan_id]) return ADAMAH_ERR_NOT_FOUND;
+  bool opened = g.batch_depth == 0;
+  if (opened) batch_begin();
+  int ret;
+  PlanGraph& pg = g_pg[plan_id];
+  if (!plan_graphs_on() || pg.disabled) ret = replay_plan(plan_id, pos, seq_len);
+  else {
+    flush_pending();                                 // what was queued before the plan runs ahead of it
+    if (pg.ready && pg.pos == pos && pg.seq == seq_len) {
+      ret = hipGraphLaunch(pg.exec[pg.cur], g.stream) == hipSuccess ? ADAMAH_OK : ADAMAH_ERR_BACKEND;
+      count_launch((int)pg.n_nodes);
+      pg.n_graph++;
+    } else {
+      ret = replay_plan(plan_id, pos, seq_len);
+      flush_pending();
+      pg.eager_steps++;
+    }
+    // the first steps run the ordinary way (scratch buffers reach their sizes); then record the next one
+    if (ret == ADAMAH_OK && pg.eager_steps >= 2 && pos != 0xFFFFFFFFu && seq_len != 0xFFFFFFFFu)
+      plan_graph_record(plan_id, pos + 1, seq_len + 1);
+    else pg.ready = false;
   }
   if (opened) batch_end();
   return ret;

@@ -208,3 +208,47 @@ def test_batched_lockstep_decode(hip, arch):
     for sq in range(4):
         for i in range(10):
             assert out[sq][i] == refs[sq][0][i] or refs[sq][1][i] < 5e-2, (sq, i, out[sq][i], refs[sq][0][i], refs[sq][1][i])
+
+
+_GRAPH_SNIPPET = """
+import sys, json
+sys.path.insert(0, {root!r})
+import numpy as np
+from adam_amd import adamah as A, synth
+from adam_amd.engine import DecodeEngine, GenerationConfig
+cfg = synth.tiny_config({arch!r}, n_layer=3, n_embd=256, n_head=4, n_head_kv=2, head_dim=64, n_ff=512, n_vocab=1000)
+tensors = synth.make_model(cfg, seed=5, sigma=0.1)
+gpu = A.init()
+eng = DecodeEngine(gpu, cfg, tensors, A=A, kv_cap=96, kv_fp16=True)
+out = []
+for prompt in ([3, 99, 512, 7, 640, 31], [5, 6]):          # a second prompt: the step sequence restarts
+    toks, _ = eng.generate(prompt, GenerationConfig(max_tokens=40))
+    out.append([int(t) for t in toks])
+hid = eng.read_slot('hidden')
+gpu.shutdown()
+print(json.dumps({{"tokens": out, "hidden": [float(v) for v in hid[:64]]}}))
+"""
+
+
+@pytest.mark.parametrize("arch", ["gemma3", "llama"])
+def test_decode_plan_from_recorded_graphs_gives_the_same_tokens(arch):
+    """ADAMAH_PLAN_GRAPH=1: the plan's launches for the next position are recorded into a HIP graph while the
+    current step runs and replayed by the next call.  Two generations (80 graph replays with the token read
+    and the embedding upload between them) give the tokens and the final hidden state, bit for bit, of the
+    ordinary replay.  Each mode runs in a process of its own (the switch is read once)."""
+    import json, os, subprocess, sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = {}
+    for mode in ("0", "1"):
+        note(f"decode plan graphs {arch} mode {mode}")
+        env = dict(os.environ, ADAMAH_PLAN_GRAPH=mode, ADAMAH_DEBUG="1")
+        p = subprocess.run([sys.executable, "-c", _GRAPH_SNIPPET.format(root=root, arch=arch)], env=env, capture_output=True,
+                           text=True, timeout=110)
+        assert p.returncode == 0, p.stderr[-2000:]
+        res[mode] = json.loads(p.stdout.strip().split("\n")[-1])
+        if mode == "1":
+            line = [l for l in p.stderr.split("\n") if "steps from graphs" in l]
+            assert line and "given up" not in line[-1], p.stderr[-1000:]
+            assert int(line[-1].split(":")[1].split()[0]) >= 60, line[-1]       # most steps came from graphs
+    assert res["0"]["tokens"] == res["1"]["tokens"]
+    assert res["0"]["hidden"] == res["1"]["hidden"]
