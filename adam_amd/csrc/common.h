@@ -81,7 +81,7 @@ struct PendOp {
   // ROPE (one token): a = src, c = dst, rpg = heads, k = head dim, n = position, eps = frequency base.
   // QKNR: h = q rows, q weights, k rows, k weights, dst; rpg/k = q rows/dim, op/d = k rows/dim, n, eps as ROPE.
   // ROWCOPY: h = spec, source base; rpg = copies, k = row size, n = destination row offset.
-  // GEMM (2..32 activation rows, block16 weights): a, b, c = X, W, Y; rpg = M; k, n = K, N; op = weight format;
+  // GEMM (two or more activation rows, block16 weights): a, b, c = X, W, Y; rpg = M; k, n = K, N; op = weight format;
   //   h = X, W, Y handles.
 };
 

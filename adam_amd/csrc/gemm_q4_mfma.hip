@@ -238,7 +238,7 @@ template <int MT, int R>
 __global__ void __launch_bounds__(256)
 k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh,
                     const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc, const float* __restrict__ scale,
-                    uint32_t M, uint32_t K, uint32_t N) {
+                    uint32_t M, uint32_t K, uint32_t N, GemmSegs segs) {
   constexpr uint32_t BM = 16u * MT, ROWB = 272u;
   __shared__ __attribute__((aligned(16))) uint8_t xs[BM * ROWB];
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -332,7 +332,13 @@ k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __r
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const uint32_t n = n0 + r * 16u + 4u * g + i;
-        if (n < N) c[n] = acc[r][t][i] * inv;
+        if (n >= N) continue;
+        if (segs.count) {   // stacked matrices: the row's own matrix and its result base
+          uint32_t sgi = 0;
+#pragma unroll
+          for (uint32_t q = 1; q < 4; q++) sgi += (q < segs.count && n >= segs.begin[q]) ? 1u : 0u;
+          out[segs.c[sgi] + (uint64_t)row * segs.n[sgi] + (n - segs.begin[sgi])] = acc[r][t][i] * inv;
+        } else c[n] = acc[r][t][i] * inv;
       }
   }
 }
@@ -605,7 +611,8 @@ void gemm_act_mark(const void* buf, uint64_t a, uint32_t M, uint32_t K) {
 int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb, const uint32_t* lc,
                         uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops, bool q8, float* out, int64_t a_host,
                         int64_t c_host, const GemmSegs* segs) {
-  if (((q8 || out || segs) && M > 32) || ((out || segs) && n_ops != 1) || (out && segs)) return ADAMAH_ERR_INVALID;
+  if (((q8 || out) && M > 32) || ((out || segs) && n_ops != 1) || (out && segs) || (segs && segs->add && M > 32))
+    return ADAMAH_ERR_INVALID;
   GemmSegs sg = {};
   if (segs) sg = *segs;
   const size_t need = (size_t)2 * M * n_ops;
@@ -683,7 +690,7 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
   R = (uint32_t)tuning("ADAMAH_GEMM_R", (int)R);
   R = R >= 4 && mt == 4 ? 4 : R >= 2 ? 2 : 1;
   dim3 grid(cdiv(N, 64 * R), cdiv(M, 16 * mt), n_ops);
-#define GT(T, RR) k_gemm_q4_f16_tiled<T, RR><<<grid, 256, 0, g.stream>>>(act, mw->buf, mw->d16, (const u4q_t*)g_xh_buf, lb, lc, g_scale_buf, M, K, N)
+#define GT(T, RR) k_gemm_q4_f16_tiled<T, RR><<<grid, 256, 0, g.stream>>>(act, mw->buf, mw->d16, (const u4q_t*)g_xh_buf, lb, lc, g_scale_buf, M, K, N, sg)
   if (mt == 4) { if (R == 4) GT(4, 4); else if (R == 2) GT(4, 2); else GT(4, 1); }
   else { if (R == 2) GT(8, 2); else GT(8, 1); }
 #undef GT

@@ -199,7 +199,8 @@ def test_rmsnorm_rows_feed_the_matmul_without_a_conversion_launch(hip, dim, rows
 
 
 @pytest.mark.parametrize("kind,M,K,Ns", [("q4", 16, 4096, (4096, 1024, 1024)), ("q4", 5, 256, (40, 24)), ("q8", 16, 512, (100, 60, 33, 7)),
-                                         ("q4", 32, 1152, (1024, 256, 256))])
+                                         ("q4", 32, 1152, (1024, 256, 256)), ("q4", 100, 256, (200, 72, 72)),
+                                         ("q4", 512, 4096, (4096, 1024, 1024))])
 def test_stacked_matmuls_place_every_result_where_its_op_asked(hip, kind, M, K, Ns):
     """Matmuls over the same rows with weight matrices back to back but results at unrelated places and of
     different widths (not multiples of 16 either): one launch, each [M, N_i] result at its own base, equal
