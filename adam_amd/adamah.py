@@ -88,6 +88,7 @@ _SIGS = {
     "adamah_clear_decode_plan": (None, [_U]), "adamah_decode_step": (i32, [_U] * 3),
     "adamah_kv_cache_fp16": (i32, [_U] * 3),
     "adamah_attn_causal_rows_dev": (i32, [_U, pu32, _U, _U, _U, pu32, _U, _U, _U, _U, _U, f32c, f32c]),
+    "adamah_qk_norm_rope_rows_dev": (i32, [_U, _U, pu32, _U, pu32, _U, pu32, _U, _U, _U, _U, _U, _U, f32c]),
     "batch_begin": (None, []), "batch_end": (None, []),
     "map_init": (i32, [_U] * 4), "map_init_dtype": (i32, [_U] * 5), "map_destroy": (i32, [_U]),
     "map_size": (u64, [_U]), "map_get_dtype": (u32, [_U]),
@@ -147,6 +148,7 @@ _OPTIONAL_FLAGS = {
     "adamah_set_dtype": "_has_dtype",
     "adamah_kv_cache_fp16": "_has_kv_cache_fp16",
     "adamah_attn_causal_rows_dev": "_has_attn_causal_rows_dev",
+    "adamah_qk_norm_rope_rows_dev": "_has_qk_norm_rope_rows_dev",
     "map_resolve_idx_dev": "_has_map_resolve_idx_dev",
     "map_sample_categorical_dev": "_has_map_sample_categorical_dev",
     "map_repeat_penalty_dev": "_has_map_repeat_penalty_dev",
@@ -419,6 +421,15 @@ class Adamah:
         oa = (ctypes.c_uint32 * m)(*out_handles)
         self._op("adamah_attn_causal_rows_dev", map_id, qa, locs_k_handle, locs_scores_handle, locs_v_handle, oa, m,
                  head_dim, n_keys0, n_heads, value_dim, scale, softcap)
+
+    def qk_norm_rope_rows_dev(self, map_act, map_wt, q_src_handles, locs_q_wt_handle, k_src_handles, locs_k_wt_handle,
+                              dst_handles, q_rows, q_dim, k_rows, k_dim, pos0, freq_base):
+        """Extension: map_qk_norm_rope_x_dev for token t = 0 .. len(q_src_handles) - 1 at position pos0 + t in one
+        native call."""
+        m = len(q_src_handles)
+        arr = lambda hs: (ctypes.c_uint32 * m)(*hs)
+        self._op("adamah_qk_norm_rope_rows_dev", map_act, map_wt, arr(q_src_handles), locs_q_wt_handle, arr(k_src_handles),
+                 locs_k_wt_handle, arr(dst_handles), m, q_rows, q_dim, k_rows, k_dim, pos0, freq_base)
 
     def map_rope_dev(self, map_id, locs_src_handle, locs_dst_handle, n_tokens, n_heads, head_dim,
                      pos_offset=0, freq_base=10000.0):

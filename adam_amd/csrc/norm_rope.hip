@@ -323,4 +323,18 @@ int map_row_copy_dev(uint32_t map_id, uint32_t hspec, uint32_t hbase, uint32_t n
   return map_row_copy_offset_dev(map_id, hspec, hbase, 0, n_copies, row_size);
 }
 
+int adamah_qk_norm_rope_rows_dev(uint32_t map_act, uint32_t map_wt, const uint32_t* q_src_handles, uint32_t locs_q_wt,
+                                 const uint32_t* k_src_handles, uint32_t locs_k_wt, const uint32_t* dst_handles,
+                                 uint32_t m, uint32_t q_rows, uint32_t q_dim, uint32_t k_rows, uint32_t k_dim,
+                                 uint32_t pos0, float freq_base) {
+  if (m == 0) return ADAMAH_OK;
+  if (!q_src_handles || !k_src_handles || !dst_handles) return ADAMAH_ERR_INVALID;
+  for (uint32_t t = 0; t < m; t++) {
+    const int r = map_qk_norm_rope_x_dev(map_act, map_wt, q_src_handles[t], locs_q_wt, k_src_handles[t], locs_k_wt,
+                                         dst_handles[t], q_rows, q_dim, k_rows, k_dim, pos0 + t, freq_base);
+    if (r != ADAMAH_OK) return r;
+  }
+  return ADAMAH_OK;
+}
+
 }  // extern "C"

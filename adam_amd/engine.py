@@ -805,7 +805,11 @@ class DecodeEngine:
             mm('normed', f'{p}.attn_q.weight', 'q', E, q_dim)
             mm('normed', f'{p}.attn_k.weight', 'k', E, k_dim)
             mm('normed', f'{p}.attn_v.weight', 'v', E, k_dim)
-            if self._chunk_qk:
+            if self._chunk_qk and not lockstep and hasattr(g, 'qk_norm_rope_rows_dev'):
+                g.qk_norm_rope_rows_dev(ws, ws, self._c_lq[:m], self._wh[f'{p}.attn_q_norm.weight'], self._c_lk[:m],
+                                        self._wh[f'{p}.attn_k_norm.weight'], self._c_qkdst[:m], c.n_head, c.head_dim,
+                                        c.n_head_kv, c.head_dim_kv, pos0, freq)
+            elif self._chunk_qk:
                 qn, kn = self._wh[f'{p}.attn_q_norm.weight'], self._wh[f'{p}.attn_k_norm.weight']
                 for t in range(m):
                     g.map_qk_norm_rope_x_dev(ws, ws, self._c_lq[t], qn, self._c_lk[t], kn, self._c_qkdst[t],

@@ -234,6 +234,14 @@ int adamah_kv_cache_fp16(uint32_t map_id, uint32_t start, uint32_t count);
 int adamah_attn_causal_rows_dev(uint32_t map_id, const uint32_t* q_handles, uint32_t locs_k, uint32_t locs_scores,
                                 uint32_t locs_v, const uint32_t* out_handles, uint32_t m, uint32_t head_dim,
                                 uint32_t n_keys0, uint32_t n_heads, uint32_t value_dim, float scale, float softcap);
+/* QK-norm + RoPE of m consecutive tokens in one call: for t = 0 .. m-1 exactly
+ * map_qk_norm_rope_x_dev(map_act, map_wt, q_src_handles[t], locs_q_wt, k_src_handles[t], locs_k_wt,
+ * dst_handles[t], q_rows, q_dim, k_rows, k_dim, pos0 + t, freq_base)  (adamah.c:8586) -- the companion of
+ * adamah_attn_causal_rows_dev for models with per-head Q/K norms.  The three lists: m handle ids each. */
+int adamah_qk_norm_rope_rows_dev(uint32_t map_act, uint32_t map_wt, const uint32_t* q_src_handles, uint32_t locs_q_wt,
+                                 const uint32_t* k_src_handles, uint32_t locs_k_wt, const uint32_t* dst_handles,
+                                 uint32_t m, uint32_t q_rows, uint32_t q_dim, uint32_t k_rows, uint32_t k_dim,
+                                 uint32_t pos0, float freq_base);
 /* HIP-event stopwatch on the library's stream (benchmarks). begin: 0 on success; end: ms or <0. */
 int adamah_hip_timer_begin(void);
 float adamah_hip_timer_end(void);

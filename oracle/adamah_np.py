@@ -565,6 +565,13 @@ class NumpyAdamah:
             self.map_attn_softmax_value_dev(map_id, locs_scores_handle, locs_v_handle, oh, n_heads, n_keys0 + t,
                                             value_dim, scale, softcap)
 
+    def qk_norm_rope_rows_dev(self, map_act, map_wt, q_src_handles, locs_q_wt_handle, k_src_handles, locs_k_wt_handle,
+                              dst_handles, q_rows, q_dim, k_rows, k_dim, pos0, freq_base):
+        """Extension shared with the HIP library: map_qk_norm_rope_x_dev of m consecutive tokens, token t at pos0 + t."""
+        for t, (qh, kh, dh) in enumerate(zip(q_src_handles, k_src_handles, dst_handles)):
+            self.map_qk_norm_rope_x_dev(map_act, map_wt, qh, locs_q_wt_handle, kh, locs_k_wt_handle, dh, q_rows, q_dim,
+                                        k_rows, k_dim, pos0 + t, freq_base)
+
     def kv_cache_fp16(self, map_id, start, count):
         """Extension shared with the HIP library: elements [start, start+count) of a float32
         map are a KV cache kept in fp16.  Values copied or scattered into that range are rounded

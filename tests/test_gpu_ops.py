@@ -74,6 +74,42 @@ def test_qk_norm_rope_gemma_shape(hip):
     assert rel_l2(outs[0], outs[1]) < 1e-5
 
 
+def test_qk_norm_rope_rows_entry_point_equals_per_token_calls(hip):
+    """adamah_qk_norm_rope_rows_dev (an extension: m tokens at pos0, pos0 + 1, ... in one native call) leaves the
+    words the m calls of map_qk_norm_rope_x_dev leave, inside a batch and outside; the oracle's form agrees."""
+    Hq, Hk, D, m, pos0 = 4, 1, 256, 9, 300
+    per = (Hq + Hk) * D
+    rng = np.random.default_rng(15)
+    x = rng.standard_normal(m * per).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, 2 * D).astype(np.float32)
+    w0, dst0 = m * per, m * per + 2 * D
+
+    def go(g, one_call, batch):
+        f32map(g, 0, dst0 + m * per, np.concatenate([x, w]))
+        qs = [up(g, [t * per + i * D for i in range(Hq)]) for t in range(m)]
+        ks = [up(g, [t * per + Hq * D]) for t in range(m)]
+        ds = [up(g, [dst0 + t * per]) for t in range(m)]
+        qw, kw = up(g, [w0] * Hq), up(g, [w0 + D])
+        if batch:
+            g.batch_begin()
+        if one_call:
+            g.qk_norm_rope_rows_dev(0, 0, qs, qw, ks, kw, ds, Hq, D, Hk, D, pos0, 1e6)
+        else:
+            for t in range(m):
+                g.map_qk_norm_rope_x_dev(0, 0, qs[t], qw, ks[t], kw, ds[t], Hq, D, Hk, D, pos0 + t, 1e6)
+        if batch:
+            g.batch_end()
+        return read(g, 0, dst0, m * per)
+
+    note("qk_norm_rope rows entry point")
+    base = go(hip, False, False)
+    for batch in (False, True):
+        assert np.array_equal(go(hip, True, batch).view(np.uint32), base.view(np.uint32))
+    assert rel_l2(base, go(oracle.init(), True, False)) < 1e-5
+    with pytest.raises(RuntimeError):
+        hip.qk_norm_rope_rows_dev(0, 0, [987654], 1, [987655], 1, [987656], Hq, D, Hk, D, pos0, 1e6)
+
+
 def test_kv_append_rounds_to_fp16_and_mirrors(hip):
     Hkv, d, cap = 2, 64, 8
     rng = np.random.default_rng(6)
