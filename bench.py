@@ -407,6 +407,19 @@ def main():
     }
     del eng
 
+    if not args.no_roofline and not args.prefill_chunk:
+        # the same prompt prefilled as one chunk (projections as [512, K] matmuls, one causal attention launch per layer)
+        try:
+            eng2 = DecodeEngine(gpu, cfg, tensors, A=A, kv_cap=n_prompt + 16, kv_fp16=True,
+                                fusion_scheduler_mode=args.scheduler, prefill_chunk=n_prompt)
+            eng2.reset(); eng2.prefill(prompt); gpu.sync()
+            t0 = time.perf_counter(); eng2.prefill(prompt); gpu.sync(); dt = time.perf_counter() - t0
+            res["prefill_one_chunk"] = {"tokens": n_prompt, "ms": round(dt * 1e3, 2), "tok/s": round(n_prompt / dt, 1),
+                                        "first_token_same_as_token_by_token": bool(eng2.read_token() == tokens[0])}
+            del eng2
+        except Exception as e:                      # never let the extra leg cost the headline line
+            res["prefill_one_chunk"] = {"error": repr(e)[:200]}
+
     if not args.no_roofline:
         shapes = measure_gemv(gpu, A, LLAMA_GEMV_SHAPES + [CONFIG1_GEMV_SHAPE])
         top = shapes["28672x4096"]
