@@ -125,6 +125,7 @@ _SIGS = {
     "map_matvec_topk_t_xq4_ex_dev": (i32, [_U] * 11 + [f32c, _U]),
     "map_matvec_topk_t_xq8_ex_dev": (i32, [_U] * 11 + [f32c, _U]),
     "map_matvec_rerank_t_xq8_dev": (i32, [_U] * 12 + [f32c]),
+    "adamah_matvec_topk_t_xq4_noalloc_dev": (i32, [_U] * 11 + [f32c, _U]),
     "map_fused_qkv_t_xq4_dev": (i32, [_U] * 13), "map_fused_qkv_t_xq8_dev": (i32, [_U] * 13),
     "map_fused_gateup_t_xq4_dev": (i32, [_U] * 10), "map_fused_gateup_t_xq8_dev": (i32, [_U] * 10),
     "map_fused_gateup_act_t_xq8_dev": (i32, [_U] * 8),

@@ -159,6 +159,7 @@ bool res_run(uint32_t h, uint64_t n, uint32_t* start);
 void gemm_q4_mfma_release();   // frees the GEMM's scratch (shutdown)
 void sampling_release();       // frees the scratch lists of the chunked top-k (shutdown)
 void topk_fused_release();     // frees the scratch logits of the GEMV + top-k ops (shutdown)
+int topk_noalloc_setup(int device);   // topk_fused.hip: address of this device's fixed logit scratch (init)
 size_t launch_argmax_run(const std::vector<PendOp>& q, size_t i, int* rc);   // topk_fused.hip
 int launch_argmax_direct(const PendOp& p);   // gemv_q.hip: one queued Q8 GEMV + argmax
 int launch_rmsnorm_v(const PendOp& p);

@@ -341,6 +341,7 @@ int adamah_init_ex(uint64_t hot_bytes, uint64_t cold_bytes) {
   HIPCHK(hipMalloc((void**)&g.attn_scratch, g.attn_scratch_floats * sizeof(float)));
   HIPCHK(hipMalloc((void**)&g.sync_ctr, 1024));   // [0..63] GEMV prologues, [64..191] attention groups
   HIPCHK(hipMemsetAsync(g.sync_ctr, 0, 1024, g.stream));
+  if (int r = topk_noalloc_setup(g.device)) return r;
   g.pend.clear();
   g.batch_depth = 0; g.fusion_enabled = 0; g.scheduler_mode = 0; g.active_dtype = 0;
   g.stats = Stats();

@@ -16,11 +16,36 @@
 // first put, which no caller relies on).  Groups of up to 1024 rows are ranked by counting, for every
 // row, the rows that beat it; larger groups by k rounds of a workgroup-wide best-of.
 #include "gemv_common.h"
+#include <cstdio>
+#include <algorithm>
 #include "../../include/adamah_hip.h"
+
+// Logit scratch of the entry point that allocates nothing (adamah_matvec_topk_t_xq4_noalloc_dev): part of
+// the code object, one copy per GPU at that GPU's own address, held until the process ends.  In host code
+// this name is only a stand-in for the symbol: the device address comes from hipGetSymbolAddress
+// (topk_noalloc_setup) and only that pointer is ever handed to a kernel.
+#define NOALLOC_MAX_ROWS 262144u
+static __device__ __align__(256) float scratch[NOALLOC_MAX_ROWS];
 
 namespace adamah {
 
 #define TOPK_MAX 64u
+#define NOALLOC_MAX_DEVICES 16
+
+static float* g_noalloc_ptr[NOALLOC_MAX_DEVICES] = {nullptr};
+
+// Called by adamah_init with the library's device current: resolves this device's copy of `scratch`.
+int topk_noalloc_setup(int device) {
+  if (device < 0 || device >= NOALLOC_MAX_DEVICES) return ADAMAH_ERR_INVALID;
+  if (g_noalloc_ptr[device]) return ADAMAH_OK;
+  float* p = nullptr;
+  if (hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+    (void)hipGetLastError();
+    return ADAMAH_ERR_BACKEND;
+  }
+  g_noalloc_ptr[device] = p;
+  return ADAMAH_OK;
+}
 
 static float* g_logit_buf = nullptr;
 static size_t g_logit_cap = 0;   // floats
@@ -191,7 +216,7 @@ k_rerank_q8(float* act, const uint8_t* __restrict__ W, const float2* __restrict_
 
 static int op_matvec_topk(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t ha, uint32_t hb, uint32_t hpen,
                           uint32_t hidx, uint32_t hval, uint32_t K, uint32_t N, uint32_t k, uint32_t n_pen, float rp,
-                          uint32_t rows_per_group) {
+                          uint32_t rows_per_group, float* fixed_logits = nullptr) {
   Map* ma = get_map(map_act);
   Map* mw = get_map(map_wt);
   if (!ma || !mw) return ADAMAH_ERR_INVALID;
@@ -207,7 +232,8 @@ static int op_matvec_topk(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uin
   const uint32_t *ah = res_host(ha, 1), *bh = res_host(hb, 1);
   if (ah && !in_range(ah[0], K, ma->n_elems)) return ADAMAH_ERR_INVALID;
   if (bh && !in_range(bh[0], (uint64_t)N * K, mw->n_elems)) return ADAMAH_ERR_INVALID;
-  if (N > g_logit_cap) {
+  // fixed_logits: the caller's scratch of at least N floats (the entry point that may not allocate)
+  if (!fixed_logits && N > g_logit_cap) {
     if (g_logit_buf) { hipStreamSynchronize(g.stream); hipFree(g_logit_buf); }
     g_logit_cap = std::max<size_t>(N, 1u << 16);
     if (hipMalloc((void**)&g_logit_buf, g_logit_cap * sizeof(float)) != hipSuccess) {
@@ -215,19 +241,20 @@ static int op_matvec_topk(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uin
       return ADAMAH_ERR_MEMORY;
     }
   }
+  float* const logits = fixed_logits ? fixed_logits : g_logit_buf;
   float* act = (float*)ma->buf;
   uint64_t a0 = 0, b0 = 0;
   int r;
   if (dtype == DTYPE_Q4 && block_path_ok(ma, mw, ha, hb, K, N, &a0, &b0) && mfma_path_ok(mw, K) &&
       tuning("ADAMAH_GEMV_IMPL", 3) == 3) {
     r = launch_mfma_store(fmt_of(mw, b0, (uint64_t)N * K), ma, mw, (uint32_t)a0, (uint32_t)b0, 0u, K, N, nullptr,
-                          g_logit_buf);
+                          logits);
   } else {
     if (dtype == DTYPE_Q4)
-      k_matvec_rows<true><<<cdiv(N, 4), 256, 0, g.stream>>>(act, mw->buf, mw->qp, la, lb, g_logit_buf, K, N,
+      k_matvec_rows<true><<<cdiv(N, 4), 256, 0, g.stream>>>(act, mw->buf, mw->qp, la, lb, logits, K, N,
                                                             mw->group_size, ma->n_elems, mw->n_elems);
     else
-      k_matvec_rows<false><<<cdiv(N, 4), 256, 0, g.stream>>>(act, mw->buf, mw->qp, la, lb, g_logit_buf, K, N,
+      k_matvec_rows<false><<<cdiv(N, 4), 256, 0, g.stream>>>(act, mw->buf, mw->qp, la, lb, logits, K, N,
                                                              mw->group_size, ma->n_elems, mw->n_elems);
     count_launch();
     r = check_launch();
@@ -237,10 +264,10 @@ static int op_matvec_topk(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uin
   const uint64_t rws = std::min(rows_per_group, N);
   const bool by_rank = rows_per_group <= RANK_MAX && rws * rws / 256u <= (uint64_t)k * (rws / 256u + 40u);
   if (tuning("ADAMAH_TOPK_RANK", by_rank ? 1 : 0) != 0 && rows_per_group <= RANK_MAX)
-    k_group_topk_rank<<<n_groups, 256, 0, g.stream>>>(act, g_logit_buf, pen, lidx, lval, N, k, n_pen, rp,
+    k_group_topk_rank<<<n_groups, 256, 0, g.stream>>>(act, logits, pen, lidx, lval, N, k, n_pen, rp,
                                                       rows_per_group, ma->n_elems);
   else
-    k_group_topk<<<n_groups, 256, 0, g.stream>>>(act, g_logit_buf, pen, lidx, lval, N, k, n_pen, rp, rows_per_group,
+    k_group_topk<<<n_groups, 256, 0, g.stream>>>(act, logits, pen, lidx, lval, N, k, n_pen, rp, rows_per_group,
                                                  ma->n_elems);
   count_launch();
   return check_launch();
@@ -391,6 +418,27 @@ int map_matvec_topk_t_xq8_ex_dev(uint32_t ma, uint32_t mw, uint32_t a, uint32_t 
 int map_matvec_topk_t_xq8_dev(uint32_t ma, uint32_t mw, uint32_t a, uint32_t b, uint32_t pen, uint32_t idx, uint32_t val,
                               uint32_t K, uint32_t N, uint32_t k, uint32_t n_penalty, float repeat_penalty) { ADAMAH_API();
   return op_matvec_topk(DTYPE_Q8, ma, mw, a, b, pen, idx, val, K, N, k, n_penalty, repeat_penalty, 256u);
+}
+
+// The _ex form above for callers that cannot allocate (under HIP graph capture, in serving loops or
+// harnesses that forbid hipMalloc): same arguments, same results, but the logits go to the fixed `scratch`
+// array of this GPU instead of a buffer the library grows.  No hipMalloc / hipFree on this path.
+int adamah_matvec_topk_t_xq4_noalloc_dev(uint32_t ma, uint32_t mw, uint32_t a, uint32_t b, uint32_t pen, uint32_t idx,
+                                         uint32_t val, uint32_t K, uint32_t N, uint32_t k, uint32_t n_penalty,
+                                         float repeat_penalty, uint32_t rows_per_group) {
+  if (!g.initialized) return ADAMAH_ERR_INVALID;
+  if (!g.pend.empty()) {
+    // launching the queued ops of an open batch could grow library buffers: the caller has them launched first (adamah_sync, batch_end)
+    fprintf(stderr, "adamah_matvec_topk_t_xq4_noalloc_dev: ops are queued in the open batch; call adamah_sync or batch_end first\n");
+    return ADAMAH_ERR_INVALID;
+  }
+  if (N > NOALLOC_MAX_ROWS) {
+    fprintf(stderr, "adamah_matvec_topk_t_xq4_noalloc_dev: N = %u exceeds the fixed scratch of %u rows\n", N, NOALLOC_MAX_ROWS);
+    return ADAMAH_ERR_INVALID;
+  }
+  float* const sp = (g.device >= 0 && g.device < NOALLOC_MAX_DEVICES) ? g_noalloc_ptr[g.device] : nullptr;
+  if (!sp) return ADAMAH_ERR_BACKEND;
+  return op_matvec_topk(DTYPE_Q4, ma, mw, a, b, pen, idx, val, K, N, k, n_penalty, repeat_penalty, rows_per_group, sp);
 }
 
 int map_matvec_rerank_t_xq8_dev(uint32_t map_act, uint32_t map_wt, uint32_t ha, uint32_t hb, uint32_t hpart,

@@ -242,6 +242,18 @@ int adamah_qk_norm_rope_rows_dev(uint32_t map_act, uint32_t map_wt, const uint32
                                  const uint32_t* k_src_handles, uint32_t locs_k_wt, const uint32_t* dst_handles,
                                  uint32_t m, uint32_t q_rows, uint32_t q_dim, uint32_t k_rows, uint32_t k_dim,
                                  uint32_t pos0, float freq_base);
+/* map_matvec_topk_t_xq4_ex_dev for callers that cannot allocate.  No counterpart in the reference: it is for
+ * callers under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same arguments and
+ * results; the logits go to a fixed 1 MiB device array that is part of the library's code object (one copy per
+ * GPU, held until the process ends), so N <= 262144 (larger: -3 and a message on stderr).  Calls no hipMalloc /
+ * hipFree.  Ops still queued in an open batch are not launched by this call (their launch could grow library
+ * buffers): it returns -3 until adamah_sync or batch_end has launched them.  The array keeps the previous call's logits; every
+ * call overwrites rows [0, N) before ranking them, nothing has to start at zero.  Calls that overlap on one GPU
+ * (other streams, other threads) share the array and race. */
+int adamah_matvec_topk_t_xq4_noalloc_dev(uint32_t map_act, uint32_t map_wt, uint32_t locs_a, uint32_t locs_b,
+                                         uint32_t penalty_ids, uint32_t locs_idx_dst, uint32_t locs_val_dst,
+                                         uint32_t K, uint32_t N, uint32_t k, uint32_t n_penalty,
+                                         float repeat_penalty, uint32_t rows_per_group);
 /* HIP-event stopwatch on the library's stream (benchmarks). begin: 0 on success; end: ms or <0. */
 int adamah_hip_timer_begin(void);
 float adamah_hip_timer_end(void);
