@@ -32,176 +32,37 @@ typedef uint32_t u2q_t __attribute__((ext_vector_type(2)));
 typedef uint32_t u4q_t __attribute__((ext_vector_type(4)));
 typedef _Float16 h8q_t __attribute__((ext_vector_type(8)));
 
-// Per activation row: s = 2^e with max|x| * s in [2^13, 2^14) (1 when the row is zero, tiny or not
-// finite), and 1 / s.  One workgroup per row.
-__global__ void __launch_bounds__(256)
-k_row_pow2_scale(const float* act, const uint32_t* __restrict__ la, uint32_t M, uint32_t K, float* scale) {
-  __shared__ float red[4];
-  const uint32_t row = blockIdx.x, op = blockIdx.y, tid = threadIdx.x;
-  const float* x = act + (uint64_t)la[op] + (uint64_t)row * K;
-  float m = 0.f;
-  for (uint32_t i = tid; i < K; i += 256u) m = fmaxf(m, fabsf(x[i]));
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
-  if ((tid & 63u) == 0) red[tid >> 6] = m;
-  __syncthreads();
-  if (tid == 0) {
-    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    const uint32_t e = (__float_as_uint(m) >> 23) & 0xFFu;
-    float s = 1.f, inv = 1.f;
-    if (e >= 14u && e <= 254u) { s = __uint_as_float((267u - e) << 23); inv = __uint_as_float((e - 13u) << 23); }
-    scale[2 * ((uint64_t)op * M + row)] = s;
-    scale[2 * ((uint64_t)op * M + row) + 1] = inv;
-  }
+// Two-term operands.  A product w * x of the reference is a float32 product of float32 values; one fp16
+// rounding of each operand (2^-12 relative) is harmless in a single projection but adds up over the ~200
+// projections of a forward pass (a 512-token chunk ended 1.3e-3 .. 6e-3 away from the token-by-token hidden
+// state).  Both operands are therefore fed as exact sums of two fp16 numbers:
+//   x * s  = xh + xl          xh = fp16(x s), xl = fp16(x s - xh)                (22 significant bits)
+//   w      = wh + wl          d = dh + dl with dh = d with its low four mantissa bits cleared, so that
+//                             wh = dh (q - 8) and wl = dl (q - 8) are exact fp16 products
+// and three matrix instructions accumulate  wh xh + wl xh + wh xl  in float32 (every product exact; the
+// dropped wl xl is below 2^-18 of the term).  Q8_0 weights (the LM head of a lockstep batch, the last
+// projection of a pass) keep the one-term form.
+__device__ __forceinline__ void split_pair(float a, float b, uint32_t* hi, uint32_t* lo) {
+  const _Float16 ah = (_Float16)a, bh = (_Float16)b;
+  const h2q_t h = {ah, bh}, l = {(_Float16)(a - (float)ah), (_Float16)(b - (float)bh)};
+  *hi = __builtin_bit_cast(uint32_t, h);
+  *lo = __builtin_bit_cast(uint32_t, l);
+}
+// eight consecutive activations (already scaled) -> the 16-byte pieces of both planes, pairs in the order the
+// nibble unpacking produces: (0,4)(1,5)(2,6)(3,7)
+__device__ __forceinline__ void split_word(const float* v, uint4* hi, uint4* lo) {
+  split_pair(v[0], v[4], &hi->x, &lo->x);
+  split_pair(v[1], v[5], &hi->y, &lo->y);
+  split_pair(v[2], v[6], &hi->z, &lo->z);
+  split_pair(v[3], v[7], &hi->w, &lo->w);
 }
 
-template <int MT, bool KSPLIT>
+// The activations are converted once per matmul (or by the kernel that produced them) to the two fp16
+// planes the matrix cores consume: rows scaled by their power of two, elements of every 8-word in the
+// order (0,4)(1,5)(2,6)(3,7).  The matmul workgroups then copy 16-byte pieces into LDS.  One workgroup per
+// row; also stores (s, 1/s).  xl = second plane (same indexing as xh).
 __global__ void __launch_bounds__(256)
-k_gemm_q4_f16(const float* act, float* out, const uint8_t* __restrict__ W, const __half* __restrict__ d16,
-              const uint32_t* __restrict__ la, const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc,
-              const float* __restrict__ scale, uint32_t M, uint32_t K, uint32_t N) {
-  constexpr uint32_t BM = 16u * MT;
-  // activation tile: [row][block 0..3][64 bytes]; a row is padded to 272 bytes so that the sixteen rows
-  // a wave reads side by side fall into different banks
-  constexpr uint32_t ROWB = 272u;
-  constexpr uint32_t TILES = KSPLIT ? 4u : 1u;       // KSPLIT: one activation tile per wave
-  __shared__ __attribute__((aligned(16))) uint8_t xs_all[TILES * BM * ROWB];
-  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-  const uint32_t r16 = lane & 15u, g = lane >> 4;
-  uint8_t* xs = xs_all + (KSPLIT ? wave * BM * ROWB : 0u);
-  const uint32_t n0 = KSPLIT ? blockIdx.x * 16u : blockIdx.x * 64u + wave * 16u, m0 = blockIdx.y * BM, op = blockIdx.z;
-  const uint64_t a_off = la[op], c_off = lc[op], gbase = (uint64_t)lb[op] >> 5;
-  const uint32_t nblk = K >> 5;
-  const uint32_t nrow = min(n0 + r16, N - 1u);          // rows past N are clamped here and not stored
-
-  f4q_t acc[MT];
-#pragma unroll
-  for (int t = 0; t < MT; t++) acc[t] = (f4q_t){0.f, 0.f, 0.f, 0.f};
-
-  uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u, nib_lo = 0x000F000Fu, nib_hi = 0x00F000F0u;
-  asm volatile("" : "+v"(magic_lo));   // opaque: lets instruction selection use the three-operand and-or
-  asm volatile("" : "+v"(magic_hi));
-  asm volatile("" : "+s"(nib_lo));
-  asm volatile("" : "+s"(nib_hi));
-  const h2q_t off_lo = {(_Float16)-1032.f, (_Float16)-1032.f}, off_hi = {(_Float16)-72.f, (_Float16)-72.f};
-
-  // One step ahead: the weights and activation words of the next step are loaded into registers while
-  // the matrix cores work on the current one.
-  constexpr uint32_t NTH = KSPLIT ? 64u : 256u, WPT = BM * 16u / NTH;   // staging threads per tile, words per thread
-  const uint32_t st = KSPLIT ? lane : tid;
-  float xr[WPT][8], rs[WPT];
-  uint4 qn;
-  _Float16 dn;
-#pragma unroll
-  for (uint32_t u = 0; u < WPT; u++) {
-    const uint32_t row = m0 + ((st + u * NTH) >> 4);
-    rs[u] = row < M ? scale[2 * ((uint64_t)op * M + row)] : 0.f;     // rows past M become zeros
-  }
-  auto fetch = [&](uint32_t kb_raw) {   // always executed; steps past K re-read the last one and are not used
-    const uint32_t kb = min(kb_raw, nblk - 4u);
-    const uint64_t gi = gbase + (uint64_t)nrow * nblk + kb + g;
-    qn = *(const uint4*)(W + (gi << 4));
-    dn = __builtin_bit_cast(_Float16, d16[gi]);
-#pragma unroll
-    for (uint32_t u = 0; u < WPT; u++) {
-      const uint32_t w = st + u * NTH, row = min(m0 + (w >> 4), M - 1u), wi = w & 15u;
-      const f4qu_t* p = (const f4qu_t*)(act + a_off + (uint64_t)row * K + (uint64_t)kb * 32u + wi * 8u);
-      const f4qu_t v0 = p[0], v1 = p[1];
-      xr[u][0] = v0.x; xr[u][1] = v0.y; xr[u][2] = v0.z; xr[u][3] = v0.w;
-      xr[u][4] = v1.x; xr[u][5] = v1.y; xr[u][6] = v1.z; xr[u][7] = v1.w;
-    }
-  };
-  fetch(KSPLIT ? wave * 4u : 0u);
-
-  for (uint32_t kb0 = 0; kb0 < nblk; kb0 += KSPLIT ? 16u : 4u) {
-    // KSPLIT: wave w takes step kb0/4 + w; a wave whose step lies past K idles through the barriers
-    const uint32_t kb_raw = kb0 + (KSPLIT ? wave * 4u : 0u);
-    const bool busy = kb_raw < nblk;
-    const uint4 q = qn;
-    const _Float16 d = dn;
-    // activations of the step -> fp16 in LDS, element order inside a word following the nibble pairs of
-    // the unpacking: (0,4)(1,5) | (2,6)(3,7)
-#pragma unroll
-    for (uint32_t u = 0; u < WPT; u++) {
-      const uint32_t w = st + u * NTH, m = w >> 4, wi = w & 15u;
-      const float sc = rs[u];
-      const h2q_t p0 = {(_Float16)(xr[u][0] * sc), (_Float16)(xr[u][4] * sc)}, p1 = {(_Float16)(xr[u][1] * sc), (_Float16)(xr[u][5] * sc)};
-      const h2q_t p2 = {(_Float16)(xr[u][2] * sc), (_Float16)(xr[u][6] * sc)}, p3 = {(_Float16)(xr[u][3] * sc), (_Float16)(xr[u][7] * sc)};
-      *(uint4*)(xs + m * ROWB + wi * 16u) =
-          make_uint4(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1),
-                     __builtin_bit_cast(uint32_t, p2), __builtin_bit_cast(uint32_t, p3));
-    }
-    // dequantise: (1024 + n) - 1032 = n - 8 and (64 + n) - 72 = n - 8 exactly, then one rounding in d * (n - 8)
-    uint32_t wq[8][2];
-    const h2q_t d2 = {d, d};
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const uint32_t w = j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w, w8 = w >> 8;
-      const h2q_t t0 = __builtin_bit_cast(h2q_t, (w & nib_lo) | magic_lo), t1 = __builtin_bit_cast(h2q_t, (w & nib_hi) | magic_hi);
-      const h2q_t t2 = __builtin_bit_cast(h2q_t, (w8 & nib_lo) | magic_lo), t3 = __builtin_bit_cast(h2q_t, (w8 & nib_hi) | magic_hi);
-      wq[2 * j][0] = __builtin_bit_cast(uint32_t, (h2q_t)((t0 + off_lo) * d2));
-      wq[2 * j][1] = __builtin_bit_cast(uint32_t, (h2q_t)((t1 + off_hi) * d2));
-      wq[2 * j + 1][0] = __builtin_bit_cast(uint32_t, (h2q_t)((t2 + off_lo) * d2));
-      wq[2 * j + 1][1] = __builtin_bit_cast(uint32_t, (h2q_t)((t3 + off_hi) * d2));
-    }
-    __syncthreads();
-    fetch(kb_raw + (KSPLIT ? 16u : 4u));
-    if (busy) {
-#pragma unroll
-    for (int t = 0; t < MT; t++) {
-      const uint8_t* xp = xs + (t * 16u + r16) * ROWB + g * 64u;
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const uint4 xv = *(const uint4*)(xp + j * 16);
-        // one K = 32 instruction over the two 4-element operand pairs (the sum over the 32 k is the same
-        // whichever lane group and slot a pair sits in, as long as A and B agree)
-        const u4q_t a = {wq[2 * j][0], wq[2 * j][1], wq[2 * j + 1][0], wq[2 * j + 1][1]};
-        const u4q_t b = {xv.x, xv.y, xv.z, xv.w};
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8q_t, a), __builtin_bit_cast(h8q_t, b), acc[t], 0, 0, 0);
-      }
-    }
-    }
-    __syncthreads();
-  }
-  if (KSPLIT) {   // sum the four waves' tiles in wave order; wave 0 stores
-    float* part = (float*)xs_all;             // 3 * 64 * 4 * MT floats, the activation tiles are done with
-    if (wave > 0) {
-#pragma unroll
-      for (int t = 0; t < MT; t++)
-#pragma unroll
-        for (int r = 0; r < 4; r++) part[(((wave - 1u) * MT + t) * 4u + r) * 64u + lane] = acc[t][r];
-    }
-    __syncthreads();
-    if (wave > 0) return;
-#pragma unroll
-    for (uint32_t w = 0; w < 3; w++)
-#pragma unroll
-      for (int t = 0; t < MT; t++)
-#pragma unroll
-        for (int r = 0; r < 4; r++) acc[t][r] += part[((w * MT + t) * 4u + r) * 64u + lane];
-  }
-  // lane (j = r16, g) holds D[4g + r][j]: weight rows n0 + 4g + r, activation row m0 + 16 t + r16
-#pragma unroll
-  for (int t = 0; t < MT; t++) {
-    const uint32_t row = m0 + t * 16u + r16;
-    if (row >= M) continue;
-    const float inv = scale[2 * ((uint64_t)op * M + row) + 1];
-    float* c = out + c_off + (uint64_t)row * N;
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-      const uint32_t n = n0 + 4u * g + r;
-      if (n < N) c[n] = acc[t][r] * inv;
-    }
-  }
-}
-
-
-// Large M: the activations are converted once, by a kernel of their own, to the fp16 form the matrix
-// cores consume (scaled per row by its power of two, elements of every 8-word in the order the nibble
-// unpacking produces: (0,4)(1,5)(2,6)(3,7)), so the matmul workgroups copy 16-byte pieces into LDS
-// instead of each converting the whole tile again.  One workgroup per row; also stores (s, 1/s).
-__global__ void __launch_bounds__(256)
-k_act_f16(const float* act, const uint32_t* __restrict__ la, uint32_t M, uint32_t K, float* scale, uint4* xh) {
+k_act_f16(const float* act, const uint32_t* __restrict__ la, uint32_t M, uint32_t K, float* scale, uint4* xh, uint4* xl) {
   __shared__ float red[4];
   const uint32_t row = blockIdx.x, op = blockIdx.y, tid = threadIdx.x;
   const float* x = act + (uint64_t)la[op] + (uint64_t)row * K;
@@ -219,28 +80,64 @@ k_act_f16(const float* act, const uint32_t* __restrict__ la, uint32_t M, uint32_
     scale[2 * ((uint64_t)op * M + row)] = s;
     scale[2 * ((uint64_t)op * M + row) + 1] = inv;
   }
-  uint4* dst = xh + ((uint64_t)op * M + row) * (K >> 3);
+  const uint64_t o0 = ((uint64_t)op * M + row) * (K >> 3);
   for (uint32_t w = tid; w < (K >> 3); w += 256u) {
     const f4qu_t v0 = *(const f4qu_t*)(x + w * 8u), v1 = *(const f4qu_t*)(x + w * 8u + 4u);
-    const h2q_t p0 = {(_Float16)(v0.x * s), (_Float16)(v1.x * s)}, p1 = {(_Float16)(v0.y * s), (_Float16)(v1.y * s)};
-    const h2q_t p2 = {(_Float16)(v0.z * s), (_Float16)(v1.z * s)}, p3 = {(_Float16)(v0.w * s), (_Float16)(v1.w * s)};
-    dst[w] = make_uint4(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1),
-                        __builtin_bit_cast(uint32_t, p2), __builtin_bit_cast(uint32_t, p3));
+    const float v[8] = {v0.x * s, v0.y * s, v0.z * s, v0.w * s, v1.x * s, v1.y * s, v1.z * s, v1.w * s};
+    uint4 hi, lo;
+    split_word(v, &hi, &lo);
+    xh[o0 + w] = hi;
+    xl[o0 + w] = lo;
   }
 }
 
+// nibbles of one 32-bit word -> the four fp16 pairs (q - 8) exactly: (1024 + n) - 1032 and (64 + n) - 72
+struct DeqK { uint32_t magic_lo, magic_hi, nib_lo, nib_hi; h2q_t off_lo, off_hi; };
+__device__ __forceinline__ void deq_ints(uint32_t w, const DeqK& c, h2q_t* t) {
+  const uint32_t w8 = w >> 8;
+  t[0] = __builtin_bit_cast(h2q_t, (w & c.nib_lo) | c.magic_lo) + c.off_lo;
+  t[1] = __builtin_bit_cast(h2q_t, (w & c.nib_hi) | c.magic_hi) + c.off_hi;
+  t[2] = __builtin_bit_cast(h2q_t, (w8 & c.nib_lo) | c.magic_lo) + c.off_lo;
+  t[3] = __builtin_bit_cast(h2q_t, (w8 & c.nib_hi) | c.magic_hi) + c.off_hi;
+}
+// one word of a block -> its operand fragment in both terms: wh = dh (q - 8), wl = dl (q - 8), exact
+__device__ __forceinline__ void deq_word2(uint32_t w, const DeqK& c, h2q_t dh2, h2q_t dl2, u4q_t* ah, u4q_t* al) {
+  h2q_t t[4];
+  deq_ints(w, c, t);
+  *ah = (u4q_t){__builtin_bit_cast(uint32_t, (h2q_t)(t[0] * dh2)), __builtin_bit_cast(uint32_t, (h2q_t)(t[1] * dh2)),
+                __builtin_bit_cast(uint32_t, (h2q_t)(t[2] * dh2)), __builtin_bit_cast(uint32_t, (h2q_t)(t[3] * dh2))};
+  *al = (u4q_t){__builtin_bit_cast(uint32_t, (h2q_t)(t[0] * dl2)), __builtin_bit_cast(uint32_t, (h2q_t)(t[1] * dl2)),
+                __builtin_bit_cast(uint32_t, (h2q_t)(t[2] * dl2)), __builtin_bit_cast(uint32_t, (h2q_t)(t[3] * dl2))};
+}
+// d = dh + dl: dh keeps the upper seven significant bits
+__device__ __forceinline__ void split_scale(_Float16 d, h2q_t* dh2, h2q_t* dl2) {
+  const _Float16 dh = __builtin_bit_cast(_Float16, (uint16_t)(__builtin_bit_cast(uint16_t, d) & 0xFFF0u));
+  const _Float16 dl = d - dh;
+  *dh2 = (h2q_t){dh, dh};
+  *dl2 = (h2q_t){dl, dl};
+}
+#define DEQK_INIT(c)                                                                           \
+  DeqK c = {0x64006400u, 0x54005400u, 0x000F000Fu, 0x00F000F0u,                                \
+            {(_Float16)-1032.f, (_Float16)-1032.f}, {(_Float16)-72.f, (_Float16)-72.f}};       \
+  asm volatile("" : "+v"(c.magic_lo)); /* opaque: lets instruction selection use the three-operand and-or */ \
+  asm volatile("" : "+v"(c.magic_hi));                                                         \
+  asm volatile("" : "+s"(c.nib_lo));                                                           \
+  asm volatile("" : "+s"(c.nib_hi))
+#define MFMA_F16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8q_t, a), __builtin_bit_cast(h8q_t, b), c, 0, 0, 0)
+
 // Workgroup = 4 waves, each with R tiles of 16 weight rows = 64 R weight rows x 16 MT activation rows.
-// An activation fragment read from LDS feeds R matrix instructions, so the LDS traffic per
-// instruction falls with R; the weights of a wave's R tiles are dequantised in its registers as in
-// the kernel above.  One step = 128 weights of K; the next step's weight words and activation
-// pieces are loaded into registers while the matrix cores work on the current one.
+// An activation fragment read from LDS feeds 3 R matrix instructions (R tiles, two weight terms for the
+// first activation plane, one for the second); the weights of a wave's R tiles are dequantised in its
+// registers, word by word as the K loop needs them.  One step = 128 weights of K; the next step's weight
+// words and activation pieces are loaded into registers while the matrix cores work on the current one.
 template <int MT, int R>
 __global__ void __launch_bounds__(256)
 k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh,
-                    const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc, const float* __restrict__ scale,
-                    uint32_t M, uint32_t K, uint32_t N, GemmSegs segs) {
+                    const u4q_t* __restrict__ xl, const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc,
+                    const float* __restrict__ scale, uint32_t M, uint32_t K, uint32_t N, GemmSegs segs) {
   constexpr uint32_t BM = 16u * MT, ROWB = 272u;
-  __shared__ __attribute__((aligned(16))) uint8_t xs[BM * ROWB];
+  __shared__ __attribute__((aligned(16))) uint8_t xs[2u * BM * ROWB];   // first plane, then second plane
+  uint8_t* const xs2 = xs + BM * ROWB;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t r16 = lane & 15u, g = lane >> 4;
   const uint32_t n0 = blockIdx.x * (64u * R) + wave * (16u * R), m0 = blockIdx.y * BM, op = blockIdx.z;
@@ -255,22 +152,16 @@ k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __r
   for (int r = 0; r < R; r++)
 #pragma unroll
     for (int t = 0; t < MT; t++) acc[r][t] = (f4q_t){0.f, 0.f, 0.f, 0.f};
+  DEQK_INIT(dk);
 
-  uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u, nib_lo = 0x000F000Fu, nib_hi = 0x00F000F0u;
-  asm volatile("" : "+v"(magic_lo));   // opaque: lets instruction selection use the three-operand and-or
-  asm volatile("" : "+v"(magic_hi));
-  asm volatile("" : "+s"(nib_lo));
-  asm volatile("" : "+s"(nib_hi));
-  const h2q_t off_lo = {(_Float16)-1032.f, (_Float16)-1032.f}, off_hi = {(_Float16)-72.f, (_Float16)-72.f};
-
-  // staging: the tile's 16 pieces per row and step; thread -> (row, piece) pairs, MT per thread
-  const u4q_t* xrow[MT];
+  // staging: the tile's 16 pieces per row, plane and step; thread -> (row, piece) pairs, MT per thread
+  uint64_t xoff[MT];
 #pragma unroll
   for (uint32_t u = 0; u < MT; u++) {
     const uint32_t w = tid + u * 256u, row = min(m0 + (w >> 4), M - 1u);   // rows past M: clamped, not stored
-    xrow[u] = xh + ((uint64_t)op * M + row) * kw + (w & 15u);
+    xoff[u] = ((uint64_t)op * M + row) * kw + (w & 15u);
   }
-  u4q_t xn[MT], qn[R];
+  u4q_t xn[MT], xln[MT], qn[R];
   _Float16 dn[R];
   // always executed; the step past K re-reads the last one and is not used
 #define GEMM_FETCH(kb_raw)                                                        \
@@ -281,7 +172,10 @@ k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __r
       qn[r] = *(const u4q_t*)(W + (gi << 4));                                     \
       dn[r] = __builtin_bit_cast(_Float16, d16[gi]);                              \
     }                                                                             \
-    _Pragma("unroll") for (uint32_t u = 0; u < MT; u++) xn[u] = xrow[u][kb_ * 4u]; \
+    _Pragma("unroll") for (uint32_t u = 0; u < MT; u++) {                         \
+      xn[u] = xh[xoff[u] + kb_ * 4u];                                             \
+      xln[u] = xl[xoff[u] + kb_ * 4u];                                            \
+    }                                                                             \
   } while (0)
   GEMM_FETCH(0u);
 
@@ -290,32 +184,30 @@ k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __r
     for (uint32_t u = 0; u < MT; u++) {
       const uint32_t w = tid + u * 256u;
       *(u4q_t*)(xs + (w >> 4) * ROWB + (w & 15u) * 16u) = xn[u];
+      *(u4q_t*)(xs2 + (w >> 4) * ROWB + (w & 15u) * 16u) = xln[u];
     }
-    // dequantise: (1024 + n) - 1032 = n - 8 and (64 + n) - 72 = n - 8 exactly, then one rounding in d * (n - 8)
-    u4q_t a[R][4];
+    u4q_t q[R];
+    h2q_t dh2[R], dl2[R];
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-      const h2q_t d2 = {dn[r], dn[r]};
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const uint32_t w = j == 0 ? qn[r].x : j == 1 ? qn[r].y : j == 2 ? qn[r].z : qn[r].w, w8 = w >> 8;
-        const h2q_t t0 = __builtin_bit_cast(h2q_t, (w & nib_lo) | magic_lo), t1 = __builtin_bit_cast(h2q_t, (w & nib_hi) | magic_hi);
-        const h2q_t t2 = __builtin_bit_cast(h2q_t, (w8 & nib_lo) | magic_lo), t3 = __builtin_bit_cast(h2q_t, (w8 & nib_hi) | magic_hi);
-        a[r][j] = (u4q_t){__builtin_bit_cast(uint32_t, (h2q_t)((t0 + off_lo) * d2)), __builtin_bit_cast(uint32_t, (h2q_t)((t1 + off_hi) * d2)),
-                          __builtin_bit_cast(uint32_t, (h2q_t)((t2 + off_lo) * d2)), __builtin_bit_cast(uint32_t, (h2q_t)((t3 + off_hi) * d2))};
-      }
-    }
+    for (int r = 0; r < R; r++) { q[r] = qn[r]; split_scale(dn[r], &dh2[r], &dl2[r]); }
     __syncthreads();
     GEMM_FETCH(kb0 + 4u);
 #pragma unroll
-    for (int t = 0; t < MT; t++) {
-      const uint8_t* xp = xs + (t * 16u + r16) * ROWB + g * 64u;
+    for (int j = 0; j < 4; j++) {
+      u4q_t ah[R], al[R];
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const u4q_t b = *(const u4q_t*)(xp + j * 16);
+      for (int r = 0; r < R; r++)
+        deq_word2(j == 0 ? q[r].x : j == 1 ? q[r].y : j == 2 ? q[r].z : q[r].w, dk, dh2[r], dl2[r], &ah[r], &al[r]);
 #pragma unroll
-        for (int r = 0; r < R; r++)
-          acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8q_t, a[r][j]), __builtin_bit_cast(h8q_t, b), acc[r][t], 0, 0, 0);
+      for (int t = 0; t < MT; t++) {
+        const uint32_t xo = (t * 16u + r16) * ROWB + g * 64u + j * 16u;
+        const u4q_t bh = *(const u4q_t*)(xs + xo), bl = *(const u4q_t*)(xs2 + xo);
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r][t] = MFMA_F16(ah[r], bh, acc[r][t]);
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r][t] = MFMA_F16(al[r], bh, acc[r][t]);
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r][t] = MFMA_F16(ah[r], bl, acc[r][t]);
       }
     }
     __syncthreads();
@@ -348,26 +240,28 @@ k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __r
 // Few activation rows (M <= 32): the weights are read once and nothing is reused, so the work is
 // bound by how fast they stream.  The NWV waves of a workgroup share R tiles of 16 weight rows and
 // take every NWV-th step of K each (a matrix with few rows still spreads over the whole chip); every
-// wave stages its own activation tile from the fp16 copy into its own piece of LDS, so no
+// wave stages its own activation tile (both planes) from the fp16 copy into its own piece of LDS, so no
 // workgroup barrier sits in the K loop.  The partial tiles are summed in wave order at the end.
-// Eight waves (16 activation rows only: the wave-private tiles of 32 rows would not fit the static
-// LDS limit) keep twice as many loads in flight for matrices with few weight rows.
+// Eight waves keep twice as many loads in flight for matrices with few weight rows.
 //
 // Q8: the weights are Q8_0 blocks in the same block16 layout (32 code bytes, w = d (code - 128)): two 16-byte
 // loads per block, bytes widened with a byte permute into the fp16 pairs (1024 + code), then -1152 and d
-// as for the nibbles.  `lc` null: the result rows go to out[row * N + n] (a scratch buffer of the caller).
+// (one term each for weights and activations).  `lc` null: the result rows go to out[row * N + n] (a scratch
+// buffer of the caller).
 template <int MT, int R, int NWV, bool Q8>
 __global__ void __launch_bounds__(64 * NWV)
 k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh,
-                     const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc, const float* __restrict__ scale,
-                     uint32_t M, uint32_t K, uint32_t N, GemmSegs segs) {
-  constexpr uint32_t BM = 16u * MT, ROWB = 272u, NP = 4u * MT;      // pieces per lane and step
+                     const u4q_t* __restrict__ xl, const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc,
+                     const float* __restrict__ scale, uint32_t M, uint32_t K, uint32_t N, GemmSegs segs) {
+  constexpr uint32_t BM = 16u * MT, ROWB = 272u, NP = 4u * MT;      // pieces per lane, plane and step
+  constexpr uint32_t PLANES = Q8 ? 1u : 2u;
   constexpr uint32_t TILE = BM * ROWB, PART = (NWV - 1u) * R * MT * 4u * 64u * 4u;
-  __shared__ __attribute__((aligned(16))) uint8_t xs_all[(NWV * TILE > PART) ? NWV * TILE : PART];
+  __shared__ __attribute__((aligned(16))) uint8_t xs_all[(NWV * PLANES * TILE > PART) ? NWV * PLANES * TILE : PART];
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
   const uint32_t r16 = lane & 15u, g = lane >> 4;
-  uint8_t* xs = xs_all + wave * TILE;
+  uint8_t* xs = xs_all + wave * PLANES * TILE;
+  uint8_t* const xs2 = xs + TILE;
   const uint32_t n0 = blockIdx.x * (16u * R), m0 = blockIdx.y * BM, op = blockIdx.z;
   const uint64_t c_off = lc ? (uint64_t)lc[op] : 0ull, gbase = (uint64_t)lb[op] >> 5;
   const uint32_t nblk = K >> 5, kw = K >> 3;
@@ -386,22 +280,16 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
   for (int r = 0; r < R; r++)
 #pragma unroll
     for (int t = 0; t < MT; t++) acc[r][t] = (f4q_t){0.f, 0.f, 0.f, 0.f};
-
-  uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u, nib_lo = 0x000F000Fu, nib_hi = 0x00F000F0u;
-  asm volatile("" : "+v"(magic_lo));
-  asm volatile("" : "+v"(magic_hi));
-  asm volatile("" : "+s"(nib_lo));
-  asm volatile("" : "+s"(nib_hi));
-  const h2q_t off_lo = {(_Float16)-1032.f, (_Float16)-1032.f}, off_hi = {(_Float16)-72.f, (_Float16)-72.f};
+  DEQK_INIT(dk);
   const h2q_t off_q8 = {(_Float16)-1152.f, (_Float16)-1152.f};
 
-  const u4q_t* xrow[NP];
+  uint64_t xoff[NP];
 #pragma unroll
   for (uint32_t u = 0; u < NP; u++) {
     const uint32_t w = lane + u * 64u, row = min(m0 + (w >> 4), M - 1u);
-    xrow[u] = xh + ((uint64_t)op * M + row) * kw + (w & 15u);
+    xoff[u] = ((uint64_t)op * M + row) * kw + (w & 15u);
   }
-  u4q_t xn[NP], qn[R], qn2[Q8 ? R : 1];
+  u4q_t xn[NP], xln[Q8 ? 1 : NP], qn[R], qn2[Q8 ? R : 1];
   _Float16 dn[R];
 #define GEMM_FETCH(kb_raw)                                                        \
   do {                                                                            \
@@ -414,7 +302,10 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
       } else qn[r] = *(const u4q_t*)(W + (gi << 4));                              \
       dn[r] = __builtin_bit_cast(_Float16, d16[gi]);                              \
     }                                                                             \
-    _Pragma("unroll") for (uint32_t u = 0; u < NP; u++) xn[u] = xrow[u][kb_ * 4u]; \
+    _Pragma("unroll") for (uint32_t u = 0; u < NP; u++) {                         \
+      xn[u] = xh[xoff[u] + kb_ * 4u];                                             \
+      if (!Q8) xln[u] = xl[xoff[u] + kb_ * 4u];                                   \
+    }                                                                             \
   } while (0)
   GEMM_FETCH(wave * 4u);
 
@@ -423,51 +314,58 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
     for (uint32_t u = 0; u < NP; u++) {
       const uint32_t w = lane + u * 64u;
       *(u4q_t*)(xs + (w >> 4) * ROWB + (w & 15u) * 16u) = xn[u];
+      if (!Q8) *(u4q_t*)(xs2 + (w >> 4) * ROWB + (w & 15u) * 16u) = xln[u];
     }
-    u4q_t a[R][4];
+    // the step's blocks and scales, moved to the lanes that consume them
+    u4q_t q[R], q2[Q8 ? R : 1];
+    h2q_t dh2[R], dl2[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-#define PERM_U4(v) (v) = (u4q_t){(uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)(v).x), (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)(v).y), \
-                                 (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)(v).z), (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)(v).w)}
-      PERM_U4(qn[r]);
-      if (Q8) PERM_U4(qn2[r]);
+#define PERM_U4(v) (u4q_t){(uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)(v).x), (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)(v).y), \
+                           (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)(v).z), (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)(v).w)}
+      q[r] = PERM_U4(qn[r]);
+      if (Q8) q2[r] = PERM_U4(qn2[r]);
 #undef PERM_U4
       const uint32_t dbits = (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)__builtin_bit_cast(uint16_t, dn[r]));
       const _Float16 dl = __builtin_bit_cast(_Float16, (uint16_t)dbits);
-      const h2q_t d2 = {dl, dl};
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        if (Q8) {
-          // piece j = code bytes 8j .. 8j+7 in two words; pair p = (byte p of the first, byte p of the second)
-          const uint32_t w0 = j == 0 ? qn[r].x : j == 1 ? qn[r].z : j == 2 ? qn2[r].x : qn2[r].z;
-          const uint32_t w1 = j == 0 ? qn[r].y : j == 1 ? qn[r].w : j == 2 ? qn2[r].y : qn2[r].w;
-          uint32_t o[4];
-#pragma unroll
-          for (uint32_t p = 0; p < 4; p++) {
-            const uint32_t t = __builtin_amdgcn_perm(w1, w0, 0x0C000C00u | ((4u + p) << 16) | p) | magic_lo;
-            o[p] = __builtin_bit_cast(uint32_t, (h2q_t)((__builtin_bit_cast(h2q_t, t) + off_q8) * d2));
-          }
-          a[r][j] = (u4q_t){o[0], o[1], o[2], o[3]};
-          continue;
-        }
-        const uint32_t w = j == 0 ? qn[r].x : j == 1 ? qn[r].y : j == 2 ? qn[r].z : qn[r].w, w8 = w >> 8;
-        const h2q_t t0 = __builtin_bit_cast(h2q_t, (w & nib_lo) | magic_lo), t1 = __builtin_bit_cast(h2q_t, (w & nib_hi) | magic_hi);
-        const h2q_t t2 = __builtin_bit_cast(h2q_t, (w8 & nib_lo) | magic_lo), t3 = __builtin_bit_cast(h2q_t, (w8 & nib_hi) | magic_hi);
-        a[r][j] = (u4q_t){__builtin_bit_cast(uint32_t, (h2q_t)((t0 + off_lo) * d2)), __builtin_bit_cast(uint32_t, (h2q_t)((t1 + off_hi) * d2)),
-                          __builtin_bit_cast(uint32_t, (h2q_t)((t2 + off_lo) * d2)), __builtin_bit_cast(uint32_t, (h2q_t)((t3 + off_hi) * d2))};
-      }
+      if (Q8) { dh2[r] = (h2q_t){dl, dl}; dl2[r] = dh2[r]; }
+      else split_scale(dl, &dh2[r], &dl2[r]);
     }
     __builtin_amdgcn_wave_barrier();
     GEMM_FETCH(kb0 + 4u * NWV);
 #pragma unroll
-    for (int t = 0; t < MT; t++) {
-      const uint8_t* xp = xs + (t * 16u + r16) * ROWB + g * 64u;
+    for (int j = 0; j < 4; j++) {
+      u4q_t ah[R], al[Q8 ? 1 : R];
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const u4q_t b = *(const u4q_t*)(xp + j * 16);
+      for (int r = 0; r < R; r++) {
+        if (Q8) {
+          // piece j = code bytes 8j .. 8j+7 in two words; pair p = (byte p of the first, byte p of the second)
+          const uint32_t w0 = j == 0 ? q[r].x : j == 1 ? q[r].z : j == 2 ? q2[r].x : q2[r].z;
+          const uint32_t w1 = j == 0 ? q[r].y : j == 1 ? q[r].w : j == 2 ? q2[r].y : q2[r].w;
+          uint32_t o[4];
 #pragma unroll
-        for (int r = 0; r < R; r++)
-          acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8q_t, a[r][j]), __builtin_bit_cast(h8q_t, b), acc[r][t], 0, 0, 0);
+          for (uint32_t p = 0; p < 4; p++) {
+            const uint32_t t = __builtin_amdgcn_perm(w1, w0, 0x0C000C00u | ((4u + p) << 16) | p) | dk.magic_lo;
+            o[p] = __builtin_bit_cast(uint32_t, (h2q_t)((__builtin_bit_cast(h2q_t, t) + off_q8) * dh2[r]));
+          }
+          ah[r] = (u4q_t){o[0], o[1], o[2], o[3]};
+        } else {
+          deq_word2(j == 0 ? q[r].x : j == 1 ? q[r].y : j == 2 ? q[r].z : q[r].w, dk, dh2[r], dl2[r], &ah[r], &al[r]);
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < MT; t++) {
+        const uint32_t xo = (t * 16u + r16) * ROWB + g * 64u + j * 16u;
+        const u4q_t bh = *(const u4q_t*)(xs + xo);
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r][t] = MFMA_F16(ah[r], bh, acc[r][t]);
+        if (!Q8) {
+          const u4q_t bl = *(const u4q_t*)(xs2 + xo);
+#pragma unroll
+          for (int r = 0; r < R; r++) acc[r][t] = MFMA_F16(al[r], bh, acc[r][t]);
+#pragma unroll
+          for (int r = 0; r < R; r++) acc[r][t] = MFMA_F16(ah[r], bl, acc[r][t]);
+        }
       }
     }
     __builtin_amdgcn_wave_barrier();
@@ -525,7 +423,7 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
 // dependent passes -- the rows of a decode batch are few and each workgroup's latency is the launch's.
 template <int NW>
 __global__ void __launch_bounds__(1024)
-k_act_f16_regs(const float* act, const uint32_t* __restrict__ la, uint32_t M, uint32_t K, float* scale, uint4* xh) {
+k_act_f16_regs(const float* act, const uint32_t* __restrict__ la, uint32_t M, uint32_t K, float* scale, uint4* xh, uint4* xl) {
   __shared__ float red[16];
   const uint32_t row = blockIdx.x, op = blockIdx.y, tid = threadIdx.x, kw = K >> 3;
   const float* x = act + (uint64_t)la[op] + (uint64_t)row * K;
@@ -555,26 +453,28 @@ k_act_f16_regs(const float* act, const uint32_t* __restrict__ la, uint32_t M, ui
     scale[2 * ((uint64_t)op * M + row)] = s;
     scale[2 * ((uint64_t)op * M + row) + 1] = inv;
   }
-  uint4* dst = xh + ((uint64_t)op * M + row) * kw;
+  const uint64_t o0 = ((uint64_t)op * M + row) * kw;
 #pragma unroll
   for (int u = 0; u < NW; u++) {
     const uint32_t w = tid + 1024u * u;
     if (w >= kw) continue;
-    const h2q_t p0 = {(_Float16)(v0[u].x * s), (_Float16)(v1[u].x * s)}, p1 = {(_Float16)(v0[u].y * s), (_Float16)(v1[u].y * s)};
-    const h2q_t p2 = {(_Float16)(v0[u].z * s), (_Float16)(v1[u].z * s)}, p3 = {(_Float16)(v0[u].w * s), (_Float16)(v1[u].w * s)};
-    dst[w] = make_uint4(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1),
-                        __builtin_bit_cast(uint32_t, p2), __builtin_bit_cast(uint32_t, p3));
+    const float v[8] = {v0[u].x * s, v0[u].y * s, v0[u].z * s, v0[u].w * s, v1[u].x * s, v1[u].y * s, v1[u].z * s, v1[u].w * s};
+    uint4 hi, lo;
+    split_word(v, &hi, &lo);
+    xh[o0 + w] = hi;
+    xl[o0 + w] = lo;
   }
 }
 
 static float* g_scale_buf = nullptr;
-static uint4* g_xh_buf = nullptr;     // fp16 activations of the tiled form
-static size_t g_xh_cap = 0;           // in bytes
+static uint4* g_xh_buf = nullptr;     // fp16 activations: first plane, then the second plane at g_xh_plane bytes
+static size_t g_xh_cap = 0;           // in bytes (both planes)
 static size_t g_scale_cap = 0;
 // The rows last converted into g_xh_buf / g_scale_buf, and the launch and upload counts right after the
 // matmul that used them: while both counts stand still nothing has written device memory since, so a
-// matmul over the same rows (K and V after Q, up after gate) skips the conversion launch.
-static struct { const void* buf; uint64_t a; uint32_t M, K; uint64_t dispatch, mem_gen; bool valid; } g_xh_key = {};
+// matmul over the same rows (K and V after Q, up after gate) skips the conversion launch.  plane = byte
+// offset of the second plane those rows were written with.
+static struct { const void* buf; uint64_t a; uint32_t M, K; uint64_t dispatch, mem_gen; size_t plane; bool valid; } g_xh_key = {};
 
 static bool ensure_act_bufs(size_t scale_floats, size_t xh_bytes) {
   if (scale_floats > g_scale_cap) {
@@ -592,18 +492,24 @@ static bool ensure_act_bufs(size_t scale_floats, size_t xh_bytes) {
   return true;
 }
 
-bool gemm_act_slots(uint32_t M, uint32_t K, float** scale, __half** xh) {
-  if (tuning("ADAMAH_GEMM_TILED", 1) == 0 || tuning("ADAMAH_GEMM_REUSE", 1) == 0) return false;
-  if (!ensure_act_bufs((size_t)2 * M, (size_t)M * K * 2)) return false;
+bool gemm_act_slots(uint32_t M, uint32_t K, float** scale, __half** xh, __half** xl) {
+  if (tuning("ADAMAH_GEMM_REUSE", 1) == 0) return false;
+  const size_t plane = (size_t)M * K * 2;
+  if (!ensure_act_bufs((size_t)2 * M, 2 * plane)) return false;
   g_xh_key.valid = false;   // the buffers are about to be rewritten
   *scale = g_scale_buf;
   *xh = (__half*)g_xh_buf;
+  *xl = (__half*)((uint8_t*)g_xh_buf + plane);
   return true;
 }
 
 void gemm_act_mark(const void* buf, uint64_t a, uint32_t M, uint32_t K) {
-  g_xh_key = {buf, a, M, K, g.stats.dispatch, g.mem_gen, true};
+  g_xh_key = {buf, a, M, K, g.stats.dispatch, g.mem_gen, (size_t)M * K * 2, true};
 }
+
+// Forget converted rows (after a stream capture: the launch count is rewound there, and the note must not
+// survive into a later state with the same count).
+void gemm_act_forget() { g_xh_key.valid = false; }
 
 // Preconditions (checked by the caller against the host copies of the handles): Q4 map whose blocks
 // in range are in the block16 layout, K a multiple of 128, weight bases block aligned, all operands
@@ -616,40 +522,29 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
   GemmSegs sg = {};
   if (segs) sg = *segs;
   const size_t need = (size_t)2 * M * n_ops;
+  const size_t plane = (size_t)n_ops * M * K * 2;
   const bool reuse = g_xh_key.valid && n_ops == 1 && a_host >= 0 && g_xh_key.buf == ma->buf && g_xh_key.a == (uint64_t)a_host &&
                      g_xh_key.M == M && g_xh_key.K == K && g_xh_key.dispatch == g.stats.dispatch &&
-                     g_xh_key.mem_gen == g.mem_gen && tuning("ADAMAH_GEMM_REUSE", 1) != 0;
+                     g_xh_key.mem_gen == g.mem_gen && g_xh_key.plane == plane && tuning("ADAMAH_GEMM_REUSE", 1) != 0;
   g_xh_key.valid = false;
   // after the matmul: the converted rows stay usable if the result did not land on them
   auto keep = [&]() {
     if (n_ops != 1 || a_host < 0 || (c_host < 0 && !out)) return;
     const uint64_t a0 = (uint64_t)a_host, a1 = a0 + (uint64_t)M * K, c0 = (uint64_t)c_host, c1 = c0 + (uint64_t)M * N;
     if (!out && c0 < a1 && a0 < c1) return;
-    g_xh_key = {ma->buf, a0, M, K, g.stats.dispatch, g.mem_gen, true};
+    g_xh_key = {ma->buf, a0, M, K, g.stats.dispatch, g.mem_gen, plane, true};
   };
-  if (!ensure_act_bufs(need, 0)) return ADAMAH_ERR_MEMORY;
+  if (!reuse && !ensure_act_bufs(need, 2 * plane)) return ADAMAH_ERR_MEMORY;
   float* act = (float*)ma->buf;
   uint32_t mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8;
-  if (!q8 && !out && !segs && tuning("ADAMAH_GEMM_TILED", 1) == 0) {
-    // the first form: every workgroup converts its activation tile from float32 itself
-    k_row_pow2_scale<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf);
-    count_launch();
-    const bool ksplit = mt <= 2;
-    dim3 grid(cdiv(N, ksplit ? 16 : 64), cdiv(M, 16 * mt), n_ops);
-#define GQ(T, S) k_gemm_q4_f16<T, S><<<grid, 256, 0, g.stream>>>(act, act, mw->buf, mw->d16, la, lb, lc, g_scale_buf, M, K, N)
-    if (mt == 1) GQ(1, true); else if (mt == 2) GQ(2, true); else if (mt == 4) GQ(4, false); else GQ(8, false);
-#undef GQ
-    count_launch();
-    return check_launch();
-  }
-  const size_t xh_need = (size_t)n_ops * M * K * 2;
-  if (!ensure_act_bufs(0, xh_need)) return ADAMAH_ERR_MEMORY;
+  uint4* const xh = g_xh_buf;
+  uint4* const xl = (uint4*)((uint8_t*)g_xh_buf + plane);
   if (!reuse) {
     if (K <= 16384 && tuning("ADAMAH_ACT_REGS", 1) != 0) {
-      if (K <= 8192) k_act_f16_regs<1><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, la, M, K, g_scale_buf, g_xh_buf);
-      else k_act_f16_regs<2><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, la, M, K, g_scale_buf, g_xh_buf);
+      if (K <= 8192) k_act_f16_regs<1><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, la, M, K, g_scale_buf, xh, xl);
+      else k_act_f16_regs<2><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, la, M, K, g_scale_buf, xh, xl);
     } else
-      k_act_f16<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf, g_xh_buf);
+      k_act_f16<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf, xh, xl);
     count_launch();
   }
   auto wgs = [&](uint32_t rows_per_wg, uint32_t t) { return (uint64_t)cdiv(N, rows_per_wg) * cdiv(M, 16 * t) * n_ops; };
@@ -665,7 +560,7 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
     const uint32_t* lcd = out ? nullptr : lc;
     // eight waves where the matrix has too few weight rows for larger tiles (measured: no gain otherwise)
     const uint32_t nwv = mt == 1 && !q8 ? (uint32_t)tuning("ADAMAH_GEMM_NWV", R == 1 ? 8 : 4) : 4u;
-#define GK(T, RR, W, Q) k_gemm_q4_f16_ksplit<T, RR, W, Q><<<grid, 64 * W, 0, g.stream>>>(dst, mw->buf, mw->d16, (const u4q_t*)g_xh_buf, lb, lcd, g_scale_buf, M, K, N, sg)
+#define GK(T, RR, W, Q) k_gemm_q4_f16_ksplit<T, RR, W, Q><<<grid, 64 * W, 0, g.stream>>>(dst, mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, lb, lcd, g_scale_buf, M, K, N, sg)
     if (q8) {
       if (mt == 1) { if (R == 2) GK(1, 2, 4, true); else GK(1, 1, 4, true); }
       else { if (R == 2) GK(2, 2, 4, true); else GK(2, 1, 4, true); }
@@ -690,7 +585,7 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
   R = (uint32_t)tuning("ADAMAH_GEMM_R", (int)R);
   R = R >= 4 && mt == 4 ? 4 : R >= 2 ? 2 : 1;
   dim3 grid(cdiv(N, 64 * R), cdiv(M, 16 * mt), n_ops);
-#define GT(T, RR) k_gemm_q4_f16_tiled<T, RR><<<grid, 256, 0, g.stream>>>(act, mw->buf, mw->d16, (const u4q_t*)g_xh_buf, lb, lc, g_scale_buf, M, K, N, sg)
+#define GT(T, RR) k_gemm_q4_f16_tiled<T, RR><<<grid, 256, 0, g.stream>>>(act, mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, lb, lc, g_scale_buf, M, K, N, sg)
   if (mt == 4) { if (R == 4) GT(4, 4); else if (R == 2) GT(4, 2); else GT(4, 1); }
   else { if (R == 2) GT(8, 2); else GT(8, 1); }
 #undef GT

@@ -126,9 +126,10 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
                         uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops, bool q8 = false, float* out = nullptr,
                         int64_t a_host = -1, int64_t c_host = -1, const GemmSegs* segs = nullptr);
 // For a kernel that produces the rows [M, K] of a coming batched matmul: the buffers of their fp16 form
-// ((s, 1/s) per row; K halves per row), grown as needed, and -- after that kernel's launch has been
+// ((s, 1/s) per row; two planes of K halves per row: fp16(x s) and the fp16 remainder), grown as needed, and -- after that kernel's launch has been
 // counted -- the note that rows [a, a + M K) of `buf` are converted, so the matmul skips its conversion.
-bool gemm_act_slots(uint32_t M, uint32_t K, float** scale, __half** xh);
+bool gemm_act_slots(uint32_t M, uint32_t K, float** scale, __half** xh, __half** xl);
+void gemm_act_forget();
 void gemm_act_mark(const void* buf, uint64_t a, uint32_t M, uint32_t K);
 // Second pass of the fused GEMV + argmax: best of the per-group partials, token id stored as float.
 int launch_argmax_pairs(const Map* ma, const uint32_t* lidx, const uint32_t* lval, const uint32_t* ldst,

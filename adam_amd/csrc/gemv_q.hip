@@ -550,8 +550,7 @@ int op_matmul_t_xq(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t h
     bool ok = true;
     for (uint32_t op = 0; ok && op < n_ops; op++)
       ok = (bh[op] & 31u) == 0 && fmt_of(mw, bh[op], (uint64_t)N * K) == want;
-    if (ok && n_ops == 1 && can_defer() && tuning("ADAMAH_GEMM_MERGE", 1) != 0 &&
-        (tuning("ADAMAH_GEMM_TILED", 1) != 0 || dtype == DTYPE_Q8)) {
+    if (ok && n_ops == 1 && can_defer() && tuning("ADAMAH_GEMM_MERGE", 1) != 0) {
       // queued: matmuls over the same rows whose matrices lie back to back (Q, K, V; gate, up) become one launch
       PendOp p;
       p.kind = PK_GEMM; p.map_act = map_act; p.map_wt = map_wt; p.a = ah[0]; p.b = bh[0]; p.c = ch[0]; p.rpg = M; p.k = K;

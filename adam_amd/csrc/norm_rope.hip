@@ -44,14 +44,14 @@ k_rmsnorm(const float* act, const float* wt, float* out, const uint32_t* __restr
 // The same row op with the row held in registers (dim <= 256 NU): one trip to memory instead of two
 // dependent passes.  Thread t owns elements t, t + 256, ... and sums their squares in that order, as the
 // kernel above does, so the results are the same bits.  EMIT: the rows are [n_rows, dim] back to back and a
-// batched matmul follows; its fp16 operand form (row scaled by a power of two, 8-element words in the
+// batched matmul follows; its fp16 operand form (row scaled by a power of two, two planes, 8-element words in the
 // order (0,4)(1,5)(2,6)(3,7), plus (s, 1/s) per row) is written here as well, which spares that
 // matmul its conversion launch.
 template <bool ADD, bool EMIT, int NU>
 __global__ void __launch_bounds__(256)
 k_rmsnorm_rows(const float* act, const float* wt, float* out, const uint32_t* __restrict__ ls,
                const uint32_t* __restrict__ lw, const uint32_t* __restrict__ lr, const uint32_t* __restrict__ ld,
-               uint32_t dim, float eps, uint64_t act_elems, uint64_t wt_elems, float* scale, __half* xh) {
+               uint32_t dim, float eps, uint64_t act_elems, uint64_t wt_elems, float* scale, __half* xh, __half* xl) {
   __shared__ float sh[4];
   const uint32_t ri = blockIdx.x, tid = threadIdx.x;
   const uint64_t sb = ls[ri], wb = lw[ri], db = ld[ri], rb = ADD ? (uint64_t)lr[ri] : 0;
@@ -89,11 +89,19 @@ k_rmsnorm_rows(const float* act, const float* wt, float* out, const uint32_t* __
   float s = 1.f, si = 1.f;
   if (e >= 14u && e <= 254u) { s = __uint_as_float((267u - e) << 23); si = __uint_as_float((e - 13u) << 23); }
   if (tid == 0) { scale[2 * ri] = s; scale[2 * ri + 1] = si; }
+  // two planes: fp16(x s) and the fp16 remainder x s - fp16(x s), as the matmul's own conversion writes them
   __half* dst = xh + (uint64_t)ri * dim;
+  __half* dstl = xl + (uint64_t)ri * dim;
 #pragma unroll
   for (int u = 0; u < NU; u++) {
     const uint32_t i = tid + 256u * u, q = i & 7u;
-    if (i < dim) dst[(i & ~7u) + (q < 4u ? 2u * q : 2u * (q - 4u) + 1u)] = __float2half(x[u] * s);
+    if (i < dim) {
+      const uint32_t at = (i & ~7u) + (q < 4u ? 2u * q : 2u * (q - 4u) + 1u);
+      const float v = x[u] * s;
+      const __half h = __float2half(v);
+      dst[at] = h;
+      dstl[at] = __float2half(v - __half2float(h));
+    }
   }
 }
 
@@ -212,10 +220,10 @@ static int rmsnorm_impl(uint32_t map_act, uint32_t map_wt, uint32_t hs, uint32_t
       emit = in_range(sh[i], dim, ma->n_elems) && in_range(dh[i], dim, ma->n_elems) && in_range(wh[i], dim, mw->n_elems) &&
              (!add || in_range(rh[i], dim, ma->n_elems));
     float* scale = nullptr;
-    __half* xh = nullptr;
-    if (emit) emit = gemm_act_slots(n_rows, dim, &scale, &xh);
+    __half *xh = nullptr, *xl = nullptr;
+    if (emit) emit = gemm_act_slots(n_rows, dim, &scale, &xh, &xl);
     const float* w = (const float*)mw->buf;
-#define RR(A, E, NU) k_rmsnorm_rows<A, E, NU><<<n_rows, 256, 0, g.stream>>>(a, w, a, ls, lw, lr, ld, dim, eps, ma->n_elems, mw->n_elems, scale, xh)
+#define RR(A, E, NU) k_rmsnorm_rows<A, E, NU><<<n_rows, 256, 0, g.stream>>>(a, w, a, ls, lw, lr, ld, dim, eps, ma->n_elems, mw->n_elems, scale, xh, xl)
 #define RN(A, E) do { if (dim <= 2048) RR(A, E, 8); else if (dim <= 4096) RR(A, E, 16); else RR(A, E, 32); } while (0)
     if (add) { if (emit) RN(true, true); else RN(true, false); }
     else { if (emit) RN(false, true); else RN(false, false); }

@@ -125,6 +125,7 @@ class CpuModel:
         nf = self.rms(hidden, t['output_norm.weight'], c.norm_eps)
         lm = 'output.weight' if 'output.weight' in t else 'token_embd.weight'
         logits = self.mv(lm, nf)
+        self.last_raw_logits = logits          # before the final soft-cap: what the LM-head product alone gives
         if c.final_softcap > 0:
             cap = f32(c.final_softcap)
             logits = (np.tanh(logits / cap) * cap).astype(np.float32)

@@ -1,7 +1,10 @@
 """Batched (M > 1) quantised matmul on the matrix cores against the oracle (needs an MI355X).
 
 BASELINE config 5 shapes: M = 512 (prefill chunk) and M = 16 (batched decode) over Llama-3-8B-shape
-Q4_0 matrices.  Bar: 1e-3 relative L2 per output row (fp16 operands, fp32 accumulation)."""
+Q4_0 matrices.  Bars, relative L2 per output row against the float64 product of the dequantised matrix:
+Q4_0 weights 3e-5 (both operands enter the matrix cores as exact two-term fp16 sums, float32 accumulation --
+a forward pass chains ~200 of these, so the single product has to sit far inside the path's 1e-3);
+Q8_0 weights (the LM head of a lockstep batch, the last product of a pass) and the element-wise kernels 1e-3."""
 import numpy as np
 import pytest
 
@@ -12,6 +15,7 @@ from gpu_util import note, up, f32map, put, read, rel_l2, load_qtensor
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
+TOL_Q4 = 3e-5
 
 
 def run(g, qt, x, n_ops=1, scale=None, zp=None):
@@ -39,7 +43,7 @@ def test_batched_q4_matmul_matches_oracle(hip, M, N, K):
     note(f"gemm q4 M={M} N={N} K={K} reference product")
     want = (x[0].astype(np.float64) @ qt.dequant().astype(np.float64).T)
     for m in range(M):
-        assert rel_l2(y[m], want[m]) < TOL, m
+        assert rel_l2(y[m], want[m]) < TOL_Q4, m
     if M * N * K <= 40 * 130 * 256:      # the oracle's own M > 1 path on the small case
         assert rel_l2(y, run(oracle.init(), qt, x)[0]) < TOL
 
@@ -59,7 +63,7 @@ def test_batched_matmul_row_scaling_and_ops(hip):
         want = x[op].astype(np.float64) @ w.T
         for m in range(M):
             if np.any(want[m]):
-                assert rel_l2(y[op, m], want[m]) < TOL, (op, m)
+                assert rel_l2(y[op, m], want[m]) < TOL_Q4, (op, m)
             else:
                 assert not np.any(y[op, m])
 
