@@ -1,15 +1,22 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized decode hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemma3-1b|llama3-8b] [--only LEG]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama3-8b|gemma3-1b] [--only LEG]
 
 A "step" is one bs=1 greedy decode step (embedding fetch, all layers, fused LM-head GEMV+argmax,
 token read-back) of a random-init Q4_0 model of the named architecture, issued through the
-ADAMAH op surface exactly as the decode harness does.  W untimed steps follow the prompt
-prefill, then exactly K steps are timed between two device synchronisations; weights, KV
-cache and activations are resident in HBM before the timed region starts.
+ADAMAH op surface exactly as the decode harness does.  The default workload is the Llama-3-8B
+shape with a Q8_0 output head; its prompt is sized so that the last timed step runs at context
+4096.  W untimed steps follow the prompt prefill, then exactly K steps are timed between two
+device synchronisations; weights, KV cache and activations are resident in HBM before the timed
+region starts.
 
 One JSON line is printed.  Besides the contract keys it carries
+  op_by_op      the same decode with every op of a step issued as its own call (no decode plan):
+                what an engine that never registers a plan gets from this library
+  config2_gemma3_1b  the Gemma-3-1B-shape decode (128 steps after a 512-token prompt), plan and op by op
+  config5_batched    16 prompts of 1024 tokens prefilled in chunks of 512, then 128 lockstep steps
+  gemm_q4_0     the batched Q4_0 matmul (M = 16, 512) at the Llama-3-8B shapes
   roofline      the Q4_0 GEMV kernel at the Llama-3-8B gate+up shape (28672x4096), timed with HIP
                 events on the library's stream while cycling through > 1 GB of distinct weights
   gemv_shapes   the same measurement for the other Llama-3-8B GEMV shapes
@@ -35,6 +42,9 @@ CONFIG1_GEMV_SHAPE = (6912, 1152)      # BASELINE config 1 (Gemma-3-1B FFN up): 
 # fetch_write.txt): FETCH_SIZE 32,528.8 counts x 1.999 KiB (factor from a plain read kernel of known
 # size) + WRITE_SIZE 130.5 counts x 1.000 KiB (factor from a plain copy kernel).
 GEMV_TRAFFIC_BYTES = int(32528.8 * 1.999 * 1024 + 130.5 * 1.000 * 1024)
+GEMV_TRAFFIC_SOURCE = ("profiles/gemv_q4_0_llama_shapes_pmc_fetch_write.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of "
+                       "`bench.py --only gemv`, scaled by the same counters of `bench.py --only probe`; a figure of that "
+                       "profile, not of this run")
 METRIC = "decode tok/s at bs=1 + Q4 GEMV achieved HBM GB/s (% of MI355X peak)"
 
 
@@ -289,18 +299,84 @@ def measure_model_batched(args, A, synth, DecodeEngine):
     return out
 
 
+def step_bytes_of(cfg, tensors, ctx_mid):
+    """Algorithmic HBM bytes of one bs=1 decode step: every weight block once + the KV rows of the context."""
+    q4_w = sum(v.size for v in tensors.values() if getattr(v, "kind", "") == "q4_0")
+    q8_w = sum(v.size for v in tensors.values() if getattr(v, "kind", "") == "q8_0")
+    kv_b = 2 * cfg.n_layer * cfg.n_head_kv * cfg.head_dim_kv * 2 * ctx_mid
+    return q4_w * 18 // 32 + q8_w * 34 // 32 + kv_b
+
+
+def measure_decode(gpu, A, DecodeEngine, cfg, tensors, prompt, steps, warmup, scheduler, prefill_chunk, decode_plan=True):
+    """bs=1 greedy decode: the prompt, `warmup` untimed steps, then exactly `steps` timed steps (token id read back
+    every step) between two device synchronisations.  decode_plan=False issues every op of a step as a call of its own
+    through the op surface, which is what the unchanged reference engine does (adam/models/engine.py:2971-3706)."""
+    n_prompt = len(prompt)
+    eng = DecodeEngine(gpu, cfg, tensors, A=A, kv_cap=n_prompt + warmup + steps + 8, kv_fp16=True,
+                       fusion_scheduler_mode=scheduler, prefill_chunk=prefill_chunk, decode_plan=decode_plan)
+    gpu.sync()
+    eng.reset()
+    t0 = time.perf_counter()
+    eng.prefill(prompt)
+    gpu.sync()
+    prefill_s = time.perf_counter() - t0
+    tokens, pos = [], n_prompt
+    for _ in range(warmup):
+        nt = eng.read_token(); tokens.append(nt)
+        eng._forward(nt, pos); pos += 1
+    gpu.sync()
+    gpu.reset_native_stats()
+    gpu.timer_begin()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        nt = eng.read_token(); tokens.append(nt)
+        eng._forward(nt, pos); pos += 1
+    gpu.sync()
+    wall = time.perf_counter() - t0
+    dev_ms = gpu.timer_end()
+    stats = gpu.get_native_stats()
+    sb = step_bytes_of(cfg, tensors, n_prompt + warmup + steps // 2)
+    ceiling = HBM_PEAK_GBPS * 1e9 / sb
+    del eng
+    return {"tok_s": steps / wall, "ms_per_step": 1e3 * wall / steps, "device_ms_per_step": dev_ms / steps,
+            "launches_per_token": stats["dispatch_count"] / max(1, steps), "prefill_s": prefill_s, "n_prompt": n_prompt,
+            "end_pos": pos, "tokens": tokens[warmup:], "step_bytes": int(sb), "ceiling": ceiling,
+            # the reference's stat keys (adam/models/engine.py:3922-3944)
+            "stats": {"n_prompt": n_prompt, "n_gen": steps, "prefill_tps": round(n_prompt / prefill_s, 1),
+                      "decode_tps": round(steps / wall, 2), "avg_ms": round(1e3 * wall / steps, 4),
+                      "sampling_mode": "gpu_matvec_argmax"}}
+
+
+def measure_lockstep(gpu, A, DecodeEngine, cfg, tensors, batch, n_prompt, steps, scheduler):
+    """BASELINE config 5: `batch` independent random prompts prefilled in chunks of 512 tokens on the matrix cores,
+    then `steps` lockstep decode steps."""
+    rng = np.random.default_rng(1)
+    eng = DecodeEngine(gpu, cfg, tensors, A=A, kv_cap=n_prompt + steps + 8, kv_fp16=True,
+                       fusion_scheduler_mode=scheduler, prefill_chunk=512, batch=batch)
+    prompts = [[int(t) for t in rng.integers(0, cfg.n_vocab, n_prompt)] for _ in range(batch)]
+    _, st = eng.generate_batch(prompts, steps)
+    del eng
+    return {"batch": batch, "prompt_tokens_per_sequence": n_prompt, "prefill_chunk": 512, "steps": steps,
+            "prefill_tok/s": round(batch * n_prompt / st["prefill_s"], 1),
+            "decode_tok/s_aggregate": round(st["decode_tps"], 1),
+            "ms_per_step": round(st["decode_s"] / steps * 1e3, 3)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--workload", default="gemma3-1b", choices=["gemma3-1b", "llama3-8b"])
-    ap.add_argument("--prompt", type=int, default=None, help="prompt length (default 512 / 3840)")
+    ap.add_argument("--workload", default="llama3-8b", choices=["gemma3-1b", "llama3-8b"])
+    ap.add_argument("--prompt", type=int, default=None,
+                    help="prompt length (default: llama3-8b 4096 - warmup - steps, so that the last timed step runs at "
+                         "context 4096; gemma3-1b 512)")
     ap.add_argument("--scheduler", default="level_batched", choices=["legacy", "level_batched"])
-    ap.add_argument("--prefill-chunk", type=int, default=0,
+    ap.add_argument("--prefill-chunk", type=int, default=None,
                     help="prompt in chunks of this many tokens on the matrix-core matmul (0: token by token, as the "
-                         "reference does; the timed region is the decode loop either way)")
-    ap.add_argument("--batch", type=int, default=16, help="--only batch: sequences decoded in lockstep")
+                         "reference does; default 512 for llama3-8b, 0 for gemma3-1b); the timed region is the decode "
+                         "loop either way")
+    ap.add_argument("--batch", type=int, default=16, help="sequences decoded in lockstep (config 5 leg, --only batch)")
     ap.add_argument("--only", default=None, choices=["roofline", "gemv", "probe", "attention", "gemm", "prefill", "batch"],
                     help="roofline: just the 28672x4096 GEMV (one kernel row in a rocprofv3 --stats table); "
                          "gemv: that shape, 4096x4096 and 4096x14336; probe: plain read/copy kernels of known "
@@ -310,7 +386,9 @@ def main():
                          "by token and in one chunk (matrix-core matmuls, causal attention in one launch per "
                          "layer); batch: --batch random prompts of --prompt (default 1024) tokens prefilled in "
                          "chunks of 512, then --steps lockstep decode steps of --workload")
-    ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--no-roofline", action="store_true", help="skip the kernel legs (GEMV shapes, attention, matmul)")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="skip the other configurations (op-by-op decode, Gemma-3-1B shape, lockstep batch)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -320,6 +398,8 @@ def main():
     from adam_amd.engine import DecodeEngine
 
     if args.only in ("prefill", "batch"):
+        if args.only == "batch" and args.steps == 256:
+            args.steps = 128
         print(json.dumps(measure_model_batched(args, A, synth, DecodeEngine)), flush=True)
         return
     if args.only:
@@ -346,95 +426,106 @@ def main():
 
     gemma = args.workload == "gemma3-1b"
     cfg = synth.gemma3_1b_config() if gemma else synth.llama3_8b_config()
-    n_prompt = args.prompt if args.prompt is not None else (512 if gemma else 4096 - 256)
-    kv_cap = n_prompt + args.warmup + args.steps + 8
+    if args.prompt is not None:
+        n_prompt = args.prompt
+    else:
+        n_prompt = 512 if gemma else max(16, 4096 - args.warmup - args.steps)
+    chunk = args.prefill_chunk if args.prefill_chunk is not None else (0 if gemma else 512)
     t0 = time.perf_counter()
     tensors = synth.make_model(cfg, seed=0, sigma=0.02)
     log(f"synthesised {args.workload} weights in {time.perf_counter() - t0:.1f}s")
 
     gpu = A.init()
-    t0 = time.perf_counter()
-    eng = DecodeEngine(gpu, cfg, tensors, A=A, kv_cap=kv_cap, kv_fp16=True,
-                       fusion_scheduler_mode=args.scheduler, prefill_chunk=args.prefill_chunk)
-    gpu.sync()
-    log(f"uploaded in {time.perf_counter() - t0:.1f}s; maps {sorted(eng._q4_sizes)}")
-
     rng = np.random.default_rng(0)
     prompt = [int(t) for t in rng.integers(0, cfg.n_vocab, n_prompt)]
-    eng.reset()
     t0 = time.perf_counter()
-    eng.prefill(prompt)
-    gpu.sync()
-    prefill_s = time.perf_counter() - t0
-    log(f"prefill {n_prompt} tokens ({'chunks of ' + str(args.prefill_chunk) if args.prefill_chunk else 'token by token'}): {prefill_s:.2f}s")
-
-    tokens, pos = [], n_prompt
-    for _ in range(args.warmup):
-        nt = eng.read_token(); tokens.append(nt)
-        eng._forward(nt, pos); pos += 1
-    gpu.sync()
-    gpu.reset_native_stats()
-    gpu.timer_begin()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        nt = eng.read_token(); tokens.append(nt)
-        eng._forward(nt, pos); pos += 1
-    gpu.sync()
-    wall = time.perf_counter() - t0
-    dev_ms = gpu.timer_end()
-    stats = gpu.get_native_stats()
-    tok_s = args.steps / wall
-    launches = stats["dispatch_count"] / max(1, args.steps)
-
-    c = cfg
-    q4_w = sum(v.size for v in tensors.values() if getattr(v, "kind", "") == "q4_0")
-    q8_w = sum(v.size for v in tensors.values() if getattr(v, "kind", "") == "q8_0")
-    kv_b = 2 * c.n_layer * c.n_head_kv * c.head_dim_kv * 2 * (n_prompt + args.warmup + args.steps // 2)
-    step_bytes = q4_w * 18 // 32 + q8_w * 34 // 32 + kv_b
-    ceiling = HBM_PEAK_GBPS * 1e9 / step_bytes
+    m = measure_decode(gpu, A, DecodeEngine, cfg, tensors, prompt, args.steps, args.warmup, args.scheduler, chunk)
+    log(f"{args.workload}: {m['tok_s']:.1f} tok/s, {m['ms_per_step']:.3f} ms/step, prefill {m['prefill_s']:.2f}s "
+        f"({time.perf_counter() - t0:.1f}s for the leg)")
 
     res = {
-        "metric": METRIC, "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(1e3 * wall / args.steps, 4), "higher_is_better": True,
+        "metric": METRIC, "value": round(m["tok_s"], 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(m["ms_per_step"], 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"{args.workload}-shape Q4_0 random-init, bs=1 greedy decode, "
-                               f"{n_prompt}-token random prompt, fp16 KV, tokens {n_prompt}..{pos}",
-                   "scheduler": args.scheduler, "launches_per_token": round(launches, 1)},
-        "device_ms_per_step": round(dev_ms / args.steps, 4),
-        "algorithmic_bytes_per_token": int(step_bytes),
-        "tok_s_at_hbm_peak": round(ceiling, 1), "frac_of_hbm_roofline": round(tok_s / ceiling, 4),
-        "prefill_tok_s": round(n_prompt / prefill_s, 1), "first_tokens": tokens[args.warmup:args.warmup + 8],
+        "config": {"workload": f"{args.workload}-shape Q4_0 random-init"
+                               + ("" if gemma else " (Q8_0 output head)") + ", bs=1 greedy decode, "
+                               f"{n_prompt}-token random prompt "
+                               f"({'chunks of ' + str(chunk) if chunk else 'token by token'}), fp16 KV, "
+                               f"timed steps at context {m['end_pos'] - args.steps + 1}..{m['end_pos']}",
+                   "baseline_config": 2 if gemma else 4,
+                   "scheduler": args.scheduler, "launches_per_token": round(m["launches_per_token"], 1),
+                   "issue": "one native decode_step call per token (registered decode plan)"},
+        "device_ms_per_step": round(m["device_ms_per_step"], 4),
+        "algorithmic_bytes_per_token": m["step_bytes"],
+        "tok_s_at_hbm_peak": round(m["ceiling"], 1), "frac_of_hbm_roofline": round(m["tok_s"] / m["ceiling"], 4),
+        "prefill_tok_s": round(n_prompt / m["prefill_s"], 1), "first_tokens": m["tokens"][:8],
+        "stats": m["stats"],
     }
-    del eng
 
-    if not args.no_roofline and not args.prefill_chunk:
-        # the same prompt prefilled as one chunk (projections as [512, K] matmuls, one causal attention launch per layer)
+    def leg(name, fn):
+        """An extra leg never costs the headline line: its failure is reported in its own object."""
+        t0 = time.perf_counter()
         try:
-            eng2 = DecodeEngine(gpu, cfg, tensors, A=A, kv_cap=n_prompt + 16, kv_fp16=True,
-                                fusion_scheduler_mode=args.scheduler, prefill_chunk=n_prompt)
-            eng2.reset(); eng2.prefill(prompt); gpu.sync()
-            t0 = time.perf_counter(); eng2.prefill(prompt); gpu.sync(); dt = time.perf_counter() - t0
-            res["prefill_one_chunk"] = {"tokens": n_prompt, "ms": round(dt * 1e3, 2), "tok/s": round(n_prompt / dt, 1),
-                                        "first_token_same_as_token_by_token": bool(eng2.read_token() == tokens[0])}
-            del eng2
-        except Exception as e:                      # never let the extra leg cost the headline line
-            res["prefill_one_chunk"] = {"error": repr(e)[:200]}
+            res[name] = fn()
+        except Exception as e:
+            res[name] = {"error": repr(e)[:300]}
+        log(f"{name}: {time.perf_counter() - t0:.1f}s")
+
+    if not args.no_extra:
+        n_obo = min(args.steps, 32)
+
+        def op_by_op(cfg_, tensors_, prompt_, chunk_, ref_tokens):
+            o = measure_decode(gpu, A, DecodeEngine, cfg_, tensors_, prompt_, n_obo, args.warmup, args.scheduler,
+                               chunk_, decode_plan=False)
+            return {"tok/s": round(o["tok_s"], 2), "ms_per_step": round(o["ms_per_step"], 4), "steps": n_obo,
+                    "launches_per_token": round(o["launches_per_token"], 1),
+                    "issue": "every op of the step as its own call through ctypes, as the reference engine issues them",
+                    "tokens_same_as_plan_replay": bool(o["tokens"][:8] == ref_tokens[:8])}
+        leg("op_by_op", lambda: op_by_op(cfg, tensors, prompt, chunk, m["tokens"]))
+
+        def other_shape():
+            g2 = not gemma
+            cfg2 = synth.gemma3_1b_config() if g2 else synth.llama3_8b_config()
+            t2 = synth.make_model(cfg2, seed=0, sigma=0.02)
+            st2 = min(args.steps, 128) if g2 else args.steps
+            np2 = 512 if g2 else max(16, 4096 - args.warmup - st2)
+            p2 = [int(t) for t in np.random.default_rng(0).integers(0, cfg2.n_vocab, np2)]
+            o = measure_decode(gpu, A, DecodeEngine, cfg2, t2, p2, st2, args.warmup, args.scheduler, 0 if g2 else 512)
+            out = {"workload": ("gemma3-1b" if g2 else "llama3-8b") + f"-shape Q4_0 random-init, bs=1 greedy decode, "
+                               f"{np2}-token random prompt, fp16 KV, timed steps at context "
+                               f"{o['end_pos'] - st2 + 1}..{o['end_pos']}",
+                   "tok/s": round(o["tok_s"], 2), "ms_per_step": round(o["ms_per_step"], 4), "steps": st2,
+                   "launches_per_token": round(o["launches_per_token"], 1),
+                   "tok_s_at_hbm_peak": round(o["ceiling"], 1), "frac_of_hbm_roofline": round(o["tok_s"] / o["ceiling"], 4),
+                   "prefill_tok_s": round(np2 / o["prefill_s"], 1), "stats": o["stats"]}
+            ob = measure_decode(gpu, A, DecodeEngine, cfg2, t2, p2, n_obo, args.warmup, args.scheduler, 0 if g2 else 512,
+                                decode_plan=False)
+            out["op_by_op_tok/s"] = round(ob["tok_s"], 2)
+            return out
+        leg("config2_gemma3_1b" if not gemma else "config4_llama3_8b", other_shape)
+
+        if not gemma:
+            leg("config5_batched", lambda: dict(
+                measure_lockstep(gpu, A, DecodeEngine, cfg, tensors, args.batch, 1024, 128, args.scheduler),
+                mfma_busy_source="profiles/gemm_q4_0_m16_m512_mfma_busy.txt"))
 
     if not args.no_roofline:
         shapes = measure_gemv(gpu, A, LLAMA_GEMV_SHAPES + [CONFIG1_GEMV_SHAPE])
         top = shapes["28672x4096"]
         res["roofline"] = {"bound": "hbm", "achieved": top["GB/s"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                            "frac": top["frac"], "traffic": GEMV_TRAFFIC_BYTES,
+                           "traffic_source": GEMV_TRAFFIC_SOURCE,
                            "kernel": "k_gemv_mfma<Q4_0 block16, store> 28672x4096, "
                                      f"{gemv_bytes(28672, 4096)} algorithmic B/launch"}
         res["gemv_shapes"] = shapes
-        res["attention_32q8kv_d128"] = measure_attention(gpu, A)
+        leg("attention_32q8kv_d128", lambda: measure_attention(gpu, A))
+        if not args.no_extra:
+            leg("gemm_q4_0", lambda: measure_gemm(gpu, A))
     gpu.shutdown()
 
     if not args.no_cpu_baseline:
         t0 = time.perf_counter()
-        n_cpu = 48 if gemma else 4
-        res["cpu_baseline"] = cpu_baseline(cfg, tensors, prompt, n_prompt=8 if gemma else 2, n_steps=n_cpu)
+        res["cpu_baseline"] = cpu_baseline(cfg, tensors, prompt, n_prompt=8 if gemma else 2, n_steps=48 if gemma else 6)
         log(f"cpu baseline {res['cpu_baseline']['value']} tok/s ({time.perf_counter() - t0:.1f}s incl. dequant)")
 
     print(json.dumps(res), flush=True)
