@@ -34,6 +34,8 @@ DECODE_RUNTIME_SEQ_LEN = 0xFFFFFFFD
  DECODE_OP_ROPE, DECODE_OP_MATMUL_T, DECODE_OP_MATMUL_T_X, DECODE_OP_MATMUL_X, DECODE_OP_MATMUL_T_XQ4,
  DECODE_OP_MATMUL_XQ4, DECODE_OP_MATMUL_T_XQ8, DECODE_OP_MATMUL_XQ8, DECODE_OP_QK_NORM_ROPE_X,
  DECODE_OP_ROW_COPY_OFFSET, DECODE_OP_ATTN_SOFTMAX_VALUE) = range(10, 26)
+(DECODE_OP_FUSED_QKV_T_XQ4, DECODE_OP_FUSED_GATEUP_T_XQ4, DECODE_OP_FUSED_QKV_T_XQ8, DECODE_OP_FUSED_GATEUP_T_XQ8,
+ DECODE_OP_FUSED_GATEUP_ACT_T_XQ8) = range(26, 31)
 
 (OP_NEG, OP_ABS, OP_SQRT, OP_EXP, OP_LOG, OP_TANH, OP_RELU, OP_GELU, OP_SIN, OP_COS, OP_TAN, OP_ASIN,
  OP_ACOS, OP_ATAN, OP_SINH, OP_COSH, OP_SIGMOID, OP_SWISH, OP_MISH, OP_SELU, OP_ELU, OP_LEAKY_RELU,

@@ -469,6 +469,7 @@ size_t launch_attn_batch(const std::vector<PendOp>& q, size_t i, int* rc) {
   if (n_groups > 65535u || (uint64_t)n_all * n_splits * (D + 2) > g.attn_scratch_floats) return 0;
   const size_t words = 3 * (size_t)n_all + 2 * (size_t)n_groups;
   if (words > g_ext_cap) {
+    layout_changed();
     if (g_ext_buf) { hipStreamSynchronize(g.stream); hipFree(g_ext_buf); }
     g_ext_cap = std::max<size_t>(words, 4096);
     if (hipMalloc((void**)&g_ext_buf, g_ext_cap * 4) != hipSuccess) { g_ext_buf = nullptr; g_ext_cap = 0; *rc = ADAMAH_ERR_MEMORY; return 2 * B; }

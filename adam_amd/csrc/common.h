@@ -129,6 +129,10 @@ struct Ctx {
   int no_defer = 0;              // > 0 while an entry point runs on library-owned scratch handles
   uint64_t mem_gen = 0;          // counts host-to-device copies (with stats.dispatch: "has device memory changed?")
   uint32_t* sync_ctr = nullptr;  // device counters for last-workgroup epilogues, zero between launches
+  int deferred_err = 0;          // first failure of a queued op's launch; returned (once) by the next call that can
+  uint64_t layout_gen = 0;       // counts events after which device pointers or offsets seen earlier may be stale:
+                                 // a map created, destroyed or given new qparams / an fp16 KV range, a library
+                                 // scratch buffer re-allocated (recorded HIP graphs are dropped when it moves)
 };
 
 extern Ctx g;
@@ -180,6 +184,7 @@ int launch_attn_combine_dev(Map* m, const float* partial, const uint32_t* lo_dev
                             uint32_t n_splits);
 void attn_decode_release();
 
+inline void layout_changed() { g.layout_gen++; }
 inline void count_launch(int n = 1) { g.stats.dispatch += n; g.stats.barrier += n; g.stats.last_batch_dispatch += n; }
 int check_launch();                              // hipGetLastError -> ADAMAH code
 

@@ -97,6 +97,25 @@ int launch_op2_v(const PendOp& p) {
 
 static bool disjoint(uint64_t a, uint64_t na, uint64_t b, uint64_t nb) { return a + na <= b || b + nb <= a; }
 
+// A prologue fold makes every workgroup of the GEMV read the norm's inputs (and workgroup 0 / the last ticket
+// store the norm's own results) while other workgroups already store result rows: whatever the GEMV writes --
+// its result rows, or the partial (index, value) lists and the token slot of a GEMV + argmax -- has to lie
+// clear of all of them, or the ops are launched one by one.
+static bool gemv_writes_clear(const PendOp& gp, const uint64_t (*rg)[2], int n_rg) {
+  auto clear_of_all = [&](uint64_t lo, uint64_t len) {
+    for (int r = 0; r < n_rg; r++)
+      if (!disjoint(lo, len, rg[r][0], rg[r][1])) return false;
+    return true;
+  };
+  if (gp.kind == PK_GEMV) return clear_of_all(gp.c, gp.n);
+  const uint32_t n_groups = cdiv(gp.n, gp.rpg);
+  const uint32_t *idx = res_host(gp.h[0], n_groups), *val = res_host(gp.h[1], n_groups), *dst = res_host(gp.h[2], 1);
+  if (!idx || !val || !dst) return false;   // locations only known on the device: cannot be checked here
+  for (uint32_t i = 0; i < n_groups; i++)
+    if (!clear_of_all(idx[i], 1) || !clear_of_all(val[i], 1)) return false;
+  return clear_of_all(dst[0], 1);
+}
+
 static int launch_gemv(const PendOp& gp, const GemvFuse* fz) {
   Map* ma = get_f32_map(gp.map_act);
   Map* mw = get_map(gp.map_wt);
@@ -122,6 +141,8 @@ void flush_pending() {
   q.swap(g.pend);   // launches below must not see a non-empty queue
   const size_t n = q.size();
   size_t i = 0;
+  // the queued ops have returned ADAMAH_OK already: the first launch that fails is kept for the next call
+  auto keep = [](int rc) { if (rc != ADAMAH_OK && !g.deferred_err) g.deferred_err = rc; };
   while (i < n) {
     const PendOp& p = q[i];
     auto is_gemv = [&](size_t j) {   // a launch of the int8 matrix-instruction kernel (Q8 argmax ops are not)
@@ -133,6 +154,7 @@ void flush_pending() {
       // rotation of the new Q / K rows and the KV append: one launch for the run
       int rc = 0;
       i += launch_row_run(q, i, &rc);
+      keep(rc);
       continue;
     }
     if (p.kind == PK_GEMM) {
@@ -175,9 +197,10 @@ void flush_pending() {
         }
       }
       const uint32_t *la = res_u32(p.h[0], 1), *lb = res_u32(p.h[1], 1), *lc = res_u32(p.h[2], 1);
-      if (ma && mw && la && lb && lc)
-        launch_gemm_q4_mfma(ma, mw, la, lb, lc, p.rpg, p.k, sg.begin[m], 1, p.op == (uint32_t)FMT_Q8_B16, nullptr, (int64_t)p.a,
-                            (m == 1 && !sg.add) ? (int64_t)p.c : -1, (m == 1 && !sg.add) ? nullptr : &sg);
+      if (!(ma && mw && la && lb && lc)) keep(ADAMAH_ERR_INVALID);
+      else
+        keep(launch_gemm_q4_mfma(ma, mw, la, lb, lc, p.rpg, p.k, sg.begin[m], 1, p.op == (uint32_t)FMT_Q8_B16, nullptr, (int64_t)p.a,
+                                 (m == 1 && !sg.add) ? (int64_t)p.c : -1, (m == 1 && !sg.add) ? nullptr : &sg));
       i += used;
       continue;
     }
@@ -185,14 +208,16 @@ void flush_pending() {
       // the LM head of several sequences in lockstep: one pass over the matrix for all their rows
       int rc = 0;
       const size_t used = launch_argmax_run(q, i, &rc);
+      keep(rc);
       if (used) { i += used; continue; }
-      if (p.op == (uint32_t)FMT_Q8_B16) { launch_argmax_direct(p); i++; continue; }
+      if (p.op == (uint32_t)FMT_Q8_B16) { keep(launch_argmax_direct(p)); i++; continue; }
     }
     if (p.kind == PK_SCORES) {
       // a prefill chunk: the attention of consecutive tokens over one growing cache, one launch
       int rc = 0;
       size_t used = launch_attn_chunk(q, i, &rc);
       if (!used) used = launch_attn_batch(q, i, &rc);   // or one token of several sequences in lockstep
+      keep(rc);
       if (used) { i += used; continue; }
     }
     if (p.kind == PK_SCORES || p.kind == PK_ATTN) {
@@ -202,18 +227,18 @@ void flush_pending() {
       size_t ai = i;
       if (p.kind == PK_SCORES) {
         if (i + 1 < n && attn_foldable(p, q[i + 1])) { sc = &p; ai = i + 1; }
-        else { launch_scores(p); i++; continue; }
+        else { keep(launch_scores(p)); i++; continue; }
       }
       const PendOp& at = q[ai];
       bool fold = false;
       if (ai + 1 < n && q[ai + 1].kind == PK_GEMV && q[ai + 1].map_act == at.map_act) {
         const PendOp& gp = q[ai + 1];
         const uint32_t* oh = res_host(at.h[2], at.rpg);
-        fold = oh && gp.a == oh[0] && gp.k == at.rpg * at.k && (at.k & 7u) == 0;
+        fold = oh && gp.a == oh[0] && gp.k == at.rpg * at.k && (at.k & 7u) == 0 && disjoint(gp.c, gp.n, gp.a, gp.k);
         for (uint32_t h = 1; fold && h < at.rpg; h++) fold = oh[h] == oh[0] + h * at.k;
       }
       AttnPartials ap = {nullptr, 1, 0, 0, 0};
-      launch_attn(sc, at, fold, &ap);
+      keep(launch_attn(sc, at, fold, &ap));
       if (fold && ap.n_splits > 1) {   // partials left for the GEMV to merge
         fz.pro = PRO_COMBINE; fz.c_partial = ap.base; fz.c_splits = ap.n_splits; fz.c_vd = at.k;
         fz.p_dst = q[ai + 1].a;
@@ -232,7 +257,8 @@ void flush_pending() {
       // overwrite any input
       const bool safe = disjoint(p.c, p.n, p.a, p.n) && (p.c == p.d || disjoint(p.c, p.n, p.d, p.n)) &&
                         disjoint(m.c, m.n, p.a, p.n) && disjoint(m.c, m.n, p.d, p.n) && disjoint(m.c, m.n, p.c, p.n);
-      if (chain && safe && mw1 && mw2 && (p.n & 31u) == 0 && row_fits(gp) && g.sync_ctr) {
+      const uint64_t rd[4][2] = {{p.a, p.n}, {p.d, p.n}, {p.c, p.n}, {m.c, m.n}};   // src, residual, t, x
+      if (chain && safe && mw1 && mw2 && (p.n & 31u) == 0 && row_fits(gp) && g.sync_ctr && gemv_writes_clear(gp, rd, 4)) {
         fz.pro = PRO_NORM2; fz.p_src = p.a; fz.p_src2 = p.b; fz.p_eps = p.eps; fz.p_wt = (const float*)mw1->buf;
         fz.p_res = p.d; fz.p_tdst = p.c; fz.p_w2 = m.b; fz.p_eps2 = m.eps; fz.p_wt2 = (const float*)mw2->buf;
         fz.p_dst = m.c; fz.counter = g.sync_ctr;
@@ -242,16 +268,16 @@ void flush_pending() {
       const PendOp& gp = q[i + 1];
       Map* mw = get_f32_map(p.map_wt);
       // the prologue reads its source in every workgroup while workgroup 0 stores its result
+      const uint64_t rd[2][2] = {{p.a, p.n}, {p.c, p.n}};   // src, x
       if (gp.map_act == p.map_act && gp.a == p.c && gp.k == p.n && disjoint(p.a, p.n, p.c, p.n) && (p.n & 31u) == 0 &&
-          mw && row_fits(gp)) {
+          mw && row_fits(gp) && gemv_writes_clear(gp, rd, 2)) {
         fz.pro = PRO_RMSNORM; fz.p_src = p.a; fz.p_src2 = p.b; fz.p_dst = p.c; fz.p_eps = p.eps;
         fz.p_wt = (const float*)mw->buf;
         gi = i + 1;
       }
     }
     if (gi == n) {   // nothing to fold: launch the op alone
-      if (p.kind == PK_RMSNORM) launch_rmsnorm_v(p);
-      else launch_op2_v(p);
+      keep(p.kind == PK_RMSNORM ? launch_rmsnorm_v(p) : launch_op2_v(p));
       i++;
       continue;
     }
@@ -294,7 +320,7 @@ void flush_pending() {
         last = gi + 1;
       }
     }
-    launch_gemv(gp, (fz.pro || fz.e_mode) ? &fz : nullptr);
+    keep(launch_gemv(gp, (fz.pro || fz.e_mode) ? &fz : nullptr));
     i = last + 1;
   }
 }

@@ -478,12 +478,14 @@ static struct { const void* buf; uint64_t a; uint32_t M, K; uint64_t dispatch, m
 
 static bool ensure_act_bufs(size_t scale_floats, size_t xh_bytes) {
   if (scale_floats > g_scale_cap) {
+    layout_changed();
     if (g_scale_buf) { hipStreamSynchronize(g.stream); hipFree(g_scale_buf); }
     g_xh_key.valid = false;
     g_scale_cap = std::max<size_t>(scale_floats, 8192);
     if (hipMalloc((void**)&g_scale_buf, g_scale_cap * sizeof(float)) != hipSuccess) { g_scale_buf = nullptr; g_scale_cap = 0; return false; }
   }
   if (xh_bytes > g_xh_cap) {
+    layout_changed();
     if (g_xh_buf) { hipStreamSynchronize(g.stream); hipFree(g_xh_buf); }
     g_xh_key.valid = false;
     g_xh_cap = xh_bytes;

@@ -5,6 +5,8 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <algorithm>
+#include <deque>
+#include "gemv_common.h"
 
 namespace adamah {
 
@@ -26,6 +28,9 @@ int check_launch() {
     if (getenv("ADAMAH_DEBUG")) fprintf(stderr, "adamah_hip: launch -> %s\n", hipGetErrorString(e));
     return ADAMAH_ERR_BACKEND;
   }
+  // An op queued earlier has already returned ADAMAH_OK to its caller; if its launch failed when the queue was
+  // flushed, the first entry point that launches afterwards reports it.
+  if (g.deferred_err && g.pend.empty()) { const int d = g.deferred_err; g.deferred_err = 0; return d; }
   return ADAMAH_OK;
 }
 
@@ -85,6 +90,13 @@ uint32_t res_alloc(uint32_t n_bytes) {
   r.contig = false;
   return id;
 }
+
+// map_gather_dev results in the order they were made.  Once more than GATHER_RING of them, or more than
+// GATHER_BYTES of their storage, are live, the oldest is handed out again (same id, same storage).
+enum : size_t { GATHER_RING = 4096, GATHER_BYTES = (size_t)256 << 20 };
+static std::deque<uint32_t> g_gather_ring;
+static size_t g_gather_bytes = 0;
+static void gather_ring_reset() { g_gather_ring.clear(); g_gather_bytes = 0; }
 
 // Remember what was uploaded into a handle, and whether it is a run of consecutive indices.
 static void note_host(Res* r, const void* data, uint32_t n_bytes) {
@@ -291,6 +303,7 @@ static size_t g_tmp_cap[3] = {0, 0, 0};
 static void* tmp_dev(int slot, size_t n) {
   if (n <= g_tmp_cap[slot]) return g_tmp[slot];
   hipStreamSynchronize(g.stream);
+  layout_changed();
   if (g_tmp[slot]) hipFree(g_tmp[slot]);
   g_tmp[slot] = nullptr;
   g_tmp_cap[slot] = 0;
@@ -302,6 +315,7 @@ static void* tmp_dev(int slot, size_t n) {
 
 static void destroy_map(Map* m) {
   hipStreamSynchronize(g.stream);
+  layout_changed();
   if (m->buf) hipFree(m->buf);
   if (m->qp) hipFree(m->qp);
   if (m->d16) hipFree(m->d16);
@@ -314,6 +328,7 @@ static void destroy_map(Map* m) {
 using namespace adamah;
 
 static void plan_graph_reset(uint32_t plan_id);   // drops the recorded graphs of a decode plan (defined with them)
+static void plan_graph_handle_rewritten(uint32_t handle);   // a recorded graph holds the old contents of a handle by value
 
 // =================================================================================================
 extern "C" {
@@ -359,6 +374,7 @@ void adamah_shutdown(void) { ADAMAH_API();
   for (uint8_t* p : g.arena_chunks) hipFree(p);
   g.arena_chunks.clear(); g.arena_cur = nullptr; g.arena_left = 0;
   g.res.clear();
+  gather_ring_reset();
   for (int i = 0; i < 8; i++) g_scratch_h[i] = 0;
   for (int i = 0; i < 3; i++) { if (g_tmp[i]) hipFree(g_tmp[i]); g_tmp[i] = nullptr; g_tmp_cap[i] = 0; }
   for (int i = 0; i < 2; i++) {
@@ -419,6 +435,8 @@ int adamah_fusion_is_enabled(void) { return g.fusion_enabled; }
 // A scheduling hint in the reference (submit what has been fused so far); results only become
 // observable at a sync or a read-back, so the pending queue is left alone.
 int adamah_fusion_flush(void) { g.stats.fusion_flush++; return ADAMAH_OK; }
+// First failure among launches of queued ops since the last call, then cleared (0 when none).
+static int take_deferred_err() { const int d = g.deferred_err; g.deferred_err = 0; return d; }
 void adamah_fusion_set_scheduler_mode(int mode) { if (mode >= 0 && mode <= 2) g.scheduler_mode = mode; }
 int adamah_fusion_get_scheduler_mode(void) { return g.scheduler_mode; }
 int adamah_register_loc_span(uint32_t h, uint32_t map_id, uint32_t, uint32_t) { ADAMAH_API();
@@ -457,6 +475,7 @@ int map_init_dtype(uint32_t id, uint32_t dtype, uint32_t pack_size, uint32_t n_p
   if (dtype == DTYPE_BF16 || dtype == DTYPE_Q6) return ADAMAH_ERR_INVALID;
   Map* m = &g.maps[id];
   g.mem_gen++;   // the fills below rewrite device memory without counting as launches
+  layout_changed();
   if (m->active) destroy_map(m);
   bool quant = dtype == DTYPE_Q8 || dtype == DTYPE_Q4;
   m->dtype = dtype; m->pack_size = pack_size; m->n_packs = n_packs;
@@ -504,6 +523,7 @@ int map_set_qparams(uint32_t map_id, const float* scales, const float* zps, uint
   Map* m = get_map(map_id);
   if (!m || !m->qp || !scales || !zps) return ADAMAH_ERR_INVALID;
   if ((uint64_t)n_groups > m->n_groups) return ADAMAH_ERR_INVALID;
+  layout_changed();   // the storage format of the map's groups (and with it the kernel chosen) may change
   const float off = m->dtype == DTYPE_Q4 ? -8.0f : -128.0f;
   uint64_t prefix = 0;
   bool conform = m->group_size == 32;
@@ -542,6 +562,7 @@ int adamah_kv_cache_fp16(uint32_t map_id, uint32_t start, uint32_t count) { ADAM
   Map* m = get_f32_map(map_id);
   if (!m || count == 0 || !in_range(start, count, m->n_elems)) return ADAMAH_ERR_INVALID;
   hipStreamSynchronize(g.stream);
+  layout_changed();
   if (m->kv16) hipFree(m->kv16);
   m->kv16 = nullptr;
   if (hipMalloc((void**)&m->kv16, (size_t)count * sizeof(__half) + 256) != hipSuccess) return ADAMAH_ERR_MEMORY;
@@ -668,7 +689,7 @@ uint64_t map_gather(uint32_t map_id, const uint32_t* locs, void* data, uint32_t 
 // ---- handles ---------------------------------------------------------------------------------------
 uint64_t map_upload_dev(uint32_t handle, const void* data, uint32_t n_bytes) {
   // a new handle cannot be an operand of anything queued; rewriting an existing one can
-  if (handle != 0) ADAMAH_API();
+  if (handle != 0) { ADAMAH_API(); plan_graph_handle_rewritten(handle); }
   if (!g.initialized || !data || n_bytes == 0) return 0;
   uint32_t id = handle;
   if (id == 0) {
@@ -697,8 +718,25 @@ uint64_t map_gather_dev(uint32_t map_id, uint32_t locs_handle, uint32_t n_locs) 
   if (m->dtype != DTYPE_F32 && !m->qp) return 0;
   uint64_t n_vals = (uint64_t)n_locs * m->pack_size;
   if (n_vals * 4 > 0xFFFFFFFFull) return 0;
-  uint32_t id = res_alloc((uint32_t)(n_vals * 4));
-  if (id == 0) return 0;
+  // Results are never released individually (as in the reference, whose table ends after 2048).  A decode loop
+  // gathers one embedding row per token, so only the latest results are kept: the storage and id of the oldest
+  // is handed out again when it is large enough, and handles and arena stop growing.
+  const uint32_t need = (uint32_t)(n_vals * 4);
+  uint32_t id = 0;
+  if (g_gather_ring.size() >= GATHER_RING || g_gather_bytes + need > GATHER_BYTES) {
+    Res* old = get_res(g_gather_ring.empty() ? 0u : g_gather_ring.front());
+    if (old && old->cap_bytes >= need) {
+      id = g_gather_ring.front();
+      g_gather_ring.pop_front();
+      old->size_bytes = need; old->host.clear(); old->host_valid = false; old->contig = false;
+    }
+  }
+  if (id == 0) {
+    id = res_alloc(need);
+    if (id == 0) return 0;
+    g_gather_bytes += g.res[id].cap_bytes;
+  }
+  g_gather_ring.push_back(id);
   float* dst = (float*)g.res[id].dptr;
   if (m->dtype == DTYPE_F32)
     k_gather_f32<<<cdiv(n_vals, 256), 256, 0, g.stream>>>((const float*)m->buf, dst, locs, n_locs, m->pack_size,
@@ -783,7 +821,13 @@ static int replay_plan(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
                                             u4, op.f0); break;
       case 24: ret = map_row_copy_offset_dev(op.map_id, op.h0, op.h1, u0, u1, u2); break;
       case 25: ret = map_attn_softmax_value_dev(op.map_id, op.h0, op.h1, op.h2, u0, u1, u2, op.f0, op.f1); break;
-      default: ret = ADAMAH_ERR_INVALID; break;   // fused qkv / gate-up kinds are not built
+      // fused projections (adamah.c:10318-10334): the seventh handle of the Q/K/V form travels in u0
+      case 26: ret = map_fused_qkv_t_xq4_dev(op.map_id, op.map_id2, op.h0, op.h1, op.h2, op.h3, op.h4, op.h5, u0, u1, u2, u3, u4); break;
+      case 27: ret = map_fused_gateup_t_xq4_dev(op.map_id, op.map_id2, op.h0, op.h1, op.h2, op.h3, op.h4, u0, u1, u2); break;
+      case 28: ret = map_fused_qkv_t_xq8_dev(op.map_id, op.map_id2, op.h0, op.h1, op.h2, op.h3, op.h4, op.h5, u0, u1, u2, u3, u4); break;
+      case 29: ret = map_fused_gateup_t_xq8_dev(op.map_id, op.map_id2, op.h0, op.h1, op.h2, op.h3, op.h4, u0, u1, u2); break;
+      case 30: ret = map_fused_gateup_act_t_xq8_dev(op.map_id, op.map_id2, op.h0, op.h1, op.h2, op.h3, u0, u1); break;
+      default: ret = ADAMAH_ERR_INVALID; break;
     }
     if (ret != ADAMAH_OK) break;
   }
@@ -805,6 +849,8 @@ struct PlanGraph {
   uint32_t pos = 0, seq = 0, n_nodes = 0;
   int eager_steps = 0;
   uint32_t n_graph = 0, n_update = 0, n_inst = 0;   // steps served by a graph, in-place updates, instantiations
+  uint64_t gen = 0;          // g.layout_gen when the graph was recorded: it holds device pointers and offsets by value
+  std::vector<uint32_t> handles;   // sorted ids of the handles the plan's ops name (their contents are baked in too)
 };
 static PlanGraph g_pg[MAX_PLANS];
 
@@ -823,7 +869,7 @@ static void plan_graph_drop(PlanGraph& pg, bool for_good) {
 static void plan_graph_record(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
   PlanGraph& pg = g_pg[plan_id];
   pg.ready = false;
-  const uint64_t gen0 = g.mem_gen;
+  const uint64_t gen0 = g.mem_gen, lay0 = g.layout_gen;
   const Stats saved = g.stats;
   if (hipStreamBeginCapture(g.stream, hipStreamCaptureModeThreadLocal) != hipSuccess) { (void)hipGetLastError(); plan_graph_drop(pg, true); return; }
   int r = replay_plan(plan_id, pos, seq_len);
@@ -832,12 +878,13 @@ static void plan_graph_record(uint32_t plan_id, uint32_t pos, uint32_t seq_len) 
   const hipError_t e = hipStreamEndCapture(g.stream, &graph);
   const uint32_t n_nodes = (uint32_t)(g.stats.dispatch - saved.dispatch);
   g.stats = saved;                                   // nothing ran: the launches are counted when the graph does
-  if (r != ADAMAH_OK || e != hipSuccess || !graph || g.mem_gen != gen0 || n_nodes == 0) {
+  if (r != ADAMAH_OK || e != hipSuccess || !graph || g.mem_gen != gen0 || g.layout_gen != lay0 || n_nodes == 0) {
     if (graph) hipGraphDestroy(graph);
     (void)hipGetLastError();
     plan_graph_drop(pg, true);
     return;
   }
+  gemm_act_forget();   // the note "these rows are converted" was taken while nothing ran
   const int slot = pg.cur ^ 1;
   if (pg.exec[slot]) {
     hipGraphNode_t bad = nullptr;
@@ -858,7 +905,15 @@ static void plan_graph_record(uint32_t plan_id, uint32_t pos, uint32_t seq_len) 
     return;
   }
   hipGraphDestroy(graph);
-  pg.cur = slot; pg.ready = true; pg.pos = pos; pg.seq = seq_len; pg.n_nodes = n_nodes;
+  pg.cur = slot; pg.ready = true; pg.pos = pos; pg.seq = seq_len; pg.n_nodes = n_nodes; pg.gen = g.layout_gen;
+}
+
+// The graph of a plan was recorded from the host copies of its handles: rewriting one of them makes it stale.
+static void plan_graph_handle_rewritten(uint32_t handle) {
+  for (int i = 0; i < MAX_PLANS; i++) {
+    PlanGraph& pg = g_pg[i];
+    if (pg.ready && std::binary_search(pg.handles.begin(), pg.handles.end(), handle)) pg.ready = false;
+  }
 }
 
 static void plan_graph_reset(uint32_t plan_id) {
@@ -881,6 +936,13 @@ int adamah_decode_step(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
   if (!plan_graphs_on() || pg.disabled) ret = replay_plan(plan_id, pos, seq_len);
   else {
     flush_pending();                                 // what was queued before the plan runs ahead of it
+    if (pg.ready && pg.gen != g.layout_gen) pg.ready = false;   // a map or scratch buffer moved since the recording
+    if (pg.handles.empty()) {
+      for (const PlanOp& op : g.plans[plan_id])
+        for (uint32_t h : {op.h0, op.h1, op.h2, op.h3, op.h4, op.h5}) if (h) pg.handles.push_back(h);
+      std::sort(pg.handles.begin(), pg.handles.end());
+      pg.handles.erase(std::unique(pg.handles.begin(), pg.handles.end()), pg.handles.end());
+    }
     if (pg.ready && pg.pos == pos && pg.seq == seq_len) {
       ret = hipGraphLaunch(pg.exec[pg.cur], g.stream) == hipSuccess ? ADAMAH_OK : ADAMAH_ERR_BACKEND;
       count_launch((int)pg.n_nodes);
@@ -896,6 +958,7 @@ int adamah_decode_step(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
     else pg.ready = false;
   }
   if (opened) batch_end();
+  if (ret == ADAMAH_OK && g.pend.empty()) ret = take_deferred_err();
   return ret;
 }
 

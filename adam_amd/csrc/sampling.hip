@@ -259,6 +259,7 @@ int map_topk_dev(uint32_t map_id, uint32_t hs, uint32_t hi, uint32_t hv, uint32_
   if (chunks > 1) {
     const size_t need = (size_t)chunks * k;
     if (need > g_topk_part_cap) {
+      layout_changed();
       if (g_topk_part) { hipStreamSynchronize(g.stream); hipFree(g_topk_part); }
       g_topk_part_cap = std::max<size_t>(need, 4096);
       if (hipMalloc((void**)&g_topk_part, g_topk_part_cap * 8) != hipSuccess) {

@@ -234,6 +234,7 @@ static int op_matvec_topk(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uin
   if (bh && !in_range(bh[0], (uint64_t)N * K, mw->n_elems)) return ADAMAH_ERR_INVALID;
   // fixed_logits: the caller's scratch of at least N floats (the entry point that may not allocate)
   if (!fixed_logits && N > g_logit_cap) {
+    layout_changed();
     if (g_logit_buf) { hipStreamSynchronize(g.stream); hipFree(g_logit_buf); }
     g_logit_cap = std::max<size_t>(N, 1u << 16);
     if (hipMalloc((void**)&g_logit_buf, g_logit_cap * sizeof(float)) != hipSuccess) {
@@ -374,6 +375,7 @@ size_t launch_argmax_run(const std::vector<PendOp>& q, size_t i, int* rc) {
   }
   const size_t need = (size_t)m * N + 2 * (size_t)m * n_groups + 2;
   if (need > g_logit_cap) {
+    layout_changed();
     if (g_logit_buf) { hipStreamSynchronize(g.stream); hipFree(g_logit_buf); }
     g_logit_cap = std::max<size_t>(need, 1u << 16);
     if (hipMalloc((void**)&g_logit_buf, g_logit_cap * sizeof(float)) != hipSuccess) {

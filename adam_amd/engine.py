@@ -582,6 +582,8 @@ class DecodeEngine:
         g.batch_begin()
         if self._tied:
             src_h, _, _, _ = g.map_gather_dev(self._map_of[self._lm_name], self._emb_gather_h, c.n_embd)
+            if src_h == 0:        # the binding reports a failed gather as handle 0, like the reference's
+                raise RuntimeError("map_gather_dev failed (embedding row)")
             g.map_scatter_dev(ws, hid_h, c.n_embd, src_h)
             if c.emb_scale != 1.0:
                 g.map_broadcast_dev(ws, A.OP_MUL, hid_h, W['emb_scale'][0], hid_h, c.n_embd)

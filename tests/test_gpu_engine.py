@@ -258,3 +258,49 @@ def test_decode_plan_from_recorded_graphs_gives_the_same_tokens(arch):
             assert int(line[-1].split(":")[1].split()[0]) >= 60, line[-1]       # most steps came from graphs
     assert res["0"]["tokens"] == res["1"]["tokens"]
     assert res["0"]["hidden"] == res["1"]["hidden"]
+
+
+_GRAPH_STALE_SNIPPET = """
+import sys, json
+sys.path.insert(0, {root!r})
+import numpy as np
+from adam_amd import adamah as A
+gpu = A.init()
+n = 4096
+gpu.set_dtype(A.DTYPE_F32)
+gpu.map_create(0, 1, 4 * n)
+rng = np.random.default_rng(0)
+vals = rng.standard_normal(3 * n).astype(np.float32)
+gpu.scatter_contiguous(0, 0, vals)
+run = lambda lo: np.arange(lo, lo + n, dtype=np.uint32)
+a_h, b_h, c_h = (gpu.upload_dev(run(lo))[0] for lo in (0, n, 3 * n))
+gpu.register_decode_plan(3, [A.DecodePlanOp(kind=A.DECODE_OP_OP2, map_id=0, op_code=A.OP_ADD, h0=a_h, h1=b_h, h2=c_h, u0=n)])
+out = []
+for step in range(8):
+    if step == 4:
+        gpu.upload_dev(run(2 * n), handle=b_h)          # the recorded graph of step 4 still holds the old offset
+    if step == 6:
+        gpu.map_create(5, 1, 1024)                      # an unrelated map appears: recorded graphs are dropped
+    gpu.decode_step(3, step, step + 1)
+    got = gpu.gather(0, run(3 * n)).view(np.float32)
+    want = vals[:n] + (vals[n:2 * n] if step < 4 else vals[2 * n:])
+    out.append(bool(np.array_equal(got, want)))
+gpu.shutdown()
+print(json.dumps(out))
+"""
+
+
+def test_recorded_graph_is_dropped_when_a_plan_handle_is_rewritten():
+    """A graph recorded one step ahead holds operand offsets by value: re-uploading a handle of the plan (or any
+    event that may move device buffers) between the recording and the launch must send that step through the
+    ordinary replay.  Every step's result is checked."""
+    import json, os, subprocess, sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    note("decode plan graphs: handle rewritten between record and launch")
+    env = dict(os.environ, ADAMAH_PLAN_GRAPH="1", ADAMAH_DEBUG="1")
+    p = subprocess.run([sys.executable, "-c", _GRAPH_STALE_SNIPPET.format(root=root)], env=env, capture_output=True, text=True,
+                       timeout=110)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert json.loads(p.stdout.strip().split("\n")[-1]) == [True] * 8, p.stdout
+    line = [l for l in p.stderr.split("\n") if "steps from graphs" in l]
+    assert line and int(line[-1].split(":")[1].split()[0]) >= 2, p.stderr[-1000:]      # graphs were in use at all

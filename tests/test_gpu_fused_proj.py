@@ -122,3 +122,44 @@ def test_errors(hip):
         hip.map_fused_gateup_t_xq4_dev(0, 1, a, b, b, c, up(hip, [250]), 32, 4, 8)     # result past the map
     with pytest.raises(RuntimeError):
         hip.map_fused_gateup_act_t_xq8_dev(0, 1, a, b, b, c, 32, 4)                    # Q8 only
+
+
+def test_fused_projection_kinds_in_a_decode_plan(hip):
+    """Decode-plan kinds 26..30 (adamah.c:10318-10334; the Q/K/V forms carry their seventh handle in u0) replay
+    the fused entry points: same words as the direct calls."""
+    K, rows, ff = 1152, (1024, 256, 256), 768
+    x = np.random.default_rng(3).standard_normal(K).astype(np.float32)
+    got = {}
+    for route in ("direct", "plan"):
+        note(f"fused kinds via {route}")
+        res = []
+        for kind, kq, kg in (("q4", A.DECODE_OP_FUSED_QKV_T_XQ4, A.DECODE_OP_FUSED_GATEUP_T_XQ4),
+                             ("q8", A.DECODE_OP_FUSED_QKV_T_XQ8, A.DECODE_OP_FUSED_GATEUP_T_XQ8)):
+            qt, bases = stacked(kind, rows + (ff, ff), K, 11)
+            load_qtensor(hip, 1, qt)
+            f32map(hip, 0, K + sum(rows) + 3 * ff + 64, x)
+            cs = np.cumsum((K,) + rows + (ff, ff))
+            hb = [up(hip, [b]) for b in bases]
+            hc = [up(hip, [int(c)]) for c in cs[:5]]
+            a = up(hip, [0])
+            if route == "direct":
+                hip.batch_begin()
+                (hip.map_fused_qkv_t_xq4_dev if kind == "q4" else hip.map_fused_qkv_t_xq8_dev)(0, 1, a, *hb[:3], *hc[:3], K, *rows)
+                (hip.map_fused_gateup_t_xq4_dev if kind == "q4" else hip.map_fused_gateup_t_xq8_dev)(0, 1, a, *hb[3:], *hc[3:], K, ff, ff)
+                if kind == "q8":
+                    hip.map_fused_gateup_act_t_xq8_dev(0, 1, a, hb[3], hb[4], up(hip, [int(cs[5])]), K, ff)
+                hip.batch_end()
+            else:
+                ops = [A.DecodePlanOp(kind=kq, map_id=0, map_id2=1, h0=a, h1=hb[0], h2=hb[1], h3=hb[2], h4=hc[0], h5=hc[1],
+                                      u0=hc[2], u1=K, u2=rows[0], u3=rows[1], u4=rows[2]),
+                       A.DecodePlanOp(kind=kg, map_id=0, map_id2=1, h0=a, h1=hb[3], h2=hb[4], h3=hc[3], h4=hc[4], u0=K, u1=ff, u2=ff)]
+                if kind == "q8":
+                    ops.append(A.DecodePlanOp(kind=A.DECODE_OP_FUSED_GATEUP_ACT_T_XQ8, map_id=0, map_id2=1, h0=a, h1=hb[3], h2=hb[4],
+                                              h3=up(hip, [int(cs[5])]), u0=K, u1=ff))
+                hip.register_decode_plan(5, ops)
+                hip.decode_step(5, 0, 1)
+                hip.clear_decode_plan(5)
+            res.append(read(hip, 0, K, sum(rows) + 3 * ff))
+        got[route] = res
+    for d, p in zip(got["direct"], got["plan"]):
+        assert np.any(d) and np.array_equal(d.view(np.uint32), p.view(np.uint32))

@@ -139,6 +139,41 @@ def test_aliasing_sequences_are_not_folded(hip):
     assert rel_l2(out["hip"]["x"], out["oracle"]["x"]) < TOL
 
 
+@pytest.mark.parametrize("case", ["result_on_norm_source", "result_on_residual", "argmax_lists_on_norm_source"])
+def test_gemv_result_over_a_prologue_operand_is_not_folded(hip, case):
+    """rmsnorm(A -> B); matvec(B -> A): legal as separate ops, but a GEMV that normalised A in every workgroup
+    while storing result rows into A would race.  The same for a result that lands on the residual of the
+    two-norm prologue, and for partial argmax lists that lie inside the norm's source."""
+    K = N = 2048
+    s = Slots(K, N)
+    qt = make_weights(N, K, 19)
+    out = {}
+    for name, g in (("hip", hip), ("oracle", oracle.init())):
+        note(f"fusion aliasing {case} {name}")
+        s.fill(g, 17)
+        load_qtensor(g, 1, qt)
+        g.batch_begin()
+        if case == "result_on_norm_source":
+            g.map_rmsnorm_dev(0, s.h(g, "src"), s.h(g, "nw"), s.h(g, "x"), 1, K, 1e-6)
+            g.map_matmul_t_xq4_dev(0, 1, s.h(g, "x"), up(g, [0]), s.h(g, "src"), 1, K, N)
+        elif case == "result_on_residual":
+            g.map_rmsnorm_add_dev(0, s.h(g, "src"), s.h(g, "nw"), s.h(g, "resk"), s.h(g, "src2"), 1, K, 1e-6)
+            g.map_rmsnorm_dev(0, s.h(g, "src2"), s.h(g, "nwk"), s.h(g, "x"), 1, K, 1e-5)
+            g.map_matmul_t_xq4_dev(0, 1, s.h(g, "x"), up(g, [0]), s.h(g, "resk"), 1, K, N)
+        else:
+            rpg = 64
+            g.map_rmsnorm_dev(0, s.h(g, "src"), s.h(g, "nw"), s.h(g, "x"), 1, K, 1e-6)
+            g.map_matvec_argmax_t_xq4_dev(0, 1, s.h(g, "x"), up(g, [0]), s.run(g, "src", N // rpg),
+                                          up(g, np.arange(s.off["src"] + 100, s.off["src"] + 100 + N // rpg, dtype=np.uint32)),
+                                          s.h(g, "tok"), K, N, rpg)
+        g.batch_end()
+        out[name] = {n: read(g, 0, s.off[n], K) for n in ("src", "src2", "x", "resk")}
+        out[name]["tok"] = read(g, 0, s.off["tok"], 1)
+    for slot in ("src", "src2", "x", "resk"):
+        assert rel_l2(out["hip"][slot], out["oracle"][slot]) < TOL, slot
+    assert out["hip"]["tok"][0] == out["oracle"]["tok"][0]
+
+
 @pytest.mark.parametrize("K,N,rpg", [(1152, 4096, 256), (2048, 1000, 64)])
 def test_rmsnorm_folded_into_matvec_argmax(hip, K, N, rpg):
     s = Slots(K, N)

@@ -277,3 +277,23 @@ def test_matvec_argmax_of_consecutive_rows_in_one_pass(hip, kind, N, K, rpg, m):
             assert logits[j, res[0][0][j]] >= top2[0] - 1e-9
     assert rel_l2(res[0][2], res[1][2]) < 1e-3
     assert (res[0][1] == res[1][1]).mean() > 0.95
+
+
+def test_gather_dev_results_stop_consuming_handles(hip):
+    """map_gather_dev returns a new result handle per call (a decode loop makes one per token); the library keeps
+    the latest few thousand and hands the oldest out again, so ids stay bounded while recent results stay valid."""
+    note("gather_dev handle ring")
+    n = 64
+    f32map(hip, 0, 4 * n, np.arange(4 * n, dtype=np.float32))
+    locs = [up(hip, np.arange(lo, lo + n)) for lo in (0, n, 2 * n)]
+    h0 = hip.map_gather_dev(0, locs[0], n)[0]
+    h1 = hip.map_gather_dev(0, locs[1], n)[0]
+    assert h0 != 0 and h1 != 0 and h0 != h1
+    assert np.array_equal(hip.download_dev(h0, n), np.arange(0, n, dtype=np.float32))      # an older result is intact
+    assert np.array_equal(hip.download_dev(h1, n), np.arange(n, 2 * n, dtype=np.float32))
+    ids = set()
+    for i in range(6000):
+        ids.add(hip.map_gather_dev(0, locs[i % 3], n)[0])
+    assert 0 not in ids and len(ids) <= 4200
+    last = hip.map_gather_dev(0, locs[2], n)[0]
+    assert np.array_equal(hip.download_dev(last, n), np.arange(2 * n, 3 * n, dtype=np.float32))
