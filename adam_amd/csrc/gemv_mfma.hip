@@ -52,6 +52,7 @@ struct PreM {
   uint4 q[MF_U];
   __half h[MF_U];
   float2 p[MF_U];
+  float res;   // EPIX_ADD: the residual of this lane's result row, fetched with the weights of the bundle's last step
 };
 
 // PRO selects where the activation vector comes from: the map as it is, or the result of preceding
@@ -129,13 +130,18 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       if (B16) R.h[u] = d16[gi];
       else R.p[u] = qp[gi];
     }
+    // The add epilogue needs one residual value per result row: asked for here, in the compute mapping (lane =
+    // 4 * column + row, column 0 stores), so it has arrived long before the row sum is complete.
+    if (EPI == EPI_STORE && fz.e_mode == EPIX_ADD && chunk + ks >= C && bcol == 0u)
+      R.res = act[(uint64_t)fz.e_res + min(row0 + l, end - 1u)];
   };
 
   PreM A, B;   // A's first loads stay in flight while the activations are staged
+  auto first_loads = [&]() { if (first < seg_end) load(A, first, kpart, seg_end); };
   // Loads come back in order: the activation loads (cache hits) go out ahead of the first weights, so
   // the conversion does not wait for the weights' trip to memory as well.
   const bool x_first = fz.x_first != 0u;
-  if (PRO == PRO_NONE && !x_first && first < seg_end) load(A, first, kpart, seg_end);
+  if (PRO == PRO_NONE && !x_first) first_loads();
 
   // ---- activations -> fixed-point digits; one 8-element word per thread and pass, four threads per
   // block.  stage() turns one word into digits; the prologues below decide what the word is. ------
@@ -205,7 +211,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       for (uint32_t u = 0; u < 4; u++) load8(act + a + (uint64_t)min(i0 + u * nthr + tid, nw - 1u) * 8u, x[u]);
       if (i0 == 0u && x_first) {
         __builtin_amdgcn_sched_barrier(0);
-        if (first < seg_end) load(A, first, kpart, seg_end);
+        first_loads();
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
@@ -216,7 +222,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
   } else if (PRO == PRO_COMBINE) {
     // Folded merge of the attention partials (same arithmetic as the stand-alone merge kernel):
     // M = max m_s, w_s = e^(m_s - M), L = sum l_s w_s, x = sum_s o_s w_s / L, per head.
-    if (first < seg_end) load(A, first, kpart, seg_end);
+    first_loads();
     const uint32_t stride = fz.c_vd + 2u;
     for (uint32_t i0 = 0; i0 < nw; i0 += nthr) {
       const uint32_t i = i0 + tid, ic = min(i, nw - 1u);
@@ -267,7 +273,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       if (PRO == PRO_NORM2) { load8(act + fz.p_res + e0, rv[u]); load8(fz.p_wt2 + fz.p_w2 + e0, w2v[u]); }
     }
     __builtin_amdgcn_sched_barrier(0);   // activation loads first: they are waited for first
-    if (first < seg_end) load(A, first, kpart, seg_end);
+    first_loads();
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (uint32_t u = 0; u < PRO_WPT; u++)
@@ -344,6 +350,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
   uint32_t best_i = INVALID_IDX;
 
   const int perm_addr = (int)((16u * l + bcol) << 2);   // the lane that loaded this lane's (row, block column)
+  float res_keep = 0.f;                                  // ks > 1: residual of the bundle, from this wave's last step
   auto compute = [&](const PreM& Rl, uint32_t row0, uint32_t chunk, uint32_t end) {
     PreM R;
 #pragma unroll
@@ -401,7 +408,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       }
     }
     if (ks > 1u) {
-      if (chunk + ks >= C) part[wave * 64u + lane] = acc;   // this wave's share of the bundle is done
+      if (chunk + ks >= C) { part[wave * 64u + lane] = acc; res_keep = Rl.res; }   // this wave's share of the bundle is done
     } else if (chunk == C - 1u) {   // row bundle complete: sum the 16 lanes that share a row
       float y = acc;
       y += __shfl_xor(y, 4, 64); y += __shfl_xor(y, 8, 64);
@@ -423,7 +430,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
         if (row < end && bcol == 0u) {
           if (EPI == EPI_STORE) {
             act_out[(uint64_t)c_out + row] = y;
-            if (fz.e_mode == EPIX_ADD) act_out[(uint64_t)fz.e_dst + row] = act[(uint64_t)fz.e_res + row] + y;
+            if (fz.e_mode == EPIX_ADD) act_out[(uint64_t)fz.e_dst + row] = Rl.res + y;
           } else if (better(y, row, best_v, best_i)) { best_v = y; best_i = row; }
         }
       }
@@ -487,7 +494,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
         const uint32_t row = first + l;
         if (row < N && bcol == 0u) {
           act_out[(uint64_t)c_out + row] = y;
-          if (fz.e_mode == EPIX_ADD) act_out[(uint64_t)fz.e_dst + row] = act[(uint64_t)fz.e_res + row] + y;
+          if (fz.e_mode == EPIX_ADD) act_out[(uint64_t)fz.e_dst + row] = res_keep + y;
         }
       }
       break;
@@ -585,14 +592,15 @@ static void mfma_shape(uint32_t K, uint32_t units, uint32_t* grid, uint32_t* thr
   *grid = std::max(1u, std::min<uint32_t>(cdiv(units, waves), (uint32_t)g.n_cu * wg_per_cu));
 }
 
-// Store launches of short matrices with long rows leave most SIMDs without work when a bundle of four
-// rows belongs to one wave: there, 2 or 4 waves share a bundle and split K (one step of 2048 at a time).
+// Store launches of short matrices leave most SIMDs without work when a bundle of four rows belongs to one wave:
+// there, 2 or 4 waves share a bundle and split K (one step of 2048 at a time), as far as that keeps the launch
+// within the 4096 waves the device holds at once.  A wave then has one or two steps, all of whose loads are in
+// flight from the start: such launches are bound by one trip to memory, not by arithmetic.
 static uint32_t mfma_ksplit(uint32_t K, uint32_t N, bool paired_rows) {
   const uint32_t C = cdiv(K, 2048u), n_q = cdiv(N, 4u);
   const uint32_t want = (uint32_t)std::max(1, tuning("ADAMAH_MFMA_KSPLIT_WAVES", 4096));
   uint32_t ks = 1;
-  // every wave keeps at least one full step and a partial one, so its loads still overlap its arithmetic
-  while (ks < 4u && ks * 2u * 3u <= C * 2u && n_q * ks * 2u <= want) ks *= 2u;
+  while (ks < 4u && ks * 2u <= C && n_q * ks * 2u <= want) ks *= 2u;
   const int forced = tuning("ADAMAH_MFMA_KS", 0);
   if (forced == 1 || forced == 2 || forced == 4) ks = std::min<uint32_t>((uint32_t)forced, std::max(1u, C));
   if (ks == 3u) ks = 2u;
@@ -602,7 +610,19 @@ static uint32_t mfma_ksplit(uint32_t K, uint32_t N, bool paired_rows) {
 static void mfma_store_shape(uint32_t K, uint32_t N, uint32_t ks, uint32_t* grid, uint32_t* threads) {
   const uint32_t n_q = cdiv(N, 4u);
   mfma_shape(K, n_q * ks, grid, threads);
-  if (ks > 1u) *grid = cdiv(n_q, *threads / 64u / ks);   // one bundle per ks waves, one round
+  if (ks > 1u) {
+    // one bundle per ks waves, one round.  Every workgroup stages the activations, so the workgroup size is the
+    // one with the fewest (rounds over the CUs) x (waves per workgroup); ties go to the larger workgroup.
+    uint32_t best_w = 4, best_cost = ~0u;
+    for (uint32_t w = 4; w <= 16; w *= 2) {
+      const uint32_t cost = cdiv(cdiv(n_q * ks, w), (uint32_t)g.n_cu) * w;
+      if (cost <= best_cost) { best_cost = cost; best_w = w; }
+    }
+    const int fw = tuning("ADAMAH_MFMA_WAVES", 0);
+    if (fw > 0) best_w = fw >= 16 ? 16 : fw >= 8 ? 8 : 4;
+    *threads = best_w * 64u;
+    *grid = cdiv(n_q, best_w / ks);
+  }
 }
 
 uint32_t mfma_store_threads(uint32_t K, uint32_t N) {
