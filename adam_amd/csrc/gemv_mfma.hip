@@ -41,6 +41,27 @@ __device__ unsigned long long g_trace[64];
 #define TR(i) do {} while (0)
 #endif
 
+// lane ^ 1 and lane ^ 2 within a quad (quad_perm [1,0,3,2] and [2,3,0,1]): a register move, no trip through LDS
+__device__ __forceinline__ float quad_x1(float v) {
+  int r = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false);
+  asm volatile("" : "+v"(r));   // kept an instruction of its own, see quad_b3
+  return __int_as_float(r);
+}
+__device__ __forceinline__ float quad_x2(float v) {
+  int r = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, false);
+  asm volatile("" : "+v"(r));
+  return __int_as_float(r);
+}
+
+// Lane 3 of every quad to the whole quad (quad_perm [3,3,3,3]).  The result is made opaque so that the move stays
+// an instruction of its own: with the move folded into the consuming subtract / multiply the kernel returned wrong
+// sums on the device although the generated code read as equivalent.
+__device__ __forceinline__ uint32_t quad_b3(uint32_t v) {
+  int r = __builtin_amdgcn_update_dpp(0, (int)v, 0xFF, 0xF, 0xF, false);
+  asm volatile("" : "+v"(r));
+  return (uint32_t)r;
+}
+
 // LDS layout: 128 bytes per activation block = 8 chunks of 16 bytes.  Chunk 2*d + h holds digit d of
 // words 2h, 2h+1 as {even(2h), odd(2h), even(2h+1), odd(2h+1)} (even/odd = elements 0,2,4,6 / 1,3,5,7 of
 // the 8-element word, one byte each, matching the byte order of the unpacked codes); chunk 6 holds
@@ -150,8 +171,9 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
     float m = 0.f, poison = 0.f;          // poison turns NaN as soon as one element is Inf or NaN
 #pragma unroll
     for (int k = 0; k < 8; k++) { m = fmaxf(m, fabsf(x[k])); poison = fmaf(x[k], 0.f, poison); }
-    m = fmaxf(m, __shfl_xor(m, 1, 64)); m = fmaxf(m, __shfl_xor(m, 2, 64));
-    poison += __shfl_xor(poison, 1, 64); poison += __shfl_xor(poison, 2, 64);
+    // the four threads of a block are a quad: lane ^ 1 and lane ^ 2 through the data-parallel crossbar
+    m = fmaxf(m, quad_x1(m)); m = fmaxf(m, quad_x2(m));
+    poison += quad_x1(poison); poison += quad_x2(poison);
     const uint32_t e = (__float_as_uint(m) >> 23) & 0xFFu;
     float s = 1.f, fs = 1.f;              // |x * s| < 2^21 when the block is finite and not tiny
     if (e >= 21u && e <= 254u) { s = __uint_as_float((274u - e) << 23); fs = __uint_as_float((e - 20u) << 23); }
@@ -164,7 +186,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       sx += xi;
       d0[k] = xi >> 14; d1[k] = (xi >> 7) & 127; d2[k] = xi & 127;
     }
-    sx += __shfl_xor(sx, 1, 64); sx += __shfl_xor(sx, 2, 64);
+    sx += __float_as_int(quad_x1(__int_as_float(sx))); sx += __float_as_int(quad_x2(__int_as_float(sx)));
     if (live) {
       const uint32_t blk = i >> 2, j = i & 3u;
       uint8_t* bp = xs + (size_t)blk * 128u;
@@ -191,10 +213,9 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
     v[0] = v0.x; v[1] = v0.y; v[2] = v0.z; v[3] = v0.w; v[4] = v1.x; v[5] = v1.y; v[6] = v1.z; v[7] = v1.w;
   };
   auto block_sum = [&](float v) {     // sum over the workgroup, same value in every thread
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    v = wave_sum_to_lane63(v);
     __syncthreads();                  // red_f may still be read from the previous use
-    if (lane == 0) red_f[wave] = v;
+    if (lane == 63u) red_f[wave] = v;
     __syncthreads();
     float t = 0.f;
     for (uint32_t w = 0; w < nwav; w++) t += red_f[w];
@@ -343,8 +364,11 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
   TR(5);
   uint32_t nib = 0x0F0F0F0Fu;
   asm volatile("" : "+s"(nib));             // opaque, so it stays in a register instead of a literal per use
-  const uint32_t dig = l < 3u ? l : 0u;     // lane 3 of a block repeats digit 0, its result row is unused
-  const uint32_t x_off0 = chunk_off(2u * dig, bcol), x_off1 = chunk_off(2u * dig + 1u, bcol), p_off = chunk_off(6u, bcol);
+  // Lanes 0..2 of a block read digit 0..2 (operand rows 0..2); the fourth operand row is not needed, so lane 3 reads
+  // the block's parameters instead and hands them to its three neighbours through the data-parallel crossbar:
+  // two LDS reads per lane and block where digits plus parameters would be three.
+  const uint32_t x_off0 = l < 3u ? chunk_off(2u * l, bcol) : chunk_off(6u, bcol);
+  const uint32_t x_off1 = l < 3u ? chunk_off(2u * l + 1u, bcol) : chunk_off(6u, bcol);
   float acc = 0.f;
   float best_v = NEG_FLT_MAX;
   uint32_t best_i = INVALID_IDX;
@@ -368,7 +392,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       }
     }
     const uint8_t* base = xs + (size_t)(chunk * 64u + bcol) * 128u;
-    uint4 xa[MF_U], xb[MF_U], prm[MF_U];
+    uint4 xa[MF_U], xb[MF_U];
     bool valid[MF_U];
     i4_t d[MF_U];
 #pragma unroll
@@ -380,7 +404,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
         valid[u] = blk_raw < nblk;
         bp = xs + (size_t)min(blk_raw, nblk - 1u) * 128u;
       }
-      xa[u] = *(const uint4*)(bp + x_off0); xb[u] = *(const uint4*)(bp + x_off1); prm[u] = *(const uint4*)(bp + p_off);
+      xa[u] = *(const uint4*)(bp + x_off0); xb[u] = *(const uint4*)(bp + x_off1);
       d[u] = (i4_t){0, 0, 0, 0};
     }
     // eight dependent matrix instructions per block; the four blocks of a step are interleaved so that
@@ -398,11 +422,16 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       // |d0| <= 15*128*32, so the recombination stays below 2^31
       const int sq = d[u][0] * 16384 + d[u][1] * 128 + d[u][2];
       // a block past the end of the row (ragged K) was clamped to a valid address: drop what it read
-      const float fsb = valid[u] ? __uint_as_float(prm[u].y) : 0.f, sxb = valid[u] ? __uint_as_float(prm[u].z) : 0.f;
+      // lane 3's first read is {zero-point term, 2^-e, block sum}: quad_perm [3,3,3,3]
+      const uint32_t prm_x = quad_b3(xa[u].x), prm_y = quad_b3(xa[u].y);
+
+      const float fsb = valid[u] ? __uint_as_float(prm_y) : 0.f;
       if (B16) {
         const float sc = valid[u] ? __half2float(R.h[u]) : 0.f;
-        acc = fmaf(sc, (float)(sq - (int)prm[u].x) * fsb, acc);
+        acc = fmaf(sc, (float)(sq - (int)prm_x) * fsb, acc);
       } else {
+        const uint32_t prm_z = quad_b3(xa[u].z);
+        const float sxb = valid[u] ? __uint_as_float(prm_z) : 0.f;
         const float sc = valid[u] ? R.p[u].x : 0.f, zp = valid[u] ? R.p[u].y : 0.f;
         acc = fmaf(sc, (float)sq * fsb, fmaf(zp, sxb, acc));
       }
