@@ -17,12 +17,6 @@ extern "C" int map_matmul_t_dev(uint32_t map_id, uint32_t ha, uint32_t hb, uint3
 
 namespace adamah {
 
-#ifdef ADAMAH_TRACE
-__device__ unsigned long long g_trace_attn[64];
-#define TRA(i) do { if (threadIdx.x == 0 && blockIdx.x == 0 && blockIdx.y == 0) g_trace_attn[i] = wall_clock64(); } while (0)
-#else
-#define TRA(i) do {} while (0)
-#endif
 
 __device__ __forceinline__ float ld(const float* p, uint64_t i) { return p[i]; }
 __device__ __forceinline__ float ld(const __half* p, uint64_t i) { return __half2float(p[i]); }
@@ -265,7 +259,6 @@ k_attn_fused(const float* data, float* out, const __half* kv, uint64_t kv_shift,
              float cap, uint32_t n_splits, uint32_t chunk, float* partial) {
   constexpr int VEC = 8;
   constexpr uint32_t lpr = LPR;
-  TRA(0);
   __shared__ float p[ATT_CHUNK];
   __shared__ float red[4];
   __shared__ float osum[2048];
@@ -283,7 +276,6 @@ k_attn_fused(const float* data, float* out, const __half* kv, uint64_t kv_shift,
 #pragma unroll
       for (int j = 0; j < VEC; j++) q[i][j] = v < nvec ? data[a + (uint64_t)v * VEC + j] : 0.f;
     }
-    TRA(1);
     if (lpr >= nvec) {
       // every lane holds one 16-byte slice of a row (head dims up to 512): sixteen row groups per trip,
       // all loads issued before the first is used; rows past the chunk are clamped and dropped
@@ -366,9 +358,7 @@ k_attn_fused(const float* data, float* out, const __half* kv, uint64_t kv_shift,
       }
     }
   }
-  TRA(2);
   __syncthreads();
-  TRA(3);
   float mx = -9.99999968e+37f;
   for (uint32_t t = tid; t < nt; t += 256u) {
     const float v = prep(p[t], scale, cap);
@@ -390,7 +380,6 @@ k_attn_fused(const float* data, float* out, const __half* kv, uint64_t kv_shift,
   if (lane == 0) red[wave] = sum;
   __syncthreads();
   sum = (red[0] + red[1]) + (red[2] + red[3]);
-  TRA(4);
   // values: vlpr lanes cover one V row, 256/vlpr rows in flight per sweep; row-slot partials meet in LDS
   const uint32_t vlpr = value_dim / VEC, slots = 256u / vlpr, sub = tid % vlpr, slot = tid / vlpr;
   float acc[VEC];
@@ -420,7 +409,6 @@ k_attn_fused(const float* data, float* out, const __half* kv, uint64_t kv_shift,
       }
     }
   }
-  TRA(5);
   const uint32_t fit = 2048u / value_dim;
   float o = 0.f;
   for (uint32_t s0 = 0; s0 < slots; s0 += fit) {
@@ -442,7 +430,6 @@ k_attn_fused(const float* data, float* out, const __half* kv, uint64_t kv_shift,
     pp[0] = mx;
     pp[1] = sum;
   }
-  TRA(6);
 }
 
 // Merge the split partials of one op: M = max m_s, w_s = e^(m_s-M), L = sum l_s w_s,
@@ -672,12 +659,6 @@ int launch_attn_combine_dev(Map* m, const float* partial, const uint32_t* lo_dev
 
 }  // namespace adamah
 
-#ifdef ADAMAH_TRACE
-extern "C" int adamah_hip_trace_read_attn(unsigned long long* out) {
-  hipStreamSynchronize(adamah::g.stream);
-  return hipMemcpyFromSymbol(out, HIP_SYMBOL(adamah::g_trace_attn), 64 * sizeof(unsigned long long)) == hipSuccess ? 0 : -1;
-}
-#endif
 
 using namespace adamah;
 

@@ -27,6 +27,7 @@ struct AttnDecodeArgs {
   uint32_t fold_floats;         // "few": at most this many partial floats
 };
 bool launch_attn_decode(const AttnDecodeArgs& a, AttnPartials* ap, bool* left, int* rc);
-int tuning(const char* name, int dflt);   // integer knob from the environment (gemv_q.hip)
+int tuning(const char* name, int dflt);   // behaviour switch from the environment (gemv_q.hip)
+int knob(const char* name, int dflt);     // launch-shape number, fixed unless built with -DADAMAH_TUNING
 
 }  // namespace adamah

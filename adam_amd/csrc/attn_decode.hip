@@ -34,12 +34,6 @@ typedef _Float16 h4a_t __attribute__((ext_vector_type(4)));
 typedef float f4a_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u2a_t __attribute__((ext_vector_type(2)));
 
-#ifdef ADAMAH_TRACE
-__device__ unsigned long long g_trace_attd[64];
-#define TRD(i) do { if (threadIdx.x == 0 && blockIdx.x == 0 && blockIdx.y == 0) g_trace_attd[i] = wall_clock64(); } while (0)
-#else
-#define TRD(i) do {} while (0)
-#endif
 
 #define ATTD_NEG (-1.0e30f)
 #define ATTD_MAX_SPLITS 256u
@@ -78,7 +72,6 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
   __shared__ uint32_t hmax[G];         // per head: bits of max |q|
   __shared__ float qinv[G];            // per head: 1 / (power-of-two scale of the queries)
 
-  TRD(0);
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));   // scalar: row numbers below are too
   const uint32_t c = lane & 15u, kc = lane >> 4;
@@ -151,7 +144,6 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
     }
     __syncthreads();
   }
-  TRD(1);
   // after the matrix product lane (c, kc) holds heads 4kc..4kc+3 of tile row c
   float inv_s[4], m_run[4], l_run[4];
   bool hval[4];
@@ -185,7 +177,6 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
       s2 = __builtin_amdgcn_mfma_f32_16x16x16f16(qop[2 * i + 1][0][lane], __builtin_bit_cast(h4a_t, b1), s2, 0, 0, 0);
       s3 = __builtin_amdgcn_mfma_f32_16x16x16f16(qop[2 * i + 1][1][lane], __builtin_bit_cast(h4a_t, b1), s3, 0, 0, 0);
     }
-    TRD(3);
     const uint32_t row = rb + c;
     const bool rok = row < t1;
     float v[4], mt[4];
@@ -208,7 +199,6 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
         if (c == 0u) abuf[wave][4u * kc + r] = alpha;
       }
     }
-    TRD(4);
     __builtin_amdgcn_wave_barrier();
     // values: rescale the running sums, then the sixteen rows of the tile
 #pragma unroll
@@ -238,7 +228,6 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
     __builtin_amdgcn_wave_barrier();
   };
 
-  TRD(2);
   if (any) {
     if (PF) {
       while (true) {
@@ -262,7 +251,6 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
       }
     }
   }
-  TRD(5);
 
   // wave results to LDS: l summed over the 16 tile rows; each lane owns its dims of the output
 #pragma unroll
@@ -276,7 +264,6 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
     for (int r = 0; r < 4; r++)
       if (hval[r]) { mlbuf[wave][4u * kc + r][0] = m_run[r]; mlbuf[wave][4u * kc + r][1] = l_run[r]; }
   }
-  TRD(6);
   __syncthreads();
   for (uint32_t idx = tid; idx < (uint32_t)(G * D); idx += NT) {
     const uint32_t h = idx / D, d = idx % D;
@@ -298,7 +285,6 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
       if (d == 0u) { pp[0] = M; pp[1] = L; }
     }
   }
-  TRD(7);
 }
 
 template <int D, int NW, bool PF>
@@ -340,10 +326,10 @@ bool launch_attn_decode(const AttnDecodeArgs& a, AttnPartials* ap, bool* left, i
   // Slices of the sequence.  Short sequences (at most one 16-row tile per wave when the chip holds
   // `target` waves): workgroups of 8 waves, one tile each, no prefetch; longer ones: 4 waves and as
   // many tiles per wave as it takes.
-  const uint32_t target = (uint32_t)std::max(1, tuning("ADAMAH_ATTN_WAVES", 4 * g.n_cu));
+  const uint32_t target = (uint32_t)std::max(1, knob("ADAMAH_ATTN_WAVES", 4 * g.n_cu));
   const uint64_t tiles = (uint64_t)n_groups * cdiv(a.row_size, 16u);
   uint32_t nw = (tiles <= target && G * D <= 1024u) ? 8u : 4u;
-  nw = (uint32_t)tuning("ADAMAH_ATTN_NW", (int)nw) == 8u && G * D <= 1024u ? 8u : 4u;
+  nw = (uint32_t)knob("ADAMAH_ATTN_NW", (int)nw) == 8u && G * D <= 1024u ? 8u : 4u;
   const uint32_t step = nw * 16u;
   uint32_t chunk = step * std::max<uint32_t>(1u, cdiv(tiles, target));
   while (cdiv(a.row_size, chunk) > ATTD_MAX_SPLITS) chunk += step;
@@ -457,7 +443,7 @@ size_t launch_attn_batch(const std::vector<PendOp>& q, size_t i, int* rc) {
   }
   const uint32_t n_all = (uint32_t)(B * H), n_groups = n_all / G;
   // slices as for a single pair, sized for all the groups
-  const uint32_t target = (uint32_t)std::max(1, tuning("ADAMAH_ATTN_WAVES", 4 * g.n_cu));
+  const uint32_t target = (uint32_t)std::max(1, knob("ADAMAH_ATTN_WAVES", 4 * g.n_cu));
   const uint64_t tiles = (uint64_t)n_groups * cdiv(rows, 16u);
   uint32_t nw = (tiles <= target && G * D <= 1024u) ? 8u : 4u;
   const uint32_t step = nw * 16u;
@@ -500,9 +486,3 @@ size_t launch_attn_batch(const std::vector<PendOp>& q, size_t i, int* rc) {
 
 }  // namespace adamah
 
-#ifdef ADAMAH_TRACE
-extern "C" int adamah_hip_trace_read_attd(unsigned long long* out) {
-  hipStreamSynchronize(adamah::g.stream);
-  return hipMemcpyFromSymbol(out, HIP_SYMBOL(adamah::g_trace_attd), 64 * sizeof(unsigned long long)) == hipSuccess ? 0 : -1;
-}
-#endif

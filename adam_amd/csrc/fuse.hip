@@ -24,8 +24,7 @@
 namespace adamah {
 
 bool can_defer() {
-  static const int off = getenv("ADAMAH_NO_FUSE") ? atoi(getenv("ADAMAH_NO_FUSE")) : 0;
-  return g.batch_depth > 0 && g.no_defer == 0 && !off;
+  return g.batch_depth > 0 && g.no_defer == 0 && tuning("ADAMAH_NO_FUSE", 0) == 0;
 }
 
 bool res_scalar(uint32_t h, uint32_t* out) {

@@ -542,7 +542,7 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
   uint4* const xh = g_xh_buf;
   uint4* const xl = (uint4*)((uint8_t*)g_xh_buf + plane);
   if (!reuse) {
-    if (K <= 16384 && tuning("ADAMAH_ACT_REGS", 1) != 0) {
+    if (K <= 16384 && knob("ADAMAH_ACT_REGS", 1) != 0) {
       if (K <= 8192) k_act_f16_regs<1><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, la, M, K, g_scale_buf, xh, xl);
       else k_act_f16_regs<2><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, la, M, K, g_scale_buf, xh, xl);
     } else
@@ -554,14 +554,14 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
   if (mt <= 2) {
     // few activation rows: the K-split form, as many weight-row tiles per workgroup as still fill the chip
     uint32_t R = wgs(64, mt) >= want ? 4 : wgs(32, mt) >= want ? 2 : 1;
-    R = (uint32_t)tuning("ADAMAH_GEMM_R", (int)R);
+    R = (uint32_t)knob("ADAMAH_GEMM_R", (int)R);
     R = R >= 4 ? 4 : R >= 2 ? 2 : 1;
     if (q8 && R > 2) R = 2;   // a Q8 tile holds twice the registers
     dim3 grid(cdiv(N, 16 * R), cdiv(M, 16 * mt), n_ops);
     float* dst = out ? out : act;
     const uint32_t* lcd = out ? nullptr : lc;
     // eight waves where the matrix has too few weight rows for larger tiles (measured: no gain otherwise)
-    const uint32_t nwv = mt == 1 && !q8 ? (uint32_t)tuning("ADAMAH_GEMM_NWV", R == 1 ? 8 : 4) : 4u;
+    const uint32_t nwv = mt == 1 && !q8 ? (uint32_t)knob("ADAMAH_GEMM_NWV", R == 1 ? 8 : 4) : 4u;
 #define GK(T, RR, W, Q) k_gemm_q4_f16_ksplit<T, RR, W, Q><<<grid, 64 * W, 0, g.stream>>>(dst, mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, lb, lcd, g_scale_buf, M, K, N, sg)
     if (q8) {
       if (mt == 1) { if (R == 2) GK(1, 2, 4, true); else GK(1, 1, 4, true); }
@@ -583,8 +583,8 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
     else if (wgs(64, 8) >= want) R = 1;
     else mt = 4;
   }
-  if (mt == 8 && tuning("ADAMAH_GEMM_MT", 8) == 4) mt = 4;
-  R = (uint32_t)tuning("ADAMAH_GEMM_R", (int)R);
+  if (mt == 8 && knob("ADAMAH_GEMM_MT", 8) == 4) mt = 4;
+  R = (uint32_t)knob("ADAMAH_GEMM_R", (int)R);
   R = R >= 4 && mt == 4 ? 4 : R >= 2 ? 2 : 1;
   dim3 grid(cdiv(N, 64 * R), cdiv(M, 16 * mt), n_ops);
 #define GT(T, RR) k_gemm_q4_f16_tiled<T, RR><<<grid, 256, 0, g.stream>>>(act, mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, lb, lc, g_scale_buf, M, K, N, sg)

@@ -134,7 +134,8 @@ void gemm_act_mark(const void* buf, uint64_t a, uint32_t M, uint32_t K);
 // Second pass of the fused GEMV + argmax: best of the per-group partials, token id stored as float.
 int launch_argmax_pairs(const Map* ma, const uint32_t* lidx, const uint32_t* lval, const uint32_t* ldst,
                         uint32_t n_groups);
-int tuning(const char* name, int dflt);
+int tuning(const char* name, int dflt);   // behaviour switch, from the environment
+int knob(const char* name, int dflt);     // launch-shape number, fixed unless built with -DADAMAH_TUNING
 // Preconditions of the block kernels, checked against the host copies of the handles: group size 32,
 // K a multiple of 32, weight base block aligned, operands in range.  Returns the two element offsets.
 bool block_path_ok(const Map* ma, const Map* mw, uint32_t ha, uint32_t hb, uint32_t K, uint32_t N, uint64_t* a_out,

@@ -33,13 +33,6 @@ typedef float f4u_t __attribute__((ext_vector_type(4), aligned(4)));
 
 enum { MF_U = 4 };   // 16-byte blocks per lane and step
 
-#ifdef ADAMAH_TRACE
-__device__ unsigned long long g_trace[64];
-#define TR(i) do { if (threadIdx.x == 0 && (blockIdx.x == 0 || blockIdx.x == gridDim.x - 1)) \
-  g_trace[(blockIdx.x == 0 ? 0 : 16) + (i)] = wall_clock64(); } while (0)
-#else
-#define TR(i) do {} while (0)
-#endif
 
 // lane ^ 1 and lane ^ 2 within a quad (quad_perm [1,0,3,2] and [2,3,0,1]): a register move, no trip through LDS
 __device__ __forceinline__ float quad_x1(float v) {
@@ -86,7 +79,6 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
             const __half* __restrict__ d16, uint32_t a, uint32_t b_off, uint32_t c_out,
             const uint32_t* __restrict__ lidx, const uint32_t* __restrict__ lval, uint32_t K, uint32_t N,
             uint32_t rows_per_group, uint32_t n_groups, uint32_t ks, GemvFuse fz) {
-  TR(0);
   constexpr bool B16 = (FMT == FMT_Q4_B16);
   extern __shared__ uint4 smem_u4[];
   uint8_t* xs = (uint8_t*)smem_u4;                    // nblk * 128 bytes
@@ -311,9 +303,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
 #pragma unroll
         for (int k = 0; k < 8; k++) asm volatile("" ::"v"(rv[u][k]));
     }
-    TR(1);
     nrm1 = 1.0f / sqrtf(block_sum(ss) / (float)K + fz.p_eps);
-    TR(2);
     const float nrm = nrm1;
     if (PRO == PRO_NORM2) {
       // Every thread of this workgroup has consumed `res` (the reduction above ends in a barrier).
@@ -332,7 +322,6 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
           }
         }
       const float nrm2 = 1.0f / sqrtf(block_sum(ss2) / (float)K + fz.p_eps2);
-      TR(3);
 #pragma unroll
       for (uint32_t u = 0; u < PRO_WPT; u++)
         if (mine[u]) {
@@ -359,9 +348,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       }
     }
   }
-  TR(4);
   __syncthreads();
-  TR(5);
   uint32_t nib = 0x0F0F0F0Fu;
   asm volatile("" : "+s"(nib));             // opaque, so it stays in a register instead of a literal per use
   // Lanes 0..2 of a block read digit 0..2 (operand rows 0..2); the fourth operand row is not needed, so lane 3 reads
@@ -510,7 +497,6 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
         compute(B, row_b, ch_b, seg_end);
       }
     }
-    TR(6);
     if (EPI == EPI_STORE && ks > 1u) {
       // the ks waves of a bundle meet: the first of them adds the shares in wave order and stores
       if (!(first < seg_end)) part[wave * 64u + lane] = 0.f;
@@ -558,9 +544,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
     best_v = NEG_FLT_MAX; best_i = INVALID_IDX;
     if (!more) break;
   }
-  TR(7);
   finish_norm2();
-  TR(8);
 }
 
 // ---- host side -----------------------------------------------------------------------------------
@@ -592,7 +576,7 @@ static int launch_mfma(int fmt, uint32_t grid, uint32_t threads, const Map* ma, 
                        uint32_t n_groups, uint32_t ks, const GemvFuse* fzp, float* out = nullptr) {
   GemvFuse fz = {};
   if (fzp) fz = *fzp;
-  const int xf = tuning("ADAMAH_MFMA_XFIRST", -1);
+  const int xf = knob("ADAMAH_MFMA_XFIRST", -1);
   fz.x_first = xf < 0 ? 1u : (uint32_t)(xf != 0);
 #define MP(P) launch_mfma_p<EPI, P>(fmt, grid, threads, ma, mw, a, b, c, lidx, lval, K, N, rpg, n_groups, ks, fz, out)
   switch (fz.pro) {
@@ -612,9 +596,9 @@ static void mfma_shape(uint32_t K, uint32_t units, uint32_t* grid, uint32_t* thr
   // largest workgroup (16, 8 or 4 waves) that still leaves a workgroup for every CU
   uint32_t waves = 16;
   while (waves > 4 && cdiv(units, waves) < (uint32_t)g.n_cu) waves >>= 1;
-  waves = (uint32_t)tuning("ADAMAH_MFMA_WAVES", (int)waves);
+  waves = (uint32_t)knob("ADAMAH_MFMA_WAVES", (int)waves);
   waves = waves >= 16 ? 16 : waves >= 8 ? 8 : 4;
-  const uint32_t per_simd = (uint32_t)std::max(1, tuning("ADAMAH_MFMA_PERSIMD", 2));
+  const uint32_t per_simd = (uint32_t)std::max(1, knob("ADAMAH_MFMA_PERSIMD", 2));
   const size_t lds_fit = std::max<size_t>(1, (160 * 1024) / (mfma_smem(K) + 256));
   const uint32_t wg_per_cu = (uint32_t)std::max<size_t>(1, std::min<size_t>(lds_fit, (size_t)per_simd * 4 / waves));
   *threads = waves * 64;
@@ -627,10 +611,10 @@ static void mfma_shape(uint32_t K, uint32_t units, uint32_t* grid, uint32_t* thr
 // flight from the start: such launches are bound by one trip to memory, not by arithmetic.
 static uint32_t mfma_ksplit(uint32_t K, uint32_t N, bool paired_rows) {
   const uint32_t C = cdiv(K, 2048u), n_q = cdiv(N, 4u);
-  const uint32_t want = (uint32_t)std::max(1, tuning("ADAMAH_MFMA_KSPLIT_WAVES", 4096));
+  const uint32_t want = (uint32_t)std::max(1, knob("ADAMAH_MFMA_KSPLIT_WAVES", 4096));
   uint32_t ks = 1;
   while (ks < 4u && ks * 2u <= C && n_q * ks * 2u <= want) ks *= 2u;
-  const int forced = tuning("ADAMAH_MFMA_KS", 0);
+  const int forced = knob("ADAMAH_MFMA_KS", 0);
   if (forced == 1 || forced == 2 || forced == 4) ks = std::min<uint32_t>((uint32_t)forced, std::max(1u, C));
   if (ks == 3u) ks = 2u;
   return paired_rows ? 1u : ks;
@@ -647,7 +631,7 @@ static void mfma_store_shape(uint32_t K, uint32_t N, uint32_t ks, uint32_t* grid
       const uint32_t cost = cdiv(cdiv(n_q * ks, w), (uint32_t)g.n_cu) * w;
       if (cost <= best_cost) { best_cost = cost; best_w = w; }
     }
-    const int fw = tuning("ADAMAH_MFMA_WAVES", 0);
+    const int fw = knob("ADAMAH_MFMA_WAVES", 0);
     if (fw > 0) best_w = fw >= 16 ? 16 : fw >= 8 ? 8 : 4;
     *threads = best_w * 64u;
     *grid = cdiv(n_q, best_w / ks);
@@ -681,9 +665,3 @@ int launch_mfma_argmax(int fmt, const Map* ma, const Map* mw, uint32_t a, uint32
 
 }  // namespace adamah
 
-#ifdef ADAMAH_TRACE
-extern "C" int adamah_hip_trace_read(unsigned long long* out) {
-  hipStreamSynchronize(adamah::g.stream);
-  return hipMemcpyFromSymbol(out, HIP_SYMBOL(adamah::g_trace), 64 * sizeof(unsigned long long)) == hipSuccess ? 0 : -1;
-}
-#endif

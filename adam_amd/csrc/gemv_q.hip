@@ -438,9 +438,22 @@ int fmt_of(const Map* mw, uint64_t b, uint64_t n_w) {
   return q4 ? (b16 ? FMT_Q4_B16 : FMT_Q4_AFF) : (b16 ? FMT_Q8_B16 : FMT_Q8_AFF);
 }
 
+// Behaviour switches of the library (each selects between code paths that the parity tests run both ways):
+// read from the environment at every call, so a test can flip one between two ops.
 int tuning(const char* name, int dflt) {
   const char* v = getenv(name);
   return v ? atoi(v) : dflt;
+}
+// Launch-shape numbers (waves per workgroup, rows per pass, ...): fixed in the library as built; a build with
+// -DADAMAH_TUNING reads them from the environment for sweeps.
+int knob(const char* name, int dflt) {
+#ifdef ADAMAH_TUNING
+  const char* v = getenv(name);
+  return v ? atoi(v) : dflt;
+#else
+  (void)name;
+  return dflt;
+#endif
 }
 
 template <int EPI>
@@ -449,7 +462,7 @@ static int launch_block(int fmt, const Map* ma, const Map* mw, const uint32_t* l
                         uint32_t rows_per_group) {
   const uint32_t n_groups = cdiv(N, rows_per_group);
   const size_t smem = (size_t)K * 4 + (size_t)(K >> 5) * 4;
-  const uint32_t per_cu = (uint32_t)tuning("ADAMAH_GEMV_PERCU", smem > 40000 ? 2 : 4);
+  const uint32_t per_cu = (uint32_t)knob("ADAMAH_GEMV_PERCU", smem > 40000 ? 2 : 4);
   const uint32_t grid = std::min<uint32_t>(n_groups, (uint32_t)g.n_cu * per_cu);
   float* act = (float*)ma->buf;
 #define LAUNCH(F)                                                                                              \
@@ -535,12 +548,12 @@ int op_matmul_t_xq(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t h
     if (impl == 1) {
       const uint32_t ks = K <= 4096 ? 1 : K <= 8192 ? 2 : 4;
       const uint32_t step = (4 / ks) * 4;                       // rows one workgroup pass covers
-      const uint32_t passes = (uint32_t)tuning("ADAMAH_GEMV_PASSES", 2);
+      const uint32_t passes = (uint32_t)knob("ADAMAH_GEMV_PASSES", 2);
       return launch_regx<EPI_STORE>(fmt, ma, mw, la, lb, lc, nullptr, nullptr, K, N, step * std::max(1u, passes));
     }
     if ((uint64_t)K * 4 + (K >> 5) * 4 > 64000) goto generic;
     return launch_block<EPI_STORE>(fmt, ma, mw, la, lb, lc, nullptr, nullptr, K, N,
-                                   (uint32_t)tuning("ADAMAH_GEMV_RPG", 16));
+                                   (uint32_t)knob("ADAMAH_GEMV_RPG", 16));
   }
   // several activation rows over Q4_0 blocks: fp16 matrix-core GEMM
   // (Q8_0 blocks: up to 32 rows)

@@ -71,7 +71,6 @@ class DecodeEngine:
     Q4_GROUP = 32
     SAMPLE_TOPK_MAX = 64       # reference engine.py:118
     SAMPLE_REPEAT_MAX = 64     # reference engine.py:120
-    SAMPLE_TOPK_MAX = 64
     SAMPLE_APPROX_SHORTLIST_MAX = 256
 
     def __init__(self, gpu, cfg, tensors, A=None, kv_cap=1024, kv_fp16=False,

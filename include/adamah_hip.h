@@ -69,6 +69,9 @@ int map_set_qparams(uint32_t map_id, const float* scales, const float* zero_poin
                     uint32_t n_groups);                       /* adamah.c:4621 */
 
 /* ---- host <-> map ------------------------------------------------------------------------- */
+/* The three scatters and map_gather are `int` in adamah.c; the reference's binding reads them as 64-bit
+ * tickets (adamah/__init__.py:578, :586, :597, :608 set restype c_uint64), which is what is declared here:
+ * 0 on success. */
 uint64_t map_scatter(uint32_t map_id, const uint32_t* locs, const void* data, uint32_t n_locs); /* adamah.c:3087 */
 uint64_t map_scatter_contiguous(uint32_t map_id, uint32_t start_pack, const void* data,
                                 uint32_t n_locs);             /* adamah.c:2896 */
@@ -254,15 +257,18 @@ int adamah_matvec_topk_t_xq4_noalloc_dev(uint32_t map_act, uint32_t map_wt, uint
                                          uint32_t penalty_ids, uint32_t locs_idx_dst, uint32_t locs_val_dst,
                                          uint32_t K, uint32_t N, uint32_t k, uint32_t n_penalty,
                                          float repeat_penalty, uint32_t rows_per_group);
-/* HIP-event stopwatch on the library's stream (benchmarks). begin: 0 on success; end: ms or <0. */
+/* ---- measurement and test helpers: not part of the op surface ------------------------------------
+ * Nothing a model engine calls.  bench.py times launches with the stopwatch and calibrates profiler counters
+ * with the probe; the parity tests read back what the kernels see through the other two. */
+/* HIP-event stopwatch on the library's stream. begin: 0 on success; end: ms or <0. */
 int adamah_hip_timer_begin(void);
 float adamah_hip_timer_end(void);
-/* Dequantise elements [start, start+count) of a Q4/Q8 map with the GEMV kernels' unpack code. */
-int adamah_hip_debug_dequant(uint32_t map_id, uint64_t start, uint64_t count, float* out);
 /* Streaming calibration: average microseconds per launch of a plain read (mode 0) or copy (mode 1)
  * of bytes_per_launch bytes, walking a pool_bytes buffer; negative = error code. */
 float adamah_hip_stream_probe(uint64_t bytes_per_launch, uint64_t pool_bytes, uint32_t mode, uint32_t wg_per_cu,
                               uint32_t launches);
+/* Dequantise elements [start, start+count) of a Q4/Q8 map with the GEMV kernels' unpack code. */
+int adamah_hip_debug_dequant(uint32_t map_id, uint64_t start, uint64_t count, float* out);
 /* 0 = affine qparams only, 1 = fp16-scale block plane in use for the whole map, <0 = error. */
 int adamah_hip_map_layout(uint32_t map_id);
 

@@ -663,6 +663,18 @@ class NumpyAdamah:
             self._mm(fn, ma, w, self._locs(fn, locs_a_handle, n_ops), self._locs(fn, locs_b_handle, n_ops),
                      self._locs(fn, locs_c_handle, n_ops), M, K, N, n_ops, True)
 
+    def map_matmul_x_dev(self, map_act, map_wt, locs_a_handle, locs_b_handle, locs_c_handle, M, K, N, n_ops=1):
+        """shaders/src/f32/map_matmul_x.comp:16-32: C[M,N] = A[M,K] . B[K,N], A and C in map_act, B row-major
+        in the f32 map map_wt, bases locs[op]."""
+        self.op_count += 1
+        fn = "map_matmul_x_dev"
+        ma = self._map(fn, map_act, DTYPE_F32); mw = self._map(fn, map_wt, DTYPE_F32)
+        def w(b, cnt):
+            self._chk(fn, mw, b, b + cnt); return mw.data[b:b + cnt]
+        if n_ops and N:
+            self._mm(fn, ma, w, self._locs(fn, locs_a_handle, n_ops), self._locs(fn, locs_b_handle, n_ops),
+                     self._locs(fn, locs_c_handle, n_ops), M, K, N, n_ops, False)
+
     def map_row_gather_xq8_dev(self, map_act, map_wt, src_base, dst_base, row_idx, row_size, scale=1.0):
         """shaders/src/f32/map_row_gather_xq8.comp: dst[e] = deq(src_base + row*row_size + e) * scale."""
         self.op_count += 1

@@ -297,3 +297,31 @@ def test_gather_dev_results_stop_consuming_handles(hip):
     assert 0 not in ids and len(ids) <= 4200
     last = hip.map_gather_dev(0, locs[2], n)[0]
     assert np.array_equal(hip.download_dev(last, n), np.arange(2 * n, 3 * n, dtype=np.float32))
+
+
+@pytest.mark.parametrize("M,K,N,n_ops", [(1, 256, 300, 1), (3, 70, 33, 2), (1, 4096, 512, 1)])
+def test_plain_float_matmuls(hip, M, K, N, n_ops):
+    """map_matmul_dev, map_matmul_t_x_dev and map_matmul_x_dev (float32 operands; the second and third read B
+    from another map -- the path a model with float weight matrices takes) against the oracle."""
+    rng = np.random.default_rng(M + K + N)
+    Aop = rng.standard_normal((n_ops, M, K)).astype(np.float32)
+    B = rng.standard_normal((n_ops, K, N)).astype(np.float32)
+    a_sz, b_sz, c_sz = M * K, K * N, M * N
+    a0, b0, c0 = 0, n_ops * a_sz + 3, n_ops * (a_sz + b_sz) + 7
+    out = {}
+    for name, g in (("hip", hip), ("oracle", oracle.init())):
+        note(f"plain matmuls {M}x{K}x{N} ops={n_ops} on {name}")
+        f32map(g, 0, c0 + 3 * n_ops * c_sz)
+        put(g, 0, a0, Aop); put(g, 0, b0, B)
+        f32map(g, 3, 2 * n_ops * b_sz + 8)
+        put(g, 3, 4, B); put(g, 3, 4 + n_ops * b_sz, B.transpose(0, 2, 1))
+        la = up(g, a0 + np.arange(n_ops) * a_sz)
+        lc = [up(g, c0 + v * n_ops * c_sz + np.arange(n_ops) * c_sz) for v in range(3)]
+        g.map_matmul_dev(0, la, up(g, b0 + np.arange(n_ops) * b_sz), lc[0], M, K, N, n_ops)
+        g.map_matmul_x_dev(0, 3, la, up(g, 4 + np.arange(n_ops) * b_sz), lc[1], M, K, N, n_ops)
+        g.map_matmul_t_x_dev(0, 3, la, up(g, 4 + n_ops * b_sz + np.arange(n_ops) * b_sz), lc[2], M, K, N, n_ops)
+        out[name] = read(g, 0, c0, 3 * n_ops * c_sz).reshape(3, -1)
+    want = np.stack([Aop[o].astype(np.float64) @ B[o].astype(np.float64) for o in range(n_ops)]).reshape(-1)
+    for v in range(3):
+        assert rel_l2(out["hip"][v], out["oracle"][v]) < 1e-5
+        assert rel_l2(out["hip"][v], want) < 1e-5

@@ -505,3 +505,91 @@ def test_fused_projections_equal_their_separate_dot_products():
     assert np.allclose(read(g, 0, K + 16, 4), exp, rtol=1e-5)
     with pytest.raises(RuntimeError):
         g.map_fused_qkv_t_xq4_dev(0, 1, up(g, [0]), up(g, [0]), 424242, up(g, [0]), up(g, [K]), up(g, [K]), up(g, [K]), K, 1, 0, 0)
+
+
+# ---------------------------------------------------------------- ops off the decode path: closed forms
+def test_plain_matmuls_on_integer_matrices_with_distinct_shapes():
+    """map_matmul_dev (B as [K, N]), map_matmul_t_x_dev (B as [N, K] in a second map) and map_matmul_x_dev (B as
+    [K, N] in a second map) on small integer matrices with M, K, N all different and several ops: the products
+    are exact in float32, and a transposed operand, a swapped dimension or a wrong base shows up as a mismatch."""
+    rng = np.random.default_rng(21)
+    M, K, N, n_ops = 3, 5, 7, 2
+    Aop = rng.integers(-4, 5, (n_ops, M, K)).astype(np.float32)
+    Bkn = rng.integers(-4, 5, (n_ops, K, N)).astype(np.float32)
+    want = np.stack([Aop[o].astype(np.int64) @ Bkn[o].astype(np.int64) for o in range(n_ops)]).astype(np.float32)
+    g = oracle.init()
+    a_sz, b_sz, c_sz = M * K, K * N, M * N
+    a0, b0, c0 = 0, n_ops * a_sz + 3, n_ops * (a_sz + b_sz) + 11
+    f32map(g, 0, c0 + n_ops * c_sz + 4)
+    g.scatter(0, np.arange(a0, a0 + n_ops * a_sz, dtype=np.uint32), Aop.reshape(-1))
+    g.scatter(0, np.arange(b0, b0 + n_ops * b_sz, dtype=np.uint32), Bkn.reshape(-1))
+    la, lb, lc = (up(g, base + np.arange(n_ops) * sz) for base, sz in ((a0, a_sz), (b0, b_sz), (c0, c_sz)))
+    g.map_matmul_dev(0, la, lb, lc, M, K, N, n_ops)
+    assert np.array_equal(read(g, 0, c0, n_ops * c_sz), want.reshape(-1))
+    # weights in a second f32 map: [K, N] for map_matmul_x_dev, [N, K] for map_matmul_t_x_dev
+    f32map(g, 3, 2 * n_ops * b_sz + 5)
+    g.scatter(3, np.arange(2, 2 + n_ops * b_sz, dtype=np.uint32), Bkn.reshape(-1))
+    g.scatter(3, np.arange(2 + n_ops * b_sz, 2 + 2 * n_ops * b_sz, dtype=np.uint32), Bkn.transpose(0, 2, 1).reshape(-1))
+    for fn, base in ((g.map_matmul_x_dev, 2), (g.map_matmul_t_x_dev, 2 + n_ops * b_sz)):
+        g.scatter(0, np.arange(c0, c0 + n_ops * c_sz, dtype=np.uint32), np.zeros(n_ops * c_sz, np.float32))
+        fn(0, 3, la, up(g, base + np.arange(n_ops) * b_sz), lc, M, K, N, n_ops)
+        assert np.array_equal(read(g, 0, c0, n_ops * c_sz), want.reshape(-1))
+
+
+def test_fma_on_exact_values():
+    g = oracle.init()
+    a = np.array([1.5, -2.0, 0.25, 3.0], np.float32); b = np.array([4.0, 0.5, -8.0, 0.0], np.float32)
+    c = np.array([0.5, 1.0, 1.0, -7.0], np.float32)
+    f32map(g, 0, 20, np.concatenate([a, b, c]))
+    g.map_fma_dev(0, up(g, np.arange(4)), up(g, 4 + np.arange(4)), up(g, 8 + np.arange(4)), up(g, [15, 14, 13, 12]), 4)
+    assert read(g, 0, 12, 4).tolist() == [-7.0, -1.0, 0.0, 6.5]          # a*b + c, scattered in reverse
+
+
+def test_row_softmax_closed_forms():
+    """Equal entries -> 1/n; entries ln(1..n) -> k / (n(n+1)/2); a constant shift changes nothing; the row base is
+    loc * row_size (not an absolute offset)."""
+    g = oracle.init()
+    n = 8
+    rows = np.stack([np.full(n, 3.25), np.log(np.arange(1, n + 1)), np.log(np.arange(1, n + 1)) + 100.0]).astype(np.float32)
+    f32map(g, 0, 8 * n, np.concatenate([np.zeros(n), rows.reshape(-1)]))          # rows 1, 2, 3 of size n
+    g.map_softmax_dev(0, up(g, [1, 2, 3]), up(g, [5, 6, 7]), n, 3)
+    out = read(g, 0, 5 * n, 3 * n).reshape(3, n)
+    assert np.allclose(out[0], 1.0 / n, rtol=1e-6)
+    tri = np.arange(1, n + 1) / (n * (n + 1) / 2)
+    assert np.allclose(out[1], tri, rtol=1e-5) and np.allclose(out[2], tri, rtol=1e-4)
+    assert np.allclose(out.sum(axis=1), 1.0, rtol=1e-6)
+
+
+def test_layernorm_closed_forms():
+    """A row a*k + b (k = 0..d-1) has mean b + a(d-1)/2 and variance a^2 (d^2-1)/12, so with gamma = 1, beta = 0
+    the result is (k - (d-1)/2) / sqrt((d^2-1)/12) whatever a > 0 and b are; gamma and beta then scale and shift
+    per element; source and destination bases are loc * dim, gamma / beta bases absolute."""
+    g = oracle.init()
+    d = 16
+    k = np.arange(d)
+    unit = (k - (d - 1) / 2) / np.sqrt((d * d - 1) / 12)
+    rows = np.stack([3.0 * k + 7.0, 0.5 * k - 2.0]).astype(np.float32)
+    gamma = np.linspace(0.5, 2.0, d).astype(np.float32); beta = np.linspace(-1.0, 1.0, d).astype(np.float32)
+    f32map(g, 0, 8 * d, np.concatenate([rows.reshape(-1), np.ones(d), np.zeros(d), gamma, beta]))
+    ones, zeros, gm, bt = 2 * d, 3 * d, 4 * d, 5 * d
+    g.map_layernorm_dev(0, up(g, [0, 1]), up(g, [6, 7]), up(g, [ones, gm]), up(g, [zeros, bt]), d, 0.0, 2)
+    out = read(g, 0, 6 * d, 2 * d).reshape(2, d)
+    assert np.allclose(out[0], unit, atol=2e-6)
+    assert np.allclose(out[1], unit * gamma + beta, atol=4e-6)
+    # eps enters under the root: a constant row gives beta exactly, whatever eps > 0
+    g.scatter(0, np.arange(0, d, dtype=np.uint32), np.full(d, 4.0, np.float32))
+    g.map_layernorm_dev(0, up(g, [0]), up(g, [6]), up(g, [gm]), up(g, [bt]), d, 1e-5, 1)
+    assert np.array_equal(read(g, 0, 6 * d, d), beta)
+
+
+def test_reduce_over_packs():
+    """Per loc, the pack's sum / max / min (op 0 / 1 / 2); source base is loc * pack_size, destination a
+    single element offset."""
+    g = oracle.init()
+    g.set_dtype(A.DTYPE_F32); g.map_create(0, 4, 6)
+    vals = np.array([[1, 2, 3, 4], [-5, 0.5, 7, -1], [2, 2, 2, 2]], np.float32)
+    g.scatter(0, np.array([0, 1, 2], np.uint32), vals.reshape(-1))
+    for op, want in ((0, [10.0, 1.5, 8.0]), (1, [4.0, 7.0, 2.0]), (2, [1.0, -5.0, 2.0])):
+        g.map_reduce_dev(0, op, up(g, [0, 1, 2]), up(g, [20, 21, 23]), 3)
+        got = g.gather(0, np.array([5], np.uint32)).view(np.float32)      # pack 5 = elements 20..23
+        assert [got[0], got[1], got[3]] == want
