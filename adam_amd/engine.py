@@ -393,6 +393,11 @@ class DecodeEngine:
                 sc[g0:g0 + s.size] = s; zp[g0:g0 + z.size] = z
             g.set_qparams(mid, sc, zp)
             for n in names:
+                if t[n].kind == 'q4_req':      # float values: the map's own quantiser makes the codes (reference engine.py:1086-1096)
+                    data = t[n].data
+                    for b in range(0, data.size, chunk):
+                        g.scatter_contiguous(mid, self._off[n] + b, data[b:b + chunk])
+                    continue
                 codes = t[n].codes
                 for b in range(0, codes.size, chunk):
                     part = codes[b:b + chunk]

@@ -14,20 +14,32 @@ to that form:
         128 bytes of nibbles (per 64 weights: low nibbles = first 32, high = next 32);
         w = d sc q - dmin m      -> scale d sc, zero point -dmin m per sub-block
 
-Only the nibble ORDER changes (the map keeps weight i in nibble i % 2 of byte i / 2); codes, scales
-and minima are the file's own, so the device computes with exactly the values a ggml decoder yields.
-F32 / F16 tensors come back as float32 arrays.  Other ggml types raise NotImplementedError naming the
-tensor.
+  Q5_0  22 B / 32 weights: fp16 d, 32 high bits, 16 nibble bytes; w = d (q - 16)
+        -> 8-bit map: code sign(d) (q - 16) + 128, scale |d|, zero point -128 |d| (exact; reference
+        engine.py:1171-1179 keeps Q5_0 with Q8_0 in its 8-bit map)
+
+For these, only the ORDER of the codes changes (the map keeps weight i in nibble i % 2 of byte i / 2); codes,
+scales and minima are the file's own, so the device computes with exactly the values a ggml decoder yields.
+
+Types without a map form of their own -- Q6_K (210 B / 256 weights: w = d sc (q - 32), 6-bit q in low nibbles
+plus bit pairs, 16 int8 sub-block scales), F16, BF16 and F32 matrices -- are decoded to float32 and take the route
+the reference gives "all other types" (engine.py:585-589, :1063-1096): into the 4-bit map with scale =
+(max - min) / 15 and zero point = min per 32 weights, the codes made by the map's own quantiser when the floats
+are scattered into it.  That step loses precision by the reference's design; the parity target is the reference,
+so it is kept.  One-dimensional tensors (norm weights) stay float32.  Any other ggml type raises
+NotImplementedError naming the tensor.
 """
 import mmap
 import struct
 
 import numpy as np
 
-from .quant import from_gguf_q4_0, from_gguf_q8_0, from_gguf_q4_k
+from .quant import (from_gguf_q4_0, from_gguf_q8_0, from_gguf_q4_k, from_gguf_q5_0, decode_gguf_q6_k, decode_bf16,
+                    requantize_q4)
 
-GGML_F32, GGML_F16, GGML_Q4_0, GGML_Q8_0, GGML_Q4_K = 0, 1, 2, 8, 12
-_BLOCK = {GGML_Q4_0: (32, 18), GGML_Q8_0: (32, 34), GGML_Q4_K: (256, 144)}   # weights, bytes per block
+GGML_F32, GGML_F16, GGML_Q4_0, GGML_Q5_0, GGML_Q8_0, GGML_Q4_K, GGML_Q6_K, GGML_BF16 = 0, 1, 2, 6, 8, 12, 14, 30
+# weights, bytes per block
+_BLOCK = {GGML_Q4_0: (32, 18), GGML_Q5_0: (32, 22), GGML_Q8_0: (32, 34), GGML_Q4_K: (256, 144), GGML_Q6_K: (256, 210)}
 _SCALAR = {0: "<B", 1: "<b", 2: "<H", 3: "<h", 4: "<I", 5: "<i", 6: "<f", 7: "<?", 10: "<Q", 11: "<q", 12: "<d"}
 _T_STRING, _T_ARRAY = 8, 9
 
@@ -110,7 +122,7 @@ class GGUFFile:
             nbytes = n // per * size
         elif gtype == GGML_F32:
             nbytes = 4 * n
-        elif gtype == GGML_F16:
+        elif gtype in (GGML_F16, GGML_BF16):
             nbytes = 2 * n
         else:
             raise NotImplementedError(f"{name}: ggml type {gtype} is not supported")
@@ -120,19 +132,26 @@ class GGUFFile:
         return np.frombuffer(self._mm, dtype=np.uint8, count=nbytes, offset=lo)
 
     def tensor(self, name):
-        """float32 array (F32 / F16) or QTensor in map form (Q4_0, Q8_0, Q4_K)."""
+        """float32 array (F32 / F16 / BF16 / Q6_K, decoded) or QTensor in map form (Q4_0, Q8_0, Q4_K blocks as
+        they are; Q5_0 as signed 8-bit codes, adam/models/engine.py:1171-1179)."""
         shape, gtype, _ = self.tensors[name]
         raw = self.raw(name)
         if gtype == GGML_F32:
             return raw.view(np.float32).reshape(shape).copy()
         if gtype == GGML_F16:
             return raw.view(np.float16).astype(np.float32).reshape(shape)
+        if gtype == GGML_BF16:
+            return decode_bf16(raw, self.numel(name)).reshape(shape)
+        if gtype == GGML_Q6_K:
+            return decode_gguf_q6_k(raw, self.numel(name)).reshape(shape)
         if len(shape) != 2:
             shape = (int(np.prod(shape[:-1], dtype=np.int64)), shape[-1])
         if gtype == GGML_Q4_0:
             return from_gguf_q4_0(raw, shape)
         if gtype == GGML_Q8_0:
             return from_gguf_q8_0(raw, shape)
+        if gtype == GGML_Q5_0:
+            return from_gguf_q5_0(raw, shape)
         return from_gguf_q4_k(raw, shape)
 
 
@@ -208,13 +227,17 @@ def load_model(path):
     for name in f.tensors:
         if name.startswith("rope_freqs") or not name.endswith(".weight"):
             continue
-        t = f.tensor(name)
-        if isinstance(t, np.ndarray) and t.ndim == 2 and name != "token_embd.weight":
-            raise NotImplementedError(f"{name}: float matrices are not uploaded by the decode path")
-        out[name] = t
-    if "output.weight" in out:
+        out[name] = f.tensor(name)
+    untied = "output.weight" in out
+    for name, t in list(out.items()):
+        # Weight matrices whose type has no map form of its own (Q6_K, F16, BF16, F32) go to the 4-bit map as the
+        # reference sends them (adam/models/engine.py:585-589, :1063-1096): group minimum / maximum as qparams, the
+        # float values quantised by the device on arrival.  Row length must fill whole groups of 32.
+        if isinstance(t, np.ndarray) and t.ndim == 2 and not (untied and name == "token_embd.weight"):
+            if t.shape[1] % 32:
+                raise NotImplementedError(f"{name}: float matrix rows of {t.shape[1]} weights do not fill groups of 32")
+            out[name] = requantize_q4(t)
+    if untied:
         out["token_embd.weight"] = RowLookup(out["token_embd.weight"])
-    elif isinstance(out.get("token_embd.weight"), np.ndarray):
-        raise NotImplementedError("token_embd.weight: a tied float embedding matrix is not uploaded by the decode path")
     f.close()
     return cfg, out

@@ -88,7 +88,56 @@ def make_q4_k(rng, n_blocks):
     return b.tobytes()
 
 
+def make_q5_0(rng, n_blocks):
+    b = np.empty((n_blocks, 22), np.uint8)
+    d = rand_f16(rng, n_blocks)
+    d[::3] = -d[::3]                                   # negative scales occur in real files
+    if n_blocks > 4:
+        d[4] = 0
+    b[:, 0:2] = d.view(np.uint8).reshape(n_blocks, 2)
+    b[:, 2:] = rng.integers(0, 256, (n_blocks, 20), dtype=np.uint8)
+    return b.tobytes()
+
+
+def make_q6_k(rng, n_blocks):
+    b = np.empty((n_blocks, 210), np.uint8)
+    b[:, 0:208] = rng.integers(0, 256, (n_blocks, 208), dtype=np.uint8)     # every nibble, bit pair and int8 scale
+    b[:, 208:210] = rand_f16(rng, n_blocks, 0.00002, 0.0002).view(np.uint8).reshape(n_blocks, 2)
+    return b.tobytes()
+
+
 # ------------------------------------------------------------------ independent decoders (ggml formulation)
+def dec_q5_0(raw):
+    """w[j] = d * ((nibble j | bit j of qh << 4) - 16); nibbles: low halves are weights 0..15, high 16..31."""
+    out = []
+    for i in range(0, len(raw), 22):
+        d = np.frombuffer(raw[i:i + 2], np.float16)[0].astype(np.float32)
+        qh = struct.unpack("<I", raw[i + 2:i + 6])[0]
+        qs = raw[i + 6:i + 22]
+        for j in range(32):
+            nib = (qs[j] & 15) if j < 16 else (qs[j - 16] >> 4)
+            out.append(d * np.float32((nib | (((qh >> j) & 1) << 4)) - 16))
+    return np.array(out, np.float32)
+
+
+def dec_q6_k(raw):
+    """Per 128 weights: weight 32 j + l (j = 0..3, l = 0..31) has its low nibble in ql[l + 32 (j & 1)] (low half for
+    j < 2, high half else), its upper two bits at bit 2 j of qh[l], and the int8 scale 2 j + l // 16 of the half;
+    w = d * scale * (q - 32), left to right in float32."""
+    out = []
+    for i in range(0, len(raw), 210):
+        ql, qh = raw[i:i + 128], raw[i + 128:i + 192]
+        sc = np.frombuffer(raw[i + 192:i + 208], np.int8)
+        d = np.frombuffer(raw[i + 208:i + 210], np.float16)[0].astype(np.float32)
+        for half in range(2):
+            for j in range(4):
+                for l in range(32):
+                    byte = ql[64 * half + l + 32 * (j & 1)]
+                    low = (byte & 15) if j < 2 else (byte >> 4)
+                    q = low | (((qh[32 * half + l] >> (2 * j)) & 3) << 4)
+                    out.append(d * np.float32(sc[8 * half + 2 * j + l // 16]) * np.float32(q - 32))
+    return np.array(out, np.float32)
+
 def dec_q4_0(raw):
     out = []
     for i in range(0, len(raw), 18):
@@ -188,7 +237,7 @@ def test_rejects_bad_files(tmp_path):
     with pytest.raises(ValueError, match="not a GGUF"):
         gguf.GGUFFile(str(p))
     rng = np.random.default_rng(3)
-    write_gguf(p, {"general.architecture": "llama"}, [("x.weight", (2, 64), 14, b"\0" * 210)])     # Q6_K
+    write_gguf(p, {"general.architecture": "llama"}, [("x.weight", (2, 128), 10, b"\0" * 84)])     # Q2_K: not read
     f = gguf.GGUFFile(str(p))
     with pytest.raises(NotImplementedError, match="x.weight"):
         f.tensor("x.weight")
@@ -200,7 +249,18 @@ def test_rejects_bad_files(tmp_path):
     f.close()
 
 
-def _model_file(path, arch, rng):
+def _float_matrix(rng, gtype, n):
+    w = (rng.standard_normal(n) * 0.05).astype(np.float32)
+    if gtype == gguf.GGML_F16:
+        return w.astype(np.float16).tobytes()
+    if gtype == gguf.GGML_BF16:
+        return (w.view(np.uint32) >> 16).astype(np.uint16).tobytes()
+    return w.tobytes()
+
+
+def _model_file(path, arch, rng, mixed=False):
+    """mixed: the tensor types of a Q4_K_M-style file and of float exports -- Q6_K for V, down and the output /
+    tied embedding matrix, Q5_0 for K, F16 / BF16 / F32 matrices for O, up and gate of the second layer."""
     L, E, H, KV, D, FF, V = 2, 256, 4, 2, 64, 512, 96
     md = {"general.architecture": arch, f"{arch}.block_count": L, f"{arch}.embedding_length": E,
           f"{arch}.feed_forward_length": FF, f"{arch}.attention.head_count": H, f"{arch}.attention.head_count_kv": KV,
@@ -219,24 +279,44 @@ def _model_file(path, arch, rng):
                (f"{p}.ffn_up.weight", (FF, E), gguf.GGML_Q4_K, make_q4_k(rng, FF * E // 256)),
                (f"{p}.ffn_down.weight", (E, FF), gguf.GGML_Q4_0, make_q4_0(rng, E * FF // 32)),
                (f"{p}.attn_norm.weight", (E,), gguf.GGML_F32, norm(E)), (f"{p}.ffn_norm.weight", (E,), gguf.GGML_F32, norm(E))]
+        if mixed:
+            repl = {f"{p}.attn_k.weight": (gguf.GGML_Q5_0, make_q5_0(rng, KV * D * E // 32)),
+                    f"{p}.attn_v.weight": (gguf.GGML_Q6_K, make_q6_k(rng, KV * D * E // 256)),
+                    f"{p}.ffn_down.weight": (gguf.GGML_Q6_K, make_q6_k(rng, E * FF // 256)),
+                    f"{p}.attn_output.weight": (gguf.GGML_F16, _float_matrix(rng, gguf.GGML_F16, E * H * D)),
+                    f"{p}.ffn_up.weight": (gguf.GGML_BF16, _float_matrix(rng, gguf.GGML_BF16, FF * E))}
+            if i == 1:
+                repl[f"{p}.ffn_gate.weight"] = (gguf.GGML_F32, _float_matrix(rng, gguf.GGML_F32, FF * E))
+            ts[-9:] = [(n, sh, *repl[n]) if n in repl else (n, sh, gt, raw) for n, sh, gt, raw in ts[-9:]]
         if arch == "gemma3":
             ts += [(f"{p}.attn_q_norm.weight", (D,), gguf.GGML_F32, norm(D)), (f"{p}.attn_k_norm.weight", (D,), gguf.GGML_F32, norm(D)),
                    (f"{p}.post_attention_norm.weight", (E,), gguf.GGML_F32, norm(E)),
                    (f"{p}.post_ffw_norm.weight", (E,), gguf.GGML_F32, norm(E))]
     ts.append(("output_norm.weight", (E,), gguf.GGML_F32, norm(E)))
-    ts.append(("token_embd.weight", (V, E), gguf.GGML_Q4_K if arch == "gemma3" else gguf.GGML_Q8_0,
-               make_q4_k(rng, V * E // 256) if arch == "gemma3" else make_q8_0(rng, V * E // 32)))
+    if mixed:      # tied: Q6_K embedding = LM head; untied: F16 embedding rows on the host, Q6_K output matrix
+        ts.append(("token_embd.weight", (V, E), gguf.GGML_Q6_K, make_q6_k(rng, V * E // 256)) if arch == "gemma3" else
+                  ("token_embd.weight", (V, E), gguf.GGML_F16, _float_matrix(rng, gguf.GGML_F16, V * E)))
+    else:
+        ts.append(("token_embd.weight", (V, E), gguf.GGML_Q4_K if arch == "gemma3" else gguf.GGML_Q8_0,
+                   make_q4_k(rng, V * E // 256) if arch == "gemma3" else make_q8_0(rng, V * E // 32)))
     if arch == "llama":
-        ts.append(("output.weight", (V, E), gguf.GGML_Q8_0, make_q8_0(rng, V * E // 32)))
+        ts.append(("output.weight", (V, E), gguf.GGML_Q6_K, make_q6_k(rng, V * E // 256)) if mixed else
+                  ("output.weight", (V, E), gguf.GGML_Q8_0, make_q8_0(rng, V * E // 32)))
         ts.append(("rope_freqs.weight", (D // 2,), gguf.GGML_F32, np.ones(D // 2, np.float32).tobytes()))
     write_gguf(path, md, ts)
 
 
+@pytest.mark.parametrize("mixed", [False, True])
 @pytest.mark.parametrize("arch", ["llama", "gemma3"])
-def test_model_from_file_decodes_like_the_reference_forward(tmp_path, arch):
+def test_model_from_file_decodes_like_the_reference_forward(tmp_path, arch, mixed):
     p = tmp_path / f"{arch}.gguf"
-    _model_file(str(p), arch, np.random.default_rng(7))
+    _model_file(str(p), arch, np.random.default_rng(7), mixed=mixed)
     cfg, tensors = gguf.load_model(str(p))
+    if mixed:
+        kinds = {n: getattr(v, "kind", None) for n, v in tensors.items()}
+        assert kinds["blk.0.attn_k.weight"] == 'q8_0' and kinds["blk.1.ffn_gate.weight"] == 'q4_req'
+        assert kinds["blk.0.attn_v.weight"] == kinds["blk.0.attn_output.weight"] == kinds["blk.1.ffn_up.weight"] == 'q4_req'
+        assert kinds["output.weight" if arch == "llama" else "token_embd.weight"] == 'q4_req' 
     assert (cfg.arch, cfg.n_layer, cfg.n_embd, cfg.n_head, cfg.n_head_kv, cfg.head_dim, cfg.n_ff, cfg.n_vocab) == \
         (arch, 2, 256, 4, 2, 64, 512, 96)
     assert cfg.ffn_act == ("gelu" if arch == "gemma3" else "silu") and (cfg.attn_softcap == 50.0) == (arch == "gemma3")
@@ -251,3 +331,48 @@ def test_model_from_file_decodes_like_the_reference_forward(tmp_path, arch):
         assert a == b or margins[i] < 1e-5, (i, a, b, margins[i])
     hid = eng.read_slot('hidden')
     assert np.linalg.norm(hid - ref.last_hidden) / np.linalg.norm(ref.last_hidden) < 1e-4
+
+
+def test_q5_0_q6_k_bf16_decoders_and_requantised_upload(tmp_path):
+    """Q5_0 -> signed 8-bit codes with scale |d|: bit-exact against the ggml form, negative and zero scales
+    included.  Q6_K and BF16 decode bit-exactly; as weight matrices they (and F16 / F32 matrices) come back from
+    load_model in the reference's re-quantised form -- scale = (max - min) / 15, zero point = min per 32 weights,
+    codes from the map's quantiser -- and what the op surface then holds equals QTensor.dequant()."""
+    rng = np.random.default_rng(5)
+    r5, r6 = make_q5_0(rng, 16), make_q6_k(rng, 4)
+    bf = (rng.standard_normal(128).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    f16 = rng.standard_normal(128).astype(np.float16)
+    f32 = rng.standard_normal(128).astype(np.float32)
+    p = tmp_path / "m.gguf"
+    write_gguf(p, {"general.architecture": "llama", "llama.vocab_size": 8},
+               [("blk.0.a.weight", (8, 64), gguf.GGML_Q5_0, r5), ("blk.0.b.weight", (4, 256), gguf.GGML_Q6_K, r6),
+                ("blk.0.c.weight", (2, 64), gguf.GGML_BF16, bf.tobytes()), ("blk.0.d.weight", (2, 64), gguf.GGML_F16, f16.tobytes()),
+                ("blk.0.e.weight", (4, 32), gguf.GGML_F32, f32.tobytes()), ("blk.0.n.weight", (128,), gguf.GGML_BF16, bf.tobytes())])
+    f = gguf.GGUFFile(str(p))
+    t5 = f.tensor("blk.0.a.weight")
+    assert t5.kind == 'q8_0' and np.array_equal(t5.dequant().reshape(-1), dec_q5_0(r5))    # equal as numbers (a d = 0
+    # block gives -0.0 for negative codes in the ggml form, +0.0 here)
+    assert np.array_equal(f.tensor("blk.0.b.weight").view(np.uint32).reshape(-1), dec_q6_k(r6).view(np.uint32))
+    assert np.array_equal(f.tensor("blk.0.c.weight").view(np.uint32).reshape(-1), bf.astype(np.uint32) << 16)
+    f.close()
+    cfg, ts = gguf.load_model(str(p))
+    assert ts["blk.0.n.weight"].dtype == np.float32 and ts["blk.0.n.weight"].ndim == 1       # 1-D tensors stay float
+    src = {"blk.0.b.weight": dec_q6_k(r6), "blk.0.c.weight": (bf.astype(np.uint32) << 16).view(np.float32),
+           "blk.0.d.weight": f16.astype(np.float32), "blk.0.e.weight": f32}
+    g = oracle.init()
+    for name, x in src.items():
+        t = ts[name]
+        assert t.kind == 'q4_req'
+        xb = x.reshape(-1, 32).astype(np.float64)
+        want_scale = np.where(xb.max(1) > xb.min(1), (xb.max(1) - xb.min(1)) / 15.0, 1.0).astype(np.float32)
+        assert np.array_equal(t.scale, want_scale) and np.array_equal(t.zp, xb.min(1).astype(np.float32))
+        # through the op surface: floats scattered into a 4-bit map, read back dequantised
+        g.map_create_typed(1, A.DTYPE_Q4, 1, t.size, 32)
+        g.set_qparams(1, *t.qparams())
+        g.scatter_contiguous(1, 0, t.data)
+        h = g.map_gather_dev(1, g.upload_dev(np.arange(t.size, dtype=np.uint32))[0], t.size)[0]
+        assert np.array_equal(g.download_dev(h, t.size), t.dequant().reshape(-1)), name
+        # the extremes of every group are kept exactly; nothing moves by more than half a step (+ rounding)
+        deq = t.dequant().reshape(-1, 32)
+        assert np.array_equal(deq.min(1), xb.min(1).astype(np.float32))
+        assert np.all(np.abs(deq - x.reshape(-1, 32)) <= 0.5 * want_scale[:, None] * (1 + 1e-5) + 1e-7)

@@ -131,15 +131,17 @@ def test_llama3_8b_full_model_tokens_match_reference_forward(hip):
     _full_model_vs_cpu(hip, synth.llama3_8b_config(), 4, 3, 0)
 
 
+@pytest.mark.parametrize("mixed", [False, True])
 @pytest.mark.parametrize("arch", ["llama", "gemma3"])
-def test_model_read_from_a_gguf_file(hip, arch, tmp_path):
-    """Q4_K, Q4_0 and Q8_0 blocks of a file uploaded in map form (nothing re-quantised): the harness on the
-    HIP library follows the harness on the oracle, and the restated reference forward over the
-    dequantised blocks."""
+def test_model_read_from_a_gguf_file(hip, arch, mixed, tmp_path):
+    """Q4_K, Q4_0 and Q8_0 blocks of a file uploaded in map form (nothing re-quantised) -- and, mixed, a file that
+    also holds Q5_0 (as signed 8-bit codes), Q6_K, F16, BF16 and F32 matrices (through the 4-bit map's own
+    quantiser, as the reference sends them): the harness on the HIP library follows the harness on the oracle,
+    and the restated reference forward over the dequantised weights."""
     from adam_amd import gguf
     from test_gguf_loader import _model_file
     p = tmp_path / f"{arch}.gguf"
-    _model_file(str(p), arch, np.random.default_rng(11))
+    _model_file(str(p), arch, np.random.default_rng(11), mixed=mixed)
     cfg, tensors = gguf.load_model(str(p))
     note(f"engine from gguf {arch}")
     prompt = [5, 17, 3, 90, 44]
