@@ -6,19 +6,21 @@
 // is the one place on the path where the work is a dense contraction and belongs on MFMA.
 //
 // v_mfma_f32_16x16x32_f16:  D[i][j] += sum_k A[i][k] B[k][j];  lane l supplies A[l % 16][8g..8g+7] and
-// B[8g..8g+7][l % 16] with g = l / 16, and receives D[4g..4g+3][l % 16].  Here i runs over 16 weight
-// rows, j over 16 activation rows, and the 32 k of one instruction are eight weights out of each of
-// four consecutive 32-weight blocks: lane (row, g) loads block g of its row as one 16-byte word
-// group, dequantises it in registers to fp16 (exactly (q - 8), then times the block's fp16 scale:
-// one rounding per weight) and feeds four instructions from it.  The activations of the tile are
-// converted once per step to fp16 in LDS, scaled per row by a power of two so that no row can
-// overflow fp16 (the scale is divided out of the fp32 result), in the element order the unpacking
-// produces.  Accumulation is fp32 in the matrix core.
+// B[8g..8g+7][l % 16] with g = l / 16, and receives D[4g..4g+3][l % 16].  Here i runs over 16 activation rows,
+// j over 16 weight rows, and the 32 k of one instruction are ONE 32-weight block: lane (row, g) loads block g of
+// the step's four blocks of its weight row as one 16-byte word group, a 4 x 4 transpose of words between the four
+// lanes of a row (gfx950 row-swap instructions) leaves it with word g of every block, and the nibbles become
+// fp16 (q - 8) exactly.  Each block's products are summed by the matrix core from zero and the block's fp16
+// scale is applied to that sum in float32 (one fused multiply-add per output and block), so the weights need no
+// rounding at all.  The activations of the tile are converted once per matmul to two fp16 planes (x s = xh + xl,
+// s a power of two per row so that no row can overflow; divided out of the float32 result), in the element order
+// the unpacking produces; two instructions per block (xh, xl), every product exact.
 //
-// Workgroup = 4 waves = 64 weight rows x (16 * MT) activation rows; one step = 128 weights of K.
-// KSPLIT (few activation rows): the four waves share 16 weight rows and take every fourth step of K
-// each, so that small matrices still spread over the whole chip; their partial tiles are summed
-// through LDS in a fixed order.
+// Tiled form: workgroup = NW waves, each with R tiles of 16 weight rows = 16 NW R weight rows x 16 MT activation
+// rows; one step = 128 weights of K (four blocks).
+// K-split form (few activation rows): the waves share R tiles of 16 weight rows and take every NWV-th step of K
+// each, so that small matrices still spread over the whole chip; their partial tiles are summed through LDS in
+// a fixed order.
 #include "gemv_common.h"
 #include <algorithm>
 
@@ -32,16 +34,13 @@ typedef uint32_t u2q_t __attribute__((ext_vector_type(2)));
 typedef uint32_t u4q_t __attribute__((ext_vector_type(4)));
 typedef _Float16 h8q_t __attribute__((ext_vector_type(8)));
 
-// Two-term operands.  A product w * x of the reference is a float32 product of float32 values; one fp16
-// rounding of each operand (2^-12 relative) is harmless in a single projection but adds up over the ~200
+// Two-term activations.  A product w * x of the reference is a float32 product of float32 values; one fp16
+// rounding of an operand (2^-12 relative) is harmless in a single projection but adds up over the ~200
 // projections of a forward pass (a 512-token chunk ended 1.3e-3 .. 6e-3 away from the token-by-token hidden
-// state).  Both operands are therefore fed as exact sums of two fp16 numbers:
-//   x * s  = xh + xl          xh = fp16(x s), xl = fp16(x s - xh)                (22 significant bits)
-//   w      = wh + wl          d = dh + dl with dh = d with its low four mantissa bits cleared, so that
-//                             wh = dh (q - 8) and wl = dl (q - 8) are exact fp16 products
-// and three matrix instructions accumulate  wh xh + wl xh + wh xl  in float32 (every product exact; the
-// dropped wl xl is below 2^-18 of the term).  Q8_0 weights (the LM head of a lockstep batch, the last
-// projection of a pass) keep the one-term form.
+// state).  The activations are therefore fed as exact sums of two fp16 numbers,
+//   x * s  = xh + xl          xh = fp16(x s), xl = fp16(x s - xh)                (22 significant bits),
+// and the weights as the integers (q - 8) with the block scale applied afterwards in float32.  Q8_0 weights (the LM
+// head of a lockstep batch, the last projection of a pass) keep one fp16 term for each operand.
 __device__ __forceinline__ void split_pair(float a, float b, uint32_t* hi, uint32_t* lo) {
   const _Float16 ah = (_Float16)a, bh = (_Float16)b;
   const h2q_t h = {ah, bh}, l = {(_Float16)(a - (float)ah), (_Float16)(b - (float)bh)};
@@ -100,21 +99,35 @@ __device__ __forceinline__ void deq_ints(uint32_t w, const DeqK& c, h2q_t* t) {
   t[2] = __builtin_bit_cast(h2q_t, (w8 & c.nib_lo) | c.magic_lo) + c.off_lo;
   t[3] = __builtin_bit_cast(h2q_t, (w8 & c.nib_hi) | c.magic_hi) + c.off_hi;
 }
-// one word of a block -> its operand fragment in both terms: wh = dh (q - 8), wl = dl (q - 8), exact
-__device__ __forceinline__ void deq_word2(uint32_t w, const DeqK& c, h2q_t dh2, h2q_t dl2, u4q_t* ah, u4q_t* al) {
+// one word of a block -> the operand fragment (q - 8), exact in fp16, eight weights in the order deq_ints makes
+__device__ __forceinline__ u4q_t deq_word(uint32_t w, const DeqK& c) {
   h2q_t t[4];
   deq_ints(w, c, t);
-  *ah = (u4q_t){__builtin_bit_cast(uint32_t, (h2q_t)(t[0] * dh2)), __builtin_bit_cast(uint32_t, (h2q_t)(t[1] * dh2)),
-                __builtin_bit_cast(uint32_t, (h2q_t)(t[2] * dh2)), __builtin_bit_cast(uint32_t, (h2q_t)(t[3] * dh2))};
-  *al = (u4q_t){__builtin_bit_cast(uint32_t, (h2q_t)(t[0] * dl2)), __builtin_bit_cast(uint32_t, (h2q_t)(t[1] * dl2)),
-                __builtin_bit_cast(uint32_t, (h2q_t)(t[2] * dl2)), __builtin_bit_cast(uint32_t, (h2q_t)(t[3] * dl2))};
+  return (u4q_t){__builtin_bit_cast(uint32_t, t[0]), __builtin_bit_cast(uint32_t, t[1]), __builtin_bit_cast(uint32_t, t[2]),
+                 __builtin_bit_cast(uint32_t, t[3])};
 }
-// d = dh + dl: dh keeps the upper seven significant bits
-__device__ __forceinline__ void split_scale(_Float16 d, h2q_t* dh2, h2q_t* dl2) {
-  const _Float16 dh = __builtin_bit_cast(_Float16, (uint16_t)(__builtin_bit_cast(uint16_t, d) & 0xFFF0u));
-  const _Float16 dl = d - dh;
-  *dh2 = (h2q_t){dh, dh};
-  *dl2 = (h2q_t){dl, dl};
+// Lanes l, l + 16, l + 32, l + 48 hold the four 32-weight blocks of one step of a weight row, four words each.
+// One matrix instruction is to cover ONE block (so that the block's scale can be applied to its result), i.e.
+// lane group g has to supply word g of that block: a 4 x 4 transpose of words between the four lanes, done with
+// the row-swap instructions of gfx950 (v_permlane32_swap: upper half of the first register <-> lower half of the
+// second; v_permlane16_swap: odd 16-lane rows of the first <-> even rows of the second).  Afterwards word b of
+// the result is word g of block b.
+typedef uint32_t u2s_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u4q_t transpose_blocks(u4q_t q) {
+  const u2s_t a = __builtin_amdgcn_permlane32_swap(q.x, q.z, false, false);
+  const u2s_t b = __builtin_amdgcn_permlane32_swap(q.y, q.w, false, false);
+  const u2s_t c = __builtin_amdgcn_permlane16_swap(a.x, b.x, false, false);
+  const u2s_t d = __builtin_amdgcn_permlane16_swap(a.y, b.y, false, false);
+  return (u4q_t){c.x, c.y, d.x, d.y};
+}
+// the scales of the four blocks (lane group g holds block g's): all four to every lane, as float
+__device__ __forceinline__ f4q_t gather_scales(_Float16 d) {
+  const uint32_t v = (uint32_t)__builtin_bit_cast(uint16_t, d);
+  const u2s_t a = __builtin_amdgcn_permlane32_swap(v, v, false, false);        // {d0 d1 d0 d1}, {d2 d3 d2 d3} by lane group
+  const u2s_t lo = __builtin_amdgcn_permlane16_swap(a.x, a.x, false, false);   // {d0 d0 d0 d0}, {d1 d1 d1 d1}
+  const u2s_t hi = __builtin_amdgcn_permlane16_swap(a.y, a.y, false, false);   // {d2 ...}, {d3 ...}
+  auto f = [](uint32_t b) { return (float)__builtin_bit_cast(_Float16, (uint16_t)b); };
+  return (f4q_t){f(lo.x), f(lo.y), f(hi.x), f(hi.y)};
 }
 #define DEQK_INIT(c)                                                                           \
   DeqK c = {0x64006400u, 0x54005400u, 0x000F000Fu, 0x00F000F0u,                                \
@@ -125,13 +138,14 @@ __device__ __forceinline__ void split_scale(_Float16 d, h2q_t* dh2, h2q_t* dl2) 
   asm volatile("" : "+s"(c.nib_hi))
 #define MFMA_F16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8q_t, a), __builtin_bit_cast(h8q_t, b), c, 0, 0, 0)
 
-// Workgroup = 4 waves, each with R tiles of 16 weight rows = 64 R weight rows x 16 MT activation rows.
-// An activation fragment read from LDS feeds 3 R matrix instructions (R tiles, two weight terms for the
-// first activation plane, one for the second); the weights of a wave's R tiles are dequantised in its
-// registers, word by word as the K loop needs them.  One step = 128 weights of K; the next step's weight
-// words and activation pieces are loaded into registers while the matrix cores work on the current one.
-template <int MT, int R>
-__global__ void __launch_bounds__(256)
+// Workgroup = NW waves, each with R tiles of 16 weight rows = 16 NW R weight rows x 16 MT activation rows.
+// A pair of activation fragments (both planes) read from LDS feeds 2 R matrix instructions; the weights of a
+// wave's R tiles are unpacked in its registers, block by block as the K loop needs them.  One step = 128 weights
+// of K; the next step's weight words and activation pieces are loaded into registers while the matrix cores work
+// on the current one.  The activation tile is staged by every workgroup, so wide workgroups (eight waves) move
+// fewer bytes per flop: 28672x4096 at M = 512 went 434 -> 344 us with 256 instead of 128 weight rows per workgroup.
+template <int MT, int R, int NW>
+__global__ void __launch_bounds__(64 * NW)
 k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh,
                     const u4q_t* __restrict__ xl, const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc,
                     const float* __restrict__ scale, uint32_t M, uint32_t K, uint32_t N, GemmSegs segs) {
@@ -140,7 +154,8 @@ k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __r
   uint8_t* const xs2 = xs + BM * ROWB;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t r16 = lane & 15u, g = lane >> 4;
-  const uint32_t n0 = blockIdx.x * (64u * R) + wave * (16u * R), m0 = blockIdx.y * BM, op = blockIdx.z;
+  constexpr uint32_t NT = 64u * NW, NP = 256u * MT / NT;       // threads; 16-byte pieces per thread, plane and step
+  const uint32_t n0 = blockIdx.x * (16u * NW * R) + wave * (16u * R), m0 = blockIdx.y * BM, op = blockIdx.z;
   const uint64_t c_off = lc[op], gbase = (uint64_t)lb[op] >> 5;
   const uint32_t nblk = K >> 5, kw = K >> 3;                   // blocks and 16-byte pieces per row
   uint32_t nrow[R];
@@ -154,14 +169,14 @@ k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __r
     for (int t = 0; t < MT; t++) acc[r][t] = (f4q_t){0.f, 0.f, 0.f, 0.f};
   DEQK_INIT(dk);
 
-  // staging: the tile's 16 pieces per row, plane and step; thread -> (row, piece) pairs, MT per thread
-  uint64_t xoff[MT];
+  // staging: the tile's 16 pieces per row, plane and step; thread -> (row, piece) pairs, NP per thread
+  uint64_t xoff[NP];
 #pragma unroll
-  for (uint32_t u = 0; u < MT; u++) {
-    const uint32_t w = tid + u * 256u, row = min(m0 + (w >> 4), M - 1u);   // rows past M: clamped, not stored
+  for (uint32_t u = 0; u < NP; u++) {
+    const uint32_t w = tid + u * NT, row = min(m0 + (w >> 4), M - 1u);   // rows past M: clamped, not stored
     xoff[u] = ((uint64_t)op * M + row) * kw + (w & 15u);
   }
-  u4q_t xn[MT], xln[MT], qn[R];
+  u4q_t xn[NP], xln[NP], qn[R];
   _Float16 dn[R];
   // always executed; the step past K re-reads the last one and is not used
 #define GEMM_FETCH(kb_raw)                                                        \
@@ -172,7 +187,7 @@ k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __r
       qn[r] = *(const u4q_t*)(W + (gi << 4));                                     \
       dn[r] = __builtin_bit_cast(_Float16, d16[gi]);                              \
     }                                                                             \
-    _Pragma("unroll") for (uint32_t u = 0; u < MT; u++) {                         \
+    _Pragma("unroll") for (uint32_t u = 0; u < NP; u++) {                         \
       xn[u] = xh[xoff[u] + kb_ * 4u];                                             \
       xln[u] = xl[xoff[u] + kb_ * 4u];                                            \
     }                                                                             \
@@ -181,49 +196,66 @@ k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __r
 
   for (uint32_t kb0 = 0; kb0 < nblk; kb0 += 4u) {
 #pragma unroll
-    for (uint32_t u = 0; u < MT; u++) {
-      const uint32_t w = tid + u * 256u;
+    for (uint32_t u = 0; u < NP; u++) {
+      const uint32_t w = tid + u * NT;
       *(u4q_t*)(xs + (w >> 4) * ROWB + (w & 15u) * 16u) = xn[u];
       *(u4q_t*)(xs2 + (w >> 4) * ROWB + (w & 15u) * 16u) = xln[u];
     }
     u4q_t q[R];
-    h2q_t dh2[R], dl2[R];
+    f4q_t ds[R];
 #pragma unroll
-    for (int r = 0; r < R; r++) { q[r] = qn[r]; split_scale(dn[r], &dh2[r], &dl2[r]); }
+    for (int r = 0; r < R; r++) { q[r] = transpose_blocks(qn[r]); ds[r] = gather_scales(dn[r]); }
     __syncthreads();
     GEMM_FETCH(kb0 + 4u);
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      u4q_t ah[R], al[R];
+    for (int b = 0; b < 4; b++) {      // one 32-weight block of the step at a time
+      u4q_t wq[R];
 #pragma unroll
-      for (int r = 0; r < R; r++)
-        deq_word2(j == 0 ? q[r].x : j == 1 ? q[r].y : j == 2 ? q[r].z : q[r].w, dk, dh2[r], dl2[r], &ah[r], &al[r]);
+      for (int r = 0; r < R; r++) wq[r] = deq_word(b == 0 ? q[r].x : b == 1 ? q[r].y : b == 2 ? q[r].z : q[r].w, dk);
+      // TG activation tiles at a time: their first-plane instructions, then the second-plane ones (each depends on
+      // one issued TG * R instructions earlier), then the scaling of the block results
+      constexpr int TG = R >= 4 ? 2 : MT >= 4 ? 4 : MT;
 #pragma unroll
-      for (int t = 0; t < MT; t++) {
-        const uint32_t xo = (t * 16u + r16) * ROWB + g * 64u + j * 16u;
-        const u4q_t bh = *(const u4q_t*)(xs + xo), bl = *(const u4q_t*)(xs2 + xo);
+      for (int t0 = 0; t0 < MT; t0 += TG) {
+        u4q_t ah[TG], al[TG];
+        f4q_t blk[TG][R];
 #pragma unroll
-        for (int r = 0; r < R; r++) acc[r][t] = MFMA_F16(ah[r], bh, acc[r][t]);
+        for (int t = 0; t < TG; t++) {
+          const uint32_t xo = ((t0 + t) * 16u + r16) * ROWB + b * 64u + g * 16u;
+          ah[t] = *(const u4q_t*)(xs + xo); al[t] = *(const u4q_t*)(xs2 + xo);
+        }
 #pragma unroll
-        for (int r = 0; r < R; r++) acc[r][t] = MFMA_F16(al[r], bh, acc[r][t]);
+        for (int t = 0; t < TG; t++)
 #pragma unroll
-        for (int r = 0; r < R; r++) acc[r][t] = MFMA_F16(ah[r], bl, acc[r][t]);
+          for (int r = 0; r < R; r++) blk[t][r] = MFMA_F16(ah[t], wq[r], ((f4q_t){0.f, 0.f, 0.f, 0.f}));
+#pragma unroll
+        for (int t = 0; t < TG; t++)
+#pragma unroll
+          for (int r = 0; r < R; r++) blk[t][r] = MFMA_F16(al[t], wq[r], blk[t][r]);
+#pragma unroll
+        for (int t = 0; t < TG; t++)
+#pragma unroll
+          for (int r = 0; r < R; r++) {
+            const float d = ds[r][b];
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[r][t0 + t][i] = fmaf(blk[t][r][i], d, acc[r][t0 + t][i]);
+          }
       }
     }
     __syncthreads();
   }
-  // lane (j = r16, g) holds D[4g + i][j]: weight rows n0 + 16 r + 4g + i, activation row m0 + 16 t + r16
+  // lane (r16, g) holds D[4g + i][r16]: activation rows m0 + 16 t + 4g + i, weight row n0 + 16 r + r16
 #pragma unroll
-  for (int t = 0; t < MT; t++) {
-    const uint32_t row = m0 + t * 16u + r16;
-    if (row >= M) continue;
-    const float inv = scale[2 * ((uint64_t)op * M + row) + 1];
-    float* c = out + c_off + (uint64_t)row * N;
+  for (int t = 0; t < MT; t++)
 #pragma unroll
-    for (int r = 0; r < R; r++)
+    for (int i = 0; i < 4; i++) {
+      const uint32_t row = m0 + t * 16u + 4u * g + i;
+      if (row >= M) continue;
+      const float inv = scale[2 * ((uint64_t)op * M + row) + 1];
+      float* c = out + c_off + (uint64_t)row * N;
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const uint32_t n = n0 + r * 16u + 4u * g + i;
+      for (int r = 0; r < R; r++) {
+        const uint32_t n = n0 + r * 16u + r16;
         if (n >= N) continue;
         if (segs.count) {   // stacked matrices: the row's own matrix and its result base
           uint32_t sgi = 0;
@@ -232,7 +264,7 @@ k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __r
           out[segs.c[sgi] + (uint64_t)row * segs.n[sgi] + (n - segs.begin[sgi])] = acc[r][t][i] * inv;
         } else c[n] = acc[r][t][i] * inv;
       }
-  }
+    }
 }
 
 #undef GEMM_FETCH
@@ -318,7 +350,8 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
     }
     // the step's blocks and scales, moved to the lanes that consume them
     u4q_t q[R], q2[Q8 ? R : 1];
-    h2q_t dh2[R], dl2[R];
+    f4q_t ds[Q8 ? 1 : R];
+    h2q_t d2[Q8 ? R : 1];
 #pragma unroll
     for (int r = 0; r < R; r++) {
 #define PERM_U4(v) (u4q_t){(uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)(v).x), (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)(v).y), \
@@ -328,17 +361,19 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
 #undef PERM_U4
       const uint32_t dbits = (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)__builtin_bit_cast(uint16_t, dn[r]));
       const _Float16 dl = __builtin_bit_cast(_Float16, (uint16_t)dbits);
-      if (Q8) { dh2[r] = (h2q_t){dl, dl}; dl2[r] = dh2[r]; }
-      else split_scale(dl, &dh2[r], &dl2[r]);
+      if (Q8) d2[r] = (h2q_t){dl, dl};
+      else { q[r] = transpose_blocks(q[r]); ds[r] = gather_scales(dl); }
     }
     __builtin_amdgcn_wave_barrier();
     GEMM_FETCH(kb0 + 4u * NWV);
+    if (Q8) {
+      // Q8_0 blocks: lane group g holds block g whole; instruction j takes code bytes 8j .. 8j+7 of each of the
+      // four blocks, scaled before the product (one term each for weights and activations)
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      u4q_t ah[R], al[Q8 ? 1 : R];
+      for (int j = 0; j < 4; j++) {
+        u4q_t wq[R];
 #pragma unroll
-      for (int r = 0; r < R; r++) {
-        if (Q8) {
+        for (int r = 0; r < R; r++) {
           // piece j = code bytes 8j .. 8j+7 in two words; pair p = (byte p of the first, byte p of the second)
           const uint32_t w0 = j == 0 ? q[r].x : j == 1 ? q[r].z : j == 2 ? q2[r].x : q2[r].z;
           const uint32_t w1 = j == 0 ? q[r].y : j == 1 ? q[r].w : j == 2 ? q2[r].y : q2[r].w;
@@ -346,25 +381,38 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
 #pragma unroll
           for (uint32_t p = 0; p < 4; p++) {
             const uint32_t t = __builtin_amdgcn_perm(w1, w0, 0x0C000C00u | ((4u + p) << 16) | p) | dk.magic_lo;
-            o[p] = __builtin_bit_cast(uint32_t, (h2q_t)((__builtin_bit_cast(h2q_t, t) + off_q8) * dh2[r]));
+            o[p] = __builtin_bit_cast(uint32_t, (h2q_t)((__builtin_bit_cast(h2q_t, t) + off_q8) * d2[r]));
           }
-          ah[r] = (u4q_t){o[0], o[1], o[2], o[3]};
-        } else {
-          deq_word2(j == 0 ? q[r].x : j == 1 ? q[r].y : j == 2 ? q[r].z : q[r].w, dk, dh2[r], dl2[r], &ah[r], &al[r]);
+          wq[r] = (u4q_t){o[0], o[1], o[2], o[3]};
+        }
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+          const u4q_t ah = *(const u4q_t*)(xs + (t * 16u + r16) * ROWB + g * 64u + j * 16u);
+#pragma unroll
+          for (int r = 0; r < R; r++) acc[r][t] = MFMA_F16(ah, wq[r], acc[r][t]);
         }
       }
+    } else {
 #pragma unroll
-      for (int t = 0; t < MT; t++) {
-        const uint32_t xo = (t * 16u + r16) * ROWB + g * 64u + j * 16u;
-        const u4q_t bh = *(const u4q_t*)(xs + xo);
+      for (int b = 0; b < 4; b++) {      // one 32-weight block of the step at a time
+        u4q_t wq[R];
 #pragma unroll
-        for (int r = 0; r < R; r++) acc[r][t] = MFMA_F16(ah[r], bh, acc[r][t]);
-        if (!Q8) {
-          const u4q_t bl = *(const u4q_t*)(xs2 + xo);
+        for (int r = 0; r < R; r++) wq[r] = deq_word(b == 0 ? q[r].x : b == 1 ? q[r].y : b == 2 ? q[r].z : q[r].w, dk);
 #pragma unroll
-          for (int r = 0; r < R; r++) acc[r][t] = MFMA_F16(al[r], bh, acc[r][t]);
+        for (int t = 0; t < MT; t++) {
+          const uint32_t xo = (t * 16u + r16) * ROWB + b * 64u + g * 16u;
+          const u4q_t ah = *(const u4q_t*)(xs + xo), al = *(const u4q_t*)(xs2 + xo);
+          f4q_t blk[R];
 #pragma unroll
-          for (int r = 0; r < R; r++) acc[r][t] = MFMA_F16(ah[r], bl, acc[r][t]);
+          for (int r = 0; r < R; r++) blk[r] = MFMA_F16(ah, wq[r], ((f4q_t){0.f, 0.f, 0.f, 0.f}));
+#pragma unroll
+          for (int r = 0; r < R; r++) blk[r] = MFMA_F16(al, wq[r], blk[r]);
+#pragma unroll
+          for (int r = 0; r < R; r++) {
+            const float d = ds[r][b];
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[r][t][i] = fmaf(blk[r][i], d, acc[r][t][i]);
+          }
         }
       }
     }
@@ -391,17 +439,18 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
       for (int t = 0; t < MT; t++)
 #pragma unroll
         for (int i = 0; i < 4; i++) acc[r][t][i] += part[(((w * R + r) * MT + t) * 4u + i) * 64u + lane];
+  // lane (r16, g) holds D[4g + i][r16]: activation rows m0 + 16 t + 4g + i, weight row n0 + 16 r + r16
 #pragma unroll
-  for (int t = 0; t < MT; t++) {
-    const uint32_t row = m0 + t * 16u + r16;
-    if (row >= M) continue;
-    const float inv = scale[2 * ((uint64_t)op * M + row) + 1];
-    float* c = out + c_off + (uint64_t)row * N;
+  for (int t = 0; t < MT; t++)
 #pragma unroll
-    for (int r = 0; r < R; r++)
+    for (int i = 0; i < 4; i++) {
+      const uint32_t row = m0 + t * 16u + 4u * g + i;
+      if (row >= M) continue;
+      const float inv = scale[2 * ((uint64_t)op * M + row) + 1];
+      float* c = out + c_off + (uint64_t)row * N;
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const uint32_t n = n0 + r * 16u + 4u * g + i;
+      for (int r = 0; r < R; r++) {
+        const uint32_t n = n0 + r * 16u + r16;
         if (n >= N) continue;
         if (segs.count) {   // stacked matrices: the row's own matrix and its result base
           uint32_t sgi = 0;
@@ -414,7 +463,7 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
           if (segs.add) out[segs.dst + (uint64_t)row * N + n] = out[segs.res + (uint64_t)row * N + n] + y;
         }
       }
-  }
+    }
 }
 #undef GEMM_FETCH
 
@@ -575,21 +624,28 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
     keep();
     return check_launch();
   }
-  // Tile per workgroup: 64 R weight rows x 16 MT activation rows.  The largest of (8,2), (8,1), (4,1)
-  // that still gives every CU two workgroups; a larger tile reads the activations and LDS less often.
-  uint32_t R = 1;
+  // Tile per workgroup: 16 NW R weight rows x 16 MT activation rows (NW waves with R tiles of 16 weight rows each).
+  // Every workgroup stages its activation tile (two fp16 planes: 64 KB per step of 128 weights at MT = 8) from L2,
+  // while its weights are 4.5 bits each, so the bytes a workgroup moves per flop fall with the number of weight
+  // rows it covers: 512 (eight waves, R = 4) where the matrix still gives most CUs a workgroup, else 128 / 64.
+  uint32_t R = 1, NW = 4;
   if (mt == 8) {
-    if (wgs(128, 8) >= want) R = 2;
+    if (wgs(256, 8) * 4 >= 3ull * (uint64_t)g.n_cu) { R = 2; NW = 8; }
+    else if (wgs(128, 8) >= want) R = 2;
     else if (wgs(64, 8) >= want) R = 1;
     else mt = 4;
   }
-  if (mt == 8 && knob("ADAMAH_GEMM_MT", 8) == 4) mt = 4;
+  if (mt == 8 && knob("ADAMAH_GEMM_MT", 8) == 4) { mt = 4; NW = 4; R = 1; }
   R = (uint32_t)knob("ADAMAH_GEMM_R", (int)R);
+  NW = (uint32_t)knob("ADAMAH_GEMM_NW", (int)NW) >= 8 ? 8 : 4;
   R = R >= 4 && mt == 4 ? 4 : R >= 2 ? 2 : 1;
-  dim3 grid(cdiv(N, 64 * R), cdiv(M, 16 * mt), n_ops);
-#define GT(T, RR) k_gemm_q4_f16_tiled<T, RR><<<grid, 256, 0, g.stream>>>(act, mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, lb, lc, g_scale_buf, M, K, N, sg)
-  if (mt == 4) { if (R == 4) GT(4, 4); else if (R == 2) GT(4, 2); else GT(4, 1); }
-  else { if (R == 2) GT(8, 2); else GT(8, 1); }
+  if (mt == 4 && NW == 8 && R == 1) R = 2;
+  dim3 grid(cdiv(N, 16 * NW * R), cdiv(M, 16 * mt), n_ops);
+#define GT(T, RR, W) k_gemm_q4_f16_tiled<T, RR, W><<<grid, 64 * W, 0, g.stream>>>(act, mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, lb, lc, g_scale_buf, M, K, N, sg)
+  if (mt == 4 && NW == 8) { if (R == 4) GT(4, 4, 8); else GT(4, 2, 8); }
+  else if (mt == 4) { if (R == 4) GT(4, 4, 4); else if (R == 2) GT(4, 2, 4); else GT(4, 1, 4); }
+  else if (NW == 8) { if (R == 2) GT(8, 2, 8); else GT(8, 1, 8); }
+  else { if (R == 2) GT(8, 2, 4); else GT(8, 1, 4); }
 #undef GT
   count_launch();
   keep();
