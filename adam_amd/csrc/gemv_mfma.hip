@@ -84,6 +84,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
   uint8_t* xs = (uint8_t*)smem_u4;                    // nblk * 128 bytes
   __shared__ float red_f[16];
   __shared__ uint32_t red_i[16];
+  __shared__ float red_g[16];                         // per-wave partial sums of the prologue's last norm
   __shared__ float part[16 * 64];                     // ks > 1: per-wave partial sums of a shared bundle
   const uint32_t nblk = K >> 5;
   const uint32_t C = (nblk + 63u) >> 6;               // steps per row bundle
@@ -214,7 +215,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
     return t;
   };
 
-  float nrm1 = 1.f;
+  float nrm1 = 1.f, nrm_late = 1.f;   // nrm_late: the prologue's last norm, applied to the row sums
   uint32_t ticket = 0;
   if (PRO == PRO_NONE) {
     // four passes of loads are issued before the first word is converted
@@ -303,9 +304,13 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
 #pragma unroll
         for (int k = 0; k < 8; k++) asm volatile("" ::"v"(rv[u][k]));
     }
-    nrm1 = 1.0f / sqrtf(block_sum(ss) / (float)K + fz.p_eps);
-    const float nrm = nrm1;
+    // The LAST norm of the prologue is not applied to the activations but to the row sums: y = W (u n) = n (W u)
+    // with u = t w (elementwise) and n = rsqrt(mean(t^2) + eps) a scalar.  The workgroup-wide sum behind n then
+    // runs beside the staging of u instead of before it; it is needed only when the first row sum is complete.
+    float ss_last = ss;
     if (PRO == PRO_NORM2) {
+      nrm1 = 1.0f / sqrtf(block_sum(ss) / (float)K + fz.p_eps);
+      const float nrm = nrm1;
       // Every thread of this workgroup has consumed `res` (the reduction above ends in a barrier).
       // t usually goes back into `res` (residual updated in place), which other workgroups may not
       // have read yet, so it is stored by whichever workgroup draws the last ticket.  The ticket is
@@ -319,36 +324,38 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
           for (int k = 0; k < 8; k++) {
             v[u][k] = v[u][k] * nrm * wv[u][k] + rv[u][k];
             if (live[u]) ss2 = fmaf(v[u][k], v[u][k], ss2);
+            v[u][k] *= w2v[u][k];
           }
         }
-      const float nrm2 = 1.0f / sqrtf(block_sum(ss2) / (float)K + fz.p_eps2);
-#pragma unroll
-      for (uint32_t u = 0; u < PRO_WPT; u++)
-        if (mine[u]) {
-#pragma unroll
-          for (int k = 0; k < 8; k++) v[u][k] = v[u][k] * nrm2 * w2v[u][k];
-        }
+      ss_last = ss2;
     } else {
 #pragma unroll
       for (uint32_t u = 0; u < PRO_WPT; u++)
         if (mine[u]) {
 #pragma unroll
-          for (int k = 0; k < 8; k++) v[u][k] = v[u][k] * nrm * wv[u][k];
+          for (int k = 0; k < 8; k++) v[u][k] *= wv[u][k];
         }
     }
 #pragma unroll
-    for (uint32_t u = 0; u < PRO_WPT; u++) {
-      const uint32_t i = u * nthr + tid;
-      if (mine[u]) {
-        if (blockIdx.x == 0 && live[u]) {
-          f4u_t* o = (f4u_t*)(act_out + fz.p_dst + (uint64_t)i * 8u);
-          o[0] = (f4u_t){v[u][0], v[u][1], v[u][2], v[u][3]}; o[1] = (f4u_t){v[u][4], v[u][5], v[u][6], v[u][7]};
+    for (uint32_t u = 0; u < PRO_WPT; u++)
+      if (mine[u]) stage(u * nthr + tid, live[u], v[u]);
+    ss_last = wave_sum_to_lane63(ss_last);
+    if (lane == 63u) red_g[wave] = ss_last;
+    __syncthreads();          // the staged activations and the waves' partial sums are in LDS
+    float tot = 0.f;
+    for (uint32_t w = 0; w < nwav; w++) tot += red_g[w];
+    nrm_late = 1.0f / sqrtf(tot / (float)K + (PRO == PRO_NORM2 ? fz.p_eps2 : fz.p_eps));
+    if (blockIdx.x == 0) {    // the normalised vector itself, where the norm op would have stored it
+#pragma unroll
+      for (uint32_t u = 0; u < PRO_WPT; u++)
+        if (mine[u] && live[u]) {
+          f4u_t* o = (f4u_t*)(act_out + fz.p_dst + (uint64_t)(u * nthr + tid) * 8u);
+          o[0] = (f4u_t){v[u][0] * nrm_late, v[u][1] * nrm_late, v[u][2] * nrm_late, v[u][3] * nrm_late};
+          o[1] = (f4u_t){v[u][4] * nrm_late, v[u][5] * nrm_late, v[u][6] * nrm_late, v[u][7] * nrm_late};
         }
-        stage(i, live[u], v[u]);
-      }
     }
   }
-  __syncthreads();
+  if (PRO == PRO_NONE || PRO == PRO_COMBINE) __syncthreads();
   uint32_t nib = 0x0F0F0F0Fu;
   asm volatile("" : "+s"(nib));             // opaque, so it stays in a register instead of a literal per use
   // Lanes 0..2 of a block read digit 0..2 (operand rows 0..2); the fourth operand row is not needed, so lane 3 reads
@@ -429,6 +436,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       float y = acc;
       y += __shfl_xor(y, 4, 64); y += __shfl_xor(y, 8, 64);
       y += __shfl_xor(y, 16, 64); y += __shfl_xor(y, 32, 64);
+      if (PRO == PRO_RMSNORM || PRO == PRO_NORM2) y *= nrm_late;
       acc = 0.f;
       if (glu) {
         // lanes 0, 1 hold gate rows, lanes 2, 3 the matching up rows
@@ -506,6 +514,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
         for (uint32_t pk = 1; pk < ks; pk++) y += part[(wave + pk) * 64u + lane];
         y += __shfl_xor(y, 4, 64); y += __shfl_xor(y, 8, 64);
         y += __shfl_xor(y, 16, 64); y += __shfl_xor(y, 32, 64);
+        if (PRO == PRO_RMSNORM || PRO == PRO_NORM2) y *= nrm_late;
         const uint32_t row = first + l;
         if (row < N && bcol == 0u) {
           act_out[(uint64_t)c_out + row] = y;
