@@ -326,11 +326,9 @@ bool launch_attn_decode(const AttnDecodeArgs& a, AttnPartials* ap, bool* left, i
   // Slices of the sequence.  Short sequences (at most one 16-row tile per wave when the chip holds
   // `target` waves): workgroups of 8 waves, one tile each, no prefetch; longer ones: 4 waves and as
   // many tiles per wave as it takes.
-  // Wave budget: four waves per CU; eight for sequences up to 8192 rows, where a wave has few tiles and more,
-  // shorter slices finish sooner (context 4096: 12.2 -> 11.0 us with the merge; 16384: 21.7 against 22.7 us)
-  const uint32_t target = (uint32_t)std::max(1, knob("ADAMAH_ATTN_WAVES", (a.row_size <= 8192u ? 8 : 4) * g.n_cu));
+  const uint32_t target = (uint32_t)std::max(1, knob("ADAMAH_ATTN_WAVES", 4 * g.n_cu));
   const uint64_t tiles = (uint64_t)n_groups * cdiv(a.row_size, 16u);
-  uint32_t nw = (tiles <= (uint32_t)(4 * g.n_cu) && G * D <= 1024u) ? 8u : 4u;
+  uint32_t nw = (tiles <= target && G * D <= 1024u) ? 8u : 4u;
   nw = (uint32_t)knob("ADAMAH_ATTN_NW", (int)nw) == 8u && G * D <= 1024u ? 8u : 4u;
   const uint32_t step = nw * 16u;
   uint32_t chunk = step * std::max<uint32_t>(1u, cdiv(tiles, target));
