@@ -437,13 +437,16 @@ k_attn_fused(const float* data, float* out, const __half* kv, uint64_t kv_shift,
 // output elements, eight groups of 32 threads take every eighth split each and meet in LDS.
 __global__ void __launch_bounds__(256)
 k_attn_combine(float* out, const float* partial, const uint32_t* __restrict__ lo, uint32_t value_dim,
-               uint32_t n_splits, uint64_t n_elems) {
+               uint32_t n_splits, uint64_t n_elems, const float* q_src, uint32_t q_dst, uint32_t q_n) {
   __shared__ float w[1024];
   __shared__ float red[4];
   __shared__ float osum[8][32];
   const uint32_t op = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t stride = value_dim + 2;
   const float* pp = partial + (uint64_t)op * n_splits * stride;
+  // queries the attention launch prepared and could not yet store over the raw ones: each workgroup its share
+  for (uint32_t i = (blockIdx.y * gridDim.x + op) * 256u + tid; i < q_n; i += gridDim.x * gridDim.y * 256u)
+    out[(uint64_t)q_dst + i] = q_src[i];
   const uint64_t ob = lo[op];
   if (ob + value_dim > n_elems) return;
   float M = -9.99999968e+37f;
@@ -581,13 +584,20 @@ bool attn_foldable(const PendOp& sc, const PendOp& at) {
   return true;
 }
 
-int launch_attn(const PendOp* sc, const PendOp& at, bool leave_partials, AttnPartials* ap) {
+int launch_attn(const PendOp* sc, const PendOp& at, bool leave_partials, AttnPartials* ap, const RowPrepCtx* prep) {
   Map* m = get_f32_map(at.map_act);
-  if (!m) return ADAMAH_ERR_INVALID;
+  // the row ops offered with the pair: launched here, ahead of the attention, unless the decode kernel takes them
+  auto rows_first = [&]() {
+    int rc = ADAMAH_OK;
+    if (prep) launch_row_run(*prep->q, prep->i0, &rc);
+    prep = nullptr;
+    return rc;
+  };
+  if (!m) { rows_first(); return ADAMAH_ERR_INVALID; }
   const uint32_t n_ops = at.rpg, row_size = at.n, value_dim = at.k;
   bool kv = false, fast = false;
   int r = attn_check(at.map_act, at.h[0], at.h[1], at.h[2], n_ops, row_size, value_dim, &kv, &fast);
-  if (r) return r;
+  if (r) { rows_first(); return r; }
   const uint32_t *ls = res_u32(at.h[0], n_ops), *lv = res_u32(at.h[1], n_ops), *lo = res_u32(at.h[2], n_ops);
   uint32_t chunk, n_splits;
   attn_split(n_ops, row_size, value_dim, leave_partials, &chunk, &n_splits);
@@ -600,17 +610,26 @@ int launch_attn(const PendOp* sc, const PendOp& at, bool leave_partials, AttnPar
                          res_u32(sc->h[0], n_ops), res_u32(sc->h[1], n_ops), ls, lv, lo,
                          res_host(sc->h[0], n_ops), res_host(sc->h[1], n_ops), res_host(at.h[0], n_ops),
                          res_host(at.h[1], n_ops), res_host(at.h[2], n_ops),
-                         n_ops, value_dim, row_size, at.eps, at.f2, leave_partials, ATT_FOLD_FLOATS};
+                         n_ops, value_dim, row_size, at.eps, at.f2, leave_partials, ATT_FOLD_FLOATS, nullptr, nullptr};
     int drc = 0;
-    bool left = false;
+    bool left = false, prep_done = false;
     AttnPartials dp = {};
-    if (launch_attn_decode(da, &dp, &left, &drc)) {
+    auto finish = [&]() {
       if (ap) ap->n_splits = 1;
       if (drc || dp.n_splits == 1) return drc;
-      if (left && ap) { *ap = dp; return ADAMAH_OK; }
+      if (left && ap) { *ap = dp; return (int)ADAMAH_OK; }
       return launch_attn_combine(at, dp);
+    };
+    if (prep) {
+      // with the preparation inside the launch, or not at all (nothing is launched then)
+      da.prep = &prep->tasks; da.prep_done = &prep_done;
+      if (launch_attn_decode(da, &dp, &left, &drc)) return finish();
+      da.prep = nullptr; da.prep_done = nullptr;
+      if ((r = rows_first())) return r;
     }
+    if (launch_attn_decode(da, &dp, &left, &drc)) return finish();
   }
+  if ((r = rows_first())) return r;
   if (sc && fast && kv) {
     const uint32_t *la = res_u32(sc->h[0], n_ops), *lb = res_u32(sc->h[1], n_ops);
     uint32_t lpr = 8;
@@ -633,7 +652,7 @@ int launch_attn(const PendOp* sc, const PendOp& at, bool leave_partials, AttnPar
   count_launch();
   r = check_launch();
   if (r || n_splits == 1) { if (ap) ap->n_splits = 1; return r; }
-  AttnPartials loc = {g.attn_scratch, n_splits, value_dim, n_ops, 0};
+  AttnPartials loc = {g.attn_scratch, n_splits, value_dim, n_ops, 0, nullptr, 0, 0};
   if (leave_partials && ap) { *ap = loc; return ADAMAH_OK; }
   if (ap) ap->n_splits = 1;
   return launch_attn_combine(at, loc);
@@ -643,7 +662,8 @@ int launch_attn_combine(const PendOp& at, const AttnPartials& ap) {
   Map* m = get_f32_map(at.map_act);
   const uint32_t* lo = res_u32(at.h[2], at.rpg);
   if (!m || !lo) return ADAMAH_ERR_INVALID;
-  k_attn_combine<<<dim3(at.rpg, cdiv(ap.value_dim, 32)), 256, 0, g.stream>>>((float*)m->buf, ap.base, lo, ap.value_dim, ap.n_splits, m->n_elems);
+  k_attn_combine<<<dim3(at.rpg, cdiv(ap.value_dim, 32)), 256, 0, g.stream>>>((float*)m->buf, ap.base, lo, ap.value_dim, ap.n_splits, m->n_elems,
+                                                                              ap.q_src, ap.q_dst, ap.q_n);
   count_launch();
   return check_launch();
 }
@@ -652,7 +672,7 @@ int launch_attn_combine(const PendOp& at, const AttnPartials& ap) {
 int launch_attn_combine_dev(Map* m, const float* partial, const uint32_t* lo_dev, uint32_t n_ops, uint32_t value_dim,
                             uint32_t n_splits) {
   k_attn_combine<<<dim3(n_ops, cdiv(value_dim, 32)), 256, 0, g.stream>>>((float*)m->buf, partial, lo_dev, value_dim, n_splits,
-                                                                        m->n_elems);
+                                                                        m->n_elems, nullptr, 0u, 0u);
   count_launch();
   return check_launch();
 }

@@ -2,6 +2,7 @@
 // decode kernel.
 #pragma once
 #include "common.h"
+#include <vector>
 
 namespace adamah {
 
@@ -11,6 +12,30 @@ __device__ __forceinline__ float prep(float v, float scale, float cap) {
   if (cap > 0.0f) v = tanhf(v / cap) * cap;
   return v;
 }
+
+// Same arithmetic as rope_cs in norm_rope.hip.
+__device__ __forceinline__ void rope_cs2(uint32_t i, uint32_t dim, uint32_t pos, float base, float* c, float* s) {
+  const float e = (float)(2u * i) / (float)dim;
+  const float p = (float)pow((double)base, (double)e);
+  const float angle = (float)pos * (1.0f / p);
+  *c = cosf(angle);
+  *s = sinf(angle);
+}
+
+// A row task of the preparation before decode attention (rowprep.hip): source row, optional norm weights,
+// optional rotation, destination row, optional cache row.
+#define ROWT_MAX 64u
+#define ROWT_NONE 0xFFFFFFFFu
+struct RowTask {
+  uint32_t src, dst, cache, w;   // element offsets; dst / cache / w may be ROWT_NONE
+  uint32_t dim, pos, flags;      // flags: 1 = RMSNorm (eps 1e-6), 2 = RoPE
+  float base;
+};
+size_t build_row_run(const std::vector<PendOp>& q, size_t i, std::vector<RowTask>* out, bool* alone);
+// The run of row ops q[i0 ...] that directly precedes a (scores, softmax . V) pair, as merged tasks.  The decode
+// attention launch does them itself when they are exactly the preparation of its own operands; otherwise
+// launch_attn launches the run on its own first.
+struct RowPrepCtx { const std::vector<PendOp>* q; size_t i0; std::vector<RowTask> tasks; };
 
 // Grouped decode attention (attn_decode.hip).  Returns false when the shape is not one it covers and
 // nothing was launched; otherwise *rc carries the launch status, *ap the partials still to be merged
@@ -25,6 +50,9 @@ struct AttnDecodeArgs {
   float scale, cap;
   bool leave_partials;          // stop before the merge of the sequence splits when there are few partials
   uint32_t fold_floats;         // "few": at most this many partial floats
+  const std::vector<RowTask>* prep;   // optional: the row tasks queued just before the pair (rotation of the new
+                                      // Q / K rows, KV append); done inside the launch when they fit its pattern
+  bool* prep_done;              // set by launch_attn_decode when it took them
 };
 bool launch_attn_decode(const AttnDecodeArgs& a, AttnPartials* ap, bool* left, int* rc);
 int tuning(const char* name, int dflt);   // behaviour switch from the environment (gemv_q.hip)

@@ -43,6 +43,28 @@ typedef uint32_t u2a_t __attribute__((ext_vector_type(2)));
 #define ATTD_MAX_OPS 64u
 struct AttdBases { uint32_t q[ATTD_MAX_OPS], sc[ATTD_MAX_OPS], o[ATTD_MAX_OPS], kb[ATTD_MAX_OPS], vb[ATTD_MAX_OPS]; };
 
+// Row preparation done by the attention launch itself (RP): the rotation (after the optional per-head RMSNorm) of
+// the token's new Q and K rows and the append of its K and V rows to the cache, which otherwise are a launch of
+// their own just before (rowprep.hip; same arithmetic in the same order, so the results are the same bits).
+// Every workgroup of a KV head prepares the group's queries for itself from the raw rows; the workgroup that
+// owns the last slice of the sequence also prepares the new K and V rows, stores them to the cache (float32 row
+// and fp16 copy) and uses them from LDS in place of the cache row it loaded.  The prepared queries usually go back
+// over the raw ones, which other workgroups of the group may not have read yet.  With one slice they are stored
+// at once; with more, the first slice's workgroup puts them into scratch memory and the launch that merges the
+// slices (the merge kernel, or the GEMV that merges while staging) copies them to their place.  (Counting the
+// workgroups in with an atomic and letting the last one store cost 2 us per launch: the atomic's reply comes back
+// in order with the wave's K / V tiles, which then wait for the contended counter.)
+struct AttdRowPrep {
+  uint32_t flags;                        // 1 = RMSNorm (eps 1e-6) before the rotation
+  uint32_t pos;                          // position the rotation is for; the new cache row is row_size - 1
+  float base;
+  uint32_t q_src, k_src, k_dst, v_src;   // element offsets: head h of Q at q_src + h D, KV head g at k_src + g D, ...;
+                                         // k_dst = ROWT_NONE: the rotated K row goes to the cache only
+  uint32_t q_w, k_w;                     // norm weights (flags & 1)
+  float* q_scratch;                      // n_splits > 1: the prepared queries, head h at q_scratch + h D
+  const float* inv_freq;                 // 1 / base^(2i/D) for i < D/2, as the stand-alone rotation computes it
+};
+
 #define ATTD_DPP(v, ctrl) __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, 0xF, 0xF, false))
 // all-reduce over each 16-lane row: quad_perm [1,0,3,2], [2,3,0,1], row_half_mirror, row_mirror
 __device__ __forceinline__ float row16_max(float v) {
@@ -55,11 +77,11 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
-template <int D, int G, int NW, bool PF, bool EXT>
+template <int D, int G, int NW, bool PF, bool EXT, bool RP>
 __global__ void __launch_bounds__(NW * 64)
 k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift, const AttdBases bs,
               uint32_t row_size, float scale, float cap, uint32_t n_splits, uint32_t chunk, float* partial,
-              const uint32_t* __restrict__ ext) {
+              const uint32_t* __restrict__ ext, const AttdRowPrep rp) {
   constexpr int NI = D / 32;           // 16-byte K loads per lane and tile
   constexpr int DPL = D / 64;          // V dims per lane (every lane sees all 16 rows of the tile)
   constexpr int DW = DPL > 2 ? DPL / 2 : 1;
@@ -71,6 +93,9 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
   __shared__ h4a_t qop[2 * NI][2][64]; // query operands of the matrix product: [k-step][hi, lo][lane]
   __shared__ uint32_t hmax[G];         // per head: bits of max |q|
   __shared__ float qinv[G];            // per head: 1 / (power-of-two scale of the queries)
+  // RP: sums of squares per 64 elements of the raw Q rows and of the raw K row; the new K and V rows as fp16
+  __shared__ float ssq[RP ? G * D / 64 : 1], ssk[RP ? D / 64 : 1], kraw_s[RP ? D : 1];
+  __shared__ __attribute__((aligned(16))) __half knew[RP ? D : 8], vnew[RP ? D : 8];
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));   // scalar: row numbers below are too
@@ -108,22 +133,132 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
   uint32_t vA[16][DW], vB[16][DW];
   uint32_t rbase = t0 + wave * 16u;
   const bool any = rbase < t1;
+  constexpr uint32_t QN = ((uint32_t)(G * D) + NT - 1u) / NT;        // query elements per thread
+  constexpr uint32_t PN = ((uint32_t)(G * D) / 2u + NT - 1u) / NT;   // RP: rotation pairs per thread
+  const bool tail_wg = RP && split + 1u == n_splits;                 // RP: this workgroup owns the sequence's last row
   {
     float* qs = &obuf[0][0][0];
     if (tid < (uint32_t)G) hmax[tid] = 0u;
-    __syncthreads();
-    for (uint32_t i = tid; i < (uint32_t)(G * D); i += NT) {   // a wave's 64 elements belong to one head
-      const uint32_t hq = (uint32_t)__builtin_amdgcn_readfirstlane((int)(i / D));   // scalar: read from the arguments
-      const float x = data[(uint64_t)(EXT ? e_q[op0 + hq] : bs.q[op0 + hq]) + i % D];
-      qs[i] = x;
-      float m = fabsf(x);
+    if (!RP) {
+      __syncthreads();
+      for (uint32_t i = tid; i < (uint32_t)(G * D); i += NT) {   // a wave's 64 elements belong to one head
+        const uint32_t hq = (uint32_t)__builtin_amdgcn_readfirstlane((int)(i / D));   // scalar: read from the arguments
+        const float x = data[(uint64_t)(EXT ? e_q[op0 + hq] : bs.q[op0 + hq]) + i % D];
+        qs[i] = x;
+        float m = fabsf(x);
 #pragma unroll
-      for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
-      if (lane == 0u) atomicMax(&hmax[i / D], __float_as_uint(m));
+        for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+        if (lane == 0u) atomicMax(&hmax[i / D], __float_as_uint(m));
+      }
+      if (any) { fetch(kA, vA, rbase); }
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+    } else {
+      constexpr uint32_t half = (uint32_t)D / 2u;
+      // raw rows first (they are waited for first), then the first tile
+      float qraw[QN], kraw = 0.f, vraw = 0.f;
+#pragma unroll
+      for (uint32_t u = 0; u < QN; u++) {
+        const uint32_t i = tid + u * NT;
+        qraw[u] = i < (uint32_t)(G * D) ? data[(uint64_t)rp.q_src + (uint64_t)op0 * D + i] : 0.f;
+      }
+      if (tail_wg && tid < (uint32_t)D) {
+        kraw = data[(uint64_t)rp.k_src + (uint64_t)group * D + tid];
+        vraw = data[(uint64_t)rp.v_src + (uint64_t)group * D + tid];
+      }
+      // what the rotation of this thread's pairs needs from memory, asked for now: its frequencies and norm weights
+      float fr[PN], wq[PN][2], wk[2] = {1.f, 1.f};
+#pragma unroll
+      for (uint32_t u = 0; u < PN; u++) {
+        const uint32_t i = (tid + u * NT) % half;
+        fr[u] = rp.inv_freq[i];
+        wq[u][0] = 1.f; wq[u][1] = 1.f;
+        if (rp.flags & 1u) { wq[u][0] = data[(uint64_t)rp.q_w + i]; wq[u][1] = data[(uint64_t)rp.q_w + i + half]; }
+      }
+      if (tail_wg && tid < half && (rp.flags & 1u)) { wk[0] = data[(uint64_t)rp.k_w + tid]; wk[1] = data[(uint64_t)rp.k_w + tid + half]; }
+      __builtin_amdgcn_sched_barrier(0);
+      if (any) { fetch(kA, vA, rbase); }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (uint32_t u = 0; u < QN; u++) {
+        const uint32_t i = tid + u * NT;
+        if (i < (uint32_t)(G * D)) {
+          qs[i] = qraw[u];
+          if (rp.flags & 1u) {
+            float ss = fmaf(qraw[u], qraw[u], 0.f);
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+            if (lane == 0u) ssq[i >> 6] = ss;
+          }
+        }
+      }
+      if (tail_wg && tid < (uint32_t)D) {   // whole waves: D is a multiple of 64
+        kraw_s[tid] = kraw;
+        if (rp.flags & 1u) {
+          float ss = fmaf(kraw, kraw, 0.f);
+#pragma unroll
+          for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+          if (lane == 0u) ssk[tid >> 6] = ss;
+        }
+        // the V row: rounded to fp16 for the copy, and the rounded value into the float32 row
+        const __half vh = __float2half(vraw);
+        const uint64_t vo = (uint64_t)bs.vb[group] + (uint64_t)(row_size - 1u) * D + tid;
+        const_cast<__half*>(kv)[vo - kv_shift] = vh;
+        out[vo] = __half2float(vh);
+        vnew[tid] = vh;
+      }
+      __syncthreads();
+      // sum over a row's 64-element pieces in the order of the stand-alone kernel: (s0 + s1) + (s2 + s3)
+      auto row_ss = [&](const float* pc) {
+        const float s0 = pc[0], s1 = pc[1], s2 = D >= 256 ? pc[D >= 256 ? 2 : 0] : 0.f, s3 = D >= 256 ? pc[D >= 256 ? 3 : 0] : 0.f;
+        return (s0 + s1) + (s2 + s3);
+      };
+#pragma unroll
+      for (uint32_t u = 0; u < PN; u++) {
+        const uint32_t pi = tid + u * NT;           // a wave's 64 pairs belong to one head (D >= 128)
+        if (pi < (uint32_t)(G * D) / 2u) {
+          const uint32_t h = pi / half, i = pi % half;
+          float y0 = qs[h * D + i], y1 = qs[h * D + i + half];
+          if (rp.flags & 1u) {
+            const float inv = 1.0f / sqrtf(row_ss(&ssq[h * (D / 64)]) / (float)D + 1e-6f);
+            y0 = y0 * inv * wq[u][0];
+            y1 = y1 * inv * wq[u][1];
+          }
+          const float angle = (float)rp.pos * fr[u];
+          const float cs = cosf(angle), sn = sinf(angle);
+          const float r0 = y0 * cs - y1 * sn, r1 = y0 * sn + y1 * cs;
+          qs[h * D + i] = r0; qs[h * D + i + half] = r1;   // only this thread touches the pair
+          if (split == 0u) {
+            float* qd = n_splits == 1u ? out + (uint64_t)bs.q[op0 + h] : rp.q_scratch + (uint64_t)(op0 + h) * D;
+            qd[i] = r0; qd[i + half] = r1;
+          }
+          float m = fmaxf(fabsf(r0), fabsf(r1));
+#pragma unroll
+          for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+          if (lane == 0u) atomicMax(&hmax[h], __float_as_uint(m));
+          if (u == 0u && tail_wg && tid < half) {
+            // the new K row: same angle as this thread's query pair (tid = i); stored as the row tasks store it
+            float k0 = kraw_s[i], k1 = kraw_s[i + half];
+            if (rp.flags & 1u) {
+              const float inv = 1.0f / sqrtf(row_ss(&ssk[0]) / (float)D + 1e-6f);
+              k0 = k0 * inv * wk[0];
+              k1 = k1 * inv * wk[1];
+            }
+            const float kr0 = k0 * cs - k1 * sn, kr1 = k0 * sn + k1 * cs;
+            if (rp.k_dst != ROWT_NONE) {
+              out[(uint64_t)rp.k_dst + (uint64_t)group * D + i] = kr0;
+              out[(uint64_t)rp.k_dst + (uint64_t)group * D + i + half] = kr1;
+            }
+            const __half h0 = __float2half(kr0), h1 = __float2half(kr1);
+            const uint64_t ko = (uint64_t)bs.kb[group] + (uint64_t)(row_size - 1u) * D + i;
+            const_cast<__half*>(kv)[ko - kv_shift] = h0; const_cast<__half*>(kv)[ko - kv_shift + half] = h1;
+            out[ko] = __half2float(h0); out[ko + half] = __half2float(h1);
+            knew[i] = h0; knew[i + half] = h1;
+          }
+        }
+      }
+      __syncthreads();
     }
-    if (any) fetch(kA, vA, rbase);
-    __builtin_amdgcn_sched_barrier(0);
-    __syncthreads();
     const uint32_t e = c < G ? (hmax[c] >> 23) & 0xFFu : 0u;
     float s = 1.f, inv = 1.f;
     if (e >= 14u && e <= 254u) { s = __uint_as_float((267u - e) << 23); inv = __uint_as_float((e - 13u) << 23); }
@@ -144,6 +279,23 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
     }
     __syncthreads();
   }
+  // RP: the tile that holds the sequence's last row (and the lanes clamped onto it) takes that row from LDS: the
+  // cache row was still being written when it was loaded
+  auto patch = [&](uint4 (&kr)[NI], uint32_t (&vr)[16][DW], uint32_t rb) {
+    if (!RP || !tail_wg || rb + 16u < t1) return;      // wave-uniform
+    if (rb + c >= t1 - 1u) {
+#pragma unroll
+      for (int i = 0; i < NI; i++) kr[i] = *(const uint4*)((const char*)knew + klane + 64u * i);
+    }
+#pragma unroll
+    for (int u = 0; u < 16; u++)
+      if (rb + u >= t1 - 1u) {
+        const char* src = (const char*)vnew + vlane;
+        if (DPL == 1) vr[u][0] = *(const uint16_t*)src;
+        else if (DPL == 2) vr[u][0] = *(const uint32_t*)src;
+        else { const uint2 t = *(const uint2*)src; vr[u][0] = t.x; vr[u][DW - 1] = t.y; }
+      }
+  };
   // after the matrix product lane (c, kc) holds heads 4kc..4kc+3 of tile row c
   float inv_s[4], m_run[4], l_run[4];
   bool hval[4];
@@ -233,17 +385,20 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
       while (true) {
         fetch(kB, vB, rbase + NW * 16u);     // next tile (clamped into the slice when there is none)
         __builtin_amdgcn_sched_barrier(0);
+        patch(kA, vA, rbase);
         tile(kA, vA, rbase);
         rbase += NW * 16u;
         if (rbase >= t1) break;
         fetch(kA, vA, rbase + NW * 16u);
         __builtin_amdgcn_sched_barrier(0);
+        patch(kB, vB, rbase);
         tile(kB, vB, rbase);
         rbase += NW * 16u;
         if (rbase >= t1) break;
       }
     } else {
       while (true) {
+        patch(kA, vA, rbase);
         tile(kA, vA, rbase);
         rbase += NW * 16u;
         if (rbase >= t1) break;
@@ -289,21 +444,106 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
 
 template <int D, int NW, bool PF>
 static void launch_dg(uint32_t G, dim3 grid, const AttnDecodeArgs& a, const AttdBases& bs, uint32_t n_splits,
-                      uint32_t chunk, const uint32_t* ext) {
-#define ADL(GG, EE)                                                                                       \
-  k_attn_decode<D, GG, NW, PF, EE><<<grid, NW * 64, 0, g.stream>>>(a.data, a.data, a.kv, a.kv_shift, bs, a.row_size, \
-                                                                   a.scale, a.cap, n_splits, chunk, g.attn_scratch, ext)
-  if (ext) { if (G == 1) ADL(1, true); else if (G == 2) ADL(2, true); else if (G == 4) ADL(4, true); else ADL(8, true); }
-  else { if (G == 1) ADL(1, false); else if (G == 2) ADL(2, false); else if (G == 4) ADL(4, false); else ADL(8, false); }
+                      uint32_t chunk, const uint32_t* ext, const AttdRowPrep* rp) {
+  const AttdRowPrep none = {};
+#define ADL(GG, EE, RR)                                                                                   \
+  k_attn_decode<D, GG, NW, PF, EE, RR><<<grid, NW * 64, 0, g.stream>>>(a.data, a.data, a.kv, a.kv_shift, bs, a.row_size, \
+                                                                       a.scale, a.cap, n_splits, chunk, g.attn_scratch, ext, RR ? *rp : none)
+  if (ext) { if (G == 1) ADL(1, true, false); else if (G == 2) ADL(2, true, false); else if (G == 4) ADL(4, true, false); else ADL(8, true, false); }
+  else if (rp && D >= 128) {
+    constexpr bool R = D >= 128;   // the row preparation is built for head sizes 128 and 256
+    if (G == 1) ADL(1, false, R); else if (G == 2) ADL(2, false, R); else if (G == 4) ADL(4, false, R); else ADL(8, false, R);
+  }
+  else { if (G == 1) ADL(1, false, false); else if (G == 2) ADL(2, false, false); else if (G == 4) ADL(4, false, false); else ADL(8, false, false); }
 #undef ADL
 }
 
 template <int D>
 static void launch_d(uint32_t G, uint32_t nw, bool pf, dim3 grid, const AttnDecodeArgs& a, const AttdBases& bs,
-                     uint32_t n_splits, uint32_t chunk, const uint32_t* ext = nullptr) {
-  if (nw == 8) launch_dg<D, 8, false>(G, grid, a, bs, n_splits, chunk, ext);
-  else if (pf) launch_dg<D, 4, true>(G, grid, a, bs, n_splits, chunk, ext);
-  else launch_dg<D, 4, false>(G, grid, a, bs, n_splits, chunk, ext);
+                     uint32_t n_splits, uint32_t chunk, const uint32_t* ext = nullptr, const AttdRowPrep* rp = nullptr) {
+  if (nw == 8) launch_dg<D, 8, false>(G, grid, a, bs, n_splits, chunk, ext, rp);
+  else if (pf) launch_dg<D, 4, true>(G, grid, a, bs, n_splits, chunk, ext, rp);
+  else launch_dg<D, 4, false>(G, grid, a, bs, n_splits, chunk, ext, rp);
+}
+
+// 1 / base^(2i/dim), i < dim / 2, with the arithmetic of the stand-alone rotation (rope_cs2), so that a kernel
+// that reads the table rotates to the same bits.  One table per (base, dim) seen, built on the device at first use.
+__global__ void k_rope_inv_freq(float* t, uint32_t dim, float base) {
+  const uint32_t i = blockIdx.x * 64u + threadIdx.x;
+  if (i >= dim / 2u) return;
+  const float e = (float)(2u * i) / (float)dim;
+  const float p = (float)pow((double)base, (double)e);
+  t[i] = 1.0f / p;
+}
+static struct { float base; uint32_t dim; float* dev; } g_freq[8];
+static int g_freq_n = 0;
+static const float* rope_inv_freq(float base, uint32_t dim) {
+  for (int i = 0; i < g_freq_n; i++)
+    if (g_freq[i].dim == dim && __builtin_bit_cast(uint32_t, g_freq[i].base) == __builtin_bit_cast(uint32_t, base)) return g_freq[i].dev;
+  if (g_freq_n == 8 || dim < 2) return nullptr;
+  float* dev = nullptr;
+  if (hipMalloc((void**)&dev, (size_t)(dim / 2u) * 4) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+  k_rope_inv_freq<<<cdiv(dim / 2u, 64u), 64, 0, g.stream>>>(dev, dim, base);
+  g_freq[g_freq_n++] = {base, dim, dev};
+  return dev;
+}
+
+// Are the queued row tasks exactly the preparation of this launch's operands?  Expected, in queue order: one
+// rotation task per query head (destination = the head's query row, sources one after the other), one per KV head
+// for the new K row (cache row = last row of the head's K rows), one copy per KV head for the new V row.
+static bool match_prep(const std::vector<RowTask>& T, const AttnDecodeArgs& a, uint32_t G, uint32_t n_groups, AttdRowPrep* rp) {
+  const uint32_t D = a.head_dim, n_ops = a.n_ops;
+  if (T.size() != (size_t)n_ops + 2u * n_groups || a.row_size == 0) return false;
+  const RowTask &q0 = T[0], &k0 = T[n_ops], &v0 = T[n_ops + n_groups];
+  const uint32_t F = q0.flags;
+  if (!(F & 2u) || k0.flags != F || v0.flags != 0u) return false;
+  const uint64_t last = (uint64_t)(a.row_size - 1u) * D;
+  for (uint32_t h = 0; h < n_ops; h++) {
+    const RowTask& t = T[h];
+    if (t.flags != F || t.dim != D || t.pos != q0.pos || t.base != q0.base || t.cache != ROWT_NONE || t.w != q0.w ||
+        t.dst != a.ha[h] || (uint64_t)t.src != (uint64_t)q0.src + (uint64_t)h * D || (uint64_t)t.dst != (uint64_t)q0.dst + (uint64_t)h * D)
+      return false;
+  }
+  for (uint32_t gi = 0; gi < n_groups; gi++) {
+    const RowTask &t = T[n_ops + gi], &v = T[n_ops + n_groups + gi];
+    if (t.flags != F || t.dim != D || t.pos != q0.pos || t.base != q0.base || t.w != k0.w ||
+        (uint64_t)t.src != (uint64_t)k0.src + (uint64_t)gi * D || (uint64_t)t.cache != (uint64_t)a.hb[gi * G] + last)
+      return false;
+    if ((k0.dst == ROWT_NONE) != (t.dst == ROWT_NONE) || (t.dst != ROWT_NONE && (uint64_t)t.dst != (uint64_t)k0.dst + (uint64_t)gi * D))
+      return false;
+    if (v.flags != 0u || v.dim != D || v.dst != ROWT_NONE || v.w != ROWT_NONE ||
+        (uint64_t)v.src != (uint64_t)v0.src + (uint64_t)gi * D || (uint64_t)v.cache != (uint64_t)a.hv[gi * G] + last)
+      return false;
+    // the new rows lie in the fp16 copy
+    if ((uint64_t)t.cache < a.kv_shift || (uint64_t)v.cache < a.kv_shift) return false;
+  }
+  if ((F & 1u) && (q0.w == ROWT_NONE || k0.w == ROWT_NONE)) return false;
+  // What the launch reads (raw rows, norm weights) against what it writes (prepared rows, cache rows, score rows,
+  // outputs).  A prepared row may go back over its own raw row (the usual case); nothing else may meet.
+  struct Iv { uint64_t lo, n; int own; };   // own: > 0 marks a raw row / prepared row pair that may coincide
+  std::vector<Iv> rd, wr;
+  rd.push_back({v0.src, (uint64_t)n_groups * D, 0});
+  if (F & 1u) { rd.push_back({q0.w, D, 0}); rd.push_back({k0.w, D, 0}); }
+  for (uint32_t h = 0; h < n_ops; h++) { rd.push_back({T[h].src, D, 1 + (int)h}); wr.push_back({T[h].dst, D, 1 + (int)h}); }
+  for (uint32_t gi = 0; gi < n_groups; gi++) {
+    const RowTask &t = T[n_ops + gi], &v = T[n_ops + n_groups + gi];
+    rd.push_back({t.src, D, 1000 + (int)gi});
+    if (t.dst != ROWT_NONE) wr.push_back({t.dst, D, 1000 + (int)gi});
+    wr.push_back({t.cache, D, 0}); wr.push_back({v.cache, D, 0});
+  }
+  for (uint32_t h = 0; h < n_ops; h++) { wr.push_back({a.hc[h], a.row_size, 0}); wr.push_back({a.ho[h], D, 0}); }
+  auto meet = [](const Iv& x, const Iv& y) { return !(x.lo + x.n <= y.lo || y.lo + y.n <= x.lo); };
+  for (const Iv& w : wr)
+    for (const Iv& r : rd)
+      if (meet(w, r) && !(w.own && w.own == r.own && w.lo == r.lo)) return false;
+  for (size_t x = 0; x < wr.size(); x++)
+    for (size_t y = x + 1; y < wr.size(); y++)
+      if (meet(wr[x], wr[y])) return false;
+  const float* inv_freq = rope_inv_freq(q0.base, D);
+  if (!inv_freq) return false;
+  *rp = AttdRowPrep{F & 1u, q0.pos, q0.base, q0.src, k0.src, k0.dst, v0.src, (F & 1u) ? q0.w : 0u, (F & 1u) ? k0.w : 0u,
+                    nullptr, inv_freq};
+  return true;
 }
 
 bool launch_attn_decode(const AttnDecodeArgs& a, AttnPartials* ap, bool* left, int* rc) {
@@ -322,6 +562,12 @@ bool launch_attn_decode(const AttnDecodeArgs& a, AttnPartials* ap, bool* left, i
   }
   const uint32_t n_groups = n_ops / G;
   if (n_groups > ATTD_MAX_GROUPS) return false;
+  AttdRowPrep rp = {};
+  if (a.prep) {   // with the row preparation inside the launch, or no launch at all
+    if (!a.prep_done || (D != 128 && D != 256) || tuning("ADAMAH_ATTN_ROWPREP", 1) == 0 ||
+        !match_prep(*a.prep, a, G, n_groups, &rp))
+      return false;
+  }
 
   // Slices of the sequence.  Short sequences (at most one 16-row tile per wave when the chip holds
   // `target` waves): workgroups of 8 waves, one tile each, no prefetch; longer ones: 4 waves and as
@@ -348,12 +594,21 @@ bool launch_attn_decode(const AttnDecodeArgs& a, AttnPartials* ap, bool* left, i
   for (uint32_t gi = 0; gi < n_groups; gi++) { bs.kb[gi] = a.hb[gi * G]; bs.vb[gi] = a.hv[gi * G]; }
   // the slices are merged by the consumer (leave) or by the caller's merge kernel
   dim3 grid(n_splits, n_groups);
+  const AttdRowPrep* rpp = a.prep ? &rp : nullptr;
+  // the prepared queries wait behind the partials until the merge copies them to their rows
+  const uint64_t part_floats = (uint64_t)n_ops * n_splits * (D + 2);
+  if (a.prep && n_splits > 1) {
+    if (part_floats + (uint64_t)n_ops * D > g.attn_scratch_floats) return false;
+    rp.q_scratch = g.attn_scratch + part_floats;
+  }
   if (D == 64) launch_d<64>(G, nw, pf, grid, a, bs, n_splits, chunk);
-  else if (D == 128) launch_d<128>(G, nw, pf, grid, a, bs, n_splits, chunk);
-  else launch_d<256>(G, nw, pf, grid, a, bs, n_splits, chunk);
+  else if (D == 128) launch_d<128>(G, nw, pf, grid, a, bs, n_splits, chunk, nullptr, rpp);
+  else launch_d<256>(G, nw, pf, grid, a, bs, n_splits, chunk, nullptr, rpp);
+  if (a.prep) *a.prep_done = true;
   count_launch();
   *rc = check_launch();
-  *ap = AttnPartials{g.attn_scratch, *rc == 0 ? n_splits : 1u, D, n_ops, 0};
+  *ap = AttnPartials{g.attn_scratch, *rc == 0 ? n_splits : 1u, D, n_ops, 0, nullptr, 0, 0};
+  if (a.prep && n_splits > 1 && *rc == 0) { ap->q_src = rp.q_scratch; ap->q_dst = (*a.prep)[0].dst; ap->q_n = n_ops * D; }
   *left = leave;
   return true;
 }
@@ -368,6 +623,8 @@ static uint32_t* g_ext_buf = nullptr;
 static size_t g_ext_cap = 0;   // words
 
 void attn_decode_release() {
+  for (int i = 0; i < g_freq_n; i++) hipFree(g_freq[i].dev);
+  g_freq_n = 0;
   if (g_ext_buf) hipFree(g_ext_buf);
   g_ext_buf = nullptr;
   g_ext_cap = 0;

@@ -9,6 +9,7 @@
 #include <stdint.h>
 #include <stddef.h>
 #include <vector>
+#include <utility>
 
 // Error codes of the reference C ABI (adamah.c:24-28).
 #define ADAMAH_OK 0
@@ -21,6 +22,7 @@
 #define MAX_RES 65536          // reference: 2048; ids stay 32-bit so a larger table is invisible to callers
 #define MAX_PLANS 8
 #define MAX_PLAN_OPS 4096
+#define T_PARK_FLOATS 65536
 
 #define DTYPE_F32 0
 #define DTYPE_BF16 1
@@ -129,6 +131,7 @@ struct Ctx {
   int no_defer = 0;              // > 0 while an entry point runs on library-owned scratch handles
   uint64_t mem_gen = 0;          // counts host-to-device copies (with stats.dispatch: "has device memory changed?")
   uint32_t* sync_ctr = nullptr;  // device counters for last-workgroup epilogues, zero between launches
+  float* t_park = nullptr;       // T_PARK_FLOATS floats: a row on its way to a place that is still being read
   int deferred_err = 0;          // first failure of a queued op's launch; returned (once) by the next call that can
   uint64_t layout_gen = 0;       // counts events after which device pointers or offsets seen earlier may be stale:
                                  // a map created, destroyed or given new qparams / an fp16 KV range, a library
@@ -168,14 +171,19 @@ size_t launch_argmax_run(const std::vector<PendOp>& q, size_t i, int* rc);   // 
 int launch_argmax_direct(const PendOp& p);   // gemv_q.hip: one queued Q8 GEMV + argmax
 int launch_rmsnorm_v(const PendOp& p);
 bool row_op_deferrable(const PendOp& p);                                  // rowprep.hip
+// Element ranges (start, length) of the activation map a queued row op reads or writes; false: not known on the host.
+bool row_op_ranges(const PendOp& p, std::vector<std::pair<uint64_t, uint64_t>>* out);   // rowprep.hip
 size_t launch_row_run(const std::vector<PendOp>& q, size_t i, int* rc);   // rowprep.hip
 int launch_op2_v(const PendOp& p);
 // Attention (attention.hip): stand-alone launches of queued ops, and the fused form.  launch_attn
 // runs scores (when sc != nullptr) and softmax . V; with leave_partials it stops before the merge
 // of the sequence splits and reports their layout so that the consumer can merge them itself.
-struct AttnPartials { const float* base; uint32_t n_splits, value_dim, n_ops, out0; };
+// q_n > 0: the launch also prepared the token's queries and left them in scratch memory; whoever merges the
+// partials copies q_n floats from q_src to element q_dst of the map (the rows the rotation writes).
+struct AttnPartials { const float* base; uint32_t n_splits, value_dim, n_ops, out0; const float* q_src; uint32_t q_dst, q_n; };
 int launch_scores(const PendOp& sc);
-int launch_attn(const PendOp* sc, const PendOp& at, bool leave_partials, AttnPartials* ap);
+struct RowPrepCtx;   // attn_common.h: the row ops queued just before the pair, offered to the attention launch
+int launch_attn(const PendOp* sc, const PendOp& at, bool leave_partials, AttnPartials* ap, const RowPrepCtx* prep = nullptr);
 int launch_attn_combine(const PendOp& at, const AttnPartials& ap);
 bool attn_foldable(const PendOp& sc, const PendOp& at);
 size_t launch_attn_chunk(const std::vector<PendOp>& q, size_t i, int* rc);   // attn_prefill.hip

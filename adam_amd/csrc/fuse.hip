@@ -14,11 +14,13 @@
 //   GEMV(-> [g; u]); GEGLU/SWIGLU(g, u -> t)              -> GEMV over paired rows that also stores t
 //   GEMV(x, W1 -> y1); GEMV(x, W2 -> y2), W2 after W1, y2 after y1 -> one GEMV over the stacked rows
 //   (scores; softmax . V) of tokens t, t+1, ... over one cache      -> one causal launch (attn_prefill.hip)
-//   RoPE(q); RoPE(k) | QK-norm+RoPE; row copy (KV append)  -> one launch of row tasks (rowprep.hip)
+//   RoPE(q); RoPE(k) | QK-norm+RoPE; row copy (KV append)  -> one launch of row tasks (rowprep.hip), or, directly
+//                                                             before one token's decode attention, done by that launch
 //
 // Every folded op still stores its own result where it would have stored it alone, so the contents
 // of the maps after a batch do not depend on whether anything was folded.
 #include "gemv_common.h"
+#include "attn_common.h"
 #include <stdlib.h>
 
 namespace adamah {
@@ -115,6 +117,61 @@ static bool gemv_writes_clear(const PendOp& gp, const uint64_t (*rg)[2], int n_r
   return clear_of_all(dst[0], 1);
 }
 
+// May the queued op read or write elements [lo, lo + n) of activation map `map`?  Conservative: true whenever its
+// operands are not known on the host.
+static bool op_touches(const PendOp& p, uint32_t map, uint64_t lo, uint64_t n) {
+  if (p.map_act != map && p.map_wt != map) return false;
+  auto hit = [&](uint64_t a, uint64_t len) { return !disjoint(a, len, lo, n); };
+  auto rows = [&](uint32_t handle, uint32_t count, uint64_t len, bool* known) {
+    const uint32_t* h = res_host(handle, count);
+    if (!h) { *known = false; return true; }
+    for (uint32_t i = 0; i < count; i++) if (hit(h[i], len)) return true;
+    return false;
+  };
+  bool known = true;
+  switch (p.kind) {
+    case PK_RMSNORM:
+      return (p.map_act == map && (hit(p.a, p.n) || hit(p.c, p.n) || (p.op == 1 && hit(p.d, p.n)))) || (p.map_wt == map && hit(p.b, p.n));
+    case PK_GEMV:
+      return p.map_act == map && (hit(p.a, p.k) || hit(p.c, p.n));
+    case PK_OP2:
+      return p.map_act == map && (hit(p.a, p.n) || hit(p.b, p.n) || hit(p.c, p.n));
+    case PK_SCORES:
+      return rows(p.h[0], p.rpg, p.k, &known) || rows(p.h[1], p.rpg, (uint64_t)p.n * p.k, &known) || rows(p.h[2], p.rpg, p.n, &known);
+    case PK_ATTN:
+      return rows(p.h[0], p.rpg, p.n, &known) || rows(p.h[1], p.rpg, (uint64_t)p.n * p.k, &known) || rows(p.h[2], p.rpg, p.k, &known);
+    case PK_ROPE: case PK_QKNR: case PK_ROWCOPY: {
+      std::vector<std::pair<uint64_t, uint64_t>> rg;
+      if (!row_op_ranges(p, &rg)) return true;
+      for (const auto& r : rg) if (hit(r.first, r.second)) return true;
+      return false;
+    }
+    default: return true;
+  }
+}
+
+// In-place t of a folded norm + residual pair (PRO_NORM2): the first later GEMV of the queue, from `from` on, that
+// can put the parked row in place, i.e. a plain store GEMV such that neither it, nor the ops that may share its
+// launch, nor anything queued before it touches the row.  n: none.
+static size_t find_unparker(const std::vector<PendOp>& q, size_t from, uint32_t map, uint64_t lo, uint64_t len) {
+  const size_t n = q.size();
+  for (size_t j = from; j < n; j++) {
+    if (op_touches(q[j], map, lo, len)) return n;
+    if (q[j].kind != PK_GEMV || q[j].map_act != map) continue;
+    // what may ride on the same launch: GEMVs stacked behind it, one element-wise op after them
+    size_t e = j + 1;
+    while (e < n && q[e].kind == PK_GEMV) { if (op_touches(q[e], map, lo, len)) return n; e++; }
+    if (e < n && q[e].kind == PK_OP2 && op_touches(q[e], map, lo, len)) return n;
+    return j;
+  }
+  return n;
+}
+
+__global__ void __launch_bounds__(256) k_copy_f32(float* data, const float* src, uint32_t dst, uint32_t n) {
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  if (i < n) data[(uint64_t)dst + i] = src[i];
+}
+
 static int launch_gemv(const PendOp& gp, const GemvFuse* fz) {
   Map* ma = get_f32_map(gp.map_act);
   Map* mw = get_map(gp.map_wt);
@@ -142,20 +199,45 @@ void flush_pending() {
   size_t i = 0;
   // the queued ops have returned ADAMAH_OK already: the first launch that fails is kept for the next call
   auto keep = [](int rc) { if (rc != ADAMAH_OK && !g.deferred_err) g.deferred_err = rc; };
+  // a row parked by a PRO_NORM2 launch, and the queue index of the GEMV that will put it in place
+  struct { bool active; size_t at; uint32_t map, dst, len; } park = {false, 0, 0, 0, 0};
+  auto unpark_now = [&]() {   // not taken by the launch it was meant for: a copy of its own
+    if (!park.active) return;
+    park.active = false;
+    Map* m = get_f32_map(park.map);
+    if (!m) { keep(ADAMAH_ERR_INVALID); return; }
+    k_copy_f32<<<cdiv(park.len, 256), 256, 0, g.stream>>>((float*)m->buf, g.t_park, park.dst, park.len);
+    count_launch();
+    keep(check_launch());
+  };
   while (i < n) {
+    if (park.active && i > park.at) unpark_now();
+    RowPrepCtx prep = {&q, i, {}};
+    bool have_prep = false;
+    if (q[i].kind == PK_ROPE || q[i].kind == PK_QKNR || q[i].kind == PK_ROWCOPY) {
+      // Rotation of the new Q / K rows and the KV append.  When the run is followed directly by the decode attention
+      // of one token, it is offered to that launch, which does the preparation of its own operands itself;
+      // otherwise: one launch for the run.
+      bool alone = false;
+      const size_t used = build_row_run(q, i, &prep.tasks, &alone);
+      const size_t s = i + used;
+      if (used && !alone && s + 1 < n && q[s].map_act == q[i].map_act && attn_foldable(q[s], q[s + 1]) &&
+          !(s + 2 < n && q[s + 2].kind == PK_SCORES)) {
+        have_prep = true;
+        i = s;
+      } else {
+        int rc = 0;
+        i += launch_row_run(q, i, &rc);
+        keep(rc);
+        continue;
+      }
+    }
     const PendOp& p = q[i];
     auto is_gemv = [&](size_t j) {   // a launch of the int8 matrix-instruction kernel (Q8 argmax ops are not)
       return j < n && (q[j].kind == PK_GEMV || (q[j].kind == PK_ARGMAX && q[j].op != (uint32_t)FMT_Q8_B16));
     };
     size_t gi = n;    // the GEMV this group is built around, if any
     GemvFuse fz = {};
-    if (p.kind == PK_ROPE || p.kind == PK_QKNR || p.kind == PK_ROWCOPY) {
-      // rotation of the new Q / K rows and the KV append: one launch for the run
-      int rc = 0;
-      i += launch_row_run(q, i, &rc);
-      keep(rc);
-      continue;
-    }
     if (p.kind == PK_GEMM) {
       // Matmuls over the same few rows whose weight matrices lie back to back: one launch over the stacked
       // rows, every result where its own op puts it.  All of them read the rows as they were before the
@@ -211,7 +293,7 @@ void flush_pending() {
       if (used) { i += used; continue; }
       if (p.op == (uint32_t)FMT_Q8_B16) { keep(launch_argmax_direct(p)); i++; continue; }
     }
-    if (p.kind == PK_SCORES) {
+    if (p.kind == PK_SCORES && !have_prep) {
       // a prefill chunk: the attention of consecutive tokens over one growing cache, one launch
       int rc = 0;
       size_t used = launch_attn_chunk(q, i, &rc);
@@ -235,11 +317,15 @@ void flush_pending() {
         const uint32_t* oh = res_host(at.h[2], at.rpg);
         fold = oh && gp.a == oh[0] && gp.k == at.rpg * at.k && (at.k & 7u) == 0 && disjoint(gp.c, gp.n, gp.a, gp.k);
         for (uint32_t h = 1; fold && h < at.rpg; h++) fold = oh[h] == oh[0] + h * at.k;
+        // a merging GEMV may also have to put the token's prepared queries in place (workgroup 0, while others
+        // already store result rows): its results must lie clear of those rows
+        if (fold && have_prep && !prep.tasks.empty()) fold = disjoint(gp.c, gp.n, prep.tasks[0].dst, (uint64_t)at.rpg * at.k);
       }
-      AttnPartials ap = {nullptr, 1, 0, 0, 0};
-      keep(launch_attn(sc, at, fold, &ap));
+      AttnPartials ap = {nullptr, 1, 0, 0, 0, nullptr, 0, 0};
+      keep(launch_attn(sc, at, fold, &ap, have_prep ? &prep : nullptr));
       if (fold && ap.n_splits > 1) {   // partials left for the GEMV to merge
         fz.pro = PRO_COMBINE; fz.c_partial = ap.base; fz.c_splits = ap.n_splits; fz.c_vd = at.k;
+        fz.c_qsrc = ap.q_src; fz.c_qdst = ap.q_dst; fz.c_qn = ap.q_n;
         fz.p_dst = q[ai + 1].a;
         gi = ai + 1;
       }
@@ -254,13 +340,17 @@ void flush_pending() {
                          gp.a == m.c && gp.k == m.n;
       // t may overwrite the residual (ticket-protected) but nothing else that is read; x must not
       // overwrite any input
-      const bool safe = disjoint(p.c, p.n, p.a, p.n) && (p.c == p.d || disjoint(p.c, p.n, p.d, p.n)) &&
-                        disjoint(m.c, m.n, p.a, p.n) && disjoint(m.c, m.n, p.d, p.n) && disjoint(m.c, m.n, p.c, p.n);
+      bool safe = disjoint(p.c, p.n, p.a, p.n) && (p.c == p.d || disjoint(p.c, p.n, p.d, p.n)) &&
+                  disjoint(m.c, m.n, p.a, p.n) && disjoint(m.c, m.n, p.d, p.n) && disjoint(m.c, m.n, p.c, p.n);
+      // norm weights that live in the activation map: neither t nor x may land on them
+      if (p.map_wt == p.map_act) safe = safe && disjoint(p.c, p.n, p.b, p.n) && disjoint(m.c, m.n, p.b, p.n);
+      if (m.map_wt == p.map_act) safe = safe && disjoint(p.c, p.n, m.b, m.n) && disjoint(m.c, m.n, m.b, m.n);
       const uint64_t rd[4][2] = {{p.a, p.n}, {p.d, p.n}, {p.c, p.n}, {m.c, m.n}};   // src, residual, t, x
       if (chain && safe && mw1 && mw2 && (p.n & 31u) == 0 && row_fits(gp) && g.sync_ctr && gemv_writes_clear(gp, rd, 4)) {
         fz.pro = PRO_NORM2; fz.p_src = p.a; fz.p_src2 = p.b; fz.p_eps = p.eps; fz.p_wt = (const float*)mw1->buf;
         fz.p_res = p.d; fz.p_tdst = p.c; fz.p_w2 = m.b; fz.p_eps2 = m.eps; fz.p_wt2 = (const float*)mw2->buf;
         fz.p_dst = m.c; fz.counter = g.sync_ctr;
+        fz.t_mode = p.c == p.d ? 0u : 1u;   // t clear of the residual (and, `safe`, of the source): stored at once
         gi = i + 2;
       }
     } else if (p.kind == PK_RMSNORM && p.op == 0 && is_gemv(i + 1)) {
@@ -284,6 +374,7 @@ void flush_pending() {
     // gate, up issued one after the other): one launch over the stacked rows.  All of them read the
     // activations as they were before the first, so no result may overlap what the launch reads.
     PendOp gp = q[gi];
+    const size_t gi0 = gi;   // queue index of the group's first GEMV
     if (gp.kind == PK_GEMV) {
       while (gi + 1 < n && q[gi + 1].kind == PK_GEMV) {
         const PendOp& nx = q[gi + 1];
@@ -294,6 +385,7 @@ void flush_pending() {
         bool clear = nn <= 0xFFFFFFFFull && disjoint(gp.c, nn, gp.a, gp.k);
         if (fz.pro == PRO_RMSNORM || fz.pro == PRO_NORM2) clear = clear && disjoint(gp.c, nn, fz.p_src, gp.k);
         if (fz.pro == PRO_NORM2) clear = clear && disjoint(gp.c, nn, fz.p_res, gp.k) && disjoint(gp.c, nn, fz.p_tdst, gp.k);
+        if (fz.pro == PRO_COMBINE && fz.c_qn) clear = clear && disjoint(gp.c, nn, fz.c_qdst, fz.c_qn);
         if (!clear) break;
         gp.n = (uint32_t)nn;
         gi++;
@@ -307,6 +399,9 @@ void flush_pending() {
       bool clear = disjoint(e.c, e.n, gp.c, gp.n) && disjoint(e.c, e.n, gp.a, gp.k);
       if (fz.pro) clear = clear && disjoint(e.c, e.n, fz.p_src, gp.k);
       if (fz.pro == PRO_NORM2) clear = clear && disjoint(e.c, e.n, fz.p_res, gp.k) && disjoint(e.c, e.n, fz.p_tdst, gp.k);
+      // the prepared queries workgroup 0 puts in place: neither written nor read (a residual) by the epilogue
+      if (fz.pro == PRO_COMBINE && fz.c_qn)
+        clear = clear && disjoint(e.c, e.n, fz.c_qdst, fz.c_qn) && disjoint(e.a, e.n, fz.c_qdst, fz.c_qn) && disjoint(e.b, e.n, fz.c_qdst, fz.c_qn);
       if (e.op == 0 && e.n == gp.n && (e.a == gp.c) != (e.b == gp.c)) {
         const uint32_t r = e.a == gp.c ? e.b : e.a;   // the residual may be updated in place
         bool ok = clear && (r == e.c || disjoint(r, e.n, e.c, e.n));
@@ -319,9 +414,19 @@ void flush_pending() {
         last = gi + 1;
       }
     }
-    keep(launch_gemv(gp, (fz.pro || fz.e_mode) ? &fz : nullptr));
+    if (park.active && park.at <= last) {
+      if (park.at == gi0 && gp.kind == PK_GEMV) { fz.d_src = g.t_park; fz.d_dst = park.dst; fz.d_n = park.len; park.active = false; }
+      else unpark_now();
+    }
+    if (fz.pro == PRO_NORM2 && fz.t_mode == 0u && !park.active && g.t_park && gp.k <= T_PARK_FLOATS &&
+        tuning("ADAMAH_NORM2_PARK", 1) != 0) {
+      const size_t at = find_unparker(q, last + 1, gp.map_act, fz.p_tdst, gp.k);
+      if (at < n) { fz.t_mode = 2u; fz.t_park = g.t_park; park = {true, at, gp.map_act, fz.p_tdst, gp.k}; }
+    }
+    keep(launch_gemv(gp, (fz.pro || fz.e_mode || fz.d_n) ? &fz : nullptr));
     i = last + 1;
   }
+  unpark_now();
 }
 
 }  // namespace adamah

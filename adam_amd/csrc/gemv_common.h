@@ -84,11 +84,25 @@ struct GemvFuse {
   uint32_t p_res, p_tdst, p_w2;   // residual, destination of t, weight w2 (element offset in p_wt2)
   float p_eps2;
   const float* p_wt2;
-  uint32_t* counter;        // PRO_NORM2: zero-initialised device counter, left at zero
+  // t usually goes back over the residual, which every workgroup reads.  Where it is stored:
+  //   t_mode 0: by whichever workgroup draws the last ticket of `counter` (zero-initialised, left at zero);
+  //   t_mode 1: by workgroup 0 at once (p_tdst lies clear of everything the launch reads);
+  //   t_mode 2: workgroup 0 parks it at t_park, and a later launch that does not touch p_tdst copies it there
+  //             (its d_src / d_dst / d_n): no atomic, whose reply would hold up the drawing wave's weight loads
+  uint32_t* counter;
+  uint32_t t_mode;
+  float* t_park;
+  // any prologue: d_n > 0: workgroup 0 copies d_n floats from d_src to element d_dst of the activation map
+  const float* d_src;
+  uint32_t d_dst, d_n;
   // PRO_COMBINE: x = merge of the split-sequence attention partials, heads side by side  -> p_dst
   //   partial[(head * c_splits + s) * (c_vd + 2)] = {max, sum, values[c_vd]}
   const float* c_partial;
   uint32_t c_splits, c_vd;
+  //   c_qn > 0: the attention launch also left the token's prepared queries in scratch memory: c_qn floats from
+  //   c_qsrc go to element c_qdst (workgroup 0)
+  const float* c_qsrc;
+  uint32_t c_qdst, c_qn;
   // EPIX_ADD:            e_dst[row] = e_res[row] + y[row]
   // EPIX_GEGLU / SWIGLU: the matrix is [gate rows; up rows], e_dst[i] = act(y[i]) * y[N/2 + i]
   uint32_t e_mode;

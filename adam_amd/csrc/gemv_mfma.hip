@@ -237,6 +237,8 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
     // Folded merge of the attention partials (same arithmetic as the stand-alone merge kernel):
     // M = max m_s, w_s = e^(m_s - M), L = sum l_s w_s, x = sum_s o_s w_s / L, per head.
     first_loads();
+    if (blockIdx.x == 0)
+      for (uint32_t i = tid; i < fz.c_qn; i += nthr) act_out[(uint64_t)fz.c_qdst + i] = fz.c_qsrc[i];
     const uint32_t stride = fz.c_vd + 2u;
     for (uint32_t i0 = 0; i0 < nw; i0 += nthr) {
       const uint32_t i = i0 + tid, ic = min(i, nw - 1u);
@@ -315,7 +317,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       // t usually goes back into `res` (residual updated in place), which other workgroups may not
       // have read yet, so it is stored by whichever workgroup draws the last ticket.  The ticket is
       // drawn here and looked at after staging, so nobody waits for the atomic's round trip.
-      if (wave == 0 && lane == 0) ticket = atomicAdd(fz.counter, 1u);
+      if (fz.t_mode == 0u && wave == 0 && lane == 0) ticket = atomicAdd(fz.counter, 1u);
       float ss2 = 0.f;
 #pragma unroll
       for (uint32_t u = 0; u < PRO_WPT; u++)
@@ -324,8 +326,14 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
           for (int k = 0; k < 8; k++) {
             v[u][k] = v[u][k] * nrm * wv[u][k] + rv[u][k];
             if (live[u]) ss2 = fmaf(v[u][k], v[u][k], ss2);
-            v[u][k] *= w2v[u][k];
           }
+          if (fz.t_mode != 0u && blockIdx.x == 0 && live[u]) {   // t: in place at once, or parked for a later launch
+            float* td = fz.t_mode == 1u ? act_out + fz.p_tdst : fz.t_park;
+            f4u_t* o = (f4u_t*)(td + (uint64_t)(u * nthr + tid) * 8u);
+            o[0] = (f4u_t){v[u][0], v[u][1], v[u][2], v[u][3]}; o[1] = (f4u_t){v[u][4], v[u][5], v[u][6], v[u][7]};
+          }
+#pragma unroll
+          for (int k = 0; k < 8; k++) v[u][k] *= w2v[u][k];
         }
       ss_last = ss2;
     } else {
@@ -465,7 +473,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
   // it.  Looked at only here, after the workgroup's own rows, so that nobody waits for the atomic; the
   // whole workgroup then recomputes t for the row.
   auto finish_norm2 = [&]() {
-    if (PRO != PRO_NORM2) return;
+    if (PRO != PRO_NORM2 || fz.t_mode != 0u) return;
     if (wave == 0 && lane == 0) red_i[0] = ticket;
     __syncthreads();
     if (red_i[0] != gridDim.x - 1u) return;
@@ -554,6 +562,9 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
     if (!more) break;
   }
   finish_norm2();
+  // a row an earlier launch parked: to its place (nothing in this launch touches it)
+  if (blockIdx.x == 0)
+    for (uint32_t i = tid; i < fz.d_n; i += nthr) const_cast<float*>(act)[(uint64_t)fz.d_dst + i] = fz.d_src[i];
 }
 
 // ---- host side -----------------------------------------------------------------------------------

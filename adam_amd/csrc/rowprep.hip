@@ -12,29 +12,13 @@
 // other overlap between a task and an earlier one ends the run, so tasks of one launch are
 // independent.  The arithmetic and its order are those of the stand-alone kernels, so results do not
 // depend on whether a run was merged.
-#include "common.h"
+#include "attn_common.h"
 #include "../../include/adamah_hip.h"
 #include <algorithm>
 
 namespace adamah {
 
-#define ROWT_MAX 64u
-#define ROWT_NONE 0xFFFFFFFFu
-struct RowTask {
-  uint32_t src, dst, cache, w;   // element offsets; dst / cache / w may be ROWT_NONE
-  uint32_t dim, pos, flags;      // flags: 1 = RMSNorm (eps 1e-6), 2 = RoPE
-  float base;
-};
 struct RowTasks { RowTask t[ROWT_MAX]; };
-
-// Same arithmetic as rope_cs in norm_rope.hip.
-__device__ __forceinline__ void rope_cs2(uint32_t i, uint32_t dim, uint32_t pos, float base, float* c, float* s) {
-  const float e = (float)(2u * i) / (float)dim;
-  const float p = (float)pow((double)base, (double)e);
-  const float angle = (float)pos * (1.0f / p);
-  *c = cosf(angle);
-  *s = sinf(angle);
-}
 
 __device__ __forceinline__ void store_row_elem(float* act, __half* kv16, uint64_t kv_start, uint64_t kv_count,
                                                uint32_t dst, uint32_t cache, uint32_t i, float v) {
@@ -136,6 +120,19 @@ bool row_op_deferrable(const PendOp& p) {
   return m && expand(p, m, &ts) && !ts.empty() && ts.size() <= ROWT_MAX;
 }
 
+bool row_op_ranges(const PendOp& p, std::vector<std::pair<uint64_t, uint64_t>>* out) {
+  Map* m = get_f32_map(p.map_act);
+  std::vector<RowTask> ts;
+  if (!m || !expand(p, m, &ts)) return false;
+  for (const RowTask& t : ts) {
+    out->push_back({t.src, t.dim});
+    if (t.dst != ROWT_NONE) out->push_back({t.dst, t.dim});
+    if (t.cache != ROWT_NONE) out->push_back({t.cache, t.dim});
+    if (t.w != ROWT_NONE) out->push_back({t.w, t.dim});
+  }
+  return true;
+}
+
 static int launch_tasks(Map* m, const std::vector<RowTask>& run) {
   if (run.empty()) return ADAMAH_OK;
   RowTasks ts;
@@ -145,17 +142,20 @@ static int launch_tasks(Map* m, const std::vector<RowTask>& run) {
   return check_launch();
 }
 
-// Launches the run of row ops that starts at q[i]; returns how many queue entries it consumed.
-size_t launch_row_run(const std::vector<PendOp>& q, size_t i, int* rc) {
-  *rc = ADAMAH_OK;
+// The merged tasks of the run of row ops that starts at q[i]; returns how many queue entries the run covers.  0:
+// the first op cannot be expanded on the host.  *alone: q[i] by itself does not fit one launch (run holds its tasks,
+// which are independent of each other).
+size_t build_row_run(const std::vector<PendOp>& q, size_t i, std::vector<RowTask>* out, bool* alone) {
+  *alone = false;
+  out->clear();
   Map* m = get_f32_map(q[i].map_act);
-  if (!m) { *rc = ADAMAH_ERR_INVALID; return 1; }
+  if (!m) return 0;
   std::vector<RowTask> run, add;
   size_t j = i;
   for (; j < q.size(); j++) {
     const PendOp& p = q[j];
     if ((p.kind != PK_ROPE && p.kind != PK_QKNR && p.kind != PK_ROWCOPY) || p.map_act != q[i].map_act) break;
-    if (!expand(p, m, &add)) { if (j == i) { *rc = ADAMAH_ERR_INVALID; return 1; } break; }
+    if (!expand(p, m, &add)) { if (j == i) return 0; break; }
     // every new task against every task already in the run
     std::vector<RowTask> next = run;
     bool ok = run.size() + add.size() <= ROWT_MAX || p.kind == PK_ROWCOPY;
@@ -189,17 +189,30 @@ size_t launch_row_run(const std::vector<PendOp>& q, size_t i, int* rc) {
       if (ok && !merged) next.push_back(nt);
     }
     if (!ok || next.size() > ROWT_MAX) {
-      if (j == i) {   // a single op that does not fit one launch: task by task in chunks (tasks of one op are independent)
-        for (size_t a = 0; a < add.size() && *rc == ADAMAH_OK; a += ROWT_MAX)
-          *rc = launch_tasks(m, std::vector<RowTask>(add.begin() + a, add.begin() + std::min(add.size(), a + (size_t)ROWT_MAX)));
-        return 1;
-      }
+      if (j == i) { *alone = true; *out = add; return 1; }
       break;
     }
     run.swap(next);
   }
-  *rc = launch_tasks(m, run);
+  *out = run;
   return j - i;
+}
+
+// Launches the run of row ops that starts at q[i]; returns how many queue entries it consumed.
+size_t launch_row_run(const std::vector<PendOp>& q, size_t i, int* rc) {
+  *rc = ADAMAH_OK;
+  Map* m = get_f32_map(q[i].map_act);
+  std::vector<RowTask> run;
+  bool alone = false;
+  const size_t used = build_row_run(q, i, &run, &alone);
+  if (!m || used == 0) { *rc = ADAMAH_ERR_INVALID; return 1; }
+  if (alone) {   // a single op that does not fit one launch: task by task in chunks (tasks of one op are independent)
+    for (size_t a = 0; a < run.size() && *rc == ADAMAH_OK; a += ROWT_MAX)
+      *rc = launch_tasks(m, std::vector<RowTask>(run.begin() + a, run.begin() + std::min(run.size(), a + (size_t)ROWT_MAX)));
+    return 1;
+  }
+  *rc = launch_tasks(m, run);
+  return used;
 }
 
 }  // namespace adamah

@@ -354,8 +354,11 @@ int adamah_init_ex(uint64_t hot_bytes, uint64_t cold_bytes) {
   g.res_next = 1;
   g.attn_scratch_floats = (size_t)4 << 20;   // 16 MiB of split-KV partials
   HIPCHK(hipMalloc((void**)&g.attn_scratch, g.attn_scratch_floats * sizeof(float)));
-  HIPCHK(hipMalloc((void**)&g.sync_ctr, 1024));   // [0..63] GEMV prologues, [64..191] attention groups
+  // counters of the GEMV prologues (1 KiB), then the row a folded norm + residual parks until a later launch puts
+  // it in place (T_PARK_FLOATS floats)
+  HIPCHK(hipMalloc((void**)&g.sync_ctr, 1024 + (size_t)T_PARK_FLOATS * 4));
   HIPCHK(hipMemsetAsync(g.sync_ctr, 0, 1024, g.stream));
+  g.t_park = (float*)((uint8_t*)g.sync_ctr + 1024);
   if (int r = topk_noalloc_setup(g.device)) return r;
   g.pend.clear();
   g.batch_depth = 0; g.fusion_enabled = 0; g.scheduler_mode = 0; g.active_dtype = 0;
@@ -387,6 +390,7 @@ void adamah_shutdown(void) { ADAMAH_API();
   g.attn_scratch = nullptr;
   if (g.sync_ctr) hipFree(g.sync_ctr);
   g.sync_ctr = nullptr;
+  g.t_park = nullptr;
   gemm_q4_mfma_release();
   topk_fused_release();
   sampling_release();

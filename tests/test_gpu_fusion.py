@@ -322,3 +322,138 @@ def test_kv_prep_run_equals_separate_ops(hip, style, Hq, Hkv, d, pos, hazard):
         assert launches == 1          # rotation(s) and append shared one launch
     elif hazard in ("rope_after_copy", "shifted_source"):
         assert launches >= 2          # the dependent op was kept out of the first launch
+
+
+# ---- the same preparation done by the decode attention launch itself ---------------------------------
+def _prep_attn_case(g, style, Hq, Hkv, d, ctx, seed, variant=None, project=False):
+    """One decode step's attention inputs, in one batch: rotation of the new Q / K rows (in place), KV append, scores,
+    softmax . V (and optionally a Q4 projection of the heads' outputs).  Layout: q | k | v | norm weights | score rows |
+    outputs | y | KV cache [K heads | V heads] of ctx + 3 rows each (fp16 mirrored); the cache rows from the new one on
+    hold NaN until the append writes them."""
+    rng = np.random.default_rng(seed)
+    cap, gs, pos, N = ctx + 3, Hq // Hkv, ctx - 1, 256
+    qn, kn = Hq * d, Hkv * d
+    q0, k0, v0, w0 = 5, 5 + qn, 5 + qn + kn, 5 + qn + 2 * kn
+    sc0 = w0 + 2 * d
+    out0 = sc0 + Hq * ctx
+    y0 = out0 + qn
+    kv_start = (y0 + N + d - 1) // d * d
+    step = cap * d
+    total = kv_start + 2 * Hkv * step
+    f32map(g, 0, total, None)
+    put(g, 0, q0, np.concatenate([rng.standard_normal(qn + 2 * kn), rng.uniform(0.5, 1.5, 2 * d)]).astype(np.float32))
+    g.kv_cache_fp16(0, kv_start, 2 * Hkv * step)
+    for h in range(2 * Hkv):
+        rows = rng.standard_normal((cap, d)).astype(np.float32)
+        rows[pos:] = np.nan
+        put(g, 0, kv_start + h * step, rows)
+    if project:
+        load_qtensor(g, 1, make_weights(N, qn, 41))
+    spec = []
+    for gi in range(Hkv):
+        spec += [gi, kv_start // d + gi * cap, gi + Hkv, kv_start // d + (Hkv + gi) * cap]
+    heads = np.arange(Hq) // gs
+    hq, hk = up(g, [q0]), up(g, [k0])
+    q_rows, k_rows = up(g, q0 + np.arange(Hq) * d), up(g, k0 + np.arange(Hkv) * d)
+    s_rows, o_rows = up(g, sc0 + np.arange(Hq) * ctx), up(g, out0 + np.arange(Hq) * d)
+    if variant == "scores_over_raw_v":            # the score rows start on the raw V row: the launch must not read it late
+        s_rows = up(g, np.concatenate([[v0], sc0 + np.arange(1, Hq) * ctx]))
+    g.batch_begin()
+    if style == "rope":
+        g.map_rope_dev(0, hq, hq, 1, Hq, d, pos, 5e5)
+        if variant != "k_not_rotated":
+            g.map_rope_dev(0, hk, hk, 1, Hkv, d, pos if variant != "other_position" else pos + 1, 5e5)
+    else:
+        g.map_qk_norm_rope_x_dev(0, 0, q_rows, up(g, [w0] * Hq), k_rows, up(g, [w0 + d] * Hkv), up(g, [q0]), Hq, d, Hkv, d, pos, 1e6)
+    g.map_row_copy_offset_dev(0, up(g, spec), up(g, [k0]), pos, 2 * Hkv, d)
+    g.map_matmul_t_dev(0, q_rows, up(g, kv_start + heads * step), s_rows, 1, d, ctx, Hq)
+    g.map_attn_softmax_value_dev(0, s_rows, up(g, kv_start + (Hkv + heads) * step), o_rows, Hq, ctx, d, float(1 / np.sqrt(d)), 0.0)
+    if project:
+        g.map_matmul_t_xq4_dev(0, 1, up(g, [out0]), up(g, [0]), up(g, [y0]), 1, qn, N)
+    g.batch_end()
+    launches = g.get_last_barrier_count() if hasattr(g, "get_last_barrier_count") else None
+    m = read(g, 0, 0, total)
+    # the untouched NaN rows of the cache (beyond the new row) stay out of the comparison of values
+    keep = np.ones(total, bool)
+    for h in range(2 * Hkv):
+        keep[kv_start + h * step + (pos + 1) * d: kv_start + (h + 1) * step] = False
+    return m, keep, launches
+
+
+@pytest.mark.parametrize("style,Hq,Hkv,d,ctx,project", [("rope", 32, 8, 128, 4096, False), ("rope", 32, 8, 128, 4096, True),
+                                                        ("rope", 8, 2, 128, 17, False), ("rope", 8, 8, 128, 300, True),
+                                                        ("qknr", 4, 1, 256, 612, True), ("qknr", 8, 4, 128, 1, False),
+                                                        ("qknr", 16, 2, 256, 2500, False)])
+def test_kv_prep_inside_the_attention_launch(hip, monkeypatch, style, Hq, Hkv, d, ctx, project):
+    note(f"kv prep in attention {style} {Hq}/{Hkv}x{d} ctx={ctx} project={project}")
+    inside, keep, n_in = _prep_attn_case(hip, style, Hq, Hkv, d, ctx, 19, project=project)
+    monkeypatch.setenv("ADAMAH_ATTN_ROWPREP", "0")
+    apart, _, n_out = _prep_attn_case(hip, style, Hq, Hkv, d, ctx, 19, project=project)
+    monkeypatch.delenv("ADAMAH_ATTN_ROWPREP")
+    assert n_in == n_out - 1                      # the preparation cost no launch of its own
+    assert not np.isnan(inside[keep]).any()
+    assert np.array_equal(inside.view(np.uint32), apart.view(np.uint32))
+    want, _, _ = _prep_attn_case(oracle.init(), style, Hq, Hkv, d, ctx, 19, project=project)
+    assert rel_l2(inside[keep], want[keep]) < (TOL if project else 1e-5)
+    # a second step on the same stream: the tickets of the first were handed back
+    again, _, _ = _prep_attn_case(hip, style, Hq, Hkv, d, ctx, 19, project=project)
+    assert np.array_equal(inside.view(np.uint32), again.view(np.uint32))
+
+
+@pytest.mark.parametrize("variant", ["k_not_rotated", "other_position", "scores_over_raw_v"])
+def test_kv_prep_that_is_not_the_attention_s_own_stays_a_launch(hip, monkeypatch, variant):
+    """Row ops before the pair that are not exactly the preparation of its operands (or whose rows the pair writes)."""
+    note(f"kv prep not folded: {variant}")
+    got, keep, n_in = _prep_attn_case(hip, "rope", 8, 2, 128, 200, 23, variant=variant)
+    monkeypatch.setenv("ADAMAH_ATTN_ROWPREP", "0")
+    apart, _, n_out = _prep_attn_case(hip, "rope", 8, 2, 128, 200, 23, variant=variant)
+    monkeypatch.delenv("ADAMAH_ATTN_ROWPREP")
+    assert n_in == n_out
+    assert np.array_equal(got.view(np.uint32), apart.view(np.uint32))
+    want, _, _ = _prep_attn_case(oracle.init(), "rope", 8, 2, 128, 200, 23, variant=variant)
+    assert rel_l2(got[keep], want[keep]) < 1e-5
+
+
+# ---- the in-place row of a folded norm + residual pair, parked until a later GEMV puts it in place ----
+def _norm2_then(g, s, qt, then):
+    """norm + residual (in place unless then == 'apart'), norm, GEMV in one batch, followed by `then`:
+    'gemv': a second GEMV that does not touch the residual (puts the parked row in place);
+    'gemv_reads_row': a second GEMV whose activations are that row; 'op_reads_row': an add over it, then the GEMV;
+    'apart': the first norm's result goes to its own place; 'nothing': the batch ends."""
+    K, N = s.K, s.N
+    t_dst = "src2" if then == "apart" else "resk"
+    g.batch_begin()
+    g.map_rmsnorm_add_dev(0, s.h(g, "src"), s.h(g, "nw"), s.h(g, "resk"), s.h(g, t_dst), 1, K, 1e-6)
+    g.map_rmsnorm_dev(0, s.h(g, t_dst), s.h(g, "nwk"), s.h(g, "x"), 1, K, 1e-5)
+    g.map_matmul_t_xq4_dev(0, 1, s.h(g, "x"), up(g, [0]), s.h(g, "y"), 1, K, N)
+    if then == "op_reads_row":
+        g.map_op2_dev(0, A.OP_ADD, s.run(g, "resk", K), s.run(g, "x", K), s.run(g, "src2", K), K)
+    if then != "nothing":
+        second_x = "resk" if then == "gemv_reads_row" else "x"
+        g.map_matmul_t_xq4_dev(0, 1, s.h(g, second_x), up(g, [0]), s.h(g, "dst"), 1, K, N)
+    g.batch_end()
+    launches = g.get_last_barrier_count() if hasattr(g, "get_last_barrier_count") else None
+    return read(g, 0, 0, s.total), launches
+
+
+@pytest.mark.parametrize("then", ["gemv", "gemv_reads_row", "op_reads_row", "apart", "nothing"])
+@pytest.mark.parametrize("K,N", [(1152, 1536), (4096, 1024)])
+def test_norm2_row_parked_until_a_later_gemv(hip, monkeypatch, K, N, then):
+    s = Slots(K, N)
+    qt = make_weights(N, K, 17)
+    got = {}
+    for name, g in (("park", hip), ("ticket", hip), ("oracle", oracle.init())):
+        note(f"norm2 then {then} K={K} N={N} {name}")
+        if name == "ticket":
+            monkeypatch.setenv("ADAMAH_NORM2_PARK", "0")
+        s.fill(g, 29)
+        load_qtensor(g, 1, qt)
+        got[name] = _norm2_then(g, s, qt, then)
+        if name == "ticket":
+            monkeypatch.delenv("ADAMAH_NORM2_PARK")
+    assert np.array_equal(got["park"][0].view(np.uint32), got["ticket"][0].view(np.uint32))
+    assert got["park"][1] == got["ticket"][1]       # parking costs no launch
+    assert rel_l2(got["park"][0], got["oracle"][0]) < TOL
+    for slot in ("resk", "x", "src2"):
+        o = s.off[slot]
+        assert rel_l2(got["park"][0][o:o + K], got["oracle"][0][o:o + K]) < 1e-5, slot
