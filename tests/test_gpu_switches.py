@@ -23,7 +23,7 @@ pytestmark = pytest.mark.gpu
 SWITCHES = [("ADAMAH_NO_FUSE", "1"), ("ADAMAH_GEMV_IMPL", "0"), ("ADAMAH_GEMV_IMPL", "1"), ("ADAMAH_GEMV_IMPL", "3"),
             ("ADAMAH_GEMM_IMPL", "0"), ("ADAMAH_GEMM_MERGE", "0"), ("ADAMAH_GEMM_EPI", "0"), ("ADAMAH_GEMM_REUSE", "0"),
             ("ADAMAH_RMSNORM_EMIT", "0"), ("ADAMAH_RMSNORM_ROWS", "0"), ("ADAMAH_ARGMAX_RUN", "0"),
-            ("ADAMAH_ATTN_CHUNK", "0"), ("ADAMAH_ATTN_BATCH", "0"), ("ADAMAH_ATTN_IMPL", "0"), ("ADAMAH_ATTN_ROWPREP", "0"), ("ADAMAH_TOPK_RANK", "0"),
+            ("ADAMAH_ATTN_CHUNK", "0"), ("ADAMAH_ATTN_BATCH", "0"), ("ADAMAH_ATTN_IMPL", "0"), ("ADAMAH_ATTN_ROWPREP", "0"), ("ADAMAH_NORM2_PARK", "0"), ("ADAMAH_TOPK_RANK", "0"),
             ("ADAMAH_TOPK_RANK", "1")]
 
 _REF = {}
@@ -108,3 +108,33 @@ def test_m1_product_kernels_at_full_row_lengths(hip, monkeypatch, impl, kind, N,
     assert rel_l2(res["hip"][1], res["oracle"][1]) < 1e-3
     assert res["hip"][2] == res["oracle"][2]
     assert rel_l2(res["hip"][3], res["oracle"][3]) < 1e-3
+
+
+@pytest.mark.parametrize("arch", ["gemma3", "llama"])
+def test_row_preparation_and_parked_row_on_a_model_with_wide_heads(hip, monkeypatch, arch):
+    """The decode attention launch takes over the token's rotation and KV append only for head sizes 128 and 256, and
+    a folded norm pair parks its in-place row only when a later GEMV can put it in place: a small model with 128-wide
+    heads decodes the same tokens and ends on the same hidden state (bit for bit) with either turned off, and
+    agrees with the reference forward pass."""
+    cfg = synth.tiny_config(arch, n_layer=3, n_embd=256, n_head=4, n_head_kv=2, head_dim=128, n_ff=512, n_vocab=1000)
+    tensors = synth.make_model(cfg, seed=6, sigma=0.1)
+    deq = {n: (v.dequant() if isinstance(v, QTensor) else v) for n, v in tensors.items()}
+    rng = np.random.default_rng(4)
+    prompt = [int(t) for t in rng.integers(0, 1000, 37)]
+    want = CpuModel(cfg, deq, kv_cap=96, kv_fp16=True).generate(prompt, 10)
+    got = {}
+    for name, env in (("default", None), ("no_rowprep", "ADAMAH_ATTN_ROWPREP"), ("no_park", "ADAMAH_NORM2_PARK")):
+        note(f"wide heads {arch}: {name}")
+        if env:
+            monkeypatch.setenv(env, "0")
+        dev = DecodeEngine(hip, cfg, tensors, A=A, kv_cap=96, kv_fp16=True, gpu_fused_rows_per_group=128)
+        tok, _ = dev.generate(prompt, GenerationConfig(max_tokens=10), forced=want[0])
+        got[name] = (tok, dev.read_slot('hidden'), hip.get_last_barrier_count())
+        if env:
+            monkeypatch.delenv(env)
+        for i in range(10):
+            assert tok[i] == want[0][i] or want[1][i] < 1e-4, (name, i)
+    for name in ("no_rowprep", "no_park"):
+        assert got[name][0] == got["default"][0]
+        assert np.array_equal(got[name][1].view(np.uint32), got["default"][1].view(np.uint32)), name
+    assert got["no_rowprep"][2] == got["default"][2] + cfg.n_layer      # one launch per layer more
