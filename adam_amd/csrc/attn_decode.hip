@@ -25,6 +25,7 @@
 // each of those writes back and invalidates the L2 of its XCD and the kernel got 4x slower.)
 #include "attn_common.h"
 #include <algorithm>
+#include <string.h>
 #include <utility>
 #include <vector>
 
@@ -619,15 +620,35 @@ bool launch_attn_decode(const AttnDecodeArgs& a, AttnPartials* ap, bool* left, i
 // parameters, the same score rows, but queries, outputs and KV cache of its own.  A run of such pairs
 // becomes one launch of the kernel above over all their heads (bases in device memory); only the
 // last pair stores raw scores, which is what the shared score rows hold after the pairs ran one by one.
-static uint32_t* g_ext_buf = nullptr;
-static size_t g_ext_cap = 0;   // words
+// The table of operand bases of a launch.  A decode loop comes back with the same tables step after step (one per
+// layer), so each distinct table is uploaded once and kept: no copy in the step, and a step without copies from the
+// host can be recorded into a graph.
+struct ExtTable { std::vector<uint32_t> host; uint32_t* dev; };
+static std::vector<ExtTable> g_ext_tables;
+#define ATTD_EXT_TABLES 1024u
 
 void attn_decode_release() {
   for (int i = 0; i < g_freq_n; i++) hipFree(g_freq[i].dev);
   g_freq_n = 0;
-  if (g_ext_buf) hipFree(g_ext_buf);
-  g_ext_buf = nullptr;
-  g_ext_cap = 0;
+  for (ExtTable& t : g_ext_tables) hipFree(t.dev);
+  g_ext_tables.clear();
+}
+
+// Device copy of the table, uploaded on first sight; nullptr: out of memory.
+static const uint32_t* ext_table(const std::vector<uint32_t>& ext, int* rc) {
+  for (const ExtTable& t : g_ext_tables)
+    if (t.host.size() == ext.size() && memcmp(t.host.data(), ext.data(), ext.size() * 4) == 0) return t.dev;
+  if (g_ext_tables.size() >= ATTD_EXT_TABLES) {   // a caller that never repeats itself: start over
+    hipStreamSynchronize(g.stream);
+    for (ExtTable& t : g_ext_tables) hipFree(t.dev);
+    g_ext_tables.clear();
+    layout_changed();
+  }
+  uint32_t* dev = nullptr;
+  if (hipMalloc((void**)&dev, ext.size() * 4) != hipSuccess) { (void)hipGetLastError(); *rc = ADAMAH_ERR_MEMORY; return nullptr; }
+  if ((*rc = h2d(dev, ext.data(), ext.size() * 4)) != ADAMAH_OK) { hipFree(dev); return nullptr; }
+  g_ext_tables.push_back({ext, dev});
+  return dev;
 }
 
 size_t launch_attn_batch(const std::vector<PendOp>& q, size_t i, int* rc) {
@@ -711,12 +732,6 @@ size_t launch_attn_batch(const std::vector<PendOp>& q, size_t i, int* rc) {
   const uint32_t n_splits = cdiv(rows, chunk);
   if (n_groups > 65535u || (uint64_t)n_all * n_splits * (D + 2) > g.attn_scratch_floats) return 0;
   const size_t words = 3 * (size_t)n_all + 2 * (size_t)n_groups;
-  if (words > g_ext_cap) {
-    layout_changed();
-    if (g_ext_buf) { hipStreamSynchronize(g.stream); hipFree(g_ext_buf); }
-    g_ext_cap = std::max<size_t>(words, 4096);
-    if (hipMalloc((void**)&g_ext_buf, g_ext_cap * 4) != hipSuccess) { g_ext_buf = nullptr; g_ext_cap = 0; *rc = ADAMAH_ERR_MEMORY; return 2 * B; }
-  }
   std::vector<uint32_t> ext(words);
   for (size_t b = 0; b < B; b++)
     for (uint32_t op = 0; op < H; op++) {
@@ -726,18 +741,19 @@ size_t launch_attn_batch(const std::vector<PendOp>& q, size_t i, int* rc) {
       ext[2 * (size_t)n_all + k] = ho[b][op];
       if (op % G == 0) { ext[3 * (size_t)n_all + k / G] = hk[b][op]; ext[3 * (size_t)n_all + n_groups + k / G] = hv[b][op]; }
     }
-  if ((*rc = h2d(g_ext_buf, ext.data(), words * 4)) != ADAMAH_OK) return 2 * B;
+  const uint32_t* ext_dev = ext_table(ext, rc);
+  if (!ext_dev) return 2 * B;
   AttnDecodeArgs da = {(float*)mp->buf, mp->kv16, mp->kv_start, nullptr, nullptr, nullptr, nullptr, nullptr,
                        nullptr, nullptr, nullptr, nullptr, nullptr, n_all, D, rows, a0.eps, a0.f2, false, 0};
   AttdBases bs = {};
   dim3 grid(n_splits, n_groups);
-  if (D == 64) launch_d<64>(G, nw, pf, grid, da, bs, n_splits, chunk, g_ext_buf);
-  else if (D == 128) launch_d<128>(G, nw, pf, grid, da, bs, n_splits, chunk, g_ext_buf);
-  else launch_d<256>(G, nw, pf, grid, da, bs, n_splits, chunk, g_ext_buf);
+  if (D == 64) launch_d<64>(G, nw, pf, grid, da, bs, n_splits, chunk, ext_dev);
+  else if (D == 128) launch_d<128>(G, nw, pf, grid, da, bs, n_splits, chunk, ext_dev);
+  else launch_d<256>(G, nw, pf, grid, da, bs, n_splits, chunk, ext_dev);
   count_launch();
   *rc = check_launch();
   if (*rc == ADAMAH_OK && n_splits > 1)
-    *rc = launch_attn_combine_dev(mp, g.attn_scratch, g_ext_buf + 2 * (size_t)n_all, n_all, D, n_splits);
+    *rc = launch_attn_combine_dev(mp, g.attn_scratch, ext_dev + 2 * (size_t)n_all, n_all, D, n_splits);
   return 2 * B;
 }
 

@@ -838,7 +838,7 @@ static int replay_plan(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
   return ret;
 }
 
-// Graph replay of a plan (ADAMAH_PLAN_GRAPH=1).  A decode loop calls the plan with pos, pos + 1, ...: after
+// Graph replay of a plan (on unless ADAMAH_PLAN_GRAPH=0).  A decode loop calls the plan with pos, pos + 1, ...: after
 // serving step (pos, seq_len) the library records the launches of step (pos + 1, seq_len + 1) into a HIP graph
 // -- stream capture of the same entry points, nothing executes -- while the device is still busy with the
 // current step, and the next call launches that graph if it asks for exactly that step (anything else is
@@ -855,19 +855,30 @@ struct PlanGraph {
   uint32_t n_graph = 0, n_update = 0, n_inst = 0;   // steps served by a graph, in-place updates, instantiations
   uint64_t gen = 0;          // g.layout_gen when the graph was recorded: it holds device pointers and offsets by value
   std::vector<uint32_t> handles;   // sorted ids of the handles the plan's ops name (their contents are baked in too)
+  std::vector<PendOp> tail;        // the recorded step's last queued norms: not in the graph, queued again behind it
 };
 static PlanGraph g_pg[MAX_PLANS];
 
 static bool plan_graphs_on() {
-  static int on = -1;
-  if (on < 0) { const char* e = getenv("ADAMAH_PLAN_GRAPH"); on = (e && e[0] == '1') ? 1 : 0; }
-  return on == 1;
+  const char* e = getenv("ADAMAH_PLAN_GRAPH");
+  return !(e && e[0] == '0');
 }
 
 static void plan_graph_drop(PlanGraph& pg, bool for_good) {
   for (int i = 0; i < 2; i++) { if (pg.exec[i]) hipGraphExecDestroy(pg.exec[i]); pg.exec[i] = nullptr; }
   pg.ready = false;
   if (for_good) pg.disabled = true;
+}
+
+// A plan usually ends in the norms that the caller's next op (the LM head) folds into its own launch.  They stay in
+// the queue when the rest of the step is launched (or recorded), so that a step from a graph leaves the queue as an
+// ordinary replay does.
+static std::vector<PendOp> take_trailing_norms() {
+  size_t n = g.pend.size(), k = 0;
+  while (k < 2 && k < n && g.pend[n - 1 - k].kind == PK_RMSNORM) k++;
+  std::vector<PendOp> tail(g.pend.end() - (long)k, g.pend.end());
+  g.pend.resize(n - k);
+  return tail;
 }
 
 static void plan_graph_record(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
@@ -877,6 +888,7 @@ static void plan_graph_record(uint32_t plan_id, uint32_t pos, uint32_t seq_len) 
   const Stats saved = g.stats;
   if (hipStreamBeginCapture(g.stream, hipStreamCaptureModeThreadLocal) != hipSuccess) { (void)hipGetLastError(); plan_graph_drop(pg, true); return; }
   int r = replay_plan(plan_id, pos, seq_len);
+  pg.tail = take_trailing_norms();
   flush_pending();
   hipGraph_t graph = nullptr;
   const hipError_t e = hipStreamEndCapture(g.stream, &graph);
@@ -951,15 +963,20 @@ int adamah_decode_step(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
       ret = hipGraphLaunch(pg.exec[pg.cur], g.stream) == hipSuccess ? ADAMAH_OK : ADAMAH_ERR_BACKEND;
       count_launch((int)pg.n_nodes);
       pg.n_graph++;
+      g.pend.insert(g.pend.end(), pg.tail.begin(), pg.tail.end());
     } else {
       ret = replay_plan(plan_id, pos, seq_len);
-      flush_pending();
       pg.eager_steps++;
     }
+    // the step's launches are out (but for its last norms, which wait for the caller's next op as they would without
+    // graphs); the recording below must find the queue without them
+    const std::vector<PendOp> tail = take_trailing_norms();
+    flush_pending();
     // the first steps run the ordinary way (scratch buffers reach their sizes); then record the next one
     if (ret == ADAMAH_OK && pg.eager_steps >= 2 && pos != 0xFFFFFFFFu && seq_len != 0xFFFFFFFFu)
       plan_graph_record(plan_id, pos + 1, seq_len + 1);
     else pg.ready = false;
+    g.pend.insert(g.pend.end(), tail.begin(), tail.end());
   }
   if (opened) batch_end();
   if (ret == ADAMAH_OK && g.pend.empty()) ret = take_deferred_err();

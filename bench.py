@@ -454,7 +454,7 @@ def main():
                                f"timed steps at context {m['end_pos'] - args.steps + 1}..{m['end_pos']}",
                    "baseline_config": 2 if gemma else 4,
                    "scheduler": args.scheduler, "launches_per_token": round(m["launches_per_token"], 1),
-                   "issue": "one native decode_step call per token (registered decode plan)"},
+                   "issue": "one native decode_step call per token (registered decode plan, launched from HIP graphs recorded one step ahead)"},
         "device_ms_per_step": round(m["device_ms_per_step"], 4),
         "algorithmic_bytes_per_token": m["step_bytes"],
         "tok_s_at_hbm_peak": round(m["ceiling"], 1), "frac_of_hbm_roofline": round(m["tok_s"] / m["ceiling"], 4),

@@ -240,10 +240,10 @@ print(json.dumps({{"tokens": out, "hidden": [float(v) for v in hid[:64]]}}))
 
 @pytest.mark.parametrize("arch", ["gemma3", "llama"])
 def test_decode_plan_from_recorded_graphs_gives_the_same_tokens(arch):
-    """ADAMAH_PLAN_GRAPH=1: the plan's launches for the next position are recorded into a HIP graph while the
-    current step runs and replayed by the next call.  Two generations (80 graph replays with the token read
+    """The plan's launches for the next position are recorded into a HIP graph while the current step runs and
+    replayed by the next call (ADAMAH_PLAN_GRAPH=0: never).  Two generations (80 graph replays with the token read
     and the embedding upload between them) give the tokens and the final hidden state, bit for bit, of the
-    ordinary replay.  Each mode runs in a process of its own (the switch is read once)."""
+    ordinary replay.  Each mode runs in a process of its own, so the library's exit report can be read."""
     import json, os, subprocess, sys
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     res = {}
