@@ -851,6 +851,7 @@ struct PlanGraph {
   int cur = 0;               // exec[cur] holds the recorded step when ready
   bool ready = false, disabled = false;
   uint32_t pos = 0, seq = 0, n_nodes = 0;
+  uint32_t last_pos = 0xFFFFFFFFu, last_seq = 0xFFFFFFFFu;   // the previous call's step
   int eager_steps = 0;
   uint32_t n_graph = 0, n_update = 0, n_inst = 0;   // steps served by a graph, in-place updates, instantiations
   uint64_t gen = 0;          // g.layout_gen when the graph was recorded: it holds device pointers and offsets by value
@@ -972,8 +973,12 @@ int adamah_decode_step(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
     // graphs); the recording below must find the queue without them
     const std::vector<PendOp> tail = take_trailing_norms();
     flush_pending();
-    // the first steps run the ordinary way (scratch buffers reach their sizes); then record the next one
-    if (ret == ADAMAH_OK && pg.eager_steps >= 2 && pos != 0xFFFFFFFFu && seq_len != 0xFFFFFFFFu)
+    // The first steps run the ordinary way (scratch buffers reach their sizes).  Then the next step is recorded, but
+    // only for a caller that is walking through positions (this call continued the previous one): a plan that is
+    // called with the same step again and again (a benchmark loop) would pay for a recording it never uses.
+    const bool walking = pg.last_pos != 0xFFFFFFFFu && pos == pg.last_pos + 1u && seq_len == pg.last_seq + 1u;
+    pg.last_pos = pos; pg.last_seq = seq_len;
+    if (ret == ADAMAH_OK && pg.eager_steps >= 2 && walking && pos != 0xFFFFFFFFu && seq_len != 0xFFFFFFFFu)
       plan_graph_record(plan_id, pos + 1, seq_len + 1);
     else pg.ready = false;
     g.pend.insert(g.pend.end(), tail.begin(), tail.end());

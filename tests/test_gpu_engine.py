@@ -306,3 +306,42 @@ def test_recorded_graph_is_dropped_when_a_plan_handle_is_rewritten():
     assert json.loads(p.stdout.strip().split("\n")[-1]) == [True] * 8, p.stdout
     line = [l for l in p.stderr.split("\n") if "steps from graphs" in l]
     assert line and int(line[-1].split(":")[1].split()[0]) >= 2, p.stderr[-1000:]      # graphs were in use at all
+
+
+_GRAPH_SAME_STEP_SNIPPET = """
+import sys, json
+sys.path.insert(0, {root!r})
+import numpy as np
+from adam_amd import adamah as A
+gpu = A.init()
+n = 4096
+gpu.set_dtype(A.DTYPE_F32)
+gpu.map_create(0, 1, 3 * n)
+vals = np.random.default_rng(0).standard_normal(2 * n).astype(np.float32)
+gpu.scatter_contiguous(0, 0, vals)
+run = lambda lo: np.arange(lo, lo + n, dtype=np.uint32)
+a_h, b_h, c_h = (gpu.upload_dev(run(lo))[0] for lo in (0, n, 2 * n))
+gpu.register_decode_plan(3, [A.DecodePlanOp(kind=A.DECODE_OP_OP2, map_id=0, op_code=A.OP_ADD, h0=a_h, h1=b_h, h2=c_h, u0=n)])
+ok = []
+for step in (5, 5, 5, 5, 5, 5, 9, 2, 2):          # a benchmark loop, not a decode loop
+    gpu.decode_step(3, step, step + 1)
+    ok.append(bool(np.array_equal(gpu.gather(0, run(2 * n)).view(np.float32), vals[:n] + vals[n:])))
+gpu.shutdown()
+print(json.dumps(ok))
+"""
+
+
+def test_a_plan_called_with_the_same_step_is_not_recorded():
+    """Graphs are recorded one step ahead for a caller that walks through positions.  A plan that is called with the same
+    (or an unrelated) step every time -- the kernel benchmarks do that -- must not pay for recordings it never uses."""
+    import json, os, subprocess, sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    note("decode plan graphs: the same step again and again")
+    env = dict(os.environ, ADAMAH_DEBUG="1")
+    env.pop("ADAMAH_PLAN_GRAPH", None)
+    p = subprocess.run([sys.executable, "-c", _GRAPH_SAME_STEP_SNIPPET.format(root=root)], env=env, capture_output=True, text=True,
+                       timeout=110)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert json.loads(p.stdout.strip().split("\n")[-1]) == [True] * 9, p.stdout
+    line = [l for l in p.stderr.split("\n") if "steps from graphs" in l]
+    assert line and " 0 steps from graphs" in line[-1] and " 0 instantiations" in line[-1], p.stderr[-1000:]
