@@ -156,29 +156,35 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
       __syncthreads();
     } else {
       constexpr uint32_t half = (uint32_t)D / 2u;
-      // raw rows first (they are waited for first), then the first tile
-      float qraw[QN], kraw = 0.f, vraw = 0.f;
+      // Raw rows first (they are waited for first), then what the rotation needs from memory (frequencies, norm
+      // weights), then the first tile.  Every load below is issued by every thread, at an address clamped into its
+      // row where the thread has no element of its own: with loads under branches the compiler no longer knows how
+      // many are in flight and waited for all of them, K / V tile included, before the queries could be staged.
+      float qraw[QN], kraw, vraw;
 #pragma unroll
-      for (uint32_t u = 0; u < QN; u++) {
-        const uint32_t i = tid + u * NT;
-        qraw[u] = i < (uint32_t)(G * D) ? data[(uint64_t)rp.q_src + (uint64_t)op0 * D + i] : 0.f;
+      for (uint32_t u = 0; u < QN; u++)
+        qraw[u] = data[(uint64_t)rp.q_src + (uint64_t)op0 * D + min(tid + u * NT, (uint32_t)(G * D) - 1u)];
+      {
+        const uint32_t d = min(tid, (uint32_t)D - 1u);
+        kraw = data[(uint64_t)rp.k_src + (uint64_t)group * D + d];
+        vraw = data[(uint64_t)rp.v_src + (uint64_t)group * D + d];
       }
-      if (tail_wg && tid < (uint32_t)D) {
-        kraw = data[(uint64_t)rp.k_src + (uint64_t)group * D + tid];
-        vraw = data[(uint64_t)rp.v_src + (uint64_t)group * D + tid];
-      }
-      // what the rotation of this thread's pairs needs from memory, asked for now: its frequencies and norm weights
-      float fr[PN], wq[PN][2], wk[2] = {1.f, 1.f};
+      float fr[PN], wq[PN][2], wk[2];
+      const bool nrm = (rp.flags & 1u) != 0u;
+      {
+        const float* wqp = nrm ? data + rp.q_w : rp.inv_freq;     // no norm: any readable address, the value is not used
+        const float* wkp = nrm ? data + rp.k_w : rp.inv_freq;
+        const uint32_t hs = nrm ? half : 0u;
 #pragma unroll
-      for (uint32_t u = 0; u < PN; u++) {
-        const uint32_t i = (tid + u * NT) % half;
-        fr[u] = rp.inv_freq[i];
-        wq[u][0] = 1.f; wq[u][1] = 1.f;
-        if (rp.flags & 1u) { wq[u][0] = data[(uint64_t)rp.q_w + i]; wq[u][1] = data[(uint64_t)rp.q_w + i + half]; }
+        for (uint32_t u = 0; u < PN; u++) {
+          const uint32_t i = (tid + u * NT) % half;
+          fr[u] = rp.inv_freq[i];
+          wq[u][0] = wqp[i]; wq[u][1] = wqp[i + hs];
+        }
+        wk[0] = wkp[tid % half]; wk[1] = wkp[tid % half + hs];
       }
-      if (tail_wg && tid < half && (rp.flags & 1u)) { wk[0] = data[(uint64_t)rp.k_w + tid]; wk[1] = data[(uint64_t)rp.k_w + tid + half]; }
       __builtin_amdgcn_sched_barrier(0);
-      if (any) { fetch(kA, vA, rbase); }
+      fetch(kA, vA, min(rbase, t1 - 1u));      // a wave without rows asks for the slice's last row: not used
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (uint32_t u = 0; u < QN; u++) {

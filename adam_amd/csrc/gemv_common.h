@@ -107,7 +107,6 @@ struct GemvFuse {
   // EPIX_GEGLU / SWIGLU: the matrix is [gate rows; up rows], e_dst[i] = act(y[i]) * y[N/2 + i]
   uint32_t e_mode;
   uint32_t e_res, e_dst;
-  uint32_t x_first;         // set by the launcher: activation loads go out ahead of the first weight loads
 };
 // Threads per workgroup the launchers will use for a matrix with N rows (store variant).
 uint32_t mfma_store_threads(uint32_t K, uint32_t N);

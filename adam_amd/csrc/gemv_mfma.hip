@@ -145,17 +145,20 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       else R.p[u] = qp[gi];
     }
     // The add epilogue needs one residual value per result row: asked for here, in the compute mapping (lane =
-    // 4 * column + row, column 0 stores), so it has arrived long before the row sum is complete.
-    if (EPI == EPI_STORE && fz.e_mode == EPIX_ADD && chunk + ks >= C && bcol == 0u)
-      R.res = act[(uint64_t)fz.e_res + min(row0 + l, end - 1u)];
+    // 4 * column + row, column 0 stores), so it has arrived long before the row sum is complete.  Every lane asks at
+    // every step (without the epilogue: for a word of the activations, not used): a load under a branch would leave
+    // the compiler unable to count the loads in flight, and it then waits for all of them wherever it waits for one.
+    if (EPI == EPI_STORE) R.res = act[fz.e_mode == EPIX_ADD ? (uint64_t)fz.e_res + min(row0 + l, end - 1u) : (uint64_t)a];
   };
 
   PreM A, B;   // A's first loads stay in flight while the activations are staged
-  auto first_loads = [&]() { if (first < seg_end) load(A, first, kpart, seg_end); };
+  // (a wave without rows asks for the matrix's first rows: same number of loads on every path, see load())
+  auto first_loads = [&]() {
+    const bool has = first < seg_end;
+    load(A, has ? first : 0u, has ? kpart : 0u, has ? seg_end : min(N, 4u));
+  };
   // Loads come back in order: the activation loads (cache hits) go out ahead of the first weights, so
   // the conversion does not wait for the weights' trip to memory as well.
-  const bool x_first = fz.x_first != 0u;
-  if (PRO == PRO_NONE && !x_first) first_loads();
 
   // ---- activations -> fixed-point digits; one 8-element word per thread and pass, four threads per
   // block.  stage() turns one word into digits; the prologues below decide what the word is. ------
@@ -218,12 +221,14 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
   float nrm1 = 1.f, nrm_late = 1.f;   // nrm_late: the prologue's last norm, applied to the row sums
   uint32_t ticket = 0;
   if (PRO == PRO_NONE) {
-    // four passes of loads are issued before the first word is converted
-    for (uint32_t i0 = 0; i0 < nw; i0 += 4u * nthr) {
+    // four passes of loads are issued before the first word is converted; the first round stands outside the loop,
+    // in straight-line code with the first weight loads behind it, so that the conversion waits for exactly the
+    // activation loads
+    auto x_round = [&](uint32_t i0, bool with_weights) {
       float x[4][8];
 #pragma unroll
       for (uint32_t u = 0; u < 4; u++) load8(act + a + (uint64_t)min(i0 + u * nthr + tid, nw - 1u) * 8u, x[u]);
-      if (i0 == 0u && x_first) {
+      if (with_weights) {
         __builtin_amdgcn_sched_barrier(0);
         first_loads();
         __builtin_amdgcn_sched_barrier(0);
@@ -232,7 +237,9 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       for (uint32_t u = 0; u < 4; u++)
         if (i0 + u * nthr + (tid & ~63u) < nw)   // wave-uniform: waves without words skip the conversion
           stage(i0 + u * nthr + tid, i0 + u * nthr + tid < nw, x[u]);
-    }
+    };
+    x_round(0u, true);
+    for (uint32_t i0 = 4u * nthr; i0 < nw; i0 += 4u * nthr) x_round(i0, false);
   } else if (PRO == PRO_COMBINE) {
     // Folded merge of the attention partials (same arithmetic as the stand-alone merge kernel):
     // M = max m_s, w_s = e^(m_s - M), L = sum l_s w_s, x = sum_s o_s w_s / L, per head.
@@ -282,7 +289,7 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       mine[u] = u * nthr + (tid & ~63u) < nw;
 #pragma unroll
       for (int k = 0; k < 8; k++) { v[u][k] = 0.f; wv[u][k] = 0.f; rv[u][k] = 0.f; w2v[u][k] = 0.f; }
-      if (!mine[u]) continue;
+      // (waves without words of their own load the row's last word: every path issues the same loads)
       const uint64_t e0 = (uint64_t)min(i, nw - 1u) * 8u;
       load8(act + fz.p_src + e0, v[u]);
       load8(fz.p_wt + fz.p_src2 + e0, wv[u]);
@@ -596,8 +603,6 @@ static int launch_mfma(int fmt, uint32_t grid, uint32_t threads, const Map* ma, 
                        uint32_t n_groups, uint32_t ks, const GemvFuse* fzp, float* out = nullptr) {
   GemvFuse fz = {};
   if (fzp) fz = *fzp;
-  const int xf = knob("ADAMAH_MFMA_XFIRST", -1);
-  fz.x_first = xf < 0 ? 1u : (uint32_t)(xf != 0);
 #define MP(P) launch_mfma_p<EPI, P>(fmt, grid, threads, ma, mw, a, b, c, lidx, lval, K, N, rpg, n_groups, ks, fz, out)
   switch (fz.pro) {
     case PRO_RMSNORM: MP(PRO_RMSNORM); break;
