@@ -141,18 +141,30 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
     float* qs = &obuf[0][0][0];
     if (tid < (uint32_t)G) hmax[tid] = 0u;
     if (!RP) {
-      __syncthreads();
-      for (uint32_t i = tid; i < (uint32_t)(G * D); i += NT) {   // a wave's 64 elements belong to one head
-        const uint32_t hq = (uint32_t)__builtin_amdgcn_readfirstlane((int)(i / D));   // scalar: read from the arguments
-        const float x = data[(uint64_t)(EXT ? e_q[op0 + hq] : bs.q[op0 + hq]) + i % D];
-        qs[i] = x;
-        float m = fabsf(x);
+      // the query loads go out first and are waited for first, with the first tile's loads already behind them
+      // (every thread issues the same loads, at clamped addresses where it has no element of its own, so that the
+      // compiler can count them: see the row preparation below)
+      float qraw[QN];
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
-        if (lane == 0u) atomicMax(&hmax[i / D], __float_as_uint(m));
+      for (uint32_t u = 0; u < QN; u++) {
+        const uint32_t i = min(tid + u * NT, (uint32_t)(G * D) - 1u), hq = i / D;   // a wave's 64 elements belong to one head
+        qraw[u] = data[(uint64_t)(EXT ? e_q[op0 + hq] : bs.q[op0 + hq]) + i % D];
       }
-      if (any) { fetch(kA, vA, rbase); }
       __builtin_amdgcn_sched_barrier(0);
+      fetch(kA, vA, min(rbase, t1 - 1u));      // a wave without rows asks for the slice's last row: not used
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();                         // hmax is zero
+#pragma unroll
+      for (uint32_t u = 0; u < QN; u++) {
+        const uint32_t i = tid + u * NT;
+        if (i < (uint32_t)(G * D)) {
+          qs[i] = qraw[u];
+          float m = fabsf(qraw[u]);
+#pragma unroll
+          for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+          if (lane == 0u) atomicMax(&hmax[i / D], __float_as_uint(m));
+        }
+      }
       __syncthreads();
     } else {
       constexpr uint32_t half = (uint32_t)D / 2u;
