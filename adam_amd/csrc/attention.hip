@@ -435,15 +435,53 @@ k_attn_fused(const float* data, float* out, const __half* kv, uint64_t kv_shift,
 // Merge the split partials of one op: M = max m_s, w_s = e^(m_s-M), L = sum l_s w_s,
 // out = sum_s o_s w_s / L.  n_splits <= 1024.  grid (n_ops, ceil(value_dim / 32)): a workgroup owns 32
 // output elements, eight groups of 32 threads take every eighth split each and meet in LDS.
+// FEW (n_splits <= 64): everything a thread needs -- its eight values, one split's (max, sum) pair per lane, the
+// output base, its element of the prepared queries -- is asked for in one round of loads, clamped rather than
+// skipped, and every wave works out M, the weights and L for itself with cross-lane operations: one trip to memory
+// and one barrier where the general form below takes three of each.  Same operations in the same order per result.
+template <bool FEW>
 __global__ void __launch_bounds__(256)
 k_attn_combine(float* out, const float* partial, const uint32_t* __restrict__ lo, uint32_t value_dim,
                uint32_t n_splits, uint64_t n_elems, const float* q_src, uint32_t q_dst, uint32_t q_n) {
-  __shared__ float w[1024];
+  __shared__ float w[FEW ? 1 : 1024];
   __shared__ float red[4];
   __shared__ float osum[8][32];
   const uint32_t op = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t stride = value_dim + 2;
   const float* pp = partial + (uint64_t)op * n_splits * stride;
+  if (FEW) {
+    const uint32_t last = n_splits - 1u, sg = tid >> 5, d = blockIdx.y * 32u + (tid & 31u), dc = min(d, value_dim - 1u);
+    const uint32_t threads = gridDim.x * gridDim.y * 256u, gi = (blockIdx.y * gridDim.x + op) * 256u + tid;
+    const float* ps = pp + (uint64_t)min(lane, last) * stride;
+    const float m_own = ps[0], l_own = ps[1];
+    float v[8];
+#pragma unroll
+    for (uint32_t k = 0; k < 8u; k++) v[k] = pp[(uint64_t)min(sg + 8u * k, last) * stride + 2 + dc];
+    const float qv = (q_n ? q_src : partial)[q_n ? min(gi, q_n - 1u) : 0u];   // (a load on every path)
+    const uint64_t ob = lo[op];
+    const float M = wave_max64(lane < n_splits ? m_own : -9.99999968e+37f);
+    const float e = lane < n_splits ? expf(m_own - M) : 0.f;
+    const float invL = 1.0f / wave_sum64(lane < n_splits ? fmaf(l_own, e, 0.f) : 0.f);
+    float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+    for (uint32_t k = 0; k < 4u; k++) {
+      const uint32_t s0 = sg + 16u * k, s1 = s0 + 8u;
+      const float w0 = __shfl(e, (int)s0, 64), w1 = __shfl(e, (int)s1, 64);
+      o0 = s0 < n_splits ? fmaf(v[2u * k], w0, o0) : o0;
+      o1 = s1 < n_splits ? fmaf(v[2u * k + 1u], w1, o1) : o1;
+    }
+    osum[sg][tid & 31u] = o0 + o1;
+    if (gi < q_n) out[(uint64_t)q_dst + gi] = qv;
+    for (uint32_t i = gi + threads; i < q_n; i += threads) out[(uint64_t)q_dst + i] = q_src[i];
+    __syncthreads();
+    if (tid < 32u && d < value_dim && ob + value_dim <= n_elems) {
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; i++) o += osum[i][tid];
+      out[ob + d] = o * invL;
+    }
+    return;
+  }
   // queries the attention launch prepared and could not yet store over the raw ones: each workgroup its share
   for (uint32_t i = (blockIdx.y * gridDim.x + op) * 256u + tid; i < q_n; i += gridDim.x * gridDim.y * 256u)
     out[(uint64_t)q_dst + i] = q_src[i];
@@ -662,8 +700,13 @@ int launch_attn_combine(const PendOp& at, const AttnPartials& ap) {
   Map* m = get_f32_map(at.map_act);
   const uint32_t* lo = res_u32(at.h[2], at.rpg);
   if (!m || !lo) return ADAMAH_ERR_INVALID;
-  k_attn_combine<<<dim3(at.rpg, cdiv(ap.value_dim, 32)), 256, 0, g.stream>>>((float*)m->buf, ap.base, lo, ap.value_dim, ap.n_splits, m->n_elems,
-                                                                              ap.q_src, ap.q_dst, ap.q_n);
+  const dim3 grid(at.rpg, cdiv(ap.value_dim, 32));
+  if (ap.n_splits <= 64u)
+    k_attn_combine<true><<<grid, 256, 0, g.stream>>>((float*)m->buf, ap.base, lo, ap.value_dim, ap.n_splits, m->n_elems, ap.q_src,
+                                                     ap.q_dst, ap.q_n);
+  else
+    k_attn_combine<false><<<grid, 256, 0, g.stream>>>((float*)m->buf, ap.base, lo, ap.value_dim, ap.n_splits, m->n_elems, ap.q_src,
+                                                      ap.q_dst, ap.q_n);
   count_launch();
   return check_launch();
 }
@@ -671,8 +714,12 @@ int launch_attn_combine(const PendOp& at, const AttnPartials& ap) {
 // Merge of the sequence slices for output rows listed in device memory.
 int launch_attn_combine_dev(Map* m, const float* partial, const uint32_t* lo_dev, uint32_t n_ops, uint32_t value_dim,
                             uint32_t n_splits) {
-  k_attn_combine<<<dim3(n_ops, cdiv(value_dim, 32)), 256, 0, g.stream>>>((float*)m->buf, partial, lo_dev, value_dim, n_splits,
-                                                                        m->n_elems, nullptr, 0u, 0u);
+  const dim3 grid(n_ops, cdiv(value_dim, 32));
+  if (n_splits <= 64u)
+    k_attn_combine<true><<<grid, 256, 0, g.stream>>>((float*)m->buf, partial, lo_dev, value_dim, n_splits, m->n_elems, nullptr, 0u, 0u);
+  else
+    k_attn_combine<false><<<grid, 256, 0, g.stream>>>((float*)m->buf, partial, lo_dev, value_dim, n_splits, m->n_elems, nullptr, 0u,
+                                                      0u);
   count_launch();
   return check_launch();
 }

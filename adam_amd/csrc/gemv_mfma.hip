@@ -243,35 +243,85 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
   } else if (PRO == PRO_COMBINE) {
     // Folded merge of the attention partials (same arithmetic as the stand-alone merge kernel):
     // M = max m_s, w_s = e^(m_s - M), L = sum l_s w_s, x = sum_s o_s w_s / L, per head.
-    first_loads();
-    if (blockIdx.x == 0)
-      for (uint32_t i = tid; i < fz.c_qn; i += nthr) act_out[(uint64_t)fz.c_qdst + i] = fz.c_qsrc[i];
     const uint32_t stride = fz.c_vd + 2u;
-    for (uint32_t i0 = 0; i0 < nw; i0 += nthr) {
-      const uint32_t i = i0 + tid, ic = min(i, nw - 1u);
-      const uint32_t head = (ic * 8u) / fz.c_vd, j0 = (ic * 8u) % fz.c_vd;
+    // At most eight slices and two threads per word: straight-line form.  A thread merges four elements: every value
+    // it needs and the slices' (max, sum) pairs are asked for in one round, ahead of the first weights (loads return
+    // in order: behind the weights they would wait for the weights' trip to memory as well).  Slices past the last
+    // are clamped, not skipped, so that the waits stay counted.  The (max, sum) pair of slice s comes from lane s of
+    // the thread's group of eight lanes, which all work on the same head (value_dim a multiple of 32).  The merged
+    // elements meet in LDS (in the digits' place, before there are digits), where each word's thread picks them up.
+    // Same order of operations per element as the loops below.
+    const bool few = EPI == EPI_STORE && fz.c_splits <= 8u && 2u * nw <= nthr && fz.c_vd % 32u == 0u;
+    if (few) {
+      const uint32_t e0 = min(tid, 2u * nw - 1u) * 4u, head = e0 / fz.c_vd, j0 = e0 % fz.c_vd, last = fz.c_splits - 1u;
       const float* pp = fz.c_partial + (uint64_t)head * fz.c_splits * stride;
-      float M = -9.99999968e+37f;
-      for (uint32_t sp = 0; sp < fz.c_splits; sp++) M = fmaxf(M, pp[(uint64_t)sp * stride]);
-      float L = 0.f, x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      for (uint32_t sp = 0; sp < fz.c_splits; sp++) {
-        const float wgt = expf(pp[(uint64_t)sp * stride] - M);
-        L = fmaf(pp[(uint64_t)sp * stride + 1], wgt, L);
-        float o[8];
-        load8(pp + (uint64_t)sp * stride + 2 + j0, o);
+      const float* pm = pp + (uint64_t)min(lane & 7u, last) * stride;
+      const float m_own = pm[0], l_own = pm[1];
+      f4u_t o[8];
 #pragma unroll
-        for (int k = 0; k < 8; k++) x[k] = fmaf(o[k], wgt, x[k]);
+      for (uint32_t sp = 0; sp < 8u; sp++) o[sp] = *(const f4u_t*)(pp + (uint64_t)min(sp, last) * stride + 2 + j0);
+      __builtin_amdgcn_sched_barrier(0);
+      first_loads();
+      __builtin_amdgcn_sched_barrier(0);
+      float mv[8], lv[8], M = -9.99999968e+37f, L = 0.f;
+#pragma unroll
+      for (uint32_t sp = 0; sp < 8u; sp++) {
+        mv[sp] = __shfl(m_own, (int)((lane & ~7u) + sp), 64);
+        lv[sp] = __shfl(l_own, (int)((lane & ~7u) + sp), 64);
+      }
+#pragma unroll
+      for (uint32_t sp = 0; sp < 8u; sp++) M = sp < fz.c_splits ? fmaxf(M, mv[sp]) : M;
+      f4u_t x4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (uint32_t sp = 0; sp < 8u; sp++) {
+        const float wgt = expf(mv[sp] - M);
+        const bool on = sp < fz.c_splits;
+        L = on ? fmaf(lv[sp], wgt, L) : L;
+        x4.x = on ? fmaf(o[sp].x, wgt, x4.x) : x4.x; x4.y = on ? fmaf(o[sp].y, wgt, x4.y) : x4.y;
+        x4.z = on ? fmaf(o[sp].z, wgt, x4.z) : x4.z; x4.w = on ? fmaf(o[sp].w, wgt, x4.w) : x4.w;
       }
       const float invL = 1.0f / L;
-#pragma unroll
-      for (int k = 0; k < 8; k++) x[k] *= invL;
-      if (i0 + (tid & ~63u) >= nw) continue;   // wave-uniform: nothing of this pass belongs to the wave
-      if (blockIdx.x == 0 && i < nw) {
-        f4u_t* o = (f4u_t*)(act_out + fz.p_dst + (uint64_t)i * 8u);
-        o[0] = (f4u_t){x[0], x[1], x[2], x[3]}; o[1] = (f4u_t){x[4], x[5], x[6], x[7]};
+      x4.x *= invL; x4.y *= invL; x4.z *= invL; x4.w *= invL;
+      float* xf = (float*)xs;
+      if (tid < 2u * nw) {
+        *(f4u_t*)(xf + tid * 4u) = x4;
+        if (blockIdx.x == 0) *(f4u_t*)(act_out + fz.p_dst + (uint64_t)tid * 4u) = x4;
       }
-      stage(i, i < nw, x);
+      __syncthreads();
+      float x[8];
+      load8(xf + min(tid, nw - 1u) * 8u, x);
+      __syncthreads();
+      if ((tid & ~63u) < nw) stage(tid, tid < nw, x);
+    } else {
+      first_loads();
+      for (uint32_t i0 = 0; i0 < nw; i0 += nthr) {
+        const uint32_t i = i0 + tid, ic = min(i, nw - 1u);
+        const uint32_t head = (ic * 8u) / fz.c_vd, j0 = (ic * 8u) % fz.c_vd;
+        const float* pp = fz.c_partial + (uint64_t)head * fz.c_splits * stride;
+        float M = -9.99999968e+37f;
+        for (uint32_t sp = 0; sp < fz.c_splits; sp++) M = fmaxf(M, pp[(uint64_t)sp * stride]);
+        float L = 0.f, x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (uint32_t sp = 0; sp < fz.c_splits; sp++) {
+          const float wgt = expf(pp[(uint64_t)sp * stride] - M);
+          L = fmaf(pp[(uint64_t)sp * stride + 1], wgt, L);
+          float o[8];
+          load8(pp + (uint64_t)sp * stride + 2 + j0, o);
+#pragma unroll
+          for (int k = 0; k < 8; k++) x[k] = fmaf(o[k], wgt, x[k]);
+        }
+        const float invL = 1.0f / L;
+#pragma unroll
+        for (int k = 0; k < 8; k++) x[k] *= invL;
+        if (i0 + (tid & ~63u) >= nw) continue;   // wave-uniform: nothing of this pass belongs to the wave
+        if (blockIdx.x == 0 && i < nw) {
+          f4u_t* o = (f4u_t*)(act_out + fz.p_dst + (uint64_t)i * 8u);
+          o[0] = (f4u_t){x[0], x[1], x[2], x[3]}; o[1] = (f4u_t){x[4], x[5], x[6], x[7]};
+        }
+        stage(i, i < nw, x);
+      }
     }
+    if (blockIdx.x == 0)
+      for (uint32_t i = tid; i < fz.c_qn; i += nthr) act_out[(uint64_t)fz.c_qdst + i] = fz.c_qsrc[i];
   } else {
     // Folded row-wise ops.  Every thread keeps its (at most PRO_WPT) words in registers from one
     // round of loads, so the norms cost block reductions but no further trips to memory.
