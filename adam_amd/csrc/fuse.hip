@@ -277,6 +277,17 @@ void flush_pending() {
           }
         }
       }
+      // gate and up stacked, followed by the gated activation over their two results: stored by the matmul as well
+      // (a workgroup then takes 16 gate rows and their 16 up rows).  The activation must not land on either result.
+      if (m == 2 && M <= 32 && sg.n[0] == sg.n[1] && (sg.n[0] & 15u) == 0 && i + 2 < n && q[i + 2].kind == PK_OP2 &&
+          (q[i + 2].op == 34u || q[i + 2].op == 35u) && q[i + 2].map_act == p.map_act && tuning("ADAMAH_GEMM_EPI", 1) != 0) {
+        const PendOp& e = q[i + 2];
+        if (e.a == sg.c[0] && e.b == sg.c[1] && e.n == M * sg.n[0] && disjoint(e.c, e.n, sg.c[0], e.n) &&
+            disjoint(e.c, e.n, sg.c[1], e.n)) {
+          sg.glu = e.op; sg.dst = e.c;
+          used = 3;
+        }
+      }
       const uint32_t *la = res_u32(p.h[0], 1), *lb = res_u32(p.h[1], 1), *lc = res_u32(p.h[2], 1);
       if (!(ma && mw && la && lb && lc)) keep(ADAMAH_ERR_INVALID);
       else
@@ -284,6 +295,19 @@ void flush_pending() {
                                  (m == 1 && !sg.add) ? (int64_t)p.c : -1, (m == 1 && !sg.add) ? nullptr : &sg));
       i += used;
       continue;
+    }
+    if (p.kind == PK_OP2 && (p.op == 34u || p.op == 35u) && i + 1 < n && q[i + 1].kind == PK_GEMM) {
+      // gated activation over the rows a batched matmul reads next: the op's launch also leaves the fp16 form of
+      // its result, and the matmul skips its conversion launch
+      const PendOp& mm = q[i + 1];
+      Map* ma = get_f32_map(p.map_act);
+      if (ma && mm.map_act == p.map_act && mm.a == p.c && (uint64_t)mm.rpg * mm.k == p.n && disjoint(p.c, p.n, p.a, p.n) &&
+          disjoint(p.c, p.n, p.b, p.n) && tuning("ADAMAH_GLU_EMIT", 1) != 0 &&
+          launch_glu_act_f16(ma, p.op, p.a, p.b, p.c, mm.rpg, mm.k)) {
+        keep(check_launch());
+        i++;
+        continue;
+      }
     }
     if (p.kind == PK_ARGMAX) {
       // the LM head of several sequences in lockstep: one pass over the matrix for all their rows

@@ -303,9 +303,15 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
   // A cross-lane permute brings each 16-byte block (and its scale) to the lane that consumes it.
   const uint32_t lrow = lane >> 2, lblk = lane & 3u;
   const int perm_addr = (int)((4u * r16 + g) << 2);
-  uint32_t nrow[R];
+  // segs.glu (R = 2, the matrix is [gate rows; up rows], N / 2 a multiple of 16): the workgroup's first tile is 16
+  // gate rows and its second the 16 up rows that belong to them, so the gated activation can be stored from here
+  const bool glum = R == 2 && segs.glu != 0u;
+  uint32_t trow0[R], nrow[R];
 #pragma unroll
-  for (int r = 0; r < R; r++) nrow[r] = min(n0 + r * 16u + lrow, N - 1u);
+  for (int r = 0; r < R; r++) {
+    trow0[r] = glum ? (uint32_t)r * (N >> 1) + blockIdx.x * 16u : n0 + r * 16u;
+    nrow[r] = min(trow0[r] + lrow, N - 1u);
+  }
 
   f4q_t acc[R][MT];
 #pragma unroll
@@ -450,7 +456,7 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
       float* c = out + c_off + (uint64_t)row * N;
 #pragma unroll
       for (int r = 0; r < R; r++) {
-        const uint32_t n = n0 + r * 16u + r16;
+        const uint32_t n = trow0[r] + r16;
         if (n >= N) continue;
         if (segs.count) {   // stacked matrices: the row's own matrix and its result base
           uint32_t sgi = 0;
@@ -463,6 +469,11 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
           if (segs.add) out[segs.dst + (uint64_t)row * N + n] = out[segs.res + (uint64_t)row * N + n] + y;
         }
       }
+      if (glum && trow0[0] + r16 < (N >> 1)) {   // act(gate) * up, as the element-wise op computes it
+        const float a = acc[0][t][i] * inv, b = acc[R - 1][t][i] * inv;
+        out[segs.dst + (uint64_t)row * (N >> 1) + trow0[0] + r16] =
+            segs.glu == 34u ? gelu_tanh(a) * b : (a / (1.0f + expf(-a))) * b;
+      }
     }
 }
 #undef GEMM_FETCH
@@ -470,12 +481,17 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
 // The same conversion with the row held in registers: 1024 threads, thread t owns the 8-element words
 // t, t + 1024, ... (NW of them; K <= 8192 NW), so the row makes one trip from memory instead of two
 // dependent passes -- the rows of a decode batch are few and each workgroup's latency is the launch's.
-template <int NW>
+// GLU: the rows are first produced here, as the gated activation of two inputs (element offsets glu.a, glu.b; the
+// float32 result goes to glu.d, as the element-wise op stores it: op2 34 = GELU(a) b, 35 = SiLU(a) b), so the op and
+// the conversion of its result are one launch and one trip.
+struct GluSrc { uint32_t op, a, b, d; };
+template <int NW, bool GLU>
 __global__ void __launch_bounds__(1024)
-k_act_f16_regs(const float* act, const uint32_t* __restrict__ la, uint32_t M, uint32_t K, float* scale, uint4* xh, uint4* xl) {
+k_act_f16_regs(const float* act, float* act_out, const uint32_t* __restrict__ la, uint32_t M, uint32_t K, float* scale, uint4* xh,
+               uint4* xl, GluSrc glu) {
   __shared__ float red[16];
   const uint32_t row = blockIdx.x, op = blockIdx.y, tid = threadIdx.x, kw = K >> 3;
-  const float* x = act + (uint64_t)la[op] + (uint64_t)row * K;
+  const float* x = act + (GLU ? (uint64_t)glu.a : (uint64_t)la[op]) + (uint64_t)row * K;
   f4qu_t v0[NW], v1[NW];
   float m = 0.f;
 #pragma unroll
@@ -484,6 +500,16 @@ k_act_f16_regs(const float* act, const uint32_t* __restrict__ la, uint32_t M, ui
     if (w < kw) {
       v0[u] = *(const f4qu_t*)(x + w * 8u);
       v1[u] = *(const f4qu_t*)(x + w * 8u + 4u);
+      if (GLU) {
+        const float* y = act + (uint64_t)glu.b + (uint64_t)row * K + w * 8u;
+        const f4qu_t y0 = *(const f4qu_t*)y, y1 = *(const f4qu_t*)(y + 4);
+        auto f = [&](float a, float b) { return glu.op == 34u ? gelu_tanh(a) * b : (a / (1.0f + expf(-a))) * b; };
+        v0[u] = (f4qu_t){f(v0[u].x, y0.x), f(v0[u].y, y0.y), f(v0[u].z, y0.z), f(v0[u].w, y0.w)};
+        v1[u] = (f4qu_t){f(v1[u].x, y1.x), f(v1[u].y, y1.y), f(v1[u].z, y1.z), f(v1[u].w, y1.w)};
+        float* d = act_out + (uint64_t)glu.d + (uint64_t)row * K + w * 8u;
+        *(f4qu_t*)d = v0[u];
+        *(f4qu_t*)(d + 4) = v1[u];
+      }
       m = fmaxf(m, fmaxf(fmaxf(fmaxf(fabsf(v0[u].x), fabsf(v0[u].y)), fmaxf(fabsf(v0[u].z), fabsf(v0[u].w))),
                          fmaxf(fmaxf(fabsf(v1[u].x), fabsf(v1[u].y)), fmaxf(fabsf(v1[u].z), fabsf(v1[u].w)))));
     }
@@ -558,6 +584,22 @@ void gemm_act_mark(const void* buf, uint64_t a, uint32_t M, uint32_t K) {
   g_xh_key = {buf, a, M, K, g.stats.dispatch, g.mem_gen, (size_t)M * K * 2, true};
 }
 
+// Gated activation (op2 34 / 35) of the [M, K] rows at a and b into the rows at d, together with the fp16 form of
+// the result that a batched matmul over those rows reads: one launch, and the matmul that follows skips its
+// conversion.  false: not taken (nothing launched).
+bool launch_glu_act_f16(const Map* ma, uint32_t op, uint32_t a, uint32_t b, uint32_t d, uint32_t M, uint32_t K) {
+  if (K > 16384u || (K & 7u) || M == 0 || knob("ADAMAH_ACT_REGS", 1) == 0) return false;
+  float* scale; __half *xh, *xl;
+  if (!gemm_act_slots(M, K, &scale, &xh, &xl)) return false;
+  float* act = (float*)ma->buf;
+  const GluSrc glu = {op, a, b, d};
+  if (K <= 8192) k_act_f16_regs<1, true><<<dim3(M, 1), 1024, 0, g.stream>>>(act, act, nullptr, M, K, scale, (uint4*)xh, (uint4*)xl, glu);
+  else k_act_f16_regs<2, true><<<dim3(M, 1), 1024, 0, g.stream>>>(act, act, nullptr, M, K, scale, (uint4*)xh, (uint4*)xl, glu);
+  count_launch();
+  gemm_act_mark(ma->buf, d, M, K);
+  return true;
+}
+
 // Forget converted rows (after a stream capture: the launch count is rewound there, and the note must not
 // survive into a later state with the same count).
 void gemm_act_forget() { g_xh_key.valid = false; }
@@ -568,7 +610,7 @@ void gemm_act_forget() { g_xh_key.valid = false; }
 int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb, const uint32_t* lc,
                         uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops, bool q8, float* out, int64_t a_host,
                         int64_t c_host, const GemmSegs* segs) {
-  if (((q8 || out) && M > 32) || ((out || segs) && n_ops != 1) || (out && segs) || (segs && segs->add && M > 32))
+  if (((q8 || out) && M > 32) || ((out || segs) && n_ops != 1) || (out && segs) || (segs && (segs->add || segs->glu) && M > 32))
     return ADAMAH_ERR_INVALID;
   GemmSegs sg = {};
   if (segs) sg = *segs;
@@ -592,8 +634,8 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
   uint4* const xl = (uint4*)((uint8_t*)g_xh_buf + plane);
   if (!reuse) {
     if (K <= 16384 && knob("ADAMAH_ACT_REGS", 1) != 0) {
-      if (K <= 8192) k_act_f16_regs<1><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, la, M, K, g_scale_buf, xh, xl);
-      else k_act_f16_regs<2><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, la, M, K, g_scale_buf, xh, xl);
+      if (K <= 8192) k_act_f16_regs<1, false><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, act, la, M, K, g_scale_buf, xh, xl, GluSrc{});
+      else k_act_f16_regs<2, false><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, act, la, M, K, g_scale_buf, xh, xl, GluSrc{});
     } else
       k_act_f16<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf, xh, xl);
     count_launch();
@@ -606,6 +648,10 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
     R = (uint32_t)knob("ADAMAH_GEMM_R", (int)R);
     R = R >= 4 ? 4 : R >= 2 ? 2 : 1;
     if (q8 && R > 2) R = 2;   // a Q8 tile holds twice the registers
+    if (sg.glu) {             // a workgroup pairs one gate tile with its up tile
+      if (sg.count != 2 || sg.n[0] != sg.n[1] || (sg.n[0] & 15u)) return ADAMAH_ERR_INVALID;
+      R = 2;
+    }
     dim3 grid(cdiv(N, 16 * R), cdiv(M, 16 * mt), n_ops);
     float* dst = out ? out : act;
     const uint32_t* lcd = out ? nullptr : lc;

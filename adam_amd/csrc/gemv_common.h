@@ -122,6 +122,8 @@ bool mfma_path_ok(const Map* mw, uint32_t K);
 // at element c[s] of the activation map.
 // add (count == 0, one matrix): a queued element-wise add that consumes the result, r + y, is stored as
 // well: y goes to its own place, r[row * N + n] + y to dst[row * N + n] (element offsets res, dst).
+// glu (count == 2, two matrices of N / 2 rows each, M <= 32): the gated activation over the two results that is
+// queued behind them (op2 code 34 GEGLU / 35 SWIGLU: act(first) * second) is stored as well, at element dst.
 struct GemmSegs {
   uint32_t count;
   uint32_t begin[5];
@@ -129,6 +131,7 @@ struct GemmSegs {
   uint64_t c[4];
   uint32_t add;
   uint64_t res, dst;
+  uint32_t glu;
 };
 // M > 1: fp16 matrix-core GEMM over Q4 block16 weights (gemm_q4_mfma.hip); operands already validated.
 // q8: Q8 block16 weights instead (M <= 32).  out: the [M, N] result goes to this buffer instead of the
@@ -143,6 +146,9 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
 // counted -- the note that rows [a, a + M K) of `buf` are converted, so the matmul skips its conversion.
 bool gemm_act_slots(uint32_t M, uint32_t K, float** scale, __half** xh, __half** xl);
 void gemm_act_forget();
+// Gated activation (op2 34 GEGLU / 35 SWIGLU) of the [M, K] rows at elements a and b into the rows at d, and the fp16
+// form of the result for the batched matmul that follows, in one launch.  false: not taken, nothing launched.
+bool launch_glu_act_f16(const Map* ma, uint32_t op, uint32_t a, uint32_t b, uint32_t d, uint32_t M, uint32_t K);
 void gemm_act_mark(const void* buf, uint64_t a, uint32_t M, uint32_t K);
 // Second pass of the fused GEMV + argmax: best of the per-group partials, token id stored as float.
 int launch_argmax_pairs(const Map* ma, const uint32_t* lidx, const uint32_t* lval, const uint32_t* ldst,

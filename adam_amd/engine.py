@@ -321,6 +321,7 @@ class DecodeEngine:
         self._c_tok_locs = np.arange(pos, pos + M, dtype=np.uint32)
         pos += M
         self._c_last = self._up(np.zeros(c.n_embd, np.uint32))
+        self._c_last_m = 0
         self._c_zero = self._up([0])
         self._c_emb_hs = {}
         self._c_wrows = {}
@@ -783,12 +784,17 @@ class DecodeEngine:
                 self._c_emb_hs[m] = self._up(locs.reshape(-1))
             emb_h = self._c_emb_hs[m]
         else:
-            rows = np.stack([self.tensors['token_embd.weight'].row(int(t)) for t in toks]).astype(np.float32)
+            emb = self.tensors['token_embd.weight']
+            rows = np.empty((m, E), np.float32)
+            for i, t in enumerate(toks):
+                rows[i] = emb.row(int(t))
             if c.emb_scale != 1.0:
-                rows = rows * np.float32(c.emb_scale)
-            g.scatter(ws, np.arange(self._cp['hidden'], self._cp['hidden'] + m * E, dtype=np.uint32), rows.reshape(-1))
-        last = self._cp['hidden'] + (m - 1) * E
-        g.upload_dev(np.arange(last, last + E, dtype=np.uint32), handle=self._c_last)
+                rows *= np.float32(c.emb_scale)
+            g.scatter_contiguous(ws, self._cp['hidden'], rows)      # one range: no list of locations to send along
+        if self._c_last_m != m:                                      # where the last row sits only depends on m
+            last = self._cp['hidden'] + (m - 1) * E
+            g.upload_dev(np.arange(last, last + E, dtype=np.uint32), handle=self._c_last)
+            self._c_last_m = m
 
         def mm(src, name, dst, K, N):
             fn = g.map_matmul_t_xq8_dev if self._kind[name] == 'q8' else g.map_matmul_t_xq4_dev

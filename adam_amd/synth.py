@@ -43,23 +43,27 @@ def tiny_config(arch="gemma3", n_layer=2, n_embd=128, n_head=4, n_head_kv=1, hea
 
 
 class SyntheticEmbedding:
-    """Untied token embedding generated row by row (the reference looks untied embeddings up on
-    the host, engine.py:2986-2992, so no [V, E] matrix has to exist anywhere)."""
+    """Untied token embedding (the reference looks untied embeddings up on the host, engine.py:2986-2992: a row
+    copy out of a float32 table).  A [V, E] float32 table of a large vocabulary would take gigabytes of host
+    memory for numbers that carry no information, so the rows come from a pool of at most POOL generated rows,
+    made on first use: a lookup is a copy, as in a real model, and tokens POOL apart (after a fixed scramble)
+    share a row."""
+
+    POOL = 4096
 
     def __init__(self, n_vocab, n_embd, seed, sigma):
         self.shape = (n_vocab, n_embd)
         self.seed, self.sigma = seed, sigma
-        self._seen = {}          # rows already generated (a real model's lookup is a copy, not a generator run)
+        self._pool = None
 
     def row(self, tok):
+        if self._pool is None:
+            rng = np.random.default_rng([self.seed, 0x0E3B])
+            n = min(self.shape[0], self.POOL)
+            self._pool = rng.standard_normal((n, self.shape[1]), dtype=np.float32) * np.float32(self.sigma)
+        n = self._pool.shape[0]
         tok = int(tok)
-        r = self._seen.get(tok)
-        if r is None:
-            rng = np.random.default_rng([self.seed, 0x0E3B, tok])
-            r = rng.standard_normal(self.shape[1], dtype=np.float32) * np.float32(self.sigma)
-            if len(self._seen) < 8192:
-                self._seen[tok] = r
-        return r
+        return self._pool[tok if self.shape[0] <= n else (tok * 40503 + 11) % n]
 
 
 def _gen(name, shape, seed, sigma, quant, rows_per_chunk=8192):

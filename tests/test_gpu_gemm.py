@@ -290,3 +290,103 @@ def test_residual_add_stored_by_the_matmul(hip, M, K, N, in_place):
     assert np.array_equal(fused.view(np.uint32), apart.view(np.uint32))
     want, _ = go(oracle.init())
     assert rel_l2(fused[y0:], want[y0:]) < TOL
+
+
+@pytest.mark.parametrize("op,M,K,N,in_place", [("swiglu", 16, 14336, 96, False), ("geglu", 5, 6912, 64, False), ("swiglu", 40, 256, 50, False),
+                                               ("geglu", 16, 1024, 96, True)])
+def test_gated_activation_feeds_the_matmul_without_a_conversion_launch(hip, op, M, K, N, in_place):
+    """act = GLU(gate, up) over M rows followed by the batched matmul over act: the activation's launch also writes
+    the matmul's fp16 operand form (two launches instead of three), and every word equals the separate ops'
+    (ADAMAH_GLU_EMIT=0).  An activation stored over its own gate rows is left as it was."""
+    import os
+    rng = np.random.default_rng(M + K)
+    qt = quant.quantize_q4_0(rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.05))
+    gate = rng.standard_normal((M, K), dtype=np.float32) * np.float32(2.0)
+    upv = rng.standard_normal((M, K), dtype=np.float32)
+    a0 = 0 if in_place else 2 * M * K
+    y0 = 3 * M * K
+    code = A.OP_SWIGLU if op == "swiglu" else A.OP_GEGLU
+
+    def go(g):
+        load_qtensor(g, 1, qt)
+        f32map(g, 0, y0 + M * N + 8, np.concatenate([gate.reshape(-1), upv.reshape(-1)]))
+        hg, hu, ha = up(g, np.arange(M * K)), up(g, M * K + np.arange(M * K)), up(g, a0 + np.arange(M * K))
+        a, b, c = up(g, [a0]), up(g, [0]), up(g, [y0])
+        g.batch_begin()
+        g.map_op2_dev(0, code, hg, hu, ha, M * K)
+        g.map_matmul_t_xq4_dev(0, 1, a, b, c, M, K, N, 1)
+        g.batch_end()
+        return read(g, 0, 0, y0 + M * N), (g.get_last_barrier_count() if g is hip else None)
+
+    note(f"{op} + matmul M={M} K={K} N={N} in_place={in_place}")
+    fused, n_fused = go(hip)
+    os.environ["ADAMAH_GLU_EMIT"] = "0"
+    try:
+        apart, n_apart = go(hip)
+    finally:
+        del os.environ["ADAMAH_GLU_EMIT"]
+    assert np.array_equal(fused.view(np.uint32), apart.view(np.uint32))
+    if K % 128 == 0:
+        assert (n_fused, n_apart) == ((3, 3) if in_place else (2, 3))
+    want, _ = go(oracle.init())
+    assert rel_l2(fused[a0:a0 + M * K], want[a0:a0 + M * K]) < 1e-5
+    assert rel_l2(fused[y0:], want[y0:]) < TOL
+
+
+@pytest.mark.parametrize("kind,op,M,K,F", [("q4", "swiglu", 16, 4096, 14336), ("q4", "geglu", 5, 256, 48), ("q8", "swiglu", 32, 512, 80),
+                                           ("q4", "swiglu", 16, 256, 40), ("q4", "geglu", 40, 256, 48)])
+def test_gated_activation_stored_by_the_stacked_gate_up_matmul(hip, kind, op, M, K, F):
+    """gate = X Wg^T, up = X Wu^T (matrices back to back), act = GLU(gate, up), then a matmul over act, as a
+    batched decode step issues them: for M <= 32 and F a multiple of 16 the stacked launch stores act as well
+    (conversion + stacked matmul + conversion + matmul = 4 launches), every word equal to the separate ops'
+    (ADAMAH_GEMM_EPI=0, ADAMAH_GLU_EMIT=0: 5); otherwise the activation's own launch leaves the fp16 form (4)."""
+    import os
+    rng = np.random.default_rng(M + K + F)
+    qfn = quant.quantize_q4_0 if kind == "q4" else quant.quantize_q8_0
+    qt = qfn(rng.standard_normal((2 * F, K), dtype=np.float32) * np.float32(0.05))
+    N2 = 24
+    fn_name = "map_matmul_t_xq4_dev" if kind == "q4" else "map_matmul_t_xq8_dev"
+    mid = 1 if kind == "q4" else 2
+    x = rng.standard_normal((M, K), dtype=np.float32)
+    g0, u0, a0 = M * K, M * K + M * F, M * K + 2 * M * F
+    y0 = a0 + M * F
+    total = y0 + M * N2 + 8
+    wd = rng.standard_normal((N2, F), dtype=np.float32) * np.float32(0.05)
+    down_ok = F % 128 == 0
+
+    def go(g):
+        load_qtensor(g, mid, qt)
+        if down_ok:
+            load_qtensor(g, 3, quant.quantize_q4_0(wd))
+        f32map(g, 0, total, x.reshape(-1))
+        a, b0, b1 = up(g, [0]), up(g, [0]), up(g, [F * K])
+        cg, cu, ca, cy = up(g, [g0]), up(g, [u0]), up(g, [a0]), up(g, [y0])
+        hg, hu, ha = up(g, g0 + np.arange(M * F)), up(g, u0 + np.arange(M * F)), up(g, a0 + np.arange(M * F))
+        g.batch_begin()
+        getattr(g, fn_name)(0, mid, a, b0, cg, M, K, F, 1)
+        getattr(g, fn_name)(0, mid, a, b1, cu, M, K, F, 1)
+        g.map_op2_dev(0, A.OP_SWIGLU if op == "swiglu" else A.OP_GEGLU, hg, hu, ha, M * F)
+        if down_ok:
+            g.map_matmul_t_xq4_dev(0, 3, ca, up(g, [0]), cy, M, F, N2, 1)
+        g.batch_end()
+        return read(g, 0, 0, total), (g.get_last_barrier_count() if g is hip else None)
+
+    note(f"gate/up + {op} {kind} M={M} K={K} F={F}")
+    fused, n_fused = go(hip)
+    os.environ["ADAMAH_GEMM_EPI"] = "0"
+    os.environ["ADAMAH_GLU_EMIT"] = "0"
+    try:
+        apart, n_apart = go(hip)
+    finally:
+        del os.environ["ADAMAH_GEMM_EPI"], os.environ["ADAMAH_GLU_EMIT"]
+    assert np.array_equal(fused.view(np.uint32), apart.view(np.uint32))
+    if down_ok:
+        assert (n_fused, n_apart) == (4, 5)
+    else:
+        assert (n_fused, n_apart) == ((2, 3) if M <= 32 and F % 16 == 0 else (3, 3))
+    want, _ = go(oracle.init())
+    assert rel_l2(fused[g0:a0], want[g0:a0]) < TOL
+    assert rel_l2(fused[a0:y0], want[a0:y0]) < TOL
+    if down_ok:
+        assert rel_l2(fused[y0:y0 + M * N2], want[y0:y0 + M * N2]) < TOL
+    assert not fused[y0 + M * N2:].any()
