@@ -478,6 +478,173 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
 }
 #undef GEMM_FETCH
 
+// M <= 16 and many weight rows: the waves of a workgroup take 16 weight rows each and share ONE activation tile per
+// step of K, staged through LDS once for all of them (the K-split form above stages a tile per wave: the tile, both
+// planes of all 16 rows, is 7x the bytes of a wave's weights, and those requests to the L1, not HBM, set its pace).
+// A macro step is two steps of K (256 weights).  Registers hold rings of what is on its way: the workgroup's next
+// four activation macro tiles (a thread's share: one or two pieces per plane each) and each wave's weights of the next
+// four macro steps, so a CU keeps ~10 KB per wave in flight; LDS holds two macro tiles, one being read by the matrix
+// instructions while the next is written, with one barrier per macro step.  Every load is issued on every path
+// (clamped to the last step of K): the waits stay counted.
+// segs.count: stacked matrices, as above.  segs.glu: [gate rows; up rows]: the first half of the waves takes gate
+// tiles, the second half the up tiles that belong to them; the up waves hand their results over in LDS and the
+// gate waves also store act(gate) * up at segs.dst.
+#define R16_MS 2u
+template <int NW>
+__global__ void __launch_bounds__(64 * NW)
+k_gemm_q4_f16_rows16(float* out, const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh,
+                     const u4q_t* __restrict__ xl, const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc,
+                     const float* __restrict__ scale, uint32_t M, uint32_t K, uint32_t N, GemmSegs segs) {
+  constexpr uint32_t ROWB = 272u, TILE = 16u * ROWB, NT = 64u * NW;
+  constexpr uint32_t PIECES = R16_MS * 256u;                 // 16-byte pieces per plane and macro step
+  constexpr uint32_t NP = (PIECES + NT - 1u) / NT;           // per thread
+  __shared__ __attribute__((aligned(16))) uint8_t xs_all[2u * 2u * R16_MS * TILE];   // [buffer][plane][step of the macro step]
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+  const uint32_t r16 = lane & 15u, g = lane >> 4, op = blockIdx.z;
+  const bool glum = segs.glu != 0u;
+  // first weight row of the wave's tile (glu: tb = the tile's first row within its half of the matrix)
+  const uint32_t tb = glum ? blockIdx.x * (8u * NW) + (wave % (NW / 2u)) * 16u : blockIdx.x * (16u * NW) + wave * 16u;
+  const uint32_t n0 = glum && wave >= NW / 2u ? (N >> 1) + tb : tb;
+  const uint64_t c_off = lc ? (uint64_t)lc[op] : 0ull, gbase = (uint64_t)lb[op] >> 5;
+  const uint32_t nblk = K >> 5, kw = K >> 3, steps = nblk >> 2, macros = (steps + R16_MS - 1u) / R16_MS;
+  const uint32_t lrow = lane >> 2, lblk = lane & 3u;
+  const int perm_addr = (int)((4u * r16 + g) << 2);
+  const uint64_t wrow = gbase + (uint64_t)min(n0 + lrow, N - 1u) * nblk + lblk;
+  DEQK_INIT(dk);
+  f4q_t acc = {0.f, 0.f, 0.f, 0.f};
+
+  // a thread's pieces of a macro tile: piece w -> (step w / 256, row (w / 16) % 16, piece w % 16)
+  uint64_t xoff[NP];
+  uint32_t xlds[NP], xst[NP];
+#pragma unroll
+  for (uint32_t u = 0; u < NP; u++) {
+    const uint32_t w = min(tid + u * NT, PIECES - 1u), row = (w >> 4) & 15u, pc = w & 15u;
+    xst[u] = w >> 8;
+    xoff[u] = ((uint64_t)op * M + min(row, M - 1u)) * kw + pc;     // + 16 pieces per step of K
+    xlds[u] = xst[u] * TILE + row * ROWB + pc * 16u;
+  }
+  struct ActR { u4q_t h[NP], l[NP]; };
+  struct WtR { u4q_t q[R16_MS]; uint32_t d[R16_MS]; };
+  ActR a0, a1, a2, a3;
+  WtR w0, w1, w2, w3;
+  // (steps past the end of K ask for the last step again: not used)
+  auto fetch_a = [&](ActR& a, uint32_t m) {
+#pragma unroll
+    for (uint32_t u = 0; u < NP; u++) {
+      const uint64_t at = xoff[u] + min(m * R16_MS + xst[u], steps - 1u) * 16u;
+      a.h[u] = xh[at]; a.l[u] = xl[at];
+    }
+  };
+  auto fetch_w = [&](WtR& w, uint32_t m) {
+#pragma unroll
+    for (uint32_t s = 0; s < R16_MS; s++) {
+      const uint64_t gi = wrow + min(m * R16_MS + s, steps - 1u) * 4u;
+      w.q[s] = *(const u4q_t*)(W + (gi << 4));
+      w.d[s] = (uint32_t)((const uint16_t*)d16)[gi];
+    }
+  };
+  auto put_a = [&](const ActR& a, uint32_t buf) {
+    uint8_t* b = xs_all + buf * (2u * R16_MS * TILE);
+#pragma unroll
+    for (uint32_t u = 0; u < NP; u++)
+      if (NT * NP == PIECES || tid + u * NT < PIECES) {
+        *(u4q_t*)(b + xlds[u]) = a.h[u];
+        *(u4q_t*)(b + R16_MS * TILE + xlds[u]) = a.l[u];
+      }
+  };
+  auto compute = [&](const WtR& w, uint32_t m, uint32_t buf) {
+    const uint8_t* b0 = xs_all + buf * (2u * R16_MS * TILE);
+#pragma unroll
+    for (uint32_t s = 0; s < R16_MS; s++) {
+      u4q_t q = {(uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)w.q[s].x), (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)w.q[s].y),
+                 (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)w.q[s].z), (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)w.q[s].w)};
+      const uint32_t dbits = (uint32_t)__builtin_amdgcn_ds_bpermute(perm_addr, (int)w.d[s]);
+      q = transpose_blocks(q);
+      const f4q_t ds = gather_scales(__builtin_bit_cast(_Float16, (uint16_t)dbits));
+      if (m * R16_MS + s < steps) {     // (uniform; the last macro step of an odd number of steps is half empty)
+        const uint8_t* xs = b0 + s * TILE;
+        const uint8_t* xs2 = xs + R16_MS * TILE;
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+          const u4q_t wq = deq_word(b == 0 ? q.x : b == 1 ? q.y : b == 2 ? q.z : q.w, dk);
+          const uint32_t xo = r16 * ROWB + b * 64u + g * 16u;
+          const u4q_t ah = *(const u4q_t*)(xs + xo), al = *(const u4q_t*)(xs2 + xo);
+          f4q_t blk = MFMA_F16(ah, wq, ((f4q_t){0.f, 0.f, 0.f, 0.f}));
+          blk = MFMA_F16(al, wq, blk);
+          const float d = ds[b];
+#pragma unroll
+          for (int i = 0; i < 4; i++) acc[i] = fmaf(blk[i], d, acc[i]);
+        }
+      }
+    }
+  };
+  // prologue: activation tiles 0 .. 4 and weights 0 .. 3, in the order the loop issues them (a tile, then the weights
+  // that go with it: loads return in order, and the tile is waited for first), so that the loop's first wait finds
+  // the same loads behind its tile whether it is entered from here or from its own end
+  fetch_a(a0, 0u);
+  fetch_a(a1, 1u); fetch_w(w0, 0u); fetch_a(a2, 2u); fetch_w(w1, 1u); fetch_a(a3, 3u); fetch_w(w2, 2u);
+  asm volatile("" ::: "memory");   // the loads stay here: none of them is moved below the first tile's wait
+  __builtin_amdgcn_sched_barrier(0);
+  put_a(a0, 0u);
+  __builtin_amdgcn_sched_barrier(0);
+  fetch_a(a0, 4u); fetch_w(w3, 3u);
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+  __syncthreads();
+  // macro step m: tile m + 1 goes to LDS, tile m + 5 and the weights of m + 4 are asked for, m is computed
+#define R16_STEP(AR, WR, mm)                                       \
+  {                                                                \
+    put_a(AR, ((mm) + 1u) & 1u);                                   \
+    __builtin_amdgcn_sched_barrier(0);                             \
+    fetch_a(AR, (mm) + 5u);                                        \
+    __builtin_amdgcn_sched_barrier(0);                             \
+    compute(WR, (mm), (mm) & 1u);                                  \
+    __builtin_amdgcn_sched_barrier(0);                             \
+    fetch_w(WR, (mm) + 4u);                                        \
+    __builtin_amdgcn_sched_barrier(0);                             \
+    __syncthreads();                                               \
+  }
+  // (four macro steps per round and one way out: steps past the end of K compute nothing)
+  for (uint32_t m = 0; m < macros; m += 4u) {
+    R16_STEP(a1, w0, m);
+    R16_STEP(a2, w1, m + 1u);
+    R16_STEP(a3, w2, m + 2u);
+    R16_STEP(a0, w3, m + 3u);
+  }
+#undef R16_STEP
+  // lane (r16, g) holds D[4g + i][r16]: activation row 4g + i, weight row n0 + r16
+  const uint32_t n = n0 + r16;
+  float y[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint32_t row = min(4u * g + i, M - 1u);
+    y[i] = acc[i] * scale[2 * ((uint64_t)op * M + row) + 1];
+  }
+  float* ybuf = (float*)xs_all;            // the up waves' tiles, [wave - NW / 2][i][lane]
+  if (glum && wave >= NW / 2u) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) ybuf[((wave - NW / 2u) * 4u + i) * 64u + lane] = y[i];
+  }
+  if (glum) __syncthreads();
+  const bool n_ok = glum ? tb + r16 < (N >> 1) : n < N;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint32_t row = 4u * g + i;
+    if (row >= M || !n_ok) continue;
+    if (segs.count) {
+      uint32_t sgi = 0;
+#pragma unroll
+      for (uint32_t q = 1; q < 4; q++) sgi += (q < segs.count && n >= segs.begin[q]) ? 1u : 0u;
+      out[segs.c[sgi] + (uint64_t)row * segs.n[sgi] + (n - segs.begin[sgi])] = y[i];
+    } else out[c_off + (uint64_t)row * N + n] = y[i];
+    if (glum && wave < NW / 2u) {
+      const float a = y[i], b = ybuf[(wave * 4u + i) * 64u + lane];
+      out[segs.dst + (uint64_t)row * (N >> 1) + n] = segs.glu == 34u ? gelu_tanh(a) * b : (a / (1.0f + expf(-a))) * b;
+    }
+  }
+}
+
 // The same conversion with the row held in registers: 1024 threads, thread t owns the 8-element words
 // t, t + 1024, ... (NW of them; K <= 8192 NW), so the row makes one trip from memory instead of two
 // dependent passes -- the rows of a decode batch are few and each workgroup's latency is the launch's.
@@ -651,6 +818,21 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
     if (sg.glu) {             // a workgroup pairs one gate tile with its up tile
       if (sg.count != 2 || sg.n[0] != sg.n[1] || (sg.n[0] & 15u)) return ADAMAH_ERR_INVALID;
       R = 2;
+    }
+    // many weight rows under at most 16 activation rows: the form whose eight waves share the activation tile, when
+    // its workgroups of 128 weight rows still cover three quarters of the CUs (28672x4096: 28.5 against 32.5 us)
+    {
+      const bool glu_ok = !sg.glu || (sg.count == 2 && sg.n[0] == sg.n[1] && (sg.n[0] & 15u) == 0);
+      const uint32_t wgs16 = cdiv(sg.glu ? N / 2 : N, sg.glu ? 64u : 128u);
+      if (mt == 1 && !q8 && !sg.add && glu_ok && (uint64_t)wgs16 * 4 >= 3ull * (uint64_t)g.n_cu &&
+          tuning("ADAMAH_GEMM_ROWS16", 1) != 0) {
+        dim3 gridr(wgs16, 1, n_ops);
+        k_gemm_q4_f16_rows16<8><<<gridr, 512, 0, g.stream>>>(out ? out : act, mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, lb,
+                                                            out ? nullptr : lc, g_scale_buf, M, K, N, sg);
+        count_launch();
+        keep();
+        return check_launch();
+      }
     }
     dim3 grid(cdiv(N, 16 * R), cdiv(M, 16 * mt), n_ops);
     float* dst = out ? out : act;

@@ -33,7 +33,7 @@ def run(g, qt, x, n_ops=1, scale=None, zp=None):
 
 
 @pytest.mark.parametrize("M,N,K", [(16, 4096, 4096), (512, 4096, 4096), (16, 4096, 14336), (512, 1000, 1152),
-                                   (2, 64, 128), (40, 130, 256), (100, 6144, 4096)])
+                                   (2, 64, 128), (40, 130, 256), (100, 6144, 4096), (16, 28672, 4096), (9, 24600, 1152)])
 def test_batched_q4_matmul_matches_oracle(hip, M, N, K):
     rng = np.random.default_rng(M + N + K)
     qt = quant.quantize_q4_0((rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.02)))
@@ -46,6 +46,14 @@ def test_batched_q4_matmul_matches_oracle(hip, M, N, K):
         assert rel_l2(y[m], want[m]) < TOL_Q4, m
     if M * N * K <= 40 * 130 * 256:      # the oracle's own M > 1 path on the small case
         assert rel_l2(y, run(oracle.init(), qt, x)[0]) < TOL
+    if M <= 16 and N >= 24576:           # wide matrices take the kernel whose waves share the activation tile
+        import os
+        os.environ["ADAMAH_GEMM_ROWS16"] = "0"
+        try:
+            y0 = run(hip, qt, x)[0]
+        finally:
+            del os.environ["ADAMAH_GEMM_ROWS16"]
+        assert not np.array_equal(y, y0) and rel_l2(y, y0) < 1e-5      # another kernel, the same product
 
 
 def test_batched_matmul_row_scaling_and_ops(hip):
