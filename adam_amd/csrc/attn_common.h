@@ -24,7 +24,7 @@ __device__ __forceinline__ void rope_cs2(uint32_t i, uint32_t dim, uint32_t pos,
 
 // A row task of the preparation before decode attention (rowprep.hip): source row, optional norm weights,
 // optional rotation, destination row, optional cache row.
-#define ROWT_MAX 64u
+#define ROWT_MAX ROW_RUN_MAX
 #define ROWT_NONE 0xFFFFFFFFu
 struct RowTask {
   uint32_t src, dst, cache, w;   // element offsets; dst / cache / w may be ROWT_NONE

@@ -80,9 +80,11 @@ struct PendOp {
   float eps = 0.f;                       // RMSNORM: eps.  ATTN: score scale
   float f2 = 0.f;                        // ATTN: soft cap
   // SCORES: k = head dim, n = sequence length.  ATTN: n = sequence length, k = value dim.
-  // ROPE (one token): a = src, c = dst, rpg = heads, k = head dim, n = position, eps = frequency base.
+  // ROPE (one token): a = src, c = dst, rpg = heads, k = head dim, n = position, eps = frequency base; op = 1: more
+  //   heads than a row run holds (h = src, dst handles).
   // QKNR: h = q rows, q weights, k rows, k weights, dst; rpg/k = q rows/dim, op/d = k rows/dim, n, eps as ROPE.
-  // ROWCOPY: h = spec, source base; rpg = copies, k = row size, n = destination row offset.
+  // ROWCOPY: h = spec, source base; rpg = copies, k = row size, n = destination row offset; op = 1: more copies than
+  //   a row run holds.
   // GEMM (two or more activation rows, block16 weights): a, b, c = X, W, Y; rpg = M; k, n = K, N; op = weight format;
   //   h = X, W, Y handles.
 };
@@ -174,6 +176,10 @@ bool row_op_deferrable(const PendOp& p);                                  // row
 // Element ranges (start, length) of the activation map a queued row op reads or writes; false: not known on the host.
 bool row_op_ranges(const PendOp& p, std::vector<std::pair<uint64_t, uint64_t>>* out);   // rowprep.hip
 size_t launch_row_run(const std::vector<PendOp>& q, size_t i, int* rc);   // rowprep.hip
+// a rotation / row copy with more rows than a row run holds (PendOp.op == 1): alone, or rotation + rotation + KV append
+// of one position in one launch; returns the queue entries used
+#define ROW_RUN_MAX 64u
+size_t launch_wide_rows(const std::vector<PendOp>& q, size_t i, int* rc);   // norm_rope.hip
 int launch_op2_v(const PendOp& p);
 // Attention (attention.hip): stand-alone launches of queued ops, and the fused form.  launch_attn
 // runs scores (when sc != nullptr) and softmax . V; with leave_partials it stops before the merge

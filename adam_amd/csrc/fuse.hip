@@ -212,6 +212,12 @@ void flush_pending() {
   };
   while (i < n) {
     if (park.active && i > park.at) unpark_now();
+    if ((q[i].kind == PK_ROPE || q[i].kind == PK_ROWCOPY) && q[i].op == 1u) {   // one token of many sequences
+      int rc = 0;
+      i += launch_wide_rows(q, i, &rc);
+      keep(rc);
+      continue;
+    }
     RowPrepCtx prep = {&q, i, {}};
     bool have_prep = false;
     if (q[i].kind == PK_ROPE || q[i].kind == PK_QKNR || q[i].kind == PK_ROWCOPY) {

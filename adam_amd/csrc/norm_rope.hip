@@ -243,6 +243,121 @@ static int rmsnorm_impl(uint32_t map_act, uint32_t map_wt, uint32_t hs, uint32_t
   return check_launch();
 }
 
+// One token of many sequences in lockstep: the rotation of all their Q heads, the rotation of all their K heads and the
+// append of the K and V rows to the caches (three ops, issued in that order) in one launch.  One workgroup per
+// row: the Q rows, then the K rows, then the copies.  A copy whose source is a K row of the launch is done by that
+// row's workgroup, which finds it in the copy list and stores the rotated row twice (in place, and to the cache with
+// the cache's fp16 rounding); its own workgroup leaves at once.  The host has checked that every copy's source is
+// either exactly one such K row (each at most once) or lies clear of both rotated ranges, and that all destinations
+// lie in the fp16 KV range, which holds no source.  Arithmetic of the three stand-alone kernels.
+__global__ void __launch_bounds__(256)
+k_rope2_copy(float* data, uint32_t qa, uint32_t q_rows, uint32_t q_dim, uint32_t ka, uint32_t k_rows, uint32_t k_dim,
+             uint32_t pos, float base, const uint32_t* __restrict__ spec, uint32_t src_base, uint32_t n_copies,
+             uint32_t dst_row_offset, __half* kv16, uint64_t kv_start, uint64_t kv_count) {
+  __shared__ uint32_t found;
+  const uint32_t b = blockIdx.x, tid = threadIdx.x;
+  auto put = [&](uint64_t dof, float v) {     // into the cache: rounded to fp16 and mirrored, as the row copy does
+    if (kv16 && dof >= kv_start && dof - kv_start < kv_count) {
+      const __half h = __float2half(v);
+      kv16[dof - kv_start] = h;
+      v = __half2float(h);
+    }
+    data[dof] = v;
+  };
+  if (b < q_rows + k_rows) {
+    const bool is_q = b < q_rows;
+    const uint32_t dim = is_q ? q_dim : k_dim, half = dim >> 1;
+    const uint64_t row = is_q ? (uint64_t)qa + (uint64_t)b * q_dim : (uint64_t)ka + (uint64_t)(b - q_rows) * k_dim;
+    uint32_t dst_row = 0xFFFFFFFFu;
+    if (!is_q) {
+      if (tid == 0) found = 0xFFFFFFFFu;
+      __syncthreads();
+      for (uint32_t ci = tid; ci < n_copies; ci += 256u)
+        if ((uint64_t)src_base + (uint64_t)spec[2 * ci] * k_dim == row) found = spec[2 * ci + 1];   // at most one
+      __syncthreads();
+      dst_row = found;
+    }
+    for (uint32_t d = tid; d < half; d += 256u) {
+      float c, s;
+      rope_cs(d, dim, pos, base, &c, &s);
+      const float x0 = data[row + d], x1 = data[row + d + half];
+      const float r0 = x0 * c - x1 * s, r1 = x0 * s + x1 * c;
+      data[row + d] = r0;
+      data[row + d + half] = r1;
+      if (dst_row != 0xFFFFFFFFu) {
+        const uint64_t dof = ((uint64_t)dst_row + dst_row_offset) * k_dim;
+        put(dof + d, r0);
+        put(dof + d + half, r1);
+      }
+    }
+    return;
+  }
+  const uint32_t ci = b - q_rows - k_rows;
+  const uint64_t so = (uint64_t)src_base + (uint64_t)spec[2 * ci] * k_dim;
+  if (so >= ka && so < (uint64_t)ka + (uint64_t)k_rows * k_dim) return;     // done by the K row's workgroup
+  const uint64_t dof = ((uint64_t)spec[2 * ci + 1] + dst_row_offset) * k_dim;
+  for (uint32_t e = tid; e < k_dim; e += 256u) put(dof + e, data[so + e]);
+}
+
+// A queued rotation (one token, more heads than a row run holds) or row copy (more copies than that) by itself.
+static int launch_wide_alone(const PendOp& p, Map* m) {
+  if (p.kind == PK_ROPE) {
+    const uint32_t *ls = res_u32(p.h[0], 1), *ld = res_u32(p.h[1], 1);
+    if (!ls || !ld) return ADAMAH_ERR_INVALID;
+    const uint64_t pairs = (uint64_t)p.rpg * (p.k / 2);
+    k_rope<<<cdiv(pairs, 256), 256, 0, g.stream>>>((float*)m->buf, ls, ld, 1, p.rpg, p.k, p.n, p.eps, m->n_elems);
+  } else {
+    const uint32_t *spec = res_u32(p.h[0], 2ull * p.rpg), *base = res_u32(p.h[1], 1);
+    if (!spec || !base) return ADAMAH_ERR_INVALID;
+    k_row_copy<<<cdiv((uint64_t)p.rpg * p.k, 256), 256, 0, g.stream>>>((float*)m->buf, spec, base, p.rpg, p.k, p.n, m->n_elems, m->kv16,
+                                                                    m->kv_start, m->kv_count);
+  }
+  count_launch();
+  return check_launch();
+}
+
+// q[i] is a wide rotation or row copy (op == 1).  Rotation of the Q heads, rotation of the K heads in place and the
+// KV append behind them, all of one position: one launch; anything else: q[i] by itself.  Returns the entries used.
+size_t launch_wide_rows(const std::vector<PendOp>& q, size_t i, int* rc) {
+  Map* m = get_f32_map(q[i].map_act);
+  if (!m) { *rc = ADAMAH_ERR_INVALID; return 1; }
+  auto fold = [&]() -> bool {
+    if (i + 2 >= q.size()) return false;
+    const PendOp &pq = q[i], &pk = q[i + 1], &pc = q[i + 2];
+    if (pq.kind != PK_ROPE || pk.kind != PK_ROPE || pc.kind != PK_ROWCOPY || pk.op != 1u || pc.op != 1u ||
+        pk.map_act != pq.map_act || pc.map_act != pq.map_act || pq.a != pq.c || pk.a != pk.c || pk.n != pq.n || pk.eps != pq.eps ||
+        pc.k != pk.k || !m->kv16)
+      return false;
+    const uint64_t q0 = pq.a, q1 = q0 + (uint64_t)pq.rpg * pq.k, k0 = pk.a, k1 = k0 + (uint64_t)pk.rpg * pk.k;
+    const uint64_t c0 = m->kv_start, c1 = c0 + m->kv_count;
+    auto apart = [](uint64_t a0, uint64_t a1, uint64_t b0, uint64_t b1) { return a1 <= b0 || b1 <= a0; };
+    if (!apart(q0, q1, k0, k1) || !apart(q0, q1, c0, c1) || !apart(k0, k1, c0, c1)) return false;
+    const uint32_t *spec = res_host(pc.h[0], 2ull * pc.rpg), *base = res_host(pc.h[1], 1);
+    if (!spec || !base || !res_u32(pc.h[0], 2ull * pc.rpg)) return false;
+    std::vector<uint8_t> seen(pk.rpg, 0);
+    for (uint32_t ci = 0; ci < pc.rpg; ci++) {
+      const uint64_t so = (uint64_t)base[0] + (uint64_t)spec[2 * ci] * pc.k, s1 = so + pc.k;
+      const uint64_t d0 = ((uint64_t)spec[2 * ci + 1] + pc.n) * pc.k, d1 = d0 + pc.k;
+      if (d0 < c0 || d1 > c1 || s1 > m->n_elems) return false;
+      if (so >= k0 && so < k1) {
+        if ((so - k0) % pk.k) return false;
+        const uint64_t j = (so - k0) / pk.k;
+        if (seen[j]) return false;
+        seen[j] = 1;
+      } else if (!apart(so, s1, k0, k1) || !apart(so, s1, q0, q1) || !apart(so, s1, c0, c1)) return false;
+    }
+    k_rope2_copy<<<pq.rpg + pk.rpg + pc.rpg, 256, 0, g.stream>>>((float*)m->buf, pq.a, pq.rpg, pq.k, pk.a, pk.rpg, pk.k, pq.n, pq.eps,
+                                                              res_u32(pc.h[0], 2ull * pc.rpg), base[0], pc.rpg, pc.n, m->kv16,
+                                                              m->kv_start, m->kv_count);
+    count_launch();
+    *rc = check_launch();
+    return true;
+  };
+  if (q[i].kind == PK_ROPE && fold()) return 3;
+  *rc = launch_wide_alone(q[i], m);
+  return 1;
+}
+
 }  // namespace adamah
 
 using namespace adamah;
@@ -271,7 +386,17 @@ int map_rope_dev(uint32_t map_id, uint32_t hs, uint32_t hd, uint32_t n_tokens, u
     // one token with operands known on the host: queue it, it may share a launch with the KV append
     PendOp p;
     p.kind = PK_ROPE; p.map_act = map_id; p.rpg = n_heads; p.k = head_dim; p.n = pos_offset; p.eps = freq_base;
-    if (res_scalar(hs, &p.a) && res_scalar(hd, &p.c) && row_op_deferrable(p)) { g.pend.push_back(p); return ADAMAH_OK; }
+    if (res_scalar(hs, &p.a) && res_scalar(hd, &p.c)) {
+      if (row_op_deferrable(p)) { g.pend.push_back(p); return ADAMAH_OK; }
+      // more heads than a row run holds (one token of many sequences): queued as well, it may share a launch with
+      // the rotation and the KV append next to it
+      if (n_heads > ROW_RUN_MAX && (head_dim & 1u) == 0 && in_range(p.a, (uint64_t)n_heads * head_dim, m->n_elems) &&
+          in_range(p.c, (uint64_t)n_heads * head_dim, m->n_elems) && tuning("ADAMAH_ROWS_WIDE", 1) != 0) {
+        p.op = 1u; p.h[0] = hs; p.h[1] = hd;
+        g.pend.push_back(p);
+        return ADAMAH_OK;
+      }
+    }
   }
   flush_pending();
   const uint32_t *ls = res_u32(hs, n_tokens), *ld = res_u32(hd, n_tokens);
@@ -318,6 +443,11 @@ int map_row_copy_offset_dev(uint32_t map_id, uint32_t hspec, uint32_t hbase, uin
     p.kind = PK_ROWCOPY; p.map_act = map_id; p.h[0] = hspec; p.h[1] = hbase; p.rpg = n_copies; p.k = row_size;
     p.n = dst_row_offset;
     if (row_op_deferrable(p)) { g.pend.push_back(p); return ADAMAH_OK; }
+    if (n_copies > ROW_RUN_MAX && res_host(hspec, 2ull * n_copies) && res_host(hbase, 1) && tuning("ADAMAH_ROWS_WIDE", 1) != 0) {
+      p.op = 1u;     // more copies than a row run holds: queued as well (see map_rope_dev); operands checked at launch
+      g.pend.push_back(p);
+      return ADAMAH_OK;
+    }
   }
   flush_pending();
   const uint32_t *spec = res_u32(hspec, 2ull * n_copies), *base = res_u32(hbase, 1);

@@ -155,6 +155,7 @@ size_t build_row_run(const std::vector<PendOp>& q, size_t i, std::vector<RowTask
   for (; j < q.size(); j++) {
     const PendOp& p = q[j];
     if ((p.kind != PK_ROPE && p.kind != PK_QKNR && p.kind != PK_ROWCOPY) || p.map_act != q[i].map_act) break;
+    if (p.kind != PK_QKNR && p.op == 1u) break;   // more rows than a run holds: launched by itself
     if (!expand(p, m, &add)) { if (j == i) return 0; break; }
     // every new task against every task already in the run
     std::vector<RowTask> next = run;

@@ -309,9 +309,11 @@ def _kv_prep_case(g, style, batch, Hq, Hkv, d, pos, seed, hazard=None):
 
 
 @pytest.mark.parametrize("style,Hq,Hkv,d,pos", [("rope", 32, 8, 128, 4095), ("rope", 4, 2, 64, 1), ("qknr", 4, 1, 256, 611),
-                                               ("qknr", 8, 4, 128, 77)])
+                                               ("qknr", 8, 4, 128, 77), ("rope", 512, 128, 128, 1030), ("rope", 80, 66, 64, 5)])
 @pytest.mark.parametrize("hazard", [None, "copy_twice", "rope_after_copy", "shifted_source"])
 def test_kv_prep_run_equals_separate_ops(hip, style, Hq, Hkv, d, pos, hazard):
+    """The last two shapes are one token of many sequences at once (the heads of a lockstep batch side by side): more
+    rows than a row run holds, taken by the launch that rotates all Q rows, all K rows and appends K and V."""
     note(f"kv prep {style} {Hq}/{Hkv}x{d} pos={pos} hazard={hazard}")
     folded, launches = _kv_prep_case(hip, style, True, Hq, Hkv, d, pos, 11, hazard)
     apart, _ = _kv_prep_case(hip, style, False, Hq, Hkv, d, pos, 11, hazard)
