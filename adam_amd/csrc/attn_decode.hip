@@ -24,6 +24,7 @@
 // finish, found with an atomic ticket, needs a device-scope release and acquire in every workgroup;
 // each of those writes back and invalidates the L2 of its XCD and the kernel got 4x slower.)
 #include "attn_common.h"
+#include "gemv_common.h"
 #include <algorithm>
 #include <string.h>
 #include <utility>
@@ -770,8 +771,23 @@ size_t launch_attn_batch(const std::vector<PendOp>& q, size_t i, int* rc) {
   else launch_d<256>(G, nw, pf, grid, da, bs, n_splits, chunk, ext_dev);
   count_launch();
   *rc = check_launch();
-  if (*rc == ADAMAH_OK && n_splits > 1)
-    *rc = launch_attn_combine_dev(mp, g.attn_scratch, ext_dev + 2 * (size_t)n_all, n_all, D, n_splits);
+  if (*rc == ADAMAH_OK && n_splits > 1) {
+    // The O-projection of all sequences next in the queue, over the heads' outputs as rows [B, H D]: the merge of
+    // the slices also writes the fp16 form of those rows, and the matmul skips its conversion launch.
+    bool merged = false;
+    const size_t nx = i + 2 * B;
+    if (n_splits <= 8 && nx < n && q[nx].kind == PK_GEMM && q[nx].map_act == s0.map_act && q[nx].rpg == B && q[nx].k == H * D &&
+        q[nx].a == ho[0][0] && tuning("ADAMAH_ATTN_MERGE_EMIT", 1) != 0) {
+      bool rows = true;
+      for (size_t b = 0; rows && b < B; b++)
+        for (uint32_t op = 0; rows && op < H; op++) rows = ho[b][op] == ho[0][0] + (b * H + op) * D;
+      if (rows && launch_attn_merge_rows_f16(mp, g.attn_scratch, ho[0][0], (uint32_t)B, H * D, D, n_splits)) {
+        merged = true;
+        *rc = check_launch();
+      }
+    }
+    if (!merged) *rc = launch_attn_combine_dev(mp, g.attn_scratch, ext_dev + 2 * (size_t)n_all, n_all, D, n_splits);
+  }
   return 2 * B;
 }
 

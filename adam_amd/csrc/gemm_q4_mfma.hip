@@ -767,6 +767,103 @@ bool launch_glu_act_f16(const Map* ma, uint32_t op, uint32_t a, uint32_t b, uint
   return true;
 }
 
+// Merge of the attention slices of a lockstep step, one workgroup per sequence: the outputs of all the sequence's
+// heads (partial[(row * heads + head) * splits + s] = {max, sum, values[D]}, at most 8 slices) are merged with the
+// operations of the stand-alone merge kernel in their order, stored as the float32 row out[o0 + row * K ...]
+// (K = heads * D), and converted to the fp16 form the O-projection's matmul reads -- the row is in registers, so its
+// maximum costs one workgroup-wide reduction instead of a launch.
+template <int NW>
+__global__ void __launch_bounds__(1024)
+k_attn_merge_rows_f16(float* out, const float* __restrict__ partial, uint32_t o0, uint32_t M, uint32_t K, uint32_t D,
+                      uint32_t splits, float* scale, uint4* xh, uint4* xl) {
+  __shared__ float red[16];
+  const uint32_t row = blockIdx.x, tid = threadIdx.x, kw = K >> 3, heads = K / D, stride = D + 2u, last = splits - 1u;
+  float v[NW][8];
+  float m = 0.f;
+#pragma unroll
+  for (int u = 0; u < NW; u++) {
+    const uint32_t w = min(tid + 1024u * u, kw - 1u), head = (w * 8u) / D, j0 = (w * 8u) % D;
+    const float* pp = partial + (uint64_t)(row * heads + head) * splits * stride;
+    float ms[8], ls[8];
+#pragma unroll
+    for (uint32_t sp = 0; sp < 8u; sp++) { const float* ps = pp + (uint64_t)min(sp, last) * stride; ms[sp] = ps[0]; ls[sp] = ps[1]; }
+    float Mx = -9.99999968e+37f;
+#pragma unroll
+    for (uint32_t sp = 0; sp < 8u; sp++) Mx = sp < splits ? fmaxf(Mx, ms[sp]) : Mx;
+    float e[8], t[8];
+#pragma unroll
+    for (uint32_t sp = 0; sp < 8u; sp++) {
+      e[sp] = sp < splits ? expf(ms[sp] - Mx) : 0.f;
+      t[sp] = sp < splits ? fmaf(ls[sp], e[sp], 0.f) : 0.f;
+    }
+    // the sum of a 64-lane butterfly over lanes 0 .. 7, as the merge kernel takes it
+    const float invL = 1.0f / (((t[0] + t[4]) + (t[2] + t[6])) + ((t[1] + t[5]) + (t[3] + t[7])));
+    float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (uint32_t half = 0; half < 2u; half++) {
+      if (half == 1u && splits <= 4u) break;
+      f4qu_t a[4], b[4];
+#pragma unroll
+      for (uint32_t q = 0; q < 4u; q++) {
+        const float* ps = pp + (uint64_t)min(half * 4u + q, last) * stride + 2 + j0;
+        a[q] = *(const f4qu_t*)ps; b[q] = *(const f4qu_t*)(ps + 4);
+      }
+#pragma unroll
+      for (uint32_t q = 0; q < 4u; q++) {
+        const uint32_t sp = half * 4u + q;
+        const float wg = e[sp];
+        if (sp < splits) {
+          o[0] += fmaf(a[q].x, wg, 0.f); o[1] += fmaf(a[q].y, wg, 0.f); o[2] += fmaf(a[q].z, wg, 0.f); o[3] += fmaf(a[q].w, wg, 0.f);
+          o[4] += fmaf(b[q].x, wg, 0.f); o[5] += fmaf(b[q].y, wg, 0.f); o[6] += fmaf(b[q].z, wg, 0.f); o[7] += fmaf(b[q].w, wg, 0.f);
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 8; k++) v[u][k] = o[k] * invL;
+    if (tid + 1024u * u < kw) {
+      float* d = out + (uint64_t)o0 + (uint64_t)row * K + w * 8u;
+      *(f4qu_t*)d = (f4qu_t){v[u][0], v[u][1], v[u][2], v[u][3]};
+      *(f4qu_t*)(d + 4) = (f4qu_t){v[u][4], v[u][5], v[u][6], v[u][7]};
+#pragma unroll
+      for (int k = 0; k < 8; k++) m = fmaxf(m, fabsf(v[u][k]));
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  if ((tid & 63u) == 0) red[tid >> 6] = m;
+  __syncthreads();
+  m = red[0];
+#pragma unroll
+  for (int i = 1; i < 16; i++) m = fmaxf(m, red[i]);
+  const uint32_t ex = (__float_as_uint(m) >> 23) & 0xFFu;
+  float s = 1.f, inv = 1.f;
+  if (ex >= 14u && ex <= 254u) { s = __uint_as_float((267u - ex) << 23); inv = __uint_as_float((ex - 13u) << 23); }
+  if (tid == 0) { scale[2 * (uint64_t)row] = s; scale[2 * (uint64_t)row + 1] = inv; }
+#pragma unroll
+  for (int u = 0; u < NW; u++) {
+    const uint32_t w = tid + 1024u * u;
+    if (w >= kw) continue;
+    const float x[8] = {v[u][0] * s, v[u][1] * s, v[u][2] * s, v[u][3] * s, v[u][4] * s, v[u][5] * s, v[u][6] * s, v[u][7] * s};
+    uint4 hi, lo;
+    split_word(x, &hi, &lo);
+    xh[(uint64_t)row * kw + w] = hi;
+    xl[(uint64_t)row * kw + w] = lo;
+  }
+}
+
+// The launch of the kernel above: M sequences' merged heads as rows [M, K] at element o0 of the map, plus their fp16
+// form for the matmul that follows.  false: not taken (nothing launched).
+bool launch_attn_merge_rows_f16(const Map* ma, const float* partial, uint32_t o0, uint32_t M, uint32_t K, uint32_t D,
+                                uint32_t splits) {
+  if (K > 8192u || (K & 7u) || (D & 7u) || K % D || splits < 2 || splits > 8 || M == 0 || knob("ADAMAH_ACT_REGS", 1) == 0) return false;
+  float* scale; __half *xh, *xl;
+  if (!gemm_act_slots(M, K, &scale, &xh, &xl)) return false;
+  k_attn_merge_rows_f16<1><<<M, 1024, 0, g.stream>>>((float*)ma->buf, partial, o0, M, K, D, splits, scale, (uint4*)xh, (uint4*)xl);
+  count_launch();
+  gemm_act_mark(ma->buf, o0, M, K);
+  return true;
+}
+
 // Forget converted rows (after a stream capture: the launch count is rewound there, and the note must not
 // survive into a later state with the same count).
 void gemm_act_forget() { g_xh_key.valid = false; }

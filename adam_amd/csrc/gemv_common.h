@@ -148,6 +148,11 @@ bool gemm_act_slots(uint32_t M, uint32_t K, float** scale, __half** xh, __half**
 void gemm_act_forget();
 // Gated activation (op2 34 GEGLU / 35 SWIGLU) of the [M, K] rows at elements a and b into the rows at d, and the fp16
 // form of the result for the batched matmul that follows, in one launch.  false: not taken, nothing launched.
+// Merge of the attention slices of M sequences (at most 8 slices, partial[(row * heads + head) * splits + s]) into the
+// rows [M, K] at element o0, and the fp16 form of those rows for the matmul that follows, in one launch.  false: not
+// taken, nothing launched.
+bool launch_attn_merge_rows_f16(const Map* ma, const float* partial, uint32_t o0, uint32_t M, uint32_t K, uint32_t D,
+                                uint32_t splits);
 bool launch_glu_act_f16(const Map* ma, uint32_t op, uint32_t a, uint32_t b, uint32_t d, uint32_t M, uint32_t K);
 void gemm_act_mark(const void* buf, uint64_t a, uint32_t M, uint32_t K);
 // Second pass of the fused GEMV + argmax: best of the per-group partials, token id stored as float.

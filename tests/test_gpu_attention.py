@@ -230,6 +230,60 @@ def test_prefill_chunk_splits_or_falls_back_when_tokens_do_not_line_up(hip, layo
     assert rel_l2(outs[0], outs[1]) < TOL
 
 
+@pytest.mark.parametrize("B,ctx,Hq,Hkv,d", [(16, 300, 8, 2, 128), (5, 2000, 32, 8, 128), (3, 40, 4, 1, 256)])
+def test_lockstep_merge_writes_the_projection_s_operand(hip, monkeypatch, B, ctx, Hq, Hkv, d):
+    """The lockstep pairs followed by the O-projection over the heads' outputs as rows [B, Hq d]: with several slices
+    of the sequence the merge launch also writes the matmul's fp16 operand form (attention, merge, matmul: 3 launches;
+    ADAMAH_ATTN_MERGE_EMIT=0: merge, conversion: 4), every word of outputs and product the same.  One slice: nothing
+    to merge, the conversion stays."""
+    from adam_amd import quant
+    from gpu_util import load_qtensor
+    rng = np.random.default_rng(B + ctx)
+    gs, N = Hq // Hkv, 64
+    scale = float(1.0 / np.sqrt(d))
+    q = rng.standard_normal((B, Hq, d)).astype(np.float32)
+    K = rng.standard_normal((B, Hkv, ctx, d)).astype(np.float32)
+    V = rng.standard_normal((B, Hkv, ctx, d)).astype(np.float32)
+    qt = quant.quantize_q4_0(rng.standard_normal((N, Hq * d), dtype=np.float32) * np.float32(0.05))
+
+    def go(g):
+        sc_sz = Hq * ctx
+        q_pos, out_pos = sc_sz, sc_sz + B * Hq * d
+        y_pos = out_pos + B * Hq * d
+        kv_start = (y_pos + B * N + d - 1) // d * d
+        step = ctx * d
+        per_seq = 2 * Hkv * step
+        load_qtensor(g, 1, qt)
+        f32map(g, 0, kv_start + B * per_seq, None)
+        g.kv_cache_fp16(0, kv_start, B * per_seq)
+        put(g, 0, q_pos, q)
+        for b in range(B):
+            put(g, 0, kv_start + b * per_seq, K[b]); put(g, 0, kv_start + b * per_seq + Hkv * step, V[b])
+        heads = np.arange(Hq) // gs
+        s_rows = up(g, np.arange(Hq) * ctx)
+        hs = [(up(g, q_pos + b * Hq * d + np.arange(Hq) * d), up(g, kv_start + b * per_seq + heads * step),
+               up(g, kv_start + b * per_seq + (Hkv + heads) * step), up(g, out_pos + b * Hq * d + np.arange(Hq) * d)) for b in range(B)]
+        a, w, c = up(g, [out_pos]), up(g, [0]), up(g, [y_pos])
+        g.batch_begin()
+        for hq, hk, hv, ho in hs:
+            g.map_matmul_t_dev(0, hq, hk, s_rows, 1, d, ctx, Hq)
+            g.map_attn_softmax_value_dev(0, s_rows, hv, ho, Hq, ctx, d, scale, 0.0)
+        g.map_matmul_t_xq4_dev(0, 1, a, w, c, B, Hq * d, N, 1)
+        g.batch_end()
+        return read(g, 0, out_pos, B * Hq * d + B * N), (g.get_last_barrier_count() if g is hip else None)
+
+    note(f"lockstep merge + projection B={B} ctx={ctx} {Hq}q/{Hkv}kv d={d}")
+    fused, n_fused = go(hip)
+    monkeypatch.setenv("ADAMAH_ATTN_MERGE_EMIT", "0")
+    apart, n_apart = go(hip)
+    monkeypatch.delenv("ADAMAH_ATTN_MERGE_EMIT")
+    assert np.array_equal(fused.view(np.uint32), apart.view(np.uint32))
+    assert (n_fused, n_apart) == ((3, 4) if ctx >= 300 else (3, 3))
+    want, _ = go(oracle.init())
+    assert rel_l2(fused[:B * Hq * d], want[:B * Hq * d]) < TOL
+    assert rel_l2(fused[B * Hq * d:], want[B * Hq * d:]) < TOL
+
+
 @pytest.mark.parametrize("B,ctx,Hq,Hkv,d,softcap", [(16, 300, 8, 2, 128, 0.0), (3, 40, 4, 1, 256, 50.0), (5, 2000, 32, 8, 128, 0.0)])
 def test_lockstep_sequences_are_one_launch(hip, B, ctx, Hq, Hkv, d, softcap):
     """One (scores, softmax.V) pair per sequence of a batch, own queries / outputs / KV cache each, shared
