@@ -81,9 +81,12 @@ __device__ __forceinline__ float row16_sum(float v) {
 
 template <int D, int G, int NW, bool PF, bool EXT, bool RP>
 __global__ void __launch_bounds__(NW * 64)
-k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift, const AttdBases bs,
-              uint32_t row_size, float scale, float cap, uint32_t n_splits, uint32_t chunk, float* partial,
-              const uint32_t* __restrict__ ext, const AttdRowPrep rp) {
+k_attn_decode(const float* data, const __half* kv, uint64_t kv_shift, uint32_t row_size, uint32_t chunk, uint32_t n_splits,
+              uint32_t rp_q_src, uint32_t rp_k_src, uint32_t rp_v_src, const float* rp_inv_freq,
+              float* out, float scale, float cap, float* partial, const uint32_t* __restrict__ ext, const AttdBases bs,
+              const AttdRowPrep rp) {
+  // (the first 14 dwords of the arguments are in registers when a wave starts: what the first loads need stands in
+  // front -- with the row preparation the raw rows' places and the frequency table, copies of rp's fields)
   constexpr int NI = D / 32;           // 16-byte K loads per lane and tile
   constexpr int DPL = D / 64;          // V dims per lane (every lane sees all 16 rows of the tile)
   constexpr int DW = DPL > 2 ? DPL / 2 : 1;
@@ -176,22 +179,22 @@ k_attn_decode(const float* data, float* out, const __half* kv, uint64_t kv_shift
       float qraw[QN], kraw, vraw;
 #pragma unroll
       for (uint32_t u = 0; u < QN; u++)
-        qraw[u] = data[(uint64_t)rp.q_src + (uint64_t)op0 * D + min(tid + u * NT, (uint32_t)(G * D) - 1u)];
+        qraw[u] = data[(uint64_t)rp_q_src + (uint64_t)op0 * D + min(tid + u * NT, (uint32_t)(G * D) - 1u)];
       {
         const uint32_t d = min(tid, (uint32_t)D - 1u);
-        kraw = data[(uint64_t)rp.k_src + (uint64_t)group * D + d];
-        vraw = data[(uint64_t)rp.v_src + (uint64_t)group * D + d];
+        kraw = data[(uint64_t)rp_k_src + (uint64_t)group * D + d];
+        vraw = data[(uint64_t)rp_v_src + (uint64_t)group * D + d];
       }
       float fr[PN], wq[PN][2], wk[2];
       const bool nrm = (rp.flags & 1u) != 0u;
       {
-        const float* wqp = nrm ? data + rp.q_w : rp.inv_freq;     // no norm: any readable address, the value is not used
-        const float* wkp = nrm ? data + rp.k_w : rp.inv_freq;
+        const float* wqp = nrm ? data + rp.q_w : rp_inv_freq;     // no norm: any readable address, the value is not used
+        const float* wkp = nrm ? data + rp.k_w : rp_inv_freq;
         const uint32_t hs = nrm ? half : 0u;
 #pragma unroll
         for (uint32_t u = 0; u < PN; u++) {
           const uint32_t i = (tid + u * NT) % half;
-          fr[u] = rp.inv_freq[i];
+          fr[u] = rp_inv_freq[i];
           wq[u][0] = wqp[i]; wq[u][1] = wqp[i + hs];
         }
         wk[0] = wkp[tid % half]; wk[1] = wkp[tid % half + hs];
@@ -467,8 +470,10 @@ static void launch_dg(uint32_t G, dim3 grid, const AttnDecodeArgs& a, const Attd
                       uint32_t chunk, const uint32_t* ext, const AttdRowPrep* rp) {
   const AttdRowPrep none = {};
 #define ADL(GG, EE, RR)                                                                                   \
-  k_attn_decode<D, GG, NW, PF, EE, RR><<<grid, NW * 64, 0, g.stream>>>(a.data, a.data, a.kv, a.kv_shift, bs, a.row_size, \
-                                                                       a.scale, a.cap, n_splits, chunk, g.attn_scratch, ext, RR ? *rp : none)
+  k_attn_decode<D, GG, NW, PF, EE, RR><<<grid, NW * 64, 0, g.stream>>>(a.data, a.kv, a.kv_shift, a.row_size, chunk, n_splits,                   \
+                                                                       (RR ? *rp : none).q_src, (RR ? *rp : none).k_src, (RR ? *rp : none).v_src, \
+                                                                       (RR ? *rp : none).inv_freq, a.data, a.scale, a.cap, g.attn_scratch, ext,  \
+                                                                       bs, RR ? *rp : none)
   if (ext) { if (G == 1) ADL(1, true, false); else if (G == 2) ADL(2, true, false); else if (G == 4) ADL(4, true, false); else ADL(8, true, false); }
   else if (rp && D >= 128) {
     constexpr bool R = D >= 128;   // the row preparation is built for head sizes 128 and 256

@@ -75,10 +75,15 @@ struct PreM {
 // stages the activations; their results are also stored where the unfused ops would have put them.
 template <int FMT, int EPI, bool RAGGED, int PRO>
 __global__ void __launch_bounds__(1024)
-k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, const float2* __restrict__ qp,
-            const __half* __restrict__ d16, uint32_t a, uint32_t b_off, uint32_t c_out,
-            const uint32_t* __restrict__ lidx, const uint32_t* __restrict__ lval, uint32_t K, uint32_t N,
-            uint32_t rows_per_group, uint32_t n_groups, uint32_t ks, GemvFuse fz) {
+k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __restrict__ d16, uint32_t K, uint32_t N, uint32_t ks,
+            uint32_t x_src, uint32_t b_off, const float* n_wt, uint32_t n_w,
+            float* act_out, uint32_t c_out, const float2* __restrict__ qp, const uint32_t* __restrict__ lidx,
+            const uint32_t* __restrict__ lval, uint32_t rows_per_group, uint32_t n_groups, GemvFuse fz) {
+  // The first 14 dwords of the arguments are in registers when a wave starts (the rest is fetched from the argument
+  // block, a trip to memory): what the first loads need stands in front -- the activations and where they start
+  // (x_src: the vector itself, or the source of the first folded norm, whose weights are n_wt + n_w), the weights,
+  // K, N and the K split.
+  const uint32_t a = x_src;
   constexpr bool B16 = (FMT == FMT_Q4_B16);
   extern __shared__ uint4 smem_u4[];
   uint8_t* xs = (uint8_t*)smem_u4;                    // nblk * 128 bytes
@@ -341,8 +346,8 @@ k_gemv_mfma(const float* act, float* act_out, const uint8_t* __restrict__ W, con
       for (int k = 0; k < 8; k++) { v[u][k] = 0.f; wv[u][k] = 0.f; rv[u][k] = 0.f; w2v[u][k] = 0.f; }
       // (waves without words of their own load the row's last word: every path issues the same loads)
       const uint64_t e0 = (uint64_t)min(i, nw - 1u) * 8u;
-      load8(act + fz.p_src + e0, v[u]);
-      load8(fz.p_wt + fz.p_src2 + e0, wv[u]);
+      load8(act + x_src + e0, v[u]);
+      load8(n_wt + n_w + e0, wv[u]);
       if (PRO == PRO_NORM2) { load8(act + fz.p_res + e0, rv[u]); load8(fz.p_wt2 + fz.p_w2 + e0, w2v[u]); }
     }
     __builtin_amdgcn_sched_barrier(0);   // activation loads first: they are waited for first
@@ -639,9 +644,12 @@ static void launch_mfma_p(int fmt, uint32_t grid, uint32_t threads, const Map* m
   float* act_out = out ? out : act;
   const size_t smem = mfma_smem(K);
   const bool ragged = (K & 2047u) != 0;
+  const bool norm = PRO == PRO_RMSNORM || PRO == PRO_NORM2;
+  const uint32_t x_src = norm ? fz.p_src : a;
+  const float* n_wt = norm ? fz.p_wt : act;
 #define MK(F, R)                                                                                                  \
-  k_gemv_mfma<F, EPI, R, PRO><<<grid, threads, smem, g.stream>>>(act, act_out, mw->buf, mw->qp, mw->d16, a, b, c, lidx, \
-                                                                 lval, K, N, rpg, n_groups, ks, fz)
+  k_gemv_mfma<F, EPI, R, PRO><<<grid, threads, smem, g.stream>>>(act, mw->buf, mw->d16, K, N, ks, x_src, b, n_wt, fz.p_src2, act_out, c, \
+                                                                 mw->qp, lidx, lval, rpg, n_groups, fz)
   if (fmt == FMT_Q4_B16) { if (ragged) MK(FMT_Q4_B16, true); else MK(FMT_Q4_B16, false); }
   else { if (ragged) MK(FMT_Q4_AFF, true); else MK(FMT_Q4_AFF, false); }
 #undef MK
