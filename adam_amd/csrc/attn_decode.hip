@@ -82,11 +82,13 @@ __device__ __forceinline__ float row16_sum(float v) {
 template <int D, int G, int NW, bool PF, bool EXT, bool RP>
 __global__ void __launch_bounds__(NW * 64)
 k_attn_decode(const float* data, const __half* kv, uint64_t kv_shift, uint32_t row_size, uint32_t chunk, uint32_t n_splits,
-              uint32_t rp_q_src, uint32_t rp_k_src, uint32_t rp_v_src, const float* rp_inv_freq,
-              float* out, float scale, float cap, float* partial, const uint32_t* __restrict__ ext, const AttdBases bs,
-              const AttdRowPrep rp) {
+              uint32_t rp_q_src, uint32_t rp_k_src, uint32_t rp_v_src, const void* early_ptr,
+              float* out, float scale, float cap, float* partial, const AttdBases bs, const AttdRowPrep rp) {
   // (the first 14 dwords of the arguments are in registers when a wave starts: what the first loads need stands in
-  // front -- with the row preparation the raw rows' places and the frequency table, copies of rp's fields)
+  // front -- with the row preparation the raw rows' places and the frequency table, copies of rp's fields; with
+  // the operand bases in device memory, the table's address)
+  const float* rp_inv_freq = (const float*)early_ptr;
+  const uint32_t* __restrict__ ext = (const uint32_t*)early_ptr;
   constexpr int NI = D / 32;           // 16-byte K loads per lane and tile
   constexpr int DPL = D / 64;          // V dims per lane (every lane sees all 16 rows of the tile)
   constexpr int DW = DPL > 2 ? DPL / 2 : 1;
@@ -472,8 +474,8 @@ static void launch_dg(uint32_t G, dim3 grid, const AttnDecodeArgs& a, const Attd
 #define ADL(GG, EE, RR)                                                                                   \
   k_attn_decode<D, GG, NW, PF, EE, RR><<<grid, NW * 64, 0, g.stream>>>(a.data, a.kv, a.kv_shift, a.row_size, chunk, n_splits,                   \
                                                                        (RR ? *rp : none).q_src, (RR ? *rp : none).k_src, (RR ? *rp : none).v_src, \
-                                                                       (RR ? *rp : none).inv_freq, a.data, a.scale, a.cap, g.attn_scratch, ext,  \
-                                                                       bs, RR ? *rp : none)
+                                                                       EE ? (const void*)ext : (const void*)(RR ? *rp : none).inv_freq,         \
+                                                                       a.data, a.scale, a.cap, g.attn_scratch, bs, RR ? *rp : none)
   if (ext) { if (G == 1) ADL(1, true, false); else if (G == 2) ADL(2, true, false); else if (G == 4) ADL(4, true, false); else ADL(8, true, false); }
   else if (rp && D >= 128) {
     constexpr bool R = D >= 128;   // the row preparation is built for head sizes 128 and 256

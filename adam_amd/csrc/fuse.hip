@@ -298,7 +298,7 @@ void flush_pending() {
       if (!(ma && mw && la && lb && lc)) keep(ADAMAH_ERR_INVALID);
       else
         keep(launch_gemm_q4_mfma(ma, mw, la, lb, lc, p.rpg, p.k, sg.begin[m], 1, p.op == (uint32_t)FMT_Q8_B16, nullptr, (int64_t)p.a,
-                                 (m == 1 && !sg.add) ? (int64_t)p.c : -1, (m == 1 && !sg.add) ? nullptr : &sg));
+                                 (m == 1 && !sg.add) ? (int64_t)p.c : -1, (m == 1 && !sg.add) ? nullptr : &sg, (int64_t)p.b));
       i += used;
       continue;
     }

@@ -146,9 +146,13 @@ __device__ __forceinline__ f4q_t gather_scales(_Float16 d) {
 // fewer bytes per flop: 28672x4096 at M = 512 went 434 -> 344 us with 256 instead of 128 weight rows per workgroup.
 template <int MT, int R, int NW>
 __global__ void __launch_bounds__(64 * NW)
-k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh,
-                    const u4q_t* __restrict__ xl, const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc,
-                    const float* __restrict__ scale, uint32_t M, uint32_t K, uint32_t N, GemmSegs segs) {
+k_gemm_q4_f16_tiled(const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh, const u4q_t* __restrict__ xl,
+                     uint32_t K, uint32_t N, uint32_t M, uint32_t b_val, uint32_t c_val, uint32_t by_val, float* out,
+                     const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc, const float* __restrict__ scale,
+                     GemmSegs segs) {
+  // (the first 14 dwords of the arguments are in registers when a wave starts; by_val bit 0 / 1: the weights' / the
+  // result's element offset of op 0 is b_val / c_val -- known on the host -- instead of a load from lb / lc, which
+  // the first weight loads would have to wait for)
   constexpr uint32_t BM = 16u * MT, ROWB = 272u;
   __shared__ __attribute__((aligned(16))) uint8_t xs[2u * BM * ROWB];   // first plane, then second plane
   uint8_t* const xs2 = xs + BM * ROWB;
@@ -156,7 +160,7 @@ k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __r
   const uint32_t r16 = lane & 15u, g = lane >> 4;
   constexpr uint32_t NT = 64u * NW, NP = 256u * MT / NT;       // threads; 16-byte pieces per thread, plane and step
   const uint32_t n0 = blockIdx.x * (16u * NW * R) + wave * (16u * R), m0 = blockIdx.y * BM, op = blockIdx.z;
-  const uint64_t c_off = lc[op], gbase = (uint64_t)lb[op] >> 5;
+  const uint64_t c_off = (by_val & 2u) ? (uint64_t)c_val : (uint64_t)lc[op], gbase = ((by_val & 1u) ? (uint64_t)b_val : (uint64_t)lb[op]) >> 5;
   const uint32_t nblk = K >> 5, kw = K >> 3;                   // blocks and 16-byte pieces per row
   uint32_t nrow[R];
 #pragma unroll
@@ -282,9 +286,13 @@ k_gemm_q4_f16_tiled(float* out, const uint8_t* __restrict__ W, const __half* __r
 // buffer of the caller).
 template <int MT, int R, int NWV, bool Q8>
 __global__ void __launch_bounds__(64 * NWV)
-k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh,
-                     const u4q_t* __restrict__ xl, const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc,
-                     const float* __restrict__ scale, uint32_t M, uint32_t K, uint32_t N, GemmSegs segs) {
+k_gemm_q4_f16_ksplit(const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh, const u4q_t* __restrict__ xl,
+                     uint32_t K, uint32_t N, uint32_t M, uint32_t b_val, uint32_t c_val, uint32_t by_val, float* out,
+                     const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc, const float* __restrict__ scale,
+                     GemmSegs segs) {
+  // (the first 14 dwords of the arguments are in registers when a wave starts; by_val bit 0 / 1: the weights' / the
+  // result's element offset of op 0 is b_val / c_val -- known on the host -- instead of a load from lb / lc, which
+  // the first weight loads would have to wait for)
   constexpr uint32_t BM = 16u * MT, ROWB = 272u, NP = 4u * MT;      // pieces per lane, plane and step
   constexpr uint32_t PLANES = Q8 ? 1u : 2u;
   constexpr uint32_t TILE = BM * ROWB, PART = (NWV - 1u) * R * MT * 4u * 64u * 4u;
@@ -295,7 +303,8 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
   uint8_t* xs = xs_all + wave * PLANES * TILE;
   uint8_t* const xs2 = xs + TILE;
   const uint32_t n0 = blockIdx.x * (16u * R), m0 = blockIdx.y * BM, op = blockIdx.z;
-  const uint64_t c_off = lc ? (uint64_t)lc[op] : 0ull, gbase = (uint64_t)lb[op] >> 5;
+  const uint64_t c_off = (by_val & 2u) ? (uint64_t)c_val : lc ? (uint64_t)lc[op] : 0ull;
+  const uint64_t gbase = ((by_val & 1u) ? (uint64_t)b_val : (uint64_t)lb[op]) >> 5;
   const uint32_t nblk = K >> 5, kw = K >> 3;
   // Weight loads: lane -> (row lane / 4, block lane % 4 of the step), so the four lanes of a quad read 64
   // contiguous bytes of one row -- one request to the L1 instead of one per lane, which is what the
@@ -492,9 +501,13 @@ k_gemm_q4_f16_ksplit(float* out, const uint8_t* __restrict__ W, const __half* __
 #define R16_MS 2u
 template <int NW>
 __global__ void __launch_bounds__(64 * NW)
-k_gemm_q4_f16_rows16(float* out, const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh,
-                     const u4q_t* __restrict__ xl, const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc,
-                     const float* __restrict__ scale, uint32_t M, uint32_t K, uint32_t N, GemmSegs segs) {
+k_gemm_q4_f16_rows16(const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh, const u4q_t* __restrict__ xl,
+                     uint32_t K, uint32_t N, uint32_t M, uint32_t b_val, uint32_t c_val, uint32_t by_val, float* out,
+                     const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc, const float* __restrict__ scale,
+                     GemmSegs segs) {
+  // (the first 14 dwords of the arguments are in registers when a wave starts; by_val bit 0 / 1: the weights' / the
+  // result's element offset of op 0 is b_val / c_val -- known on the host -- instead of a load from lb / lc, which
+  // the first weight loads would have to wait for)
   constexpr uint32_t ROWB = 272u, TILE = 16u * ROWB, NT = 64u * NW;
   constexpr uint32_t PIECES = R16_MS * 256u;                 // 16-byte pieces per plane and macro step
   constexpr uint32_t NP = (PIECES + NT - 1u) / NT;           // per thread
@@ -506,7 +519,8 @@ k_gemm_q4_f16_rows16(float* out, const uint8_t* __restrict__ W, const __half* __
   // first weight row of the wave's tile (glu: tb = the tile's first row within its half of the matrix)
   const uint32_t tb = glum ? blockIdx.x * (8u * NW) + (wave % (NW / 2u)) * 16u : blockIdx.x * (16u * NW) + wave * 16u;
   const uint32_t n0 = glum && wave >= NW / 2u ? (N >> 1) + tb : tb;
-  const uint64_t c_off = lc ? (uint64_t)lc[op] : 0ull, gbase = (uint64_t)lb[op] >> 5;
+  const uint64_t c_off = (by_val & 2u) ? (uint64_t)c_val : lc ? (uint64_t)lc[op] : 0ull;
+  const uint64_t gbase = ((by_val & 1u) ? (uint64_t)b_val : (uint64_t)lb[op]) >> 5;
   const uint32_t nblk = K >> 5, kw = K >> 3, steps = nblk >> 2, macros = (steps + R16_MS - 1u) / R16_MS;
   const uint32_t lrow = lane >> 2, lblk = lane & 3u;
   const int perm_addr = (int)((4u * r16 + g) << 2);
@@ -654,11 +668,13 @@ k_gemm_q4_f16_rows16(float* out, const uint8_t* __restrict__ W, const __half* __
 struct GluSrc { uint32_t op, a, b, d; };
 template <int NW, bool GLU>
 __global__ void __launch_bounds__(1024)
-k_act_f16_regs(const float* act, float* act_out, const uint32_t* __restrict__ la, uint32_t M, uint32_t K, float* scale, uint4* xh,
-               uint4* xl, GluSrc glu) {
+k_act_f16_regs(const float* act, uint32_t K, uint32_t M, uint32_t a_val, uint32_t a_by_val, uint4* xh, uint4* xl, float* scale,
+               float* act_out, const uint32_t* __restrict__ la, GluSrc glu) {
+  // (a_by_val: the rows start at element a_val -- known on the host -- instead of la[op], a load the rows' loads
+  // would wait for; with GLU a_val is glu.a)
   __shared__ float red[16];
   const uint32_t row = blockIdx.x, op = blockIdx.y, tid = threadIdx.x, kw = K >> 3;
-  const float* x = act + (GLU ? (uint64_t)glu.a : (uint64_t)la[op]) + (uint64_t)row * K;
+  const float* x = act + (a_by_val ? (uint64_t)a_val : (uint64_t)la[op]) + (uint64_t)row * K;
   f4qu_t v0[NW], v1[NW];
   float m = 0.f;
 #pragma unroll
@@ -760,8 +776,8 @@ bool launch_glu_act_f16(const Map* ma, uint32_t op, uint32_t a, uint32_t b, uint
   if (!gemm_act_slots(M, K, &scale, &xh, &xl)) return false;
   float* act = (float*)ma->buf;
   const GluSrc glu = {op, a, b, d};
-  if (K <= 8192) k_act_f16_regs<1, true><<<dim3(M, 1), 1024, 0, g.stream>>>(act, act, nullptr, M, K, scale, (uint4*)xh, (uint4*)xl, glu);
-  else k_act_f16_regs<2, true><<<dim3(M, 1), 1024, 0, g.stream>>>(act, act, nullptr, M, K, scale, (uint4*)xh, (uint4*)xl, glu);
+  if (K <= 8192) k_act_f16_regs<1, true><<<dim3(M, 1), 1024, 0, g.stream>>>(act, K, M, a, 1u, (uint4*)xh, (uint4*)xl, scale, act, nullptr, glu);
+  else k_act_f16_regs<2, true><<<dim3(M, 1), 1024, 0, g.stream>>>(act, K, M, a, 1u, (uint4*)xh, (uint4*)xl, scale, act, nullptr, glu);
   count_launch();
   gemm_act_mark(ma->buf, d, M, K);
   return true;
@@ -873,7 +889,10 @@ void gemm_act_forget() { g_xh_key.valid = false; }
 // in range.
 int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb, const uint32_t* lc,
                         uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops, bool q8, float* out, int64_t a_host,
-                        int64_t c_host, const GemmSegs* segs) {
+                        int64_t c_host, const GemmSegs* segs, int64_t b_host) {
+  // offsets of op 0 the host knows go to the kernels by value
+  const uint32_t b_val = b_host >= 0 ? (uint32_t)b_host : 0u, c_val = c_host >= 0 ? (uint32_t)c_host : 0u;
+  const uint32_t by_val = n_ops == 1 ? ((b_host >= 0 ? 1u : 0u) | (c_host >= 0 ? 2u : 0u)) : 0u;
   if (((q8 || out) && M > 32) || ((out || segs) && n_ops != 1) || (out && segs) || (segs && (segs->add || segs->glu) && M > 32))
     return ADAMAH_ERR_INVALID;
   GemmSegs sg = {};
@@ -898,8 +917,8 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
   uint4* const xl = (uint4*)((uint8_t*)g_xh_buf + plane);
   if (!reuse) {
     if (K <= 16384 && knob("ADAMAH_ACT_REGS", 1) != 0) {
-      if (K <= 8192) k_act_f16_regs<1, false><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, act, la, M, K, g_scale_buf, xh, xl, GluSrc{});
-      else k_act_f16_regs<2, false><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, act, la, M, K, g_scale_buf, xh, xl, GluSrc{});
+      if (K <= 8192) k_act_f16_regs<1, false><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, K, M, a_host >= 0 ? (uint32_t)a_host : 0u, (a_host >= 0 && n_ops == 1) ? 1u : 0u, xh, xl, g_scale_buf, act, la, GluSrc{});
+      else k_act_f16_regs<2, false><<<dim3(M, n_ops), 1024, 0, g.stream>>>(act, K, M, a_host >= 0 ? (uint32_t)a_host : 0u, (a_host >= 0 && n_ops == 1) ? 1u : 0u, xh, xl, g_scale_buf, act, la, GluSrc{});
     } else
       k_act_f16<<<dim3(M, n_ops), 256, 0, g.stream>>>(act, la, M, K, g_scale_buf, xh, xl);
     count_launch();
@@ -924,8 +943,9 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
       if (mt == 1 && !q8 && !sg.add && glu_ok && (uint64_t)wgs16 * 4 >= 3ull * (uint64_t)g.n_cu &&
           tuning("ADAMAH_GEMM_ROWS16", 1) != 0) {
         dim3 gridr(wgs16, 1, n_ops);
-        k_gemm_q4_f16_rows16<8><<<gridr, 512, 0, g.stream>>>(out ? out : act, mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, lb,
-                                                            out ? nullptr : lc, g_scale_buf, M, K, N, sg);
+        k_gemm_q4_f16_rows16<8><<<gridr, 512, 0, g.stream>>>(mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, K, N, M, b_val, c_val,
+                                                            out ? (by_val & 1u) : by_val, out ? out : act, lb, out ? nullptr : lc,
+                                                            g_scale_buf, sg);
         count_launch();
         keep();
         return check_launch();
@@ -936,7 +956,7 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
     const uint32_t* lcd = out ? nullptr : lc;
     // eight waves where the matrix has too few weight rows for larger tiles (measured: no gain otherwise)
     const uint32_t nwv = mt == 1 && !q8 ? (uint32_t)knob("ADAMAH_GEMM_NWV", R == 1 ? 8 : 4) : 4u;
-#define GK(T, RR, W, Q) k_gemm_q4_f16_ksplit<T, RR, W, Q><<<grid, 64 * W, 0, g.stream>>>(dst, mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, lb, lcd, g_scale_buf, M, K, N, sg)
+#define GK(T, RR, W, Q) k_gemm_q4_f16_ksplit<T, RR, W, Q><<<grid, 64 * W, 0, g.stream>>>(mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, K, N, M, b_val, c_val, out ? (by_val & 1u) : by_val, dst, lb, lcd, g_scale_buf, sg)
     if (q8) {
       if (mt == 1) { if (R == 2) GK(1, 2, 4, true); else GK(1, 1, 4, true); }
       else { if (R == 2) GK(2, 2, 4, true); else GK(2, 1, 4, true); }
@@ -966,7 +986,7 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
   R = R >= 4 && mt == 4 ? 4 : R >= 2 ? 2 : 1;
   if (mt == 4 && NW == 8 && R == 1) R = 2;
   dim3 grid(cdiv(N, 16 * NW * R), cdiv(M, 16 * mt), n_ops);
-#define GT(T, RR, W) k_gemm_q4_f16_tiled<T, RR, W><<<grid, 64 * W, 0, g.stream>>>(act, mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, lb, lc, g_scale_buf, M, K, N, sg)
+#define GT(T, RR, W) k_gemm_q4_f16_tiled<T, RR, W><<<grid, 64 * W, 0, g.stream>>>(mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, K, N, M, b_val, c_val, by_val, act, lb, lc, g_scale_buf, sg)
   if (mt == 4 && NW == 8) { if (R == 4) GT(4, 4, 8); else GT(4, 2, 8); }
   else if (mt == 4) { if (R == 4) GT(4, 4, 4); else if (R == 2) GT(4, 2, 4); else GT(4, 1, 4); }
   else if (NW == 8) { if (R == 2) GT(8, 2, 8); else GT(8, 1, 8); }

@@ -136,11 +136,12 @@ struct GemmSegs {
 // M > 1: fp16 matrix-core GEMM over Q4 block16 weights (gemm_q4_mfma.hip); operands already validated.
 // q8: Q8 block16 weights instead (M <= 32).  out: the [M, N] result goes to this buffer instead of the
 // activation map (one op).  a_host / c_host: element offsets of op 0's activations and result when the
-// host knows them (n_ops == 1): lets consecutive matmuls over the same rows share one conversion.
+// host knows them (n_ops == 1): lets consecutive matmuls over the same rows share one conversion.  b_host: likewise
+// the element offset of op 0's weights; known offsets go to the kernels by value (no load in front of their first loads).
 // segs (M <= 32, one op): the weights are several matrices back to back, results placed per segment.
 int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb, const uint32_t* lc,
                         uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops, bool q8 = false, float* out = nullptr,
-                        int64_t a_host = -1, int64_t c_host = -1, const GemmSegs* segs = nullptr);
+                        int64_t a_host = -1, int64_t c_host = -1, const GemmSegs* segs = nullptr, int64_t b_host = -1);
 // For a kernel that produces the rows [M, K] of a coming batched matmul: the buffers of their fp16 form
 // ((s, 1/s) per row; two planes of K halves per row: fp16(x s) and the fp16 remainder), grown as needed, and -- after that kernel's launch has been
 // counted -- the note that rows [a, a + M K) of `buf` are converted, so the matmul skips its conversion.

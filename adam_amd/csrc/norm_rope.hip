@@ -47,14 +47,25 @@ k_rmsnorm(const float* act, const float* wt, float* out, const uint32_t* __restr
 // batched matmul follows; its fp16 operand form (row scaled by a power of two, two planes, 8-element words in the
 // order (0,4)(1,5)(2,6)(3,7), plus (s, 1/s) per row) is written here as well, which spares that
 // matmul its conversion launch.
+struct RowsByValue { uint32_t on, s0, ss, w0, ws, d0, ds, r0, rs; };   // host side only
 template <bool ADD, bool EMIT, int NU>
 __global__ void __launch_bounds__(256)
-k_rmsnorm_rows(const float* act, const float* wt, float* out, const uint32_t* __restrict__ ls,
-               const uint32_t* __restrict__ lw, const uint32_t* __restrict__ lr, const uint32_t* __restrict__ ld,
-               uint32_t dim, float eps, uint64_t act_elems, uint64_t wt_elems, float* scale, __half* xh, __half* xl) {
+k_rmsnorm_rows(const float* act, const float* wt, uint32_t dim_on, float eps, uint32_t s0, uint32_t ss_, uint32_t w0, uint32_t ws,
+               uint32_t d0, uint32_t ds, uint32_t r0, uint32_t rs, float* out,
+               const uint32_t* __restrict__ ls, const uint32_t* __restrict__ lw, const uint32_t* __restrict__ lr,
+               const uint32_t* __restrict__ ld, uint64_t act_elems, uint64_t wt_elems, float* scale, __half* xh, __half* xl) {
+  // (these 14 dwords are in registers when a wave starts.  Top bit of dim_on: row i's source / weights / destination /
+  // residual start at x0 + i xs -- the host found the rows evenly spaced -- instead of four loads from the row
+  // tables, which the rows' own loads would have to wait for)
   __shared__ float sh[4];
-  const uint32_t ri = blockIdx.x, tid = threadIdx.x;
-  const uint64_t sb = ls[ri], wb = lw[ri], db = ld[ri], rb = ADD ? (uint64_t)lr[ri] : 0;
+  const uint32_t ri = blockIdx.x, tid = threadIdx.x, dim = dim_on & 0x7FFFFFFFu;
+  uint64_t sb, wb, db, rb = 0;
+  if (dim_on >> 31) {
+    sb = (uint64_t)s0 + (uint64_t)ri * ss_; wb = (uint64_t)w0 + (uint64_t)ri * ws;
+    db = (uint64_t)d0 + (uint64_t)ri * ds; if (ADD) rb = (uint64_t)r0 + (uint64_t)ri * rs;
+  } else {
+    sb = ls[ri]; wb = lw[ri]; db = ld[ri]; if (ADD) rb = lr[ri];
+  }
   if (sb + dim > act_elems || db + dim > act_elems || wb + dim > wt_elems || (ADD && rb + dim > act_elems)) return;
   float x[NU], w[NU], r[NU];
 #pragma unroll
@@ -223,7 +234,21 @@ static int rmsnorm_impl(uint32_t map_act, uint32_t map_wt, uint32_t hs, uint32_t
     __half *xh = nullptr, *xl = nullptr;
     if (emit) emit = gemm_act_slots(n_rows, dim, &scale, &xh, &xl);
     const float* w = (const float*)mw->buf;
-#define RR(A, E, NU) k_rmsnorm_rows<A, E, NU><<<n_rows, 256, 0, g.stream>>>(a, w, a, ls, lw, lr, ld, dim, eps, ma->n_elems, mw->n_elems, scale, xh, xl)
+    // evenly spaced rows (the usual case: rows of a matrix, one weight vector): their places go by value
+    RowsByValue rv = {};
+    {
+      const uint32_t *s_h = res_host(hs, n_rows), *w_h = res_host(hw, n_rows), *d_h = res_host(hd, n_rows);
+      const uint32_t* r_h = add ? res_host(hr, n_rows) : s_h;
+      bool even = s_h && w_h && d_h && r_h && s_h[1] >= s_h[0] && w_h[1] >= w_h[0] && d_h[1] >= d_h[0] && r_h[1] >= r_h[0];
+      if (even) {
+        rv = {1u, s_h[0], s_h[1] - s_h[0], w_h[0], w_h[1] - w_h[0], d_h[0], d_h[1] - d_h[0], r_h[0], r_h[1] - r_h[0]};
+        for (uint32_t i = 1; even && i < n_rows; i++)
+          even = s_h[i] == s_h[0] + i * rv.ss && w_h[i] == w_h[0] + i * rv.ws && d_h[i] == d_h[0] + i * rv.ds &&
+                 r_h[i] == r_h[0] + i * rv.rs;
+      }
+      if (!even) rv.on = 0u;
+    }
+#define RR(A, E, NU) k_rmsnorm_rows<A, E, NU><<<n_rows, 256, 0, g.stream>>>(a, w, dim | (rv.on << 31), eps, rv.s0, rv.ss, rv.w0, rv.ws, rv.d0, rv.ds, rv.r0, rv.rs, a, ls, lw, lr, ld, ma->n_elems, mw->n_elems, scale, xh, xl)
 #define RN(A, E) do { if (dim <= 2048) RR(A, E, 8); else if (dim <= 4096) RR(A, E, 16); else RR(A, E, 32); } while (0)
     if (add) { if (emit) RN(true, true); else RN(true, false); }
     else { if (emit) RN(false, true); else RN(false, false); }
