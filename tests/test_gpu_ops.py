@@ -42,6 +42,38 @@ def test_rmsnorm_family(hip, dim, rows):
         assert rel_l2(u, v) < 1e-5
 
 
+@pytest.mark.parametrize("dim,add", [(256, False), (1152, True)])
+def test_rmsnorm_rows_at_irregular_places(hip, dim, add):
+    """Several rows whose sources, destinations (and residuals) are NOT evenly spaced, in another order than they lie
+    in memory, and a weight vector of their own per row: the multi-row kernel takes the rows' places from the tables
+    on the device (evenly spaced rows get them by value) and gives the oracle's rows."""
+    rng = np.random.default_rng(dim)
+    rows = 5
+    src = [7 * dim + 3, 0, 3 * dim + 1, 11 * dim, 5 * dim + 2]
+    res = [20 * dim + o for o in (4 * dim, 0, 9 * dim + 5, 2 * dim, 6 * dim + 1)]
+    dst = [40 * dim + o for o in (3 * dim, 8 * dim + 2, 0, 5 * dim + 7, dim + 1)]
+    wts = [60 * dim + o for o in (2 * dim, 0, dim, 4 * dim, 3 * dim)]
+    total = 66 * dim
+    data = rng.standard_normal(total).astype(np.float32)
+    outs = []
+    for g in pair(hip):
+        note(f"rmsnorm rows at irregular places dim={dim} add={add}")
+        f32map(g, 0, total, data)
+        hs, hr, hd, hw = up(g, src), up(g, res), up(g, dst), up(g, wts)
+        if add:
+            g.map_rmsnorm_add_dev(0, hs, hw, hr, hd, rows, dim, 1e-6)
+        else:
+            g.map_rmsnorm_dev(0, hs, hw, hd, rows, dim, 1e-6)
+        outs.append(read(g, 0, 0, total))
+    assert rel_l2(outs[0], outs[1]) < 1e-5
+    for i in range(rows):                      # every row by the closed form as well
+        x = data[src[i]:src[i] + dim].astype(np.float64)
+        y = x / np.sqrt(np.mean(x * x) + 1e-6) * data[wts[i]:wts[i] + dim]
+        if add:
+            y = y + data[res[i]:res[i] + dim]
+        assert rel_l2(outs[0][dst[i]:dst[i] + dim], y) < 1e-5, i
+
+
 @pytest.mark.parametrize("heads,dim,pos,base", [(32, 128, 0, 500000.0), (8, 128, 4095, 500000.0),
                                                (4, 256, 639, 1e6), (1, 256, 16383, 1e4)])
 def test_rope(hip, heads, dim, pos, base):
