@@ -128,6 +128,8 @@ _SIGS = {
     "map_matvec_topk_t_xq8_ex_dev": (i32, [_U] * 11 + [f32c, _U]),
     "map_matvec_rerank_t_xq8_dev": (i32, [_U] * 12 + [f32c]),
     "adamah_matvec_topk_t_xq4_noalloc_dev": (i32, [_U] * 11 + [f32c, _U]),
+    "adamah_hip_embed_tokens_dev": (i32, [_U] * 8 + [f32c]),
+    "adamah_hip_token_post": (i32, [_U] * 3 + [pu32]), "adamah_hip_token_wait": (i32, [_U, pf32, _U]),
     "map_fused_qkv_t_xq4_dev": (i32, [_U] * 13), "map_fused_qkv_t_xq8_dev": (i32, [_U] * 13),
     "map_fused_gateup_t_xq4_dev": (i32, [_U] * 10), "map_fused_gateup_t_xq8_dev": (i32, [_U] * 10),
     "map_fused_gateup_act_t_xq8_dev": (i32, [_U] * 8),
@@ -152,6 +154,7 @@ _OPTIONAL_FLAGS = {
     "adamah_kv_cache_fp16": "_has_kv_cache_fp16",
     "adamah_attn_causal_rows_dev": "_has_attn_causal_rows_dev",
     "adamah_qk_norm_rope_rows_dev": "_has_qk_norm_rope_rows_dev",
+    "adamah_hip_embed_tokens_dev": "_has_token_feed",
     "map_resolve_idx_dev": "_has_map_resolve_idx_dev",
     "map_sample_categorical_dev": "_has_map_sample_categorical_dev",
     "map_repeat_penalty_dev": "_has_map_repeat_penalty_dev",
@@ -424,6 +427,28 @@ class Adamah:
         oa = (ctypes.c_uint32 * m)(*out_handles)
         self._op("adamah_attn_causal_rows_dev", map_id, qa, locs_k_handle, locs_scores_handle, locs_v_handle, oa, m,
                  head_dim, n_keys0, n_heads, value_dim, scale, softcap)
+
+    def embed_tokens_dev(self, map_act, map_src, locs_tokens_handle, src_row0, dst_start, m, E, V, scale=1.0):
+        """Extension: embedding rows of m tokens whose ids (float32) are still on the device, scaled, into
+        m consecutive rows of map_act -- what map_gather_dev + map_scatter_dev + a multiplication give."""
+        self._op("adamah_hip_embed_tokens_dev", map_act, map_src, locs_tokens_handle, src_row0, dst_start, m, E, V,
+                 scale)
+
+    def token_post(self, map_id, locs_handle, n):
+        """Extension: in stream order, hand the n float32 values at the handle's elements to the host (ring of 8
+        in pinned memory); returns the ticket to wait on."""
+        t = ctypes.c_uint32(0)
+        self._op("adamah_hip_token_post", map_id, locs_handle, n, ctypes.byref(t))
+        return t.value
+
+    def token_wait(self, ticket, n=1):
+        """Extension: the values posted under `ticket`, as soon as the post has run -- work queued behind it is
+        not waited for."""
+        out = np.empty(n, np.float32)
+        ret = self._lib.adamah_hip_token_wait(ticket, out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), n)
+        if ret != 0:
+            raise RuntimeError(f"adamah_hip_token_wait failed with code {ret}")
+        return out
 
     def qk_norm_rope_rows_dev(self, map_act, map_wt, q_src_handles, locs_q_wt_handle, k_src_handles, locs_k_wt_handle,
                               dst_handles, q_rows, q_dim, k_rows, k_dim, pos0, freq_base):

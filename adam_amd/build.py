@@ -7,7 +7,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libadamah_hip.so")
-SOURCES = ["runtime.hip", "gemv_q.hip", "gemv_mfma.hip", "gemm_q4_mfma.hip", "fuse.hip", "norm_rope.hip", "rowprep.hip", "attention.hip", "attn_decode.hip", "attn_prefill.hip", "elementwise.hip", "sampling.hip", "topk_fused.hip", "fused_proj.hip", "probe.hip"]
+SOURCES = ["runtime.hip", "gemv_q.hip", "gemv_mfma.hip", "gemm_q4_mfma.hip", "fuse.hip", "norm_rope.hip", "rowprep.hip", "attention.hip", "attn_decode.hip", "attn_prefill.hip", "elementwise.hip", "sampling.hip", "topk_fused.hip", "fused_proj.hip", "token_feed.hip", "probe.hip"]
 # -amdgpu-kernarg-preload-count: the first 14 dwords of a kernel's arguments (whole scalars / pointers, in order) are
 # in SGPRs when a wave starts instead of being fetched from the argument block -- one trip to memory less before a
 # kernel's first loads (Q4 GEMV 5.8 -> 5.4 us at 4096x4096).  The hot kernels order their arguments for it.

@@ -395,6 +395,7 @@ void adamah_shutdown(void) { ADAMAH_API();
   topk_fused_release();
   sampling_release();
   attn_decode_release();
+  token_feed_release();
   g.pend.clear();
   for (int i = 0; i < MAX_PLANS; i++) { g.plans[i].clear(); g.plan_active[i] = false; plan_graph_reset(i); }
   hipStreamDestroy(g.stream);
@@ -843,11 +844,17 @@ static int replay_plan(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
 // -- stream capture of the same entry points, nothing executes -- while the device is still busy with the
 // current step, and the next call launches that graph if it asks for exactly that step (anything else is
 // replayed the ordinary way).  Kernels of a graph start ~0.7 us sooner after their predecessor than
-// stream launches do.  Two executable graphs alternate, so the one being updated is never in flight.
+// stream launches do.  Three executable graphs take turns and each launch is followed by an event: before a graph is
+// updated (its kernels' arguments are rewritten in place) the host waits for that graph's last launch to have
+// finished.  With three, a caller that issues step n + 1 before it has seen the result of step n (one step of
+// lookahead) never waits: the graph being rewritten last ran step n - 1.
 // A plan whose ops copy from the host (tables of operand bases) or fail to capture is left to the
 // ordinary replay for good.
+#define PLAN_EXECS 3
 struct PlanGraph {
-  hipGraphExec_t exec[2] = {nullptr, nullptr};
+  hipGraphExec_t exec[PLAN_EXECS] = {nullptr, nullptr, nullptr};
+  hipEvent_t done[PLAN_EXECS] = {nullptr, nullptr, nullptr};   // recorded behind the last launch of exec[i]
+  bool launched[PLAN_EXECS] = {false, false, false};
   int cur = 0;               // exec[cur] holds the recorded step when ready
   bool ready = false, disabled = false;
   uint32_t pos = 0, seq = 0, n_nodes = 0;
@@ -866,7 +873,12 @@ static bool plan_graphs_on() {
 }
 
 static void plan_graph_drop(PlanGraph& pg, bool for_good) {
-  for (int i = 0; i < 2; i++) { if (pg.exec[i]) hipGraphExecDestroy(pg.exec[i]); pg.exec[i] = nullptr; }
+  for (int i = 0; i < PLAN_EXECS; i++) {
+    if (pg.launched[i] && pg.done[i]) hipEventSynchronize(pg.done[i]);
+    pg.launched[i] = false;
+    if (pg.exec[i]) hipGraphExecDestroy(pg.exec[i]);
+    pg.exec[i] = nullptr;
+  }
   pg.ready = false;
   if (for_good) pg.disabled = true;
 }
@@ -902,7 +914,11 @@ static void plan_graph_record(uint32_t plan_id, uint32_t pos, uint32_t seq_len) 
     return;
   }
   gemm_act_forget();   // the note "these rows are converted" was taken while nothing ran
-  const int slot = pg.cur ^ 1;
+  const int slot = (pg.cur + 1) % PLAN_EXECS;
+  if (pg.launched[slot]) {                           // its kernels read their arguments from the graph's own memory
+    hipEventSynchronize(pg.done[slot]);
+    pg.launched[slot] = false;
+  }
   if (pg.exec[slot]) {
     hipGraphNode_t bad = nullptr;
     hipGraphExecUpdateResult res;
@@ -940,6 +956,7 @@ static void plan_graph_reset(uint32_t plan_id) {
             o.n_graph, o.eager_steps, o.n_update, o.n_inst, o.n_nodes, o.disabled ? ", graphs given up" : "");
   hipStreamSynchronize(g.stream);
   plan_graph_drop(g_pg[plan_id], false);
+  for (int i = 0; i < PLAN_EXECS; i++) if (g_pg[plan_id].done[i]) hipEventDestroy(g_pg[plan_id].done[i]);
   g_pg[plan_id] = PlanGraph();
 }
 
@@ -962,6 +979,9 @@ int adamah_decode_step(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
     }
     if (pg.ready && pg.pos == pos && pg.seq == seq_len) {
       ret = hipGraphLaunch(pg.exec[pg.cur], g.stream) == hipSuccess ? ADAMAH_OK : ADAMAH_ERR_BACKEND;
+      if (!pg.done[pg.cur] && hipEventCreateWithFlags(&pg.done[pg.cur], hipEventDisableTiming) != hipSuccess) ret = ADAMAH_ERR_BACKEND;
+      if (ret == ADAMAH_OK && hipEventRecord(pg.done[pg.cur], g.stream) != hipSuccess) ret = ADAMAH_ERR_BACKEND;
+      pg.launched[pg.cur] = ret == ADAMAH_OK;
       count_launch((int)pg.n_nodes);
       pg.n_graph++;
       g.pend.insert(g.pend.end(), pg.tail.begin(), pg.tail.end());

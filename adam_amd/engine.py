@@ -76,7 +76,7 @@ class DecodeEngine:
     def __init__(self, gpu, cfg, tensors, A=None, kv_cap=1024, kv_fp16=False,
                  fusion_scheduler_mode='legacy', gpu_fused_rows_per_group=256,
                  q4_map_elem_limit=(1 << 32) - 64, verbose=False, decode_plan=True, plan_id=0,
-                 prefill_chunk=0, batch=1):
+                 prefill_chunk=0, batch=1, lookahead=True):
         if A is None:
             from . import adamah as A
         self.gpu, self.cfg, self.tensors, self.A = gpu, cfg, tensors, A
@@ -99,6 +99,10 @@ class DecodeEngine:
         gpu.fusion_enable(True)
         self._sample_token_ready = False
         self.n_ops_last_forward = 0
+        # One step of lookahead in the greedy loops (embedding rows gathered on the device from the token the
+        # previous step left there, tokens handed to the host through the library's ring): set up on first use.
+        self._lookahead = bool(lookahead) and getattr(gpu, '_has_token_feed', False)
+        self._feed = None
         # The per-token op list is the same every step except for pos / seq_len, so it is registered
         # once as a native decode plan (reference API adamah.c:10341-10398) and replayed with one call.
         self._plan_id = None
@@ -563,9 +567,48 @@ class DecodeEngine:
         rms(hid_h, 'output_norm.weight', normed_h, c.n_embd)
         return ops
 
+    # ------------------------------------------------------------------ token feed (lookahead)
+    EMB_MAP = 15
+
+    def _token_feed(self):
+        """(map, first element) of the [V, E] table the device gathers embedding rows from, plus the handles of the
+        token slots.  Tied models read the LM head's quantised rows, as their host-driven gather does; untied
+        ones get their float32 table uploaded once into a map of its own (the reference keeps it on the host,
+        engine.py:2986-2992, which forces a round trip per token).  None: no room for the table."""
+        if self._feed is not None:
+            return self._feed or None
+        c, g, A = self.cfg, self.gpu, self.A
+        if self._tied:
+            src = (self._map_of[self._lm_name], self._off[self._lm_name])
+        else:
+            emb = self.tensors['token_embd.weight']
+            if self.EMB_MAP in self._q4_sizes or c.n_vocab * c.n_embd > self._q4_limit:
+                self._feed = False
+                return None
+            g.map_create(self.EMB_MAP, 1, c.n_vocab * c.n_embd)
+            step = max(1, (1 << 24) // c.n_embd)
+            for lo in range(0, c.n_vocab, step):
+                hi = min(c.n_vocab, lo + step)
+                rows = emb.rows(lo, hi) if hasattr(emb, 'rows') else np.stack([emb.row(t) for t in range(lo, hi)])
+                g.scatter_contiguous(self.EMB_MAP, lo * c.n_embd, np.ascontiguousarray(rows, np.float32).reshape(-1))
+            src = (self.EMB_MAP, 0)
+        self._feed = {'src': src, 'tok_h': self._up(self._sample_locs),
+                      'tok_hs': {self._batch: self._up(self._c_tok_locs[:self._batch])} if self._batch > 1 else {}}
+        return self._feed
+
+    def _post_token(self, m=1):
+        """Hand the token(s) the step just issued will choose to the host; returns the ticket to wait on."""
+        f = self._token_feed()
+        return self.gpu.token_post(self.WS_MAP, f['tok_h'] if m == 1 else f['tok_hs'][m], m)
+
+    def _wait_tokens(self, ticket, m=1):
+        return [int(t) for t in self.gpu.token_wait(ticket, m)]
+
     # ------------------------------------------------------------------ forward
-    def _forward(self, tok, pos, sample=True, sample_cfg=None, sample_prev=()):
-        """One decode step; op order of reference engine.py:2971-3402 (default discrete-GPU path)."""
+    def _forward(self, tok, pos, sample=True, sample_cfg=None, sample_prev=(), from_device=False):
+        """One decode step; op order of reference engine.py:2971-3402 (default discrete-GPU path).
+        `from_device`: the input token is the one the previous step's LM head left in the token slot (`tok` is
+        not looked at); its embedding row is gathered on the device."""
         c, g, A, ws = self.cfg, self.gpu, self.A, self.WS_MAP
         q_dim, k_dim = c.n_head * c.head_dim, c.n_head_kv * c.head_dim_kv
         seq_len = pos + 1
@@ -575,7 +618,9 @@ class DecodeEngine:
             W[n][0] for n in ('attn_out', 'o_proj', 'normed2', 'gate', 'up', 'act', 'ffn_out'))
         alias_fast = self._sched != 'legacy'
 
-        if self._tied:
+        if from_device:
+            feed = self._token_feed()
+        elif self._tied:
             np.add(self._emb_base, np.uint32(tok * c.n_embd), out=self._emb_locs)
             g.upload_dev(self._emb_locs, handle=self._emb_gather_h)
         else:
@@ -585,7 +630,10 @@ class DecodeEngine:
             g.scatter(ws, self._hid_locs, row)
 
         g.batch_begin()
-        if self._tied:
+        if from_device:
+            g.embed_tokens_dev(ws, feed['src'][0], feed['tok_h'], feed['src'][1], int(self._hid_locs[0]), 1, c.n_embd,
+                               c.n_vocab, float(c.emb_scale))
+        elif self._tied:
             src_h, _, _, _ = g.map_gather_dev(self._map_of[self._lm_name], self._emb_gather_h, c.n_embd)
             if src_h == 0:        # the binding reports a failed gather as handle 0, like the reference's
                 raise RuntimeError("map_gather_dev failed (embedding row)")
@@ -758,7 +806,7 @@ class DecodeEngine:
             residual('ffn_out', f'{p}.post_ffw_norm.weight')
         return ops
 
-    def _forward_chunk(self, toks, pos0, sample=True, seq=0, lockstep=False):
+    def _forward_chunk(self, toks, pos0, sample=True, seq=0, lockstep=False, from_device=False):
         """m <= prefill_chunk prompt tokens at positions pos0 .. pos0 + m - 1 in one pass: the row-wise ops
         over m rows, the projections as [m, K] x [N, K]^T matmuls (the fp16 matrix-core kernel for Q4
         blocks), RoPE and the KV append for all tokens at once, attention token by token over the growing
@@ -767,16 +815,23 @@ class DecodeEngine:
 
         `lockstep`: the rows are one token of each of the first m sequences of the batch instead, all at
         position pos0 -- a batched decode step: every row is rotated for pos0, appended to and attended
-        over its own sequence's cache, and gets its own LM head pass (tokens in `read_tokens`)."""
+        over its own sequence's cache, and gets its own LM head pass (tokens in `read_tokens`).
+        `from_device` (a lockstep step of the full batch): the rows' tokens are the ones the previous step left in
+        the token slots (`toks` is not looked at); their embedding rows are gathered on the device."""
         c, g, A, ws = self.cfg, self.gpu, self.A, self.WS_MAP
-        m = len(toks)
+        m = self._batch if from_device else len(toks)
         if not self._chunk or m == 0 or m > self._chunk:
             raise RuntimeError(f"chunk of {m} tokens does not fit prefill_chunk={self._chunk}")
         E, FF = c.n_embd, c.n_ff
         q_dim, k_dim = c.n_head * c.head_dim, c.n_head_kv * c.head_dim_kv
         C1, CR, CS, W = self._c1, self._crow, self._cspan, self._ws
-        toks = np.asarray(toks, np.int64)
-        if self._tied:
+        if from_device:
+            feed = self._token_feed()
+        else:
+            toks = np.asarray(toks, np.int64)
+        if from_device:
+            pass                                      # nothing to send: the tokens are on the device
+        elif self._tied:
             locs = (np.uint32(self._off[self._lm_name]) + (toks[:, None] * E + np.arange(E)[None, :])).astype(np.uint32)
             if m in self._c_emb_hs:                   # a handle can be re-uploaded at its own size only
                 g.upload_dev(np.ascontiguousarray(locs.reshape(-1)), handle=self._c_emb_hs[m])
@@ -801,7 +856,10 @@ class DecodeEngine:
             fn(ws, self._map_of[name], C1[src], self._wh[name], C1[dst], m, K, N)
 
         g.batch_begin()
-        if self._tied:
+        if from_device:
+            g.embed_tokens_dev(ws, feed['src'][0], feed['tok_hs'][m], feed['src'][1], self._cp['hidden'], m, E, c.n_vocab,
+                               float(c.emb_scale))
+        elif self._tied:
             src_h, _, _, _ = g.map_gather_dev(self._map_of[self._lm_name], emb_h, m * E)
             g.map_scatter_dev(ws, CS['hidden'], m * E, src_h)
             if c.emb_scale != 1.0:
@@ -916,6 +974,9 @@ class DecodeEngine:
         if P + max_tokens > self._kv_cap:
             raise RuntimeError(f"KV cache too small: need {P + max_tokens} tokens but kv_cap={self._kv_cap}.")
         self.reset()
+        # (the device-side embedding table of an untied model is filled on first use: before the clock starts)
+        ahead = (forced is None and self._lookahead and B == self._batch and B > 1 and max_tokens > 1
+                 and self._token_feed() is not None)
         t0 = time.perf_counter()
         cur = []
         for sq, pr in enumerate(prompts):
@@ -925,7 +986,21 @@ class DecodeEngine:
         t_pre = time.perf_counter() - t0
         out = [[] for _ in range(B)]
         t0 = time.perf_counter()
-        for step in range(max_tokens):
+        if ahead:
+            # One step of lookahead: step n + 1 takes its tokens from the slots step n's LM head passes write and is
+            # issued before the host has seen them; the host still reads every step's tokens, in order, one issue late.
+            for sq in range(B):
+                out[sq].append(cur[sq])
+            self._forward_chunk(cur, P, lockstep=True)
+            ticket = self._post_token(B)
+            for step in range(1, max_tokens):
+                self._forward_chunk(None, P + step, lockstep=True, from_device=True)
+                nxt = self._post_token(B)
+                cur = self._wait_tokens(ticket, B)
+                ticket = nxt
+                for sq in range(B):
+                    out[sq].append(cur[sq])
+        for step in range(0 if not ahead else max_tokens, max_tokens):
             for sq in range(B):
                 out[sq].append(cur[sq])
             feed = cur if forced is None else [int(forced[sq][step]) for sq in range(B)]
@@ -952,9 +1027,10 @@ class DecodeEngine:
         (top-k, top-p and repeat penalty on the device, one uniform number per token from a host
         generator seeded with `config.seed`).  Prefill is the same `_forward` once per prompt token, LM head only
         on the last one; `decode_tps = n_gen / wall(decode loop)` including the per-token
-        read-back (reference engine.py:3838-3931).  `forced`, when given, is a token list fed
-        back instead of the model's own choices (teacher forcing) while the choices are still
-        returned."""
+        read-back (reference engine.py:3838-3931).  Greedy decoding without `forced` runs one step ahead of the
+        read-back unless the engine was built with `lookahead=False`: same tokens, same number of steps.
+        `forced`, when given, is a token list fed back instead of the model's own choices (teacher forcing)
+        while the choices are still returned."""
         config = config or GenerationConfig()
         if len(token_ids) + config.max_tokens > self._kv_cap:
             raise RuntimeError(
@@ -962,6 +1038,9 @@ class DecodeEngine:
                 f"kv_cap={self._kv_cap}. Reinitialize with kv_cap>={len(token_ids) + config.max_tokens}.")
         self.reset()
         sampled = config.temperature > 0.0 and config.top_k > 1
+        # (the device-side embedding table of an untied model is filled on first use: before the clock starts)
+        ahead = (not sampled and forced is None and self._lookahead and config.max_tokens > 0
+                 and self._token_feed() is not None)
         self._rng = np.random.default_rng(config.seed)
         hist = [int(t) for t in token_ids]
         tp = time.perf_counter()
@@ -975,7 +1054,23 @@ class DecodeEngine:
         t_pre = time.perf_counter() - tp
         out, ttimes = [], []
         td = time.perf_counter()
-        for step in range(config.max_tokens):
+        if ahead:
+            # One step of lookahead: the step that consumes token n takes it from the device slot and is issued
+            # before the host has seen token n; the host reads every token, in order, one issue late.  A stop token
+            # is therefore noticed after one step too many was issued (its KV row is never read).
+            ticket = self._post_token()
+            for step in range(config.max_tokens):
+                t0 = time.perf_counter()
+                self._forward(None, len(token_ids) + step, from_device=True)
+                nxt = self._post_token()
+                nt = self._wait_tokens(ticket)[0]
+                ticket = nxt
+                if nt in config.eos_token_ids:
+                    break
+                out.append(nt)
+                hist.append(nt)
+                ttimes.append(time.perf_counter() - t0)
+        for step in range(0 if not ahead else config.max_tokens, config.max_tokens):
             t0 = time.perf_counter()
             nt = self.read_token()
             if nt in config.eos_token_ids:

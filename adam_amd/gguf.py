@@ -169,6 +169,13 @@ class RowLookup:
             return np.ascontiguousarray(t[int(tok)], np.float32)
         return t.dequant_rows(int(tok), 1).reshape(k)
 
+    def rows(self, lo, hi):
+        """Rows lo .. hi-1 as one float32 [hi - lo, E] array (what a device-side table is filled from)."""
+        t, k = self._t, self.shape[1]
+        if isinstance(t, np.ndarray):
+            return np.ascontiguousarray(t[lo:hi], np.float32)
+        return t.dequant_rows(int(lo), int(hi - lo)).reshape(hi - lo, k)
+
 
 def config_from_metadata(md, tensors):
     """ModelConfig from the file's metadata, with the reference's defaults

@@ -56,14 +56,20 @@ class SyntheticEmbedding:
         self.seed, self.sigma = seed, sigma
         self._pool = None
 
-    def row(self, tok):
+    def _rows_of(self, toks):
         if self._pool is None:
             rng = np.random.default_rng([self.seed, 0x0E3B])
             n = min(self.shape[0], self.POOL)
             self._pool = rng.standard_normal((n, self.shape[1]), dtype=np.float32) * np.float32(self.sigma)
         n = self._pool.shape[0]
-        tok = int(tok)
-        return self._pool[tok if self.shape[0] <= n else (tok * 40503 + 11) % n]
+        return self._pool[toks if self.shape[0] <= n else (toks * 40503 + 11) % n]
+
+    def row(self, tok):
+        return self._rows_of(int(tok))
+
+    def rows(self, lo, hi):
+        """Rows lo .. hi-1 as one [hi - lo, E] array (what a device-side table is filled from)."""
+        return self._rows_of(np.arange(lo, hi, dtype=np.int64))
 
 
 def _gen(name, shape, seed, sigma, quant, rows_per_chunk=8192):

@@ -307,13 +307,19 @@ def step_bytes_of(cfg, tensors, ctx_mid):
     return q4_w * 18 // 32 + q8_w * 34 // 32 + kv_b
 
 
-def measure_decode(gpu, A, DecodeEngine, cfg, tensors, prompt, steps, warmup, scheduler, prefill_chunk, decode_plan=True):
+def measure_decode(gpu, A, DecodeEngine, cfg, tensors, prompt, steps, warmup, scheduler, prefill_chunk, decode_plan=True,
+                   lookahead=True):
     """bs=1 greedy decode: the prompt, `warmup` untimed steps, then exactly `steps` timed steps (token id read back
     every step) between two device synchronisations.  decode_plan=False issues every op of a step as a call of its own
-    through the op surface, which is what the unchanged reference engine does (adam/models/engine.py:2971-3706)."""
+    through the op surface, which is what the unchanged reference engine does (adam/models/engine.py:2971-3706).
+    lookahead (the engine's default greedy loop): every step takes its input token from the device slot the previous
+    step's LM head wrote and is issued before the host has read that token; the host reads every token, in order, one
+    issue late.  lookahead=False: read the token, then issue the step that consumes it, as the reference's loop does."""
     n_prompt = len(prompt)
     eng = DecodeEngine(gpu, cfg, tensors, A=A, kv_cap=n_prompt + warmup + steps + 8, kv_fp16=True,
-                       fusion_scheduler_mode=scheduler, prefill_chunk=prefill_chunk, decode_plan=decode_plan)
+                       fusion_scheduler_mode=scheduler, prefill_chunk=prefill_chunk, decode_plan=decode_plan,
+                       lookahead=lookahead)
+    lookahead = lookahead and eng._lookahead and eng._token_feed() is not None
     gpu.sync()
     eng.reset()
     t0 = time.perf_counter()
@@ -321,16 +327,28 @@ def measure_decode(gpu, A, DecodeEngine, cfg, tensors, prompt, steps, warmup, sc
     gpu.sync()
     prefill_s = time.perf_counter() - t0
     tokens, pos = [], n_prompt
-    for _ in range(warmup):
-        nt = eng.read_token(); tokens.append(nt)
-        eng._forward(nt, pos); pos += 1
+
+    def run(n, ticket):
+        nonlocal pos
+        for _ in range(n):
+            if lookahead:
+                eng._forward(None, pos, from_device=True)
+                nxt = eng._post_token()
+                nt = eng._wait_tokens(ticket)[0]
+                ticket = nxt
+            else:
+                nt = eng.read_token()
+                eng._forward(nt, pos)
+            tokens.append(nt)
+            pos += 1
+        return ticket
+
+    ticket = run(warmup, eng._post_token() if lookahead else 0)
     gpu.sync()
     gpu.reset_native_stats()
     gpu.timer_begin()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        nt = eng.read_token(); tokens.append(nt)
-        eng._forward(nt, pos); pos += 1
+    run(steps, ticket)
     gpu.sync()
     wall = time.perf_counter() - t0
     dev_ms = gpu.timer_end()
@@ -454,7 +472,10 @@ def main():
                                f"timed steps at context {m['end_pos'] - args.steps + 1}..{m['end_pos']}",
                    "baseline_config": 2 if gemma else 4,
                    "scheduler": args.scheduler, "launches_per_token": round(m["launches_per_token"], 1),
-                   "issue": "one native decode_step call per token (registered decode plan, launched from HIP graphs recorded one step ahead)"},
+                   "issue": "one native decode_step call per token (registered decode plan, launched from HIP graphs "
+                            "recorded one step ahead); every token id is read back, in order, but the step that consumes "
+                            "token n takes it from the device and is issued before the host has read it (one step of "
+                            "lookahead; 'read_then_issue' is the same loop without it)"},
         "device_ms_per_step": round(m["device_ms_per_step"], 4),
         "algorithmic_bytes_per_token": m["step_bytes"],
         "tok_s_at_hbm_peak": round(m["ceiling"], 1), "frac_of_hbm_roofline": round(m["tok_s"] / m["ceiling"], 4),
@@ -476,12 +497,21 @@ def main():
 
         def op_by_op(cfg_, tensors_, prompt_, chunk_, ref_tokens):
             o = measure_decode(gpu, A, DecodeEngine, cfg_, tensors_, prompt_, n_obo, args.warmup, args.scheduler,
-                               chunk_, decode_plan=False)
+                               chunk_, decode_plan=False, lookahead=False)
             return {"tok/s": round(o["tok_s"], 2), "ms_per_step": round(o["ms_per_step"], 4), "steps": n_obo,
                     "launches_per_token": round(o["launches_per_token"], 1),
                     "issue": "every op of the step as its own call through ctypes, as the reference engine issues them",
                     "tokens_same_as_plan_replay": bool(o["tokens"][:8] == ref_tokens[:8])}
         leg("op_by_op", lambda: op_by_op(cfg, tensors, prompt, chunk, m["tokens"]))
+
+        def read_then_issue():
+            o = measure_decode(gpu, A, DecodeEngine, cfg, tensors, prompt, args.steps, args.warmup, args.scheduler, chunk,
+                               lookahead=False)
+            return {"tok/s": round(o["tok_s"], 2), "ms_per_step": round(o["ms_per_step"], 4), "steps": args.steps,
+                    "issue": "the headline loop without lookahead: the host reads token n, then issues the step that "
+                             "consumes it (embedding row looked up with host-made locations), as the reference's loop does",
+                    "tokens_same_as_headline": bool(o["tokens"] == m["tokens"])}
+        leg("read_then_issue", read_then_issue)
 
         def other_shape():
             g2 = not gemma
@@ -499,8 +529,11 @@ def main():
                    "tok_s_at_hbm_peak": round(o["ceiling"], 1), "frac_of_hbm_roofline": round(o["tok_s"] / o["ceiling"], 4),
                    "prefill_tok_s": round(np2 / o["prefill_s"], 1), "stats": o["stats"]}
             ob = measure_decode(gpu, A, DecodeEngine, cfg2, t2, p2, n_obo, args.warmup, args.scheduler, 0 if g2 else 512,
-                                decode_plan=False)
+                                decode_plan=False, lookahead=False)
             out["op_by_op_tok/s"] = round(ob["tok_s"], 2)
+            rt = measure_decode(gpu, A, DecodeEngine, cfg2, t2, p2, st2, args.warmup, args.scheduler, 0 if g2 else 512,
+                                lookahead=False)
+            out["read_then_issue_tok/s"] = round(rt["tok_s"], 2)
             return out
         leg("config2_gemma3_1b" if not gemma else "config4_llama3_8b", other_shape)
 

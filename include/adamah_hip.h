@@ -257,6 +257,25 @@ int adamah_matvec_topk_t_xq4_noalloc_dev(uint32_t map_act, uint32_t map_wt, uint
                                          uint32_t penalty_ids, uint32_t locs_idx_dst, uint32_t locs_val_dst,
                                          uint32_t K, uint32_t N, uint32_t k, uint32_t n_penalty,
                                          float repeat_penalty, uint32_t rows_per_group);
+/* Token feedback without a host round trip per step.  No counterpart in the reference, whose loop reads the chosen
+ * token back, looks its embedding row up (on the host for untied embeddings, adam/models/engine.py:2986-2992; with a
+ * gather of host-made locations for tied ones, engine.py:2993-3010) and only then issues the next step.
+ * embed_tokens: for r = 0 .. m-1, with tok_r = the float32 token id at element locs_tokens[r] of map_act, elements
+ * [dst_start + r*E, dst_start + (r+1)*E) of map_act = scale * row tok_r of the [V, E] table that starts at element
+ * src_row0 of map_src (float32, Q4 or Q8 map; quantised values decoded as map_gather_dev decodes them).  The result
+ * is what map_gather_dev + map_scatter_dev + a multiplication by scale give for the same token.  A token id outside
+ * [0, V) gives a row of zeros.  The destination must lie outside an fp16 KV range. */
+int adamah_hip_embed_tokens_dev(uint32_t map_act, uint32_t map_src, uint32_t locs_tokens, uint32_t src_row0,
+                                uint32_t dst_start, uint32_t m, uint32_t E, uint32_t V, float scale);
+/* token_post: in stream order, copy the n <= 62 float32 values at locs_handle's elements of map_id into a ring of 8
+ * slots in pinned host memory and then mark the slot with the post's ticket, which the call returns in *ticket
+ * (1, 2, 3, ...: the library hands every ticket out once; slot = ticket % 8).
+ * token_wait: poll the ticket's slot until it carries `ticket`, then copy its first n values to out.  It neither
+ * synchronises the stream nor waits for work queued behind the post, so a caller can issue the next step first and
+ * still read every token in order.  Returns ADAMAH_ERR_NOT_FOUND when the stream has drained and the ticket is not
+ * there (never posted, or its slot taken by the post 8 tickets later). */
+int adamah_hip_token_post(uint32_t map_id, uint32_t locs_handle, uint32_t n, uint32_t* ticket);
+int adamah_hip_token_wait(uint32_t ticket, float* out, uint32_t n);
 /* ---- measurement and test helpers: not part of the op surface ------------------------------------
  * Nothing a model engine calls.  bench.py times launches with the stopwatch and calibrates profiler counters
  * with the probe; the parity tests read back what the kernels see through the other two. */
