@@ -31,7 +31,9 @@ namespace adamah {
 typedef int i4_t __attribute__((ext_vector_type(4)));
 typedef float f4u_t __attribute__((ext_vector_type(4), aligned(4)));
 
-enum { MF_U = 4 };   // 16-byte blocks per lane and step
+// A step of the row loop covers 16 * U blocks of a 4-row bundle: U 16-byte blocks per lane.  U = 4 for rows that fill
+// whole steps (K a multiple of 2048); U = 3 wastes fewer block slots on some rows that do not (K = 1152: 36 blocks
+// in one step of 48 instead of one of 64).
 
 
 // lane ^ 1 and lane ^ 2 within a quad (quad_perm [1,0,3,2] and [2,3,0,1]): a register move, no trip through LDS
@@ -62,10 +64,11 @@ __device__ __forceinline__ uint32_t quad_b3(uint32_t v) {
 // spreads the 16 blocks a wave reads at once over all banks.
 __device__ __forceinline__ uint32_t chunk_off(uint32_t c, uint32_t blk) { return ((c ^ (blk & 7u)) << 4); }
 
-struct PreM {
-  uint4 q[MF_U];
-  __half h[MF_U];
-  float2 p[MF_U];
+template <int U>
+struct PreMT {
+  uint4 q[U];
+  __half h[U];
+  float2 p[U];
   float res;   // EPIX_ADD: the residual of this lane's result row, fetched with the weights of the bundle's last step
 };
 
@@ -73,7 +76,7 @@ struct PreM {
 // row-wise ops that have been folded into this kernel (RMSNorm of another vector; or RMSNorm +
 // residual followed by a second RMSNorm).  Every workgroup recomputes those small ops while it
 // stages the activations; their results are also stored where the unfused ops would have put them.
-template <int FMT, int EPI, bool RAGGED, int PRO>
+template <int FMT, int EPI, bool RAGGED, int PRO, int MF_U>
 __global__ void __launch_bounds__(1024)
 k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __restrict__ d16, uint32_t K, uint32_t N, uint32_t ks,
             uint32_t x_src, uint32_t b_off, const float* n_wt, uint32_t n_w,
@@ -84,6 +87,8 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
   // (x_src: the vector itself, or the source of the first folded norm, whose weights are n_wt + n_w), the weights,
   // K, N and the K split.
   const uint32_t a = x_src;
+  using PreM = PreMT<MF_U>;
+  constexpr uint32_t SB = 16u * MF_U;                 // blocks per step
   constexpr bool B16 = (FMT == FMT_Q4_B16);
   extern __shared__ uint4 smem_u4[];
   uint8_t* xs = (uint8_t*)smem_u4;                    // nblk * 128 bytes
@@ -92,7 +97,7 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
   __shared__ float red_g[16];                         // per-wave partial sums of the prologue's last norm
   __shared__ float part[16 * 64];                     // ks > 1: per-wave partial sums of a shared bundle
   const uint32_t nblk = K >> 5;
-  const uint32_t C = (nblk + 63u) >> 6;               // steps per row bundle
+  const uint32_t C = (nblk + SB - 1u) / SB;           // steps per row bundle
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, nthr = blockDim.x, nwav = nthr >> 6;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -138,13 +143,13 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
   const uint32_t ll = lane >> 4, lbcol = lane & 15u;
   auto load = [&](PreM& R, uint32_t row0, uint32_t chunk, uint32_t end) {
     const uint32_t row = glu ? (row0 >> 1) + (ll & 1u) + (ll >> 1) * (N >> 1) : min(row0 + ll, end - 1u);
-    const uint64_t g0 = gbase + (uint64_t)row * nblk + chunk * 64u + lbcol;
+    const uint64_t g0 = gbase + (uint64_t)row * nblk + chunk * SB + lbcol;
 #pragma unroll
     for (uint32_t u = 0; u < MF_U; u++) {
       uint64_t gi = g0 + u * 16u;
       // blocks past the end of the row are clamped, not skipped: the number of loads per step has to be
       // fixed for the prefetch to stay ahead (see the step loop)
-      if (RAGGED) gi = gbase + (uint64_t)row * nblk + min(chunk * 64u + u * 16u + lbcol, nblk - 1u);
+      if (RAGGED) gi = gbase + (uint64_t)row * nblk + min(chunk * SB + u * 16u + lbcol, nblk - 1u);
       R.q[u] = *(const uint4*)(W + (gi << 4));
       if (B16) R.h[u] = d16[gi];
       else R.p[u] = qp[gi];
@@ -455,7 +460,7 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
         R.p[u].y = __int_as_float(__builtin_amdgcn_ds_bpermute(perm_addr, __float_as_int(Rl.p[u].y)));
       }
     }
-    const uint8_t* base = xs + (size_t)(chunk * 64u + bcol) * 128u;
+    const uint8_t* base = xs + (size_t)(chunk * SB + bcol) * 128u;
     uint4 xa[MF_U], xb[MF_U];
     bool valid[MF_U];
     i4_t d[MF_U];
@@ -464,14 +469,14 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
       valid[u] = true;
       const uint8_t* bp = base + u * 2048u;
       if (RAGGED) {
-        const uint32_t blk_raw = chunk * 64u + u * 16u + bcol;
+        const uint32_t blk_raw = chunk * SB + u * 16u + bcol;
         valid[u] = blk_raw < nblk;
         bp = xs + (size_t)min(blk_raw, nblk - 1u) * 128u;
       }
       xa[u] = *(const uint4*)(bp + x_off0); xb[u] = *(const uint4*)(bp + x_off1);
       d[u] = (i4_t){0, 0, 0, 0};
     }
-    // eight dependent matrix instructions per block; the four blocks of a step are interleaved so that
+    // eight dependent matrix instructions per block; the U blocks of a step are interleaved so that
     // consecutive instructions are independent
 #define MF_STEP(XV, WV, SH)                                                                                   \
   _Pragma("unroll") for (uint32_t u = 0; u < MF_U; u++)                                                       \
@@ -636,6 +641,19 @@ bool mfma_path_ok(const Map* mw, uint32_t K) {
   return mw->dtype == DTYPE_Q4 && mw->group_size == 32 && K >= 32 && (K & 31u) == 0 && mfma_smem(K) <= 64000;
 }
 
+// Blocks per lane and step for rows of K elements (the block16 format; the affine format always takes 4): 3 where
+// that takes no more steps than 4 and leaves fewer block slots of the last step empty (K = 1152: one step of 48 slots
+// for 36 blocks instead of one of 64; 13824 x 1152 6.4 -> 5.5 us, 6912 x 1152 4.6 -> 4.4 us).  More but shorter steps
+// lose: K = 6912 in five steps of 48 instead of four of 64, 5.1 -> 5.7 us.
+static uint32_t mfma_step_u(uint32_t K) {
+  const uint32_t nblk = K >> 5;
+  const uint32_t c4 = cdiv(nblk, 64u), c3 = cdiv(nblk, 48u);
+  uint32_t best = (c3 <= c4 && c3 * 48u < c4 * 64u) ? 3u : 4u;
+  const int forced = knob("ADAMAH_MFMA_U", 0);
+  if (forced == 3 || forced == 4) best = (uint32_t)forced;
+  return best;
+}
+
 template <int EPI, int PRO>
 static void launch_mfma_p(int fmt, uint32_t grid, uint32_t threads, const Map* ma, const Map* mw, uint32_t a, uint32_t b,
                           uint32_t c, const uint32_t* lidx, const uint32_t* lval, uint32_t K, uint32_t N, uint32_t rpg,
@@ -643,15 +661,20 @@ static void launch_mfma_p(int fmt, uint32_t grid, uint32_t threads, const Map* m
   float* act = (float*)ma->buf;
   float* act_out = out ? out : act;
   const size_t smem = mfma_smem(K);
-  const bool ragged = (K & 2047u) != 0;
+  const uint32_t U = fmt == FMT_Q4_B16 ? mfma_step_u(K) : 4u;
+  const bool ragged = (K & 2047u) != 0;              // of steps of 64 blocks
   const bool norm = PRO == PRO_RMSNORM || PRO == PRO_NORM2;
   const uint32_t x_src = norm ? fz.p_src : a;
   const float* n_wt = norm ? fz.p_wt : act;
-#define MK(F, R)                                                                                                  \
-  k_gemv_mfma<F, EPI, R, PRO><<<grid, threads, smem, g.stream>>>(act, mw->buf, mw->d16, K, N, ks, x_src, b, n_wt, fz.p_src2, act_out, c, \
-                                                                 mw->qp, lidx, lval, rpg, n_groups, fz)
-  if (fmt == FMT_Q4_B16) { if (ragged) MK(FMT_Q4_B16, true); else MK(FMT_Q4_B16, false); }
-  else { if (ragged) MK(FMT_Q4_AFF, true); else MK(FMT_Q4_AFF, false); }
+#define MK(F, R, UU)                                                                                              \
+  k_gemv_mfma<F, EPI, R, PRO, UU><<<grid, threads, smem, g.stream>>>(act, mw->buf, mw->d16, K, N, ks, x_src, b, n_wt, fz.p_src2, act_out, c, \
+                                                                     mw->qp, lidx, lval, rpg, n_groups, fz)
+  // (the shorter steps exist in the clamping form only: they are chosen for rows that do not fill steps of 64)
+  if (fmt == FMT_Q4_B16) {
+    if (U == 3u) MK(FMT_Q4_B16, true, 3);
+    else if (ragged) MK(FMT_Q4_B16, true, 4);
+    else MK(FMT_Q4_B16, false, 4);
+  } else { if (ragged) MK(FMT_Q4_AFF, true, 4); else MK(FMT_Q4_AFF, false, 4); }
 #undef MK
 }
 
@@ -693,7 +716,7 @@ static void mfma_shape(uint32_t K, uint32_t units, uint32_t* grid, uint32_t* thr
 // within the 4096 waves the device holds at once.  A wave then has one or two steps, all of whose loads are in
 // flight from the start: such launches are bound by one trip to memory, not by arithmetic.
 static uint32_t mfma_ksplit(uint32_t K, uint32_t N, bool paired_rows) {
-  const uint32_t C = cdiv(K, 2048u), n_q = cdiv(N, 4u);
+  const uint32_t C = cdiv(K, 512u * mfma_step_u(K)), n_q = cdiv(N, 4u);
   const uint32_t want = (uint32_t)std::max(1, knob("ADAMAH_MFMA_KSPLIT_WAVES", 4096));
   uint32_t ks = 1;
   while (ks < 4u && ks * 2u <= C && n_q * ks * 2u <= want) ks *= 2u;
