@@ -159,8 +159,8 @@ def test_matmul_batched_rows_ops_and_non_transposed(hip):
 
 
 # row lengths on either side of the kernel's choice of step (48 or 64 blocks): one short step (1152, 1536), several
-# short steps with the last one part empty (3072 -> 2 x 48, 4000 -> 125 blocks in 3 x 48), long steps with a ragged
-# last one (6912, 2080), exact long steps (2048)
+# short steps with the last one part empty (3072 -> 2 x 48, 2080 -> 65 blocks in 2 x 48, 4000 -> 125 blocks in
+# 3 x 48 where 2 x 64 would do: long steps), long steps with a ragged last one (6912), exact long steps (2048)
 @pytest.mark.parametrize("N,K", [(1, 32), (17, 64), (33, 4096), (16, 15872), (1153, 1152), (130, 1536), (66, 3072),
                                  (259, 4000), (1152, 6912), (40, 2080), (77, 2048)])
 def test_gemv_edge_shapes(hip, N, K):
