@@ -30,6 +30,7 @@ namespace adamah {
 
 typedef int i4_t __attribute__((ext_vector_type(4)));
 typedef float f4u_t __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u4v_t __attribute__((ext_vector_type(4)));
 
 // A step of the row loop covers 16 * U blocks of a 4-row bundle: U 16-byte blocks per lane.  U = 4 for rows that fill
 // whole steps (K a multiple of 2048); U = 3 wastes fewer block slots on some rows that do not (K = 1152: 36 blocks
@@ -150,7 +151,10 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
       // blocks past the end of the row are clamped, not skipped: the number of loads per step has to be
       // fixed for the prefetch to stay ahead (see the step loop)
       if (RAGGED) gi = gbase + (uint64_t)row * nblk + min(chunk * SB + u * 16u + lbcol, nblk - 1u);
-      R.q[u] = *(const uint4*)(W + (gi << 4));
+      // the codes are read once per launch and not again before the next token: non-temporal, so that they do not
+      // push the step's small, re-read data (activations, KV rows, slice partials) out of the L2
+      const u4v_t t = __builtin_nontemporal_load((const u4v_t*)(W + (gi << 4)));
+      R.q[u] = make_uint4(t.x, t.y, t.z, t.w);
       if (B16) R.h[u] = d16[gi];
       else R.p[u] = qp[gi];
     }

@@ -585,6 +585,7 @@ class DecodeEngine:
             if self.EMB_MAP in self._q4_sizes or c.n_vocab * c.n_embd > self._q4_limit:
                 self._feed = False
                 return None
+            g.set_dtype(A.DTYPE_F32)
             g.map_create(self.EMB_MAP, 1, c.n_vocab * c.n_embd)
             step = max(1, (1 << 24) // c.n_embd)
             for lo in range(0, c.n_vocab, step):
