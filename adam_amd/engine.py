@@ -68,6 +68,7 @@ class ModelConfig:
 class DecodeEngine:
     WS_MAP = 0
     Q8_MAP = 2
+    EMB_MAP = 15          # float32 copy of an untied embedding table, made when the greedy loops run ahead
     Q4_GROUP = 32
     SAMPLE_TOPK_MAX = 64       # reference engine.py:118
     SAMPLE_REPEAT_MAX = 64     # reference engine.py:120
@@ -568,8 +569,6 @@ class DecodeEngine:
         return ops
 
     # ------------------------------------------------------------------ token feed (lookahead)
-    EMB_MAP = 15
-
     def _token_feed(self):
         """(map, first element) of the [V, E] table the device gathers embedding rows from, plus the handles of the
         token slots.  Tied models read the LM head's quantised rows, as their host-driven gather does; untied
