@@ -708,7 +708,11 @@ static void mfma_shape(uint32_t K, uint32_t units, uint32_t* grid, uint32_t* thr
   while (waves > 4 && cdiv(units, waves) < (uint32_t)g.n_cu) waves >>= 1;
   waves = (uint32_t)knob("ADAMAH_MFMA_WAVES", (int)waves);
   waves = waves >= 16 ? 16 : waves >= 8 ? 8 : 4;
-  const uint32_t per_simd = (uint32_t)std::max(1, knob("ADAMAH_MFMA_PERSIMD", 2));
+  uint32_t per_simd = (uint32_t)std::max(1, knob("ADAMAH_MFMA_PERSIMD", 2));
+  // rows of at most 4096 elements (16 KB of staged activations): two workgroups of 8 waves per CU instead of one of 16,
+  // so that one's staging and barriers run beside the other's arithmetic (28672x4096 alone 15.8 -> 14.7 us, LM head
+  // 262144x1152 + argmax 49 -> 41 us; inside the Llama-shape step, behind a norm prologue, no difference)
+  if (waves == 16u && mfma_smem(K) <= (size_t)knob("ADAMAH_MFMA_SMALLWG", 16384)) { waves = 8u; per_simd = 4u; }
   const size_t lds_fit = std::max<size_t>(1, (160 * 1024) / (mfma_smem(K) + 256));
   const uint32_t wg_per_cu = (uint32_t)std::max<size_t>(1, std::min<size_t>(lds_fit, (size_t)per_simd * 4 / waves));
   *threads = waves * 64;
