@@ -826,11 +826,11 @@ class DecodeEngine:
         q_dim, k_dim = c.n_head * c.head_dim, c.n_head_kv * c.head_dim_kv
         C1, CR, CS, W = self._c1, self._crow, self._cspan, self._ws
         if from_device:
-            feed = self._token_feed()
+            feed = self._token_feed()                 # nothing to send: the tokens are on the device
         else:
             toks = np.asarray(toks, np.int64)
         if from_device:
-            pass                                      # nothing to send: the tokens are on the device
+            pass
         elif self._tied:
             locs = (np.uint32(self._off[self._lm_name]) + (toks[:, None] * E + np.arange(E)[None, :])).astype(np.uint32)
             if m in self._c_emb_hs:                   # a handle can be re-uploaded at its own size only
