@@ -129,6 +129,7 @@ _SIGS = {
     "map_matvec_rerank_t_xq8_dev": (i32, [_U] * 12 + [f32c]),
     "adamah_matvec_topk_t_xq4_noalloc_dev": (i32, [_U] * 11 + [f32c, _U]),
     "adamah_hip_embed_tokens_dev": (i32, [_U] * 8 + [f32c]),
+    "adamah_hip_embed_post_tokens_dev": (i32, [_U] * 8 + [f32c, pu32]),
     "adamah_hip_token_post": (i32, [_U] * 3 + [pu32]), "adamah_hip_token_wait": (i32, [_U, pf32, _U]),
     "map_fused_qkv_t_xq4_dev": (i32, [_U] * 13), "map_fused_qkv_t_xq8_dev": (i32, [_U] * 13),
     "map_fused_gateup_t_xq4_dev": (i32, [_U] * 10), "map_fused_gateup_t_xq8_dev": (i32, [_U] * 10),
@@ -433,6 +434,14 @@ class Adamah:
         m consecutive rows of map_act -- what map_gather_dev + map_scatter_dev + a multiplication give."""
         self._op("adamah_hip_embed_tokens_dev", map_act, map_src, locs_tokens_handle, src_row0, dst_start, m, E, V,
                  scale)
+
+    def embed_post_tokens_dev(self, map_act, map_src, locs_tokens_handle, src_row0, dst_start, m, E, V, scale=1.0):
+        """Extension: embed_tokens_dev whose launch also hands the m token values it reads to the host, as
+        token_post does; returns the ticket to wait on."""
+        t = ctypes.c_uint32(0)
+        self._op("adamah_hip_embed_post_tokens_dev", map_act, map_src, locs_tokens_handle, src_row0, dst_start, m, E, V,
+                 scale, ctypes.byref(t))
+        return t.value
 
     def token_post(self, map_id, locs_handle, n):
         """Extension: in stream order, hand the n float32 values at the handle's elements to the host (ring of 8

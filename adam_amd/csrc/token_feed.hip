@@ -32,8 +32,21 @@ template <int FMT>   // 0 = float32, 1 = Q4 (two codes a byte), 2 = Q8
 __global__ void __launch_bounds__(256)
 k_embed_tokens(float* act, uint64_t act_elems, const uint8_t* __restrict__ src, uint64_t src_elems, uint64_t row0,
                uint32_t E, uint32_t V, uint32_t total, uint32_t dst0, uint32_t tok0, uint32_t tok_by_val, float scale,
-               const uint32_t* __restrict__ tok_locs, const float2* __restrict__ qp, uint32_t group) {
+               const uint32_t* __restrict__ tok_locs, const float2* __restrict__ qp, uint32_t group, uint32_t m,
+               TokenMail* mail, uint32_t ticket) {
   const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  // mail: the launch also hands the m token values to the host, as k_token_post would (wave 0 of workgroup 0)
+  if (mail && blockIdx.x == 0 && threadIdx.x < 64u) {
+    if (threadIdx.x < m) {
+      const uint32_t ml = tok_by_val ? tok0 + threadIdx.x : tok_locs[threadIdx.x];
+      mail->val[threadIdx.x] = ml < act_elems ? act[ml] : 0.0f;
+    }
+    __threadfence_system();
+    if (threadIdx.x == 0) {
+      mail->n = m;
+      __hip_atomic_store(&mail->ticket, ticket, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+  }
   if (i >= total) return;
   const uint32_t r = i / E, e = i - r * E;
   const uint32_t tl = tok_by_val ? tok0 + r : tok_locs[r];
@@ -96,10 +109,9 @@ void token_feed_release() {
 
 using namespace adamah;
 
-extern "C" {
-
-int adamah_hip_embed_tokens_dev(uint32_t map_act, uint32_t map_src, uint32_t locs_tokens, uint32_t src_row0,
-                                uint32_t dst_start, uint32_t m, uint32_t E, uint32_t V, float scale) { ADAMAH_API();
+// ticket_out: the launch also posts the tokens it reads (adamah_hip_embed_post_tokens_dev)
+static int embed_tokens(uint32_t map_act, uint32_t map_src, uint32_t locs_tokens, uint32_t src_row0, uint32_t dst_start,
+                        uint32_t m, uint32_t E, uint32_t V, float scale, uint32_t* ticket_out) {
   Map* ma = get_f32_map(map_act);
   Map* ms = get_map(map_src);
   if (!ma || !ms || m == 0 || E == 0 || V == 0 || ms->pack_size != 1 || ma->pack_size != 1) return ADAMAH_ERR_INVALID;
@@ -115,13 +127,37 @@ int adamah_hip_embed_tokens_dev(uint32_t map_act, uint32_t map_src, uint32_t loc
   if (!tl) return ADAMAH_ERR_INVALID;
   uint32_t tok0 = 0;
   const uint32_t by_val = res_run(locs_tokens, m, &tok0) && in_range(tok0, m, ma->n_elems) ? 1u : 0u;
+  TokenMail* mail = nullptr;
+  uint32_t ticket = 0;
+  if (ticket_out) {
+    if (m > MAIL_MAX) return ADAMAH_ERR_INVALID;
+    if (int r = mail_setup()) return r;
+    ticket = g_ticket = g_ticket >= 0x7FFFFFFFu ? 1u : g_ticket + 1u;
+    *ticket_out = ticket;
+    mail = g_mail_dev + ticket % MAIL_SLOTS;
+  }
   const dim3 grid(cdiv(total, 256));
 #define EMBED(F) k_embed_tokens<F><<<grid, 256, 0, g.stream>>>((float*)ma->buf, ma->n_elems, ms->buf, ms->n_elems, src_row0, E, V, \
-                                                          total, dst_start, tok0, by_val, scale, tl, ms->qp, ms->group_size)
+                                                          total, dst_start, tok0, by_val, scale, tl, ms->qp, ms->group_size, m, mail, ticket)
   if (fmt == 0) EMBED(0); else if (fmt == 1) EMBED(1); else EMBED(2);
 #undef EMBED
   count_launch();
   return check_launch();
+}
+
+extern "C" {
+
+
+int adamah_hip_embed_tokens_dev(uint32_t map_act, uint32_t map_src, uint32_t locs_tokens, uint32_t src_row0,
+                                uint32_t dst_start, uint32_t m, uint32_t E, uint32_t V, float scale) { ADAMAH_API();
+  return embed_tokens(map_act, map_src, locs_tokens, src_row0, dst_start, m, E, V, scale, nullptr);
+}
+
+int adamah_hip_embed_post_tokens_dev(uint32_t map_act, uint32_t map_src, uint32_t locs_tokens, uint32_t src_row0,
+                                     uint32_t dst_start, uint32_t m, uint32_t E, uint32_t V, float scale,
+                                     uint32_t* ticket) { ADAMAH_API();
+  if (!ticket) return ADAMAH_ERR_INVALID;
+  return embed_tokens(map_act, map_src, locs_tokens, src_row0, dst_start, m, E, V, scale, ticket);
 }
 
 int adamah_hip_token_post(uint32_t map_id, uint32_t locs_handle, uint32_t n, uint32_t* ticket_out) { ADAMAH_API();

@@ -104,6 +104,7 @@ class DecodeEngine:
         # previous step left there, tokens handed to the host through the library's ring): set up on first use.
         self._lookahead = bool(lookahead) and getattr(gpu, '_has_token_feed', False)
         self._feed = None
+        self._feed_ticket = 0
         # The per-token op list is the same every step except for pos / seq_len, so it is registered
         # once as a native decode plan (reference API adamah.c:10341-10398) and replayed with one call.
         self._plan_id = None
@@ -596,11 +597,6 @@ class DecodeEngine:
                       'tok_hs': {self._batch: self._up(self._c_tok_locs[:self._batch])} if self._batch > 1 else {}}
         return self._feed
 
-    def _post_token(self, m=1):
-        """Hand the token(s) the step just issued will choose to the host; returns the ticket to wait on."""
-        f = self._token_feed()
-        return self.gpu.token_post(self.WS_MAP, f['tok_h'] if m == 1 else f['tok_hs'][m], m)
-
     def _wait_tokens(self, ticket, m=1):
         return [int(t) for t in self.gpu.token_wait(ticket, m)]
 
@@ -630,9 +626,9 @@ class DecodeEngine:
             g.scatter(ws, self._hid_locs, row)
 
         g.batch_begin()
-        if from_device:
-            g.embed_tokens_dev(ws, feed['src'][0], feed['tok_h'], feed['src'][1], int(self._hid_locs[0]), 1, c.n_embd,
-                               c.n_vocab, float(c.emb_scale))
+        if from_device:     # (the same launch hands the token to the host: _wait_tokens(self._feed_ticket))
+            self._feed_ticket = g.embed_post_tokens_dev(ws, feed['src'][0], feed['tok_h'], feed['src'][1],
+                                                        int(self._hid_locs[0]), 1, c.n_embd, c.n_vocab, float(c.emb_scale))
         elif self._tied:
             src_h, _, _, _ = g.map_gather_dev(self._map_of[self._lm_name], self._emb_gather_h, c.n_embd)
             if src_h == 0:        # the binding reports a failed gather as handle 0, like the reference's
@@ -856,9 +852,9 @@ class DecodeEngine:
             fn(ws, self._map_of[name], C1[src], self._wh[name], C1[dst], m, K, N)
 
         g.batch_begin()
-        if from_device:
-            g.embed_tokens_dev(ws, feed['src'][0], feed['tok_hs'][m], feed['src'][1], self._cp['hidden'], m, E, c.n_vocab,
-                               float(c.emb_scale))
+        if from_device:     # (the same launch hands the tokens to the host: _wait_tokens(self._feed_ticket, m))
+            self._feed_ticket = g.embed_post_tokens_dev(ws, feed['src'][0], feed['tok_hs'][m], feed['src'][1],
+                                                        self._cp['hidden'], m, E, c.n_vocab, float(c.emb_scale))
         elif self._tied:
             src_h, _, _, _ = g.map_gather_dev(self._map_of[self._lm_name], emb_h, m * E)
             g.map_scatter_dev(ws, CS['hidden'], m * E, src_h)
@@ -992,12 +988,9 @@ class DecodeEngine:
             for sq in range(B):
                 out[sq].append(cur[sq])
             self._forward_chunk(cur, P, lockstep=True)
-            ticket = self._post_token(B)
             for step in range(1, max_tokens):
                 self._forward_chunk(None, P + step, lockstep=True, from_device=True)
-                nxt = self._post_token(B)
-                cur = self._wait_tokens(ticket, B)
-                ticket = nxt
+                cur = self._wait_tokens(self._feed_ticket, B)      # the tokens that step consumes
                 for sq in range(B):
                     out[sq].append(cur[sq])
         for step in range(0 if not ahead else max_tokens, max_tokens):
@@ -1058,13 +1051,10 @@ class DecodeEngine:
             # One step of lookahead: the step that consumes token n takes it from the device slot and is issued
             # before the host has seen token n; the host reads every token, in order, one issue late.  A stop token
             # is therefore noticed after one step too many was issued (its KV row is never read).
-            ticket = self._post_token()
             for step in range(config.max_tokens):
                 t0 = time.perf_counter()
                 self._forward(None, len(token_ids) + step, from_device=True)
-                nxt = self._post_token()
-                nt = self._wait_tokens(ticket)[0]
-                ticket = nxt
+                nt = self._wait_tokens(self._feed_ticket)[0]       # the token that step consumes
                 if nt in config.eos_token_ids:
                     break
                 out.append(nt)

@@ -328,27 +328,24 @@ def measure_decode(gpu, A, DecodeEngine, cfg, tensors, prompt, steps, warmup, sc
     prefill_s = time.perf_counter() - t0
     tokens, pos = [], n_prompt
 
-    def run(n, ticket):
+    def run(n):
         nonlocal pos
         for _ in range(n):
             if lookahead:
                 eng._forward(None, pos, from_device=True)
-                nxt = eng._post_token()
-                nt = eng._wait_tokens(ticket)[0]
-                ticket = nxt
+                nt = eng._wait_tokens(eng._feed_ticket)[0]      # the token that step consumes
             else:
                 nt = eng.read_token()
                 eng._forward(nt, pos)
             tokens.append(nt)
             pos += 1
-        return ticket
 
-    ticket = run(warmup, eng._post_token() if lookahead else 0)
+    run(warmup)
     gpu.sync()
     gpu.reset_native_stats()
     gpu.timer_begin()
     t0 = time.perf_counter()
-    run(steps, ticket)
+    run(steps)
     gpu.sync()
     wall = time.perf_counter() - t0
     dev_ms = gpu.timer_end()

@@ -275,6 +275,11 @@ int adamah_hip_embed_tokens_dev(uint32_t map_act, uint32_t map_src, uint32_t loc
  * still read every token in order.  Returns ADAMAH_ERR_NOT_FOUND when the stream has drained and the ticket is not
  * there (never posted, or its slot taken by the post 8 tickets later). */
 int adamah_hip_token_post(uint32_t map_id, uint32_t locs_handle, uint32_t n, uint32_t* ticket);
+/* embed_post_tokens: embed_tokens and, in the same launch, token_post of the m <= 62 token values it reads (the
+ * ticket comes back in *ticket): a loop that runs one step ahead then needs no launch of its own to hand step n's
+ * token to the host -- the embedding launch of step n + 1 does it. */
+int adamah_hip_embed_post_tokens_dev(uint32_t map_act, uint32_t map_src, uint32_t locs_tokens, uint32_t src_row0,
+                                     uint32_t dst_start, uint32_t m, uint32_t E, uint32_t V, float scale, uint32_t* ticket);
 int adamah_hip_token_wait(uint32_t ticket, float* out, uint32_t n);
 /* ---- measurement and test helpers: not part of the op surface ------------------------------------
  * Nothing a model engine calls.  bench.py times launches with the stopwatch and calibrates profiler counters

@@ -64,6 +64,13 @@ def test_embed_tokens_matches_the_host_lookup(hip, kind, V, E, m, scale):
         want = table[toks] * np.float32(scale)
         assert np.array_equal(got, want)
         assert np.all(read(g, ACT, 0, 10) == 7.0)
+        # the form that also hands the token values to the host: same rows, and the tokens under its ticket
+        put(g, ACT, dst, np.zeros(m * E, np.float32))
+        g.batch_begin()
+        ticket = g.embed_post_tokens_dev(ACT, SRC, h, row0, dst, m, E, V, scale)
+        g.batch_end()
+        assert g.token_wait(ticket, m).tolist() == [float(t) for t in toks]
+        assert np.array_equal(read(g, ACT, dst, m * E).reshape(m, E), want)
     # the library's own three-op path leaves the same bits
     locs = (row0 + toks[:, None] * E + np.arange(E)[None, :]).astype(np.uint32).reshape(-1)
     lh = up(g, locs)
