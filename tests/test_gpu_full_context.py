@@ -71,6 +71,17 @@ def test_llama3_8b_shape_decode_step_at_position_4095(hip):
     preload_kv(eng2, cpu2, 4095, seed=7)
     eng2._forward(tok, 4095)
     check_step(eng2.read_slot('hidden'), device_logits(eng2), eng2.read_token(), cpu, cpu_logits)
+    # the next step fed from the device (the token the LM head just left in its slot, its embedding row gathered
+    # from the table on the device, the token handed to the host by that launch) against the same step fed from the
+    # host: same token reported, same hidden state, same choice
+    nt = eng2.read_token()
+    note("the step at position 4096 fed from the device")
+    eng2._forward(None, 4096, from_device=True)
+    assert eng2._wait_tokens(eng2._feed_ticket) == [nt]
+    h_dev, t_dev = eng2.read_slot('hidden'), eng2.read_token()
+    eng2._forward(nt, 4096)
+    assert np.array_equal(h_dev, eng2.read_slot('hidden'))
+    assert t_dev == eng2.read_token()
 
 
 def test_llama3_8b_shape_chunk_of_512_rows_and_16_sequences_in_lockstep(hip):
