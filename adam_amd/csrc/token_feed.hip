@@ -173,7 +173,9 @@ int adamah_hip_token_post(uint32_t map_id, uint32_t locs_handle, uint32_t n, uin
   return check_launch();
 }
 
-int adamah_hip_token_wait(uint32_t ticket, float* out, uint32_t n) { ADAMAH_API();
+// (no launch of queued ops here: a post is launched by its own call, so the ticket never depends on the queue, and a
+// caller may wait in the middle of a batch without breaking up the folds of the ops it has queued so far)
+int adamah_hip_token_wait(uint32_t ticket, float* out, uint32_t n) {
   if (!g_mail || !out || n == 0 || n > MAIL_MAX || ticket == 0 || ticket > 0x7FFFFFFFu) return ADAMAH_ERR_INVALID;
   TokenMail* s = g_mail + ticket % MAIL_SLOTS;
   for (uint32_t spins = 1;; spins++) {

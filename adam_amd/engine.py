@@ -601,10 +601,12 @@ class DecodeEngine:
         return [int(t) for t in self.gpu.token_wait(ticket, m)]
 
     # ------------------------------------------------------------------ forward
-    def _forward(self, tok, pos, sample=True, sample_cfg=None, sample_prev=(), from_device=False):
+    def _forward(self, tok, pos, sample=True, sample_cfg=None, sample_prev=(), from_device=False, on_token=None):
         """One decode step; op order of reference engine.py:2971-3402 (default discrete-GPU path).
         `from_device`: the input token is the one the previous step's LM head left in the token slot (`tok` is
-        not looked at); its embedding row is gathered on the device."""
+        not looked at); its embedding row is gathered on the device.  `on_token` (with `from_device`): called with
+        that token once it has reached the host -- after the layers have been issued, before the LM head's ops are
+        (their repeat-penalty list may depend on it); returning False ends the step there."""
         c, g, A, ws = self.cfg, self.gpu, self.A, self.WS_MAP
         q_dim, k_dim = c.n_head * c.head_dim, c.n_head_kv * c.head_dim_kv
         seq_len = pos + 1
@@ -692,6 +694,9 @@ class DecodeEngine:
             self._rms(hid_h, 'output_norm.weight', normed_h, 1, c.n_embd)
         else:
             g.decode_step(self._plan_id, pos, seq_len)
+        if from_device and on_token is not None and not on_token(self._wait_tokens(self._feed_ticket)[0]):
+            g.batch_end()
+            return
         if sample and sample_cfg is not None and sample_cfg.temperature > 0.0 and sample_cfg.top_k > 1:
             self._sample_fused_topk(sample_cfg, sample_prev, normed_h)
         elif sample:
@@ -1032,8 +1037,7 @@ class DecodeEngine:
         self.reset()
         sampled = config.temperature > 0.0 and config.top_k > 1
         # (the device-side embedding table of an untied model is filled on first use: before the clock starts)
-        ahead = (not sampled and forced is None and self._lookahead and config.max_tokens > 0
-                 and self._token_feed() is not None)
+        ahead = (forced is None and self._lookahead and config.max_tokens > 0 and self._token_feed() is not None)
         self._rng = np.random.default_rng(config.seed)
         hist = [int(t) for t in token_ids]
         tp = time.perf_counter()
@@ -1047,7 +1051,25 @@ class DecodeEngine:
         t_pre = time.perf_counter() - tp
         out, ttimes = [], []
         td = time.perf_counter()
-        if ahead:
+        if ahead and sampled:
+            # Sampled decoding one step ahead: the layers of the step that consumes token n are issued at once (the
+            # token's embedding row is gathered on the device); the host reads token n while they run, builds the
+            # repeat-penalty list that includes it and only then issues the step's LM head and sampling ops.
+            def seen(nt):
+                if nt in config.eos_token_ids:
+                    return False
+                out.append(nt)
+                hist.append(nt)
+                return True
+            for step in range(config.max_tokens):
+                t0 = time.perf_counter()
+                n_before = len(out)
+                self._forward(None, len(token_ids) + step, sample=True, sample_cfg=config, sample_prev=hist,
+                              from_device=True, on_token=seen)
+                if len(out) == n_before:
+                    break
+                ttimes.append(time.perf_counter() - t0)
+        elif ahead:
             # One step of lookahead: the step that consumes token n takes it from the device slot and is issued
             # before the host has seen token n; the host reads every token, in order, one issue late.  A stop token
             # is therefore noticed after one step too many was issued (its KV row is never read).

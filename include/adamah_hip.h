@@ -272,7 +272,7 @@ int adamah_hip_embed_tokens_dev(uint32_t map_act, uint32_t map_src, uint32_t loc
  * (1, 2, 3, ...: the library hands every ticket out once; slot = ticket % 8).
  * token_wait: poll the ticket's slot until it carries `ticket`, then copy its first n values to out.  It neither
  * synchronises the stream nor waits for work queued behind the post, so a caller can issue the next step first and
- * still read every token in order.  Returns ADAMAH_ERR_NOT_FOUND when the stream has drained and the ticket is not
+ * still read every token in order; ops queued in an open batch stay queued.  Returns ADAMAH_ERR_NOT_FOUND when the stream has drained and the ticket is not
  * there (never posted, or its slot taken by the post 8 tickets later). */
 int adamah_hip_token_post(uint32_t map_id, uint32_t locs_handle, uint32_t n, uint32_t* ticket);
 /* embed_post_tokens: embed_tokens and, in the same launch, token_post of the m <= 62 token values it reads (the

@@ -15,12 +15,19 @@ def pair(hip):
     return [hip, oracle.init()]
 
 
-@pytest.mark.parametrize("n,k,seed", [(6, 3, 0), (100, 64, 1), (262144, 8, 2), (1000, 40, 3), (5, 9, 4), (257, 1, 5)])
+# 4096 < n <= 40960 takes the selection kernel (one launch), everything else the rounds: sizes on both sides of both
+# limits, the sampled LM head's 1024 lists of 40, a list with more ties than k at the k-th value
+@pytest.mark.parametrize("n,k,seed", [(6, 3, 0), (100, 64, 1), (262144, 8, 2), (1000, 40, 3), (5, 9, 4), (257, 1, 5),
+                                      (4096, 40, 6), (4097, 40, 7), (40960, 40, 8), (40961, 40, 9), (12345, 64, 10),
+                                      (30000, 1, 11), (8000, 33, 12)])
 def test_topk(hip, n, k, seed):
     rng = np.random.default_rng(seed)
     v = (rng.integers(-50, 50, n) / 4).astype(np.float32)         # ties on purpose
     if n > 8:
         v[rng.integers(0, n, 3)] = np.nan
+    if seed == 12:
+        v[:] = np.float32(1.5)                                     # every candidate ties: the lowest indices win
+        v[7000] = np.float32(2.0)
     outs = []
     for g in pair(hip):
         note(f"topk n={n} k={k}")
