@@ -260,34 +260,45 @@ k_topp(float* data, const uint32_t* __restrict__ ls, const uint32_t* __restrict_
     lg[tid] = v;
   }
   __syncthreads();
-  if (tid != 0) return;
+  // One lane per candidate for the exponentials, the divisions and the stores; the sums run over the candidates in
+  // order in lane 0, as the reference's single invocation adds them up (same values, same order, same bits).
+  __shared__ float s_sum, s_ks;
+  __shared__ uint32_t s_keep;
   auto put = [&](uint32_t i, float v) { if (ld[i] < n_elems) data[ld[i]] = v; };
   const float temp = fmaxf(temperature, 1e-6f);
   const float keep_p = fminf(fmaxf(top_p, 0.f), 1.f);
-  float mx = SMP_NEG_INF;
-  for (uint32_t i = 0; i < n; i++) if (lg[i] > mx) mx = lg[i];
-  if (mx == SMP_NEG_INF) { for (uint32_t i = 0; i < n; i++) put(i, 0.f); return; }
-  float sum = 0.f;
-  for (uint32_t i = 0; i < n; i++) {
-    if (lg[i] == SMP_NEG_INF) { pr[i] = 0.f; continue; }
-    const float p = expf((lg[i] - mx) / temp);
-    pr[i] = p;
-    sum += p;
+  float mx = lg[tid];
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  if (mx == SMP_NEG_INF) { if (tid < n) put(tid, 0.f); return; }
+  if (tid < n) pr[tid] = lg[tid] == SMP_NEG_INF ? 0.f : expf((lg[tid] - mx) / temp);
+  __syncthreads();
+  if (tid == 0) {
+    float sum = 0.f;
+    for (uint32_t i = 0; i < n; i++) if (lg[i] != SMP_NEG_INF) sum += pr[i];
+    s_sum = sum;
   }
-  if (sum <= 0.f) { for (uint32_t i = 0; i < n; i++) put(i, i == 0 ? 1.f : 0.f); return; }
-  for (uint32_t i = 0; i < n; i++) pr[i] /= sum;
-  uint32_t keep = 0;
-  float csum = 0.f;
-  for (uint32_t i = 0; i < n; i++) {
-    csum += pr[i];
-    keep = i + 1;
-    if (keep_p >= 0.999999f || csum >= keep_p) break;
+  __syncthreads();
+  const float sum = s_sum;
+  if (sum <= 0.f) { if (tid < n) put(tid, tid == 0 ? 1.f : 0.f); return; }
+  if (tid < n) pr[tid] /= sum;
+  __syncthreads();
+  if (tid == 0) {
+    uint32_t keep = 0;
+    float csum = 0.f;
+    for (uint32_t i = 0; i < n; i++) {
+      csum += pr[i];
+      keep = i + 1;
+      if (keep_p >= 0.999999f || csum >= keep_p) break;
+    }
+    if (keep == 0 && n > 0) keep = 1;
+    float ks = 0.f;
+    for (uint32_t i = 0; i < keep; i++) ks += pr[i];
+    if (ks <= 0.f) ks = 1.f;
+    s_keep = keep; s_ks = ks;
   }
-  if (keep == 0 && n > 0) keep = 1;
-  float ks = 0.f;
-  for (uint32_t i = 0; i < keep; i++) ks += pr[i];
-  if (ks <= 0.f) ks = 1.f;
-  for (uint32_t i = 0; i < n; i++) put(i, i < keep ? pr[i] / ks : 0.f);
+  __syncthreads();
+  if (tid < n) put(tid, tid < s_keep ? pr[tid] / s_ks : 0.f);
 }
 
 // dst[i] = data[base + uint(data[sel[i]])]  (candidate position -> token id), negatives / non-finite -> 0
@@ -308,16 +319,22 @@ k_resolve_idx(float* data, const uint32_t* __restrict__ lbase, const uint32_t* _
 __global__ void __launch_bounds__(64)
 k_sample_categorical(float* data, const uint32_t* __restrict__ lidx, const uint32_t* __restrict__ lprob,
                      const uint32_t* __restrict__ lrand, const uint32_t* __restrict__ ldst, uint32_t n, uint64_t n_elems) {
-  if (threadIdx.x != 0 || n == 0) return;
-  auto prob = [&](uint32_t i) {
-    float p = lprob[i] < n_elems ? data[lprob[i]] : 0.f;
+  // the probabilities come in with one load per lane; the sums run over them in order in lane 0 (same bits as a
+  // single invocation that reads them one after the other)
+  __shared__ float ps[SMP_MAX];
+  const uint32_t tid = threadIdx.x;
+  if (n == 0) return;
+  if (tid < n) {
+    float p = lprob[tid] < n_elems ? data[lprob[tid]] : 0.f;
     if (isnan(p) || isinf(p) || p < 0.f) p = 0.f;
-    return p;
-  };
+    ps[tid] = p;
+  }
+  __syncthreads();
+  if (tid != 0) return;
   auto idx = [&](uint32_t i) { return lidx[i] < n_elems ? data[lidx[i]] : 0.f; };
   if (ldst[0] >= n_elems) return;
   float total = 0.f;
-  for (uint32_t i = 0; i < n; i++) total += prob(i);
+  for (uint32_t i = 0; i < n; i++) total += ps[i];
   if (!(total > 0.f)) { data[ldst[0]] = idx(0); return; }
   float r = lrand[0] < n_elems ? data[lrand[0]] : 0.f;
   if (isnan(r) || isinf(r)) r = 0.f;
@@ -326,7 +343,7 @@ k_sample_categorical(float* data, const uint32_t* __restrict__ lidx, const uint3
   float acc = 0.f;
   uint32_t chosen = n - 1;
   for (uint32_t i = 0; i < n; i++) {
-    acc += prob(i);
+    acc += ps[i];
     if (target < acc) { chosen = i; break; }
   }
   data[ldst[0]] = idx(chosen);
