@@ -159,7 +159,12 @@ def test_greedy_loops_one_step_ahead_give_the_same_tokens(hip, arch):
         stop = one[7]
         cut, _ = eng.generate(prompt, GenerationConfig(max_tokens=40, eos_token_ids=(stop,)))
         many, _ = eng.generate_batch(prompts, 24)
-        res[la] = (one, again, cut, many)
+        gc = GenerationConfig(max_tokens=24, temperature=2.0, top_k=40, top_p=0.95, repeat_penalty=1.3, seed=5)
+        drawn, _ = eng.generate(prompt, gc)          # sampled: the layers run ahead, the LM head waits for the token
+        drawn_cut, _ = eng.generate(prompt, GenerationConfig(max_tokens=24, temperature=2.0, top_k=40, top_p=0.95,
+                                                             repeat_penalty=1.3, seed=5, eos_token_ids=(drawn[5],)))
+        assert drawn_cut == drawn[:drawn.index(drawn[5])]
+        res[la] = (one, again, cut, many, drawn)
         assert st["n_gen"] == 40
         assert cut == one[:one.index(stop)]
         del eng
