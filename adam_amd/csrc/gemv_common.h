@@ -167,5 +167,8 @@ bool block_path_ok(const Map* ma, const Map* mw, uint32_t ha, uint32_t hb, uint3
                    uint64_t* b_out);
 // Storage format (FMT_*) of the weights [b, b + n_w) of a quantised map.
 int fmt_of(const Map* mw, uint64_t b, uint64_t n_w);
+// gemv_q.hip: the block-layout GEMV (Q4 or Q8) with the result rows in `out`, device memory outside the maps
+int launch_block_store_to(int fmt, const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb, uint32_t K,
+                          uint32_t N, float* out);
 
 }  // namespace adamah

@@ -250,6 +250,11 @@ static int op_matvec_topk(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uin
       tuning("ADAMAH_GEMV_IMPL", 3) == 3) {
     r = launch_mfma_store(fmt_of(mw, b0, (uint64_t)N * K), ma, mw, (uint32_t)a0, (uint32_t)b0, 0u, K, N, nullptr,
                           logits);
+  } else if (block_path_ok(ma, mw, ha, hb, K, N, &a0, &b0) && (uint64_t)K * 4 + (K >> 5) * 4 <= 64000 &&
+             tuning("ADAMAH_TOPK_BLOCK", 1) != 0) {
+    // block layout without the matrix-instruction kernel (Q8_0 LM heads): the fp32 block GEMV, 5-6 x the rate of
+    // the one-wave-per-row kernel below (128256 x 4096 Q8_0: 637 -> 100 us)
+    r = launch_block_store_to(fmt_of(mw, b0, (uint64_t)N * K), ma, mw, la, lb, K, N, logits);
   } else {
     if (dtype == DTYPE_Q4)
       k_matvec_rows<true><<<cdiv(N, 4), 256, 0, g.stream>>>(act, mw->buf, mw->qp, la, lb, logits, K, N,
