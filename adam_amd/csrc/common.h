@@ -94,6 +94,8 @@ struct Stats {
   uint32_t last_batch_dispatch = 0;
 };
 
+enum : uint32_t { ZERO_WORD = 64 };   // index into Ctx::sync_ctr
+
 struct PlanOp {  // mirrors DecodePlanOp (adamah.c:175-194)
   uint32_t kind, map_id, map_id2, op_code, h0, h1, h2, h3, h4, h5, u0, u1, u2, u3, u4, u5;
   float f0, f1;
@@ -132,7 +134,8 @@ struct Ctx {
   std::vector<PendOp> pend;
   int no_defer = 0;              // > 0 while an entry point runs on library-owned scratch handles
   uint64_t mem_gen = 0;          // counts host-to-device copies (with stats.dispatch: "has device memory changed?")
-  uint32_t* sync_ctr = nullptr;  // device counters for last-workgroup epilogues, zero between launches
+  uint32_t* sync_ctr = nullptr;  // device counters for last-workgroup epilogues, zero between launches (word 0 in use);
+                                 // word ZERO_WORD is cleared at init and never written: a constant zero for kernels
   float* t_park = nullptr;       // T_PARK_FLOATS floats: a row on its way to a place that is still being read
   int deferred_err = 0;          // first failure of a queued op's launch; returned (once) by the next call that can
   uint64_t layout_gen = 0;       // counts events after which device pointers or offsets seen earlier may be stale:

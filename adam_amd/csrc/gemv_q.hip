@@ -663,8 +663,8 @@ int op_matvec_argmax(uint32_t dtype, uint32_t map_act, uint32_t map_wt, uint32_t
 // A queued Q8 GEMV + argmax that did not join a run: the float32 block kernels, as when launched at once.
 // The block-layout GEMV with its result rows written to `out` (device memory outside the maps: the scratch logits of
 // the GEMV + top-k ops) instead of a range of the activation map.  The kernel adds the row number to the word behind
-// `lc`: the first of the zero-initialised launch counters serves as that word (it is zero whenever no launch is in
-// flight on the stream).
+// `lc`: a word of the zero-initialised counter block that no kernel ever writes (ZERO_WORD; the ticket counter of the
+// GEMV prologues is word 0 of that block) serves as that word.
 int launch_block_store_to(int fmt, const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb, uint32_t K,
                           uint32_t N, float* out) {
   const size_t smem = (size_t)K * 4 + (size_t)(K >> 5) * 4;
@@ -673,7 +673,7 @@ int launch_block_store_to(int fmt, const Map* ma, const Map* mw, const uint32_t*
   const uint32_t per_cu = (uint32_t)knob("ADAMAH_GEMV_PERCU", smem > 40000 ? 2 : 4);
   const uint32_t grid = std::min<uint32_t>(n_groups, (uint32_t)g.n_cu * per_cu);
   const float* act = (const float*)ma->buf;
-  const uint32_t* zero = (const uint32_t*)g.sync_ctr;
+  const uint32_t* zero = (const uint32_t*)g.sync_ctr + ZERO_WORD;
 #define LAUNCH(F)                                                                                                \
   k_gemv_block<F, EPI_STORE, 4><<<grid, 256, smem, g.stream>>>(act, out, mw->buf, mw->qp, mw->d16, la, lb, zero, nullptr, \
                                                               nullptr, K, N, rpg, n_groups)

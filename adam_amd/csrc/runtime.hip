@@ -91,12 +91,22 @@ uint32_t res_alloc(uint32_t n_bytes) {
   return id;
 }
 
-// map_gather_dev results in the order they were made.  Once more than GATHER_RING of them, or more than
-// GATHER_BYTES of their storage, are live, the oldest is handed out again (same id, same storage).
-enum : size_t { GATHER_RING = 4096, GATHER_BYTES = (size_t)256 << 20 };
-static std::deque<uint32_t> g_gather_ring;
-static size_t g_gather_bytes = 0;
-static void gather_ring_reset() { g_gather_ring.clear(); g_gather_bytes = 0; }
+// map_gather_dev results, one ring per size class (storage rounded up to a power of two, 256 B at least), each in
+// the order the results were made.  Once a class holds gather_class_limit() results its oldest is handed out again
+// (same id, same storage), so ids and arena bytes stay bounded whatever sizes a caller alternates between: a class
+// keeps at most 64 MiB (two results for the classes above 32 MiB) and at most 4096 results.
+enum : uint32_t { GATHER_CLASSES = 33, GATHER_MIN_LOG2 = 8 };
+static std::deque<uint32_t> g_gather_ring[GATHER_CLASSES];
+static inline uint32_t gather_class(uint32_t need) {
+  uint32_t c = GATHER_MIN_LOG2;
+  while (c < 32 && ((uint64_t)1 << c) < need) ++c;
+  return c;
+}
+static inline size_t gather_class_limit(uint32_t c) {
+  const uint64_t n = ((uint64_t)64 << 20) >> c;
+  return (size_t)(n < 2 ? 2 : n > 4096 ? 4096 : n);
+}
+static void gather_ring_reset() { for (auto& r : g_gather_ring) r.clear(); }
 
 // Remember what was uploaded into a handle, and whether it is a run of consecutive indices.
 static void note_host(Res* r, const void* data, uint32_t n_bytes) {
@@ -724,24 +734,28 @@ uint64_t map_gather_dev(uint32_t map_id, uint32_t locs_handle, uint32_t n_locs) 
   uint64_t n_vals = (uint64_t)n_locs * m->pack_size;
   if (n_vals * 4 > 0xFFFFFFFFull) return 0;
   // Results are never released individually (as in the reference, whose table ends after 2048).  A decode loop
-  // gathers one embedding row per token, so only the latest results are kept: the storage and id of the oldest
-  // is handed out again when it is large enough, and handles and arena stop growing.
+  // gathers one embedding row per token and a chunked prefill a block of rows per chunk, so only the latest results
+  // of a size class are kept: the storage and id of the class's oldest is handed out again, and handles and arena
+  // stop growing.  A caller that still holds the id of a result older than the class limit sees the newer contents.
   const uint32_t need = (uint32_t)(n_vals * 4);
+  const uint32_t cls = gather_class(need);
+  std::deque<uint32_t>& ring = g_gather_ring[cls];
   uint32_t id = 0;
-  if (g_gather_ring.size() >= GATHER_RING || g_gather_bytes + need > GATHER_BYTES) {
-    Res* old = get_res(g_gather_ring.empty() ? 0u : g_gather_ring.front());
+  if (ring.size() >= gather_class_limit(cls)) {
+    Res* old = get_res(ring.front());
     if (old && old->cap_bytes >= need) {
-      id = g_gather_ring.front();
-      g_gather_ring.pop_front();
+      id = ring.front();
       old->size_bytes = need; old->host.clear(); old->host_valid = false; old->contig = false;
     }
+    ring.pop_front();
   }
   if (id == 0) {
-    id = res_alloc(need);
+    const uint64_t cap = (uint64_t)1 << cls;
+    id = res_alloc(cap > 0xFFFFFFFFull ? need : (uint32_t)cap);
     if (id == 0) return 0;
-    g_gather_bytes += g.res[id].cap_bytes;
+    g.res[id].size_bytes = need;
   }
-  g_gather_ring.push_back(id);
+  ring.push_back(id);
   float* dst = (float*)g.res[id].dptr;
   if (m->dtype == DTYPE_F32)
     k_gather_f32<<<cdiv(n_vals, 256), 256, 0, g.stream>>>((const float*)m->buf, dst, locs, n_locs, m->pack_size,
@@ -972,8 +986,10 @@ int adamah_decode_step(uint32_t plan_id, uint32_t pos, uint32_t seq_len) {
     flush_pending();                                 // what was queued before the plan runs ahead of it
     if (pg.ready && pg.gen != g.layout_gen) pg.ready = false;   // a map or scratch buffer moved since the recording
     if (pg.handles.empty()) {
-      for (const PlanOp& op : g.plans[plan_id])
+      for (const PlanOp& op : g.plans[plan_id]) {
         for (uint32_t h : {op.h0, op.h1, op.h2, op.h3, op.h4, op.h5}) if (h) pg.handles.push_back(h);
+        if ((op.kind == 26 || op.kind == 28) && op.u0) pg.handles.push_back(op.u0);   // their seventh handle
+      }
       std::sort(pg.handles.begin(), pg.handles.end());
       pg.handles.erase(std::unique(pg.handles.begin(), pg.handles.end()), pg.handles.end());
     }

@@ -104,6 +104,8 @@ class DecodeEngine:
         # previous step left there, tokens handed to the host through the library's ring): set up on first use.
         self._lookahead = bool(lookahead) and getattr(gpu, '_has_token_feed', False)
         self._feed = None
+        self.feed_table_bytes = 0          # device bytes of the float32 embedding table of an untied model's token feed
+        self.feed_table_upload_s = 0.0
         self._feed_ticket = 0
         # The per-token op list is the same every step except for pos / seq_len, so it is registered
         # once as a native decode plan (reference API adamah.c:10341-10398) and replayed with one call.
@@ -585,13 +587,21 @@ class DecodeEngine:
             if self.EMB_MAP in self._q4_sizes or c.n_vocab * c.n_embd > self._q4_limit:
                 self._feed = False
                 return None
-            g.set_dtype(A.DTYPE_F32)
-            g.map_create(self.EMB_MAP, 1, c.n_vocab * c.n_embd)
-            step = max(1, (1 << 24) // c.n_embd)
-            for lo in range(0, c.n_vocab, step):
-                hi = min(c.n_vocab, lo + step)
-                rows = emb.rows(lo, hi) if hasattr(emb, 'rows') else np.stack([emb.row(t) for t in range(lo, hi)])
-                g.scatter_contiguous(self.EMB_MAP, lo * c.n_embd, np.ascontiguousarray(rows, np.float32).reshape(-1))
+            t0 = time.perf_counter()
+            try:
+                g.set_dtype(A.DTYPE_F32)
+                g.map_create(self.EMB_MAP, 1, c.n_vocab * c.n_embd)
+                step = max(1, (1 << 24) // c.n_embd)
+                for lo in range(0, c.n_vocab, step):
+                    hi = min(c.n_vocab, lo + step)
+                    rows = emb.rows(lo, hi) if hasattr(emb, 'rows') else np.stack([emb.row(t) for t in range(lo, hi)])
+                    g.scatter_contiguous(self.EMB_MAP, lo * c.n_embd, np.ascontiguousarray(rows, np.float32).reshape(-1))
+            except (RuntimeError, MemoryError):
+                # no room for the table (or the upload failed): the loops fall back to the host lookup per token
+                self._feed = False
+                return None
+            self.feed_table_bytes = 4 * c.n_vocab * c.n_embd
+            self.feed_table_upload_s = time.perf_counter() - t0
             src = (self.EMB_MAP, 0)
         self._feed = {'src': src, 'tok_h': self._up(self._sample_locs),
                       'tok_hs': {self._batch: self._up(self._c_tok_locs[:self._batch])} if self._batch > 1 else {}}

@@ -154,10 +154,13 @@ def from_gguf_q4_k(raw, shape):
     return QTensor('q4_aff', tuple(shape), None, (c[0::2] | (c[1::2] << 4)).astype(np.uint8), scale, zp)
 
 
-def from_gguf_q5_0(raw, shape):
+def from_gguf_q5_0(raw, shape, clip=True):
     """GGUF Q5_0 bytes (22 B/block: fp16 d, 32 high bits, 16 nibble bytes; w = d (q - 16), q = nibble | bit << 4)
-    -> QTensor 'q8_0': the reference keeps such tensors in the 8-bit map with scale |d| and the signed 5-bit
-    value (times the sign of d) as code (adam/models/engine.py:1171-1179), which is exact.  A block with d = 0
+    -> QTensor 'q8_0': the reference keeps such tensors in the 8-bit map with scale |d| and, as code, the signed
+    5-bit value times the sign of d.  Its default path gets there by rounding w / |d| and clipping to [-16, 15]
+    (adam/models/engine.py:1171-1179): exact except for q = 0 in a block with d < 0, whose value +16 is stored as
+    15.  `clip=True` (default) gives those codes; `clip=False` keeps +16, which is what the reference's raw decode
+    stores (engine.py:1155-1169, taken on one device family only) and is exact for every block.  A block with d = 0
     gets scale 1 and codes 0, as there."""
     n = int(shape[0]) * int(shape[1])
     nb = n // QK
@@ -169,6 +172,8 @@ def from_gguf_q5_0(raw, shape):
     hi = ((qh[:, None] >> np.arange(32, dtype=np.uint32)[None, :]) & 1).astype(np.int16)
     q = (lo | (hi << 4)) - 16
     q = q * np.where(d < 0, -1, 1).astype(np.int16)[:, None]
+    if clip:
+        q = q.clip(-16, 15)
     q[d == 0] = 0
     scale = np.where(d != 0, np.abs(d), np.float32(1.0)).astype(np.float16)
     return QTensor('q8_0', tuple(shape), scale, (q + 128).astype(np.uint8).reshape(-1))

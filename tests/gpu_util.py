@@ -58,3 +58,13 @@ def load_qtensor(g, mid, qt, offset=0, total=None, scale=None, zp=None):
         g.scatter_q4_packed_contiguous(mid, offset, qt.codes, n_locs=n)
     else:
         g.scatter_contiguous(mid, offset, qt.codes)
+
+
+def device_free_bytes():
+    """Free device memory as the HIP runtime reports it (hipMemGetInfo); used to show that a call allocates nothing."""
+    import ctypes
+    rt = ctypes.CDLL("libamdhip64.so")
+    free, total = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    rc = rt.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total))
+    assert rc == 0, f"hipMemGetInfo returned {rc}"
+    return free.value

@@ -16,7 +16,7 @@ import pytest
 import oracle
 from oracle.forward_cpu import CpuModel
 from adam_amd import adamah as A
-from adam_amd import gguf
+from adam_amd import gguf, quant
 from adam_amd.engine import DecodeEngine, GenerationConfig
 from adam_amd.quant import QTensor
 
@@ -350,8 +350,22 @@ def test_q5_0_q6_k_bf16_decoders_and_requantised_upload(tmp_path):
                 ("blk.0.e.weight", (4, 32), gguf.GGML_F32, f32.tobytes()), ("blk.0.n.weight", (128,), gguf.GGML_BF16, bf.tobytes())])
     f = gguf.GGUFFile(str(p))
     t5 = f.tensor("blk.0.a.weight")
-    assert t5.kind == 'q8_0' and np.array_equal(t5.dequant().reshape(-1), dec_q5_0(r5))    # equal as numbers (a d = 0
-    # block gives -0.0 for negative codes in the ggml form, +0.0 here)
+    # default: the codes of the reference's default path, round(w / |d|) clipped to [-16, 15] (engine.py:1171-1179) --
+    # the ggml values except for q = 0 under a negative d, whose +16 becomes 15
+    w5 = dec_q5_0(r5).reshape(-1, 32)
+    d5 = np.abs(np.frombuffer(r5, np.uint8).reshape(-1, 22)[:, 0:2].copy().view(np.float16).astype(np.float32).reshape(-1))
+    d5 = np.where(d5 > 0, d5, np.float32(1.0))
+    ref_codes = np.round(w5 / d5[:, None]).astype(np.int16).clip(-16, 15)
+    assert t5.kind == 'q8_0' and np.array_equal(t5.codes.reshape(-1, 32).astype(np.int16) - 128, ref_codes)
+    assert np.array_equal(t5.d.astype(np.float32), d5)
+    neg = np.frombuffer(r5, np.uint8).reshape(-1, 22)[:, 0:2].copy().view(np.float16).reshape(-1) < 0
+    assert np.any((np.round(w5 / d5[:, None]) == 16)[neg]), "the fixture must hold a q = 0 under a negative d"
+    # clip=False: exact for every block -- equal to the ggml form as numbers (a d = 0 block gives -0.0 for negative
+    # codes in the ggml form, +0.0 here)
+    t5x = quant.from_gguf_q5_0(r5, (8, 64), clip=False)
+    assert np.array_equal(t5x.dequant().reshape(-1), dec_q5_0(r5))
+    differ = t5x.codes != t5.codes
+    assert np.array_equal(differ.reshape(-1, 32), np.round(w5 / d5[:, None]) == 16)
     assert np.array_equal(f.tensor("blk.0.b.weight").view(np.uint32).reshape(-1), dec_q6_k(r6).view(np.uint32))
     assert np.array_equal(f.tensor("blk.0.c.weight").view(np.uint32).reshape(-1), bf.astype(np.uint32) << 16)
     f.close()

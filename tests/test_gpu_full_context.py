@@ -84,6 +84,40 @@ def test_llama3_8b_shape_decode_step_at_position_4095(hip):
     assert t_dev == eng2.read_token()
 
 
+def _full_depth_step(hip, cfg, ctx, seed, tok):
+    """One decode step of the full-size model at position `ctx` over preloaded caches: from the decode plan (the
+    launches the benchmark times) and again with every op issued by itself, each against the reference forward."""
+    tensors = synth.make_model(cfg, seed=seed, sigma=0.02)
+    cpu = CpuModel(cfg, dequantised(tensors), kv_cap=ctx + 4, kv_fp16=True, acc64=False)
+    eng = DecodeEngine(hip, cfg, tensors, A=A, kv_cap=ctx + 4, kv_fp16=True, fusion_scheduler_mode="level_batched")
+    assert eng._plan_id is not None
+    preload_kv(eng, cpu, ctx, seed=seed + 4)
+    cpu_logits = cpu.forward(tok, ctx)
+    eng._forward(tok, ctx)
+    check_step(eng.read_slot('hidden'), device_logits(eng), eng.read_token(), cpu, cpu_logits)
+    plan_id, eng._plan_id = eng._plan_id, None          # the same step op by op (rows of position ctx written again)
+    try:
+        note("... the same step op by op")
+        eng._forward(tok, ctx)
+        check_step(eng.read_slot('hidden'), device_logits(eng), eng.read_token(), cpu, cpu_logits)
+    finally:
+        eng._plan_id = plan_id
+
+
+def test_llama3_8b_all_32_layers_at_position_4095(hip):
+    """BASELINE config 4 at full depth and full context together: 32 layers of slice merges over 4095 cached
+    positions, Q8_0 head over the whole vocabulary, one reference pass on the CPU."""
+    note("llama-3-8b shape, all 32 layers, bs=1 step at position 4095")
+    _full_depth_step(hip, synth.llama3_8b_config(), 4095, seed=6, tok=4321)
+
+
+def test_gemma3_1b_all_26_layers_at_position_639(hip):
+    """BASELINE config 2's last position (512-token prompt + 128 tokens): 26 layers, one KV head of 256, attention
+    soft-cap on, tied Q4_0 head over 262144 rows."""
+    note("gemma-3-1b shape, all 26 layers, bs=1 step at position 639")
+    _full_depth_step(hip, synth.gemma3_1b_config(), 639, seed=8, tok=98765)
+
+
 def test_llama3_8b_shape_chunk_of_512_rows_and_16_sequences_in_lockstep(hip):
     """BASELINE config 5 at full width, one layer: a 512-token prompt chunk (projections as [512, K] matmuls,
     one causal attention launch) against 512 token-by-token reference passes, then one lockstep step of 16

@@ -163,3 +163,43 @@ def test_fused_projection_kinds_in_a_decode_plan(hip):
         got[route] = res
     for d, p in zip(got["direct"], got["plan"]):
         assert np.any(d) and np.array_equal(d.view(np.uint32), p.view(np.uint32))
+
+
+@pytest.mark.parametrize("kind", ["q4", "q8"])
+def test_graph_of_a_fused_qkv_plan_is_dropped_when_its_seventh_handle_is_rewritten(hip, kind):
+    """The Q/K/V kinds keep the V result's handle in u0.  A graph recorded one step ahead holds that offset by
+    value, so re-uploading the handle between two steps must send the next step through the ordinary replay:
+    V lands at the new place from that step on, and the old place is no longer written."""
+    K, rows = 1152, (256, 64, 64)
+    x = np.random.default_rng(5).standard_normal(K).astype(np.float32)
+    qt, bases = stacked(kind, rows, K, 17)
+    load_qtensor(hip, 1, qt)
+    total = K + sum(rows) + rows[2] + 64
+    f32map(hip, 0, total, x)
+    cs = np.cumsum((K,) + rows)                    # Q, K, V results back to back; a second V place behind them
+    v_old, v_new = int(cs[2]), int(cs[3]) + 32
+    hb = [up(hip, [b]) for b in bases]
+    hq, hk, hv = up(hip, [int(cs[0])]), up(hip, [int(cs[1])]), up(hip, [v_old])
+    a = up(hip, [0])
+    kq = A.DECODE_OP_FUSED_QKV_T_XQ4 if kind == "q4" else A.DECODE_OP_FUSED_QKV_T_XQ8
+    hip.register_decode_plan(6, [A.DecodePlanOp(kind=kq, map_id=0, map_id2=1, h0=a, h1=hb[0], h2=hb[1], h3=hb[2], h4=hq,
+                                                h5=hk, u0=hv, u1=K, u2=rows[0], u3=rows[1], u4=rows[2])])
+    try:
+        want = None
+        for step in range(8):
+            note(f"fused qkv plan {kind}, step {step}")
+            if step == 4:
+                hip.upload_dev(np.array([v_new], np.uint32), handle=hv)
+            hip.scatter_contiguous(0, K, np.zeros(total - K, np.float32))
+            hip.decode_step(6, step, step + 1)
+            out = read(hip, 0, K, total - K)
+            v_at_old, v_at_new = out[v_old - K: v_old - K + rows[2]], out[v_new - K: v_new - K + rows[2]]
+            if want is None:
+                want = v_at_old.copy()
+                assert np.any(want)
+            if step < 4:
+                assert np.array_equal(v_at_old, want) and not np.any(v_at_new), step
+            else:
+                assert np.array_equal(v_at_new, want) and not np.any(v_at_old), step
+    finally:
+        hip.clear_decode_plan(6)

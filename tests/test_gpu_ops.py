@@ -5,7 +5,7 @@ import pytest
 import oracle
 from adam_amd import adamah as A
 from adam_amd import quant
-from gpu_util import note, up, f32map, put, read, rel_l2, load_qtensor
+from gpu_util import note, up, f32map, put, read, rel_l2, load_qtensor, device_free_bytes
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
@@ -329,6 +329,32 @@ def test_gather_dev_results_stop_consuming_handles(hip):
     assert 0 not in ids and len(ids) <= 4200
     last = hip.map_gather_dev(0, locs[2], n)[0]
     assert np.array_equal(hip.download_dev(last, n), np.arange(2 * n, 3 * n, dtype=np.float32))
+
+
+def test_gather_dev_results_of_alternating_sizes_stay_bounded(hip):
+    """A small result (one embedding row) and a large one (a prefill chunk's rows) asked for in turn, far past the
+    limits of the result rings: every size class hands its own oldest result out again, so neither the ids nor the
+    device memory behind them keep growing, and the results stay right."""
+    note("gather_dev size-class rings")
+    small, large = 64, 65536
+    f32map(hip, 0, large, np.arange(large, dtype=np.float32))
+    ls, ll = up(hip, np.arange(small)), up(hip, np.arange(large))
+    ids_s, ids_l = set(), set()
+    free_mid = None
+    for i in range(9000):
+        ids_s.add(hip.map_gather_dev(0, ls, small)[0])
+        if i % 2 == 0:
+            ids_l.add(hip.map_gather_dev(0, ll, large)[0])
+        if i == 6000:
+            hip.sync()
+            free_mid = device_free_bytes()       # both classes are past their limits here
+    hip.sync()
+    assert 0 not in ids_s and 0 not in ids_l and not (ids_s & ids_l)
+    assert len(ids_s) <= 4096 and len(ids_l) <= 256, (len(ids_s), len(ids_l))
+    assert device_free_bytes() >= free_mid, "the arena grew after both rings were full"
+    hs, hl = hip.map_gather_dev(0, ls, small)[0], hip.map_gather_dev(0, ll, large)[0]
+    assert np.array_equal(hip.download_dev(hs, small), np.arange(small, dtype=np.float32))
+    assert np.array_equal(hip.download_dev(hl, large), np.arange(large, dtype=np.float32))
 
 
 @pytest.mark.parametrize("M,K,N,n_ops", [(1, 256, 300, 1), (3, 70, 33, 2), (1, 4096, 512, 1)])

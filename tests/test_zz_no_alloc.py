@@ -2,7 +2,8 @@
 is a variant of, map_matvec_topk_t_xq4_ex_dev: both called through the C ABI on the same inputs, outputs
 compared bit for bit (same kernels, same order of arithmetic; only the logit buffer differs).  Two calls in a
 row, the second with a smaller matrix, so that what the first call left in the fixed array would show.
-The limit (N <= 262144) and the refusal while ops are queued in an open batch are checked too."""
+The limit (N <= 262144) and the refusal while ops are queued in an open batch are checked too, and that the free
+device memory the HIP runtime reports is the same before and after the call."""
 import ctypes
 import os
 
@@ -10,7 +11,7 @@ import numpy as np
 import pytest
 
 from adam_amd import quant
-from gpu_util import note, up, f32map, read, load_qtensor
+from gpu_util import note, up, f32map, read, load_qtensor, device_free_bytes
 
 pytestmark = pytest.mark.gpu
 
@@ -36,9 +37,12 @@ def _both(hip, N, K, k, rpg, n_pen, seed):
         hip.scatter_contiguous(0, K, np.full(2 * ng * k, 12345.0, np.float32))
         hip.sync()
         note(f"{name} N={N} K={K} k={k} rows_per_group={rpg}")
+        free_before = device_free_bytes()
         rc = getattr(lib, name)(*[ctypes.c_uint32(v) for v in args], ctypes.c_float(1.3), ctypes.c_uint32(rpg))
         assert rc == 0, (name, rc)
         hip.sync()
+        if name.endswith("_noalloc_dev"):        # its kernels have run before (the sibling launches the same ones)
+            assert device_free_bytes() == free_before, "the entry point that allocates nothing changed free device memory"
         outs.append(_lists(hip, K, ng, k))
     return outs
 
