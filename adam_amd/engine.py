@@ -28,13 +28,21 @@ from .quant import QTensor
 
 @dataclass
 class GenerationConfig:
+    """Field names of the reference's GenerationConfig (adam/models/engine.py:24-29).  The defaults here are
+    greedy decoding with no stop token (what the parity tests and the benchmark want); `reference_defaults()`
+    gives the reference's own (temperature 0.8, top-k 40, top-p 0.95, repeat penalty 1.1, stop token 1)."""
     max_tokens: int = 128
     temperature: float = 0.0
     top_k: int = 1
     top_p: float = 1.0
     repeat_penalty: float = 1.0
     seed: Optional[int] = None
+    repeat_on_prompt: bool = False
     eos_token_ids: tuple = ()
+
+    @classmethod
+    def reference_defaults(cls, **kw):
+        return cls(**{**dict(temperature=0.8, top_k=40, top_p=0.95, repeat_penalty=1.1, eos_token_ids=(1,)), **kw})
 
 
 @dataclass
@@ -77,10 +85,29 @@ class DecodeEngine:
     def __init__(self, gpu, cfg, tensors, A=None, kv_cap=1024, kv_fp16=False,
                  fusion_scheduler_mode='legacy', gpu_fused_rows_per_group=256,
                  q4_map_elem_limit=(1 << 32) - 64, verbose=False, decode_plan=True, plan_id=0,
-                 prefill_chunk=0, batch=1, lookahead=True):
+                 prefill_chunk=0, batch=1, lookahead=True, gpu_fused_topk=True, gpu_approx_rerank=False,
+                 gpu_approx_partial_k=None, sampling_mode=None):
+        """`gpu_fused_topk`, `gpu_approx_rerank`, `gpu_approx_partial_k`: the reference engine's switches of the
+        same names (engine.py:333-338), which decide among the LM-head / sampling modes (`_select_sampling_mode`).
+        `sampling_mode` names one of them outright ('gpu_matvec_argmax', 'gpu_fused_topk', 'gpu_argmax',
+        'gpu_approx_rerank', 'gpu_topk', 'cpu'); a mode the configuration cannot serve raises at generate()."""
         if A is None:
             from . import adamah as A
-        self.gpu, self.cfg, self.tensors, self.A = gpu, cfg, tensors, A
+        self.gpu, self.cfg, self.A = gpu, cfg, A
+        self.tensors = tensors = dict(tensors)
+        self._gpu_fused_topk = bool(gpu_fused_topk)
+        self._gpu_approx_rerank = bool(gpu_approx_rerank)
+        self._gpu_approx_partial_k = max(1, min(self.SAMPLE_TOPK_MAX, int(gpu_approx_partial_k or self.SAMPLE_TOPK_MAX)))
+        self._force_mode = sampling_mode
+        self._lm_q4_approx_name = None
+        head = tensors.get('output.weight')
+        if self._gpu_approx_rerank and isinstance(head, QTensor) and head.kind == 'q8_0':
+            # a 4-bit copy of the 8-bit LM head for the shortlist pass, made as the reference makes it: the
+            # dequantised matrix through the 4-bit map's own quantiser with min / max qparams (engine.py:578-583,
+            # :1077-1085, :1100-1110)
+            from .quant import requantize_q4
+            self._lm_q4_approx_name = 'output.weight.q4_approx'
+            tensors[self._lm_q4_approx_name] = requantize_q4(head.dequant())
         self.verbose = verbose
         self._kv_cap = int(kv_cap)
         self._kv_fp16 = bool(kv_fp16)
@@ -195,7 +222,8 @@ class DecodeEngine:
             self._pos_attn_cap = pos; pos += 1
         if c.final_softcap > 0:
             self._pos_final_cap = pos
-            self._final_cap_h = self._up(np.full(self.SAMPLE_TOPK_MAX, pos))
+            # one entry per logit: the broadcast ops take a location per element (reference engine.py:1282-1287)
+            self._final_cap_h = self._up(np.full(c.n_vocab, pos))
             g.register_loc_span(self._final_cap_h, 0, pos, 1)
             pos += 1
 
@@ -206,7 +234,9 @@ class DecodeEngine:
                  ('sample_fused_idx', self._fused_groups * self.SAMPLE_TOPK_MAX),
                  ('sample_fused_val', self._fused_groups * self.SAMPLE_TOPK_MAX),
                  ('sample_topk_idx', self.SAMPLE_TOPK_MAX), ('sample_topk_val', self.SAMPLE_TOPK_MAX),
-                 ('sample_topk_prob', self.SAMPLE_TOPK_MAX), ('sample_short_sel', self.SAMPLE_TOPK_MAX),
+                 ('sample_topk_prob', self.SAMPLE_TOPK_MAX), ('sample_short_sel', self.SAMPLE_APPROX_SHORTLIST_MAX),
+                 ('sample_exact_idx', self.SAMPLE_APPROX_SHORTLIST_MAX),
+                 ('sample_exact_val', self.SAMPLE_APPROX_SHORTLIST_MAX),
                  ('normed2', c.n_embd)]
         for name, sz in slots:
             span(name, sz, pos); pos += sz
@@ -282,6 +312,20 @@ class DecodeEngine:
         self._sample_locs = np.array([self._ws['sample_token'][2]], dtype=np.uint32)
         self._rand_locs = np.array([self._ws['sample_rand'][2]], dtype=np.uint32)
         self._sample_fused_base_h = self._up([self._ws['sample_fused_idx'][2]])
+        self._sample_exact_base_h = self._up([self._ws['sample_exact_idx'][2]])
+        span_of = lambda n: np.arange(self._ws[n][2], self._ws[n][2] + self._ws[n][1], dtype=np.uint32)
+        self._logit_locs = span_of('logits')
+        self._fused_val_locs = span_of('sample_fused_val')
+        self._short_sel_locs, self._exact_idx_locs, self._exact_val_locs = (
+            span_of('sample_short_sel'), span_of('sample_exact_idx'), span_of('sample_exact_val'))
+        self._short_sel_chunk_h, self._exact_idx_chunk_h, self._exact_val_chunk_h = [], [], []
+        for lo in range(0, self.SAMPLE_APPROX_SHORTLIST_MAX, self.SAMPLE_TOPK_MAX):      # rerank runs in chunks of 64
+            hi = lo + self.SAMPLE_TOPK_MAX
+            self._short_sel_chunk_h.append(self._up(self._short_sel_locs[lo:hi]))
+            self._exact_idx_chunk_h.append(self._up(self._exact_idx_locs[lo:hi]))
+            self._exact_val_chunk_h.append(self._up(self._exact_val_locs[lo:hi]))
+        self._sample_rerank_n = 0
+        self._sample_fused_partial_n = 0
         self._sample_repeat_ids = np.zeros(self.SAMPLE_REPEAT_MAX, np.uint32)
         self._sample_repeat_ids_h = self._up(self._sample_repeat_ids)
         self._ws_total = pos
@@ -611,8 +655,12 @@ class DecodeEngine:
         return [int(t) for t in self.gpu.token_wait(ticket, m)]
 
     # ------------------------------------------------------------------ forward
-    def _forward(self, tok, pos, sample=True, sample_cfg=None, sample_prev=(), from_device=False, on_token=None):
+    def _forward(self, tok, pos, sample=True, sample_cfg=None, sample_prev=(), from_device=False, on_token=None,
+                 sample_mode=None, return_logits=False):
         """One decode step; op order of reference engine.py:2971-3402 (default discrete-GPU path).
+        `sample_mode`: the LM-head / sampling tail to issue (reference engine.py:3318-3640); None picks
+        'gpu_fused_topk' for a sampling configuration and 'gpu_matvec_argmax' otherwise, as before the other
+        modes existed.  `return_logits`: the full logits (final soft-cap applied) are computed and returned.
         `from_device`: the input token is the one the previous step's LM head left in the token slot (`tok` is
         not looked at); its embedding row is gathered on the device.  `on_token` (with `from_device`): called with
         that token once it has reached the host -- after the layers have been issued, before the LM head's ops are
@@ -707,43 +755,246 @@ class DecodeEngine:
         if from_device and on_token is not None and not on_token(self._wait_tokens(self._feed_ticket)[0]):
             g.batch_end()
             return
-        if sample and sample_cfg is not None and sample_cfg.temperature > 0.0 and sample_cfg.top_k > 1:
+        if callable(sample_prev):                            # evaluated late: it may include the token just read
+            sample_prev = sample_prev()
+        mode = sample_mode
+        if mode is None and sample:
+            mode = ('gpu_fused_topk' if sample_cfg is not None and sample_cfg.temperature > 0.0 and sample_cfg.top_k > 1
+                    else 'gpu_matvec_argmax')
+        if not sample:
+            mode = None
+        if mode == 'gpu_fused_topk':
             self._sample_fused_topk(sample_cfg, sample_prev, normed_h)
-        elif sample:
+        elif mode == 'gpu_matvec_argmax':
             fn = (g.map_matvec_argmax_t_xq8_dev if self._kind[self._lm_name] == 'q8'
                   else g.map_matvec_argmax_t_xq4_dev)
             fn(ws, self._map_of[self._lm_name], normed_h, self._wh[self._lm_name],
                W['sample_fused_idx'][0], W['sample_fused_val'][0], W['sample_token'][0],
                c.n_embd, c.n_vocab, self._rows_per_group)
             self._sample_token_ready = True
+        elif mode == 'gpu_approx_rerank':
+            self._issue_approx_shortlist(sample_cfg, sample_prev, normed_h)
+        elif mode in ('gpu_argmax', 'gpu_topk', 'cpu') or return_logits:
+            self._issue_full_logits(mode, sample_cfg, sample_prev, normed_h)
         g.batch_end()
+        if mode == 'gpu_approx_rerank':
+            self._rerank_shortlist(sample_cfg, normed_h)
+        if return_logits or mode == 'cpu':
+            return g.gather(ws, self._logit_locs).view(np.float32).copy()
+        return None
+
+    # ------------------------------------------------------------------ LM-head / sampling modes
+    def _effective_top_k(self, cfg):
+        """Deterministic decoding collapses to top-1 (reference engine.py:1843-1850)."""
+        if cfg.temperature <= 0.0:
+            return 1
+        k = int(cfg.top_k)
+        return 0 if k <= 0 else min(k, self.SAMPLE_TOPK_MAX, self.cfg.n_vocab)
+
+    def _select_sampling_mode(self, cfg):
+        """The reference's order of preference (engine.py:3783-3805, predicates :1852-1958) without its host-side
+        top-1 mode, which exists for one device family only."""
+        g, k = self.gpu, self._effective_top_k(cfg)
+        kind = self._kind[self._lm_name]
+        has = lambda n: bool(getattr(g, n, False)) or hasattr(g, n.replace('_has_', '', 1))
+        matvec_argmax = (k == 1 and cfg.repeat_penalty == 1.0 and has(f'_has_map_matvec_argmax_t_x{kind}_dev'))
+        can_topk = 0 < k <= self.SAMPLE_TOPK_MAX
+        fused = self._gpu_fused_topk and can_topk and has(f'_has_map_matvec_topk_t_x{kind}_dev')
+        rerank = (k > 1 and self._gpu_approx_rerank and self._lm_q4_approx_name is not None and kind == 'q8'
+                  and has('_has_map_matvec_topk_t_xq4_ex_dev') and has('_has_map_matvec_rerank_t_xq8_dev'))
+        gpu_argmax = k == 1 and cfg.repeat_penalty == 1.0
+        if self._force_mode is not None:
+            ok = {'gpu_matvec_argmax': matvec_argmax, 'gpu_fused_topk': fused, 'gpu_argmax': gpu_argmax,
+                  'gpu_approx_rerank': rerank, 'gpu_topk': can_topk, 'cpu': True}
+            if not ok.get(self._force_mode, False):
+                raise RuntimeError(f"sampling mode '{self._force_mode}' cannot serve this configuration")
+            return self._force_mode
+        if k == 1 and matvec_argmax:
+            return 'gpu_matvec_argmax'
+        if k == 1 and fused:
+            return 'gpu_fused_topk'
+        if gpu_argmax:
+            return 'gpu_argmax'
+        if rerank:
+            return 'gpu_approx_rerank'
+        if fused:
+            return 'gpu_fused_topk'
+        if can_topk:
+            return 'gpu_topk'
+        return 'cpu'
+
+    def _repeat_history(self, prompt, generated, cfg):
+        """reference engine.py:3731-3738"""
+        if cfg.repeat_penalty == 1.0:
+            return None
+        hist = (list(prompt) + list(generated)) if cfg.repeat_on_prompt else list(generated)
+        return hist or None
+
+    def _prepare_repeat_ids(self, prev):
+        """The distinct ids among the last SAMPLE_REPEAT_MAX tokens, ascending, into the penalty list's handle
+        (reference engine.py:1960-1967); returns how many."""
+        recent = sorted({int(t) for t in list(prev)[-self.SAMPLE_REPEAT_MAX:] if 0 <= int(t) < self.cfg.n_vocab})
+        if not recent:
+            return 0
+        self._sample_repeat_ids[:] = 0
+        self._sample_repeat_ids[:len(recent)] = recent
+        self.gpu.upload_dev(self._sample_repeat_ids, handle=self._sample_repeat_ids_h)
+        return len(recent)
+
+    def _write_rand(self):
+        self.gpu.scatter(self.WS_MAP, self._rand_locs, np.array([self._rng.random()], np.float32))
+
+    def _softcap(self, val_h, n):
+        c, g, A, ws = self.cfg, self.gpu, self.A, self.WS_MAP
+        if c.final_softcap > 0:
+            g.map_broadcast_dev(ws, A.OP_DIV, val_h, self._final_cap_h, val_h, n)
+            g.map_op1_dev(ws, A.OP_TANH, val_h, val_h, n)
+            g.map_broadcast_dev(ws, A.OP_MUL, val_h, self._final_cap_h, val_h, n)
+
+    def _issue_full_logits(self, mode, cfg, prev, normed_h):
+        """Full logits with the final soft-cap, then, inside the same batch, the arg-max ('gpu_argmax') or
+        repeat penalty, top-k, top-p and the draw ('gpu_topk'); reference engine.py:3509-3548."""
+        c, g, ws, W = self.cfg, self.gpu, self.WS_MAP, self._ws
+        lo_h = W['logits'][0]
+        self._proj(normed_h, self._lm_name, lo_h, c.n_embd, c.n_vocab)
+        self._softcap(lo_h, c.n_vocab)
+        if mode == 'gpu_argmax':
+            g.map_argmax_dev(ws, lo_h, W['sample_token'][0], c.n_vocab)
+            self._sample_token_ready = True
+        elif mode == 'gpu_topk' and cfg is not None:
+            if cfg.repeat_penalty != 1.0 and prev:
+                n_rep = self._prepare_repeat_ids(prev)
+                if n_rep:
+                    g.map_repeat_penalty_dev(ws, lo_h, self._sample_repeat_ids_h, n_rep, float(cfg.repeat_penalty))
+            k = self._effective_top_k(cfg)
+            idx_h, val_h, prob_h = W['sample_topk_idx'][0], W['sample_topk_val'][0], W['sample_topk_prob'][0]
+            g.map_topk_dev(ws, lo_h, idx_h, val_h, c.n_vocab, k)
+            if cfg.temperature > 0.0:
+                g.map_topp_dev(ws, val_h, prob_h, k, float(cfg.temperature), float(cfg.top_p))
+                self._write_rand()
+                g.map_sample_categorical_dev(ws, idx_h, prob_h, W['sample_rand'][0], W['sample_token'][0], k)
+                self._sample_token_ready = True
+            # (deterministic decoding reaches this mode only under a repeat penalty with the fused modes switched
+            # off: the token is then the first entry of the top-k list, which generate() reads.  The reference
+            # applies the penalty a second time on that path, engine.py:2046-2051 after :3524-3529; here it is
+            # applied once.)
+
+    def _issue_approx_shortlist(self, cfg, prev, normed_h):
+        """First pass of 'gpu_approx_rerank' (reference engine.py:3331-3356): partial top-k per group of rows over
+        the 4-bit copy of the LM head, repeat penalty applied."""
+        c, g, ws, W = self.cfg, self.gpu, self.WS_MAP, self._ws
+        k = min(self._gpu_approx_partial_k, c.n_vocab)
+        self._approx_penalty_n = self._prepare_repeat_ids(prev) if (cfg.repeat_penalty != 1.0 and prev) else 0
+        self._sample_fused_partial_n = self._fused_groups * k
+        self._sample_rerank_n = 0
+        name = self._lm_q4_approx_name
+        g.map_matvec_topk_t_xq4_ex_dev(ws, self._map_of[name], normed_h, self._wh[name], self._sample_repeat_ids_h,
+                                       W['sample_fused_idx'][0], W['sample_fused_val'][0], c.n_embd, c.n_vocab, k,
+                                       self._approx_penalty_n, float(cfg.repeat_penalty), self._rows_per_group)
+
+    def _rerank_shortlist(self, cfg, normed_h):
+        """Second pass (reference engine.py:3641-3700): the best SAMPLE_APPROX_SHORTLIST_MAX partial values are
+        picked on the host, their rows recomputed exactly over the 8-bit head in chunks of SAMPLE_TOPK_MAX."""
+        g, ws, c = self.gpu, self.WS_MAP, self.cfg
+        n_part = self._sample_fused_partial_n
+        if n_part <= 0:
+            return
+        vals = g.gather(ws, self._fused_val_locs[:n_part]).view(np.float32)
+        # (unused slots of a group shorter than k hold -FLT_MAX with row 0: finite, so the reference's test for
+        # finiteness lets them through when the whole list is shorter than the shortlist; they are left out here)
+        valid = np.flatnonzero(np.isfinite(vals) & (vals > np.float32(-3.0e38)))
+        if not valid.size:
+            return
+        n = min(self.SAMPLE_APPROX_SHORTLIST_MAX, int(valid.size))
+        keep = valid[np.argpartition(vals[valid], -n)[-n:]] if n < valid.size else valid
+        keep = keep[np.argsort(vals[keep], kind='stable')[::-1]]
+        g.batch_begin()
+        try:
+            g.scatter(ws, self._short_sel_locs[:n], keep.astype(np.float32))
+            for ci, lo in enumerate(range(0, n, self.SAMPLE_TOPK_MAX)):
+                m = min(self.SAMPLE_TOPK_MAX, n - lo)
+                g.map_matvec_rerank_t_xq8_dev(ws, self._map_of[self._lm_name], normed_h, self._wh[self._lm_name],
+                                              self._sample_fused_base_h, self._short_sel_chunk_h[ci],
+                                              self._sample_repeat_ids_h, self._exact_idx_chunk_h[ci],
+                                              self._exact_val_chunk_h[ci], c.n_embd, m, self._approx_penalty_n,
+                                              float(cfg.repeat_penalty))
+        finally:
+            g.batch_end()
+        self._sample_rerank_n = n
+
+    def _sample_approx_rerank(self, cfg):
+        """Token of 'gpu_approx_rerank' (reference engine.py:2100-2145, device path): top-k of the exact values,
+        final soft-cap, then the best one, or top-p and a draw."""
+        n, self._sample_rerank_n = self._sample_rerank_n, 0
+        if n <= 0:
+            return 0
+        c, g, ws, W = self.cfg, self.gpu, self.WS_MAP, self._ws
+        idx_h, val_h, prob_h = W['sample_topk_idx'][0], W['sample_topk_val'][0], W['sample_topk_prob'][0]
+        k = min(self._effective_top_k(cfg), n, self.SAMPLE_TOPK_MAX)
+        if k <= 0:
+            k = min(n, self.SAMPLE_TOPK_MAX)
+        g.batch_begin()
+        try:
+            g.map_topk_dev(ws, W['sample_exact_val'][0], idx_h, val_h, n, k)
+            self._softcap(val_h, k)
+            if cfg.temperature <= 0.0:
+                g.map_resolve_idx_dev(ws, self._sample_exact_base_h, idx_h, W['sample_token'][0], 1)
+            else:
+                sel_h = W['sample_short_sel'][0]
+                g.map_resolve_idx_dev(ws, self._sample_exact_base_h, idx_h, sel_h, k)
+                g.map_topp_dev(ws, val_h, prob_h, k, float(cfg.temperature), float(cfg.top_p))
+                self._write_rand()
+                g.map_sample_categorical_dev(ws, sel_h, prob_h, W['sample_rand'][0], W['sample_token'][0], k)
+        finally:
+            g.batch_end()
+        return self.read_token()
+
+    def _sample_host(self, logits, cfg, prev):
+        """'cpu' mode: the reference's host sampler (engine.py:3708-3729) on the full logits, with this engine's
+        seeded generator in place of NumPy's global one."""
+        logits = np.array(logits, dtype=np.float32)
+        if cfg.repeat_penalty != 1.0 and prev:
+            for t in set(prev[-64:]):
+                if t < len(logits):
+                    logits[t] = logits[t] / cfg.repeat_penalty if logits[t] > 0 else logits[t] * cfg.repeat_penalty
+        if cfg.temperature <= 0:
+            return int(np.argmax(logits))
+        logits /= np.float32(cfg.temperature)
+        if cfg.top_k > 0:
+            tk = min(cfg.top_k, len(logits))
+            ti = np.argpartition(logits, -tk)[-tk:]
+            m = np.full_like(logits, -np.inf); m[ti] = logits[ti]; logits = m
+        pr = np.exp(logits - np.max(logits)); pr /= pr.sum()
+        if cfg.top_p < 1.0:
+            si = np.argsort(pr)[::-1]; cs = np.cumsum(pr[si])
+            co = int(np.searchsorted(cs, cfg.top_p)) + 1
+            m = np.zeros_like(pr); m[si[:co]] = pr[si[:co]]; pr = m / m.sum()
+        return int(self._rng.choice(len(pr), p=pr.astype(np.float64) / float(pr.astype(np.float64).sum())))
 
     def _sample_fused_topk(self, cfg, prev, normed_h):
         """Sampled LM head inside the forward batch, the reference's 'gpu_fused_topk' mode
         (engine.py:3404-3508): partial top-k per group of rows with the repeat penalty, top-k of the
         partial values, final soft-cap on the k survivors, temperature / top-p, token ids resolved
-        through the partial list, one categorical draw with a uniform number from the host."""
+        through the partial list, one categorical draw with a uniform number from the host.  With an
+        effective k of 1 (deterministic decoding under a repeat penalty): arg-max of the partial values, resolved."""
         c, g, A, ws, W = self.cfg, self.gpu, self.A, self.WS_MAP, self._ws
-        top_k = max(1, min(int(cfg.top_k), self.SAMPLE_TOPK_MAX, c.n_vocab))
-        n_pen = 0
-        if cfg.repeat_penalty != 1.0 and len(prev):
-            ids = list(dict.fromkeys(int(t) for t in reversed(list(prev))))[:self.SAMPLE_REPEAT_MAX]
-            n_pen = len(ids)
-            self._sample_repeat_ids[:] = 0
-            self._sample_repeat_ids[:n_pen] = ids
-            g.upload_dev(self._sample_repeat_ids, handle=self._sample_repeat_ids_h)
-        g.scatter(ws, self._rand_locs, np.array([self._rng.random()], np.float32))
+        top_k = max(1, self._effective_top_k(cfg))
+        n_pen = self._prepare_repeat_ids(prev) if (cfg.repeat_penalty != 1.0 and prev) else 0
+        if top_k > 1:
+            self._write_rand()            # ahead of the ops: a host write in their middle would split the queue
         pidx_h, pval_h = W['sample_fused_idx'][0], W['sample_fused_val'][0]
         fn = (g.map_matvec_topk_t_xq8_ex_dev if self._kind[self._lm_name] == 'q8' else g.map_matvec_topk_t_xq4_ex_dev)
         fn(ws, self._map_of[self._lm_name], normed_h, self._wh[self._lm_name], self._sample_repeat_ids_h, pidx_h, pval_h,
            c.n_embd, c.n_vocab, top_k, n_pen, float(cfg.repeat_penalty), self._rows_per_group)
+        self._sample_fused_partial_n = self._fused_groups * top_k
         idx_h, val_h, prob_h = W['sample_topk_idx'][0], W['sample_topk_val'][0], W['sample_topk_prob'][0]
-        g.map_topk_dev(ws, pval_h, idx_h, val_h, self._fused_groups * top_k, top_k)
-        if c.final_softcap > 0:
-            cap_h = self._final_cap_h
-            g.map_broadcast_dev(ws, A.OP_DIV, val_h, cap_h, val_h, top_k)
-            g.map_op1_dev(ws, A.OP_TANH, val_h, val_h, top_k)
-            g.map_broadcast_dev(ws, A.OP_MUL, val_h, cap_h, val_h, top_k)
+        if top_k == 1:
+            g.map_argmax_dev(ws, pval_h, idx_h, self._sample_fused_partial_n)
+            g.map_resolve_idx_dev(ws, self._sample_fused_base_h, idx_h, W['sample_token'][0], 1)
+            self._sample_token_ready = True
+            return
+        g.map_topk_dev(ws, pval_h, idx_h, val_h, self._sample_fused_partial_n, top_k)
+        self._softcap(val_h, top_k)
         g.map_topp_dev(ws, val_h, prob_h, top_k, float(cfg.temperature), float(cfg.top_p))
         sel_h = W['sample_short_sel'][0]
         g.map_resolve_idx_dev(ws, self._sample_fused_base_h, idx_h, sel_h, top_k)
@@ -1030,38 +1281,56 @@ class DecodeEngine:
         self._sample_token_ready = False
 
     # ------------------------------------------------------------------ generate
-    def generate(self, token_ids, config=None, forced=None):
-        """Greedy generation, or sampled generation when `config.temperature > 0` and `config.top_k > 1`
-        (top-k, top-p and repeat penalty on the device, one uniform number per token from a host
-        generator seeded with `config.seed`).  Prefill is the same `_forward` once per prompt token, LM head only
-        on the last one; `decode_tps = n_gen / wall(decode loop)` including the per-token
-        read-back (reference engine.py:3838-3931).  Greedy decoding without `forced` runs one step ahead of the
-        read-back unless the engine was built with `lookahead=False`: same tokens, same number of steps.
+    def generate(self, token_ids, config=None, forced=None, reuse_prefix=0):
+        """Generation with the LM-head / sampling mode the configuration selects (`_select_sampling_mode`: greedy
+        GEMV + arg-max, partial top-k fused into the LM head, full logits + arg-max / top-k, approximate shortlist
+        + exact rerank, or the host sampler; one uniform number per drawn token from a host generator seeded with
+        `config.seed`).  Prefill is the same `_forward` once per prompt token (in chunks on the matrix cores when
+        the engine was built with `prefill_chunk`), LM head only on the last one; `decode_tps = n_gen /
+        wall(decode loop)` including the per-token read-back (reference engine.py:3838-3931).  The greedy and the
+        fused top-k loops run one step ahead of the read-back unless `forced` is given or the engine was built
+        with `lookahead=False`: same tokens, same number of steps.
         `forced`, when given, is a token list fed back instead of the model's own choices (teacher forcing)
-        while the choices are still returned."""
+        while the choices are still returned.
+        `reuse_prefix=n`: the caches still hold the rows of the first n prompt tokens from the previous call (same
+        tokens, e.g. the earlier turns of a conversation); prefill starts at position n (reference
+        engine.py:3815-3833)."""
         config = config or GenerationConfig()
+        token_ids = [int(t) for t in token_ids]
         if len(token_ids) + config.max_tokens > self._kv_cap:
             raise RuntimeError(
                 f"KV cache too small: need {len(token_ids) + config.max_tokens} tokens but "
                 f"kv_cap={self._kv_cap}. Reinitialize with kv_cap>={len(token_ids) + config.max_tokens}.")
+        mode = self._select_sampling_mode(config)
+        reuse = max(0, int(reuse_prefix or 0))
+        if reuse >= len(token_ids):
+            reuse = 0
         self.reset()
-        sampled = config.temperature > 0.0 and config.top_k > 1
         # (the device-side embedding table of an untied model is filled on first use: before the clock starts)
-        ahead = (forced is None and self._lookahead and config.max_tokens > 0 and self._token_feed() is not None)
+        ahead = (forced is None and self._lookahead and config.max_tokens > 0
+                 and mode in ('gpu_matvec_argmax', 'gpu_fused_topk') and self._token_feed() is not None)
         self._rng = np.random.default_rng(config.seed)
-        hist = [int(t) for t in token_ids]
+        fed = []                                             # tokens fed back after the prompt
+        prev = lambda: self._repeat_history(token_ids, fed, config)
         tp = time.perf_counter()
         last = len(token_ids) - 1
-        if self._chunk and not sampled:
-            self.prefill([int(t) for t in token_ids])
+        logits = None
+        todo = token_ids[reuse:]
+        if self._chunk and mode == 'gpu_matvec_argmax':
+            self.prefill(todo, pos0=reuse)
         else:
-            for i, t in enumerate(token_ids):
-                self._forward(int(t), i, sample=(i == last), sample_cfg=config, sample_prev=hist)
+            if self._chunk and len(todo) > 1:                # all but the last token: no LM head needed
+                self.prefill(todo[:-1], pos0=reuse, sample=False)
+                reuse = last
+            for i in range(reuse, len(token_ids)):
+                logits = self._forward(token_ids[i], i, sample=(i == last), sample_cfg=config, sample_prev=prev,
+                                       sample_mode=mode if i == last else None)
+        n_reused = len(token_ids) - len(todo)
         self.gpu.sync()
         t_pre = time.perf_counter() - tp
         out, ttimes = [], []
         td = time.perf_counter()
-        if ahead and sampled:
+        if ahead and mode == 'gpu_fused_topk':
             # Sampled decoding one step ahead: the layers of the step that consumes token n are issued at once (the
             # token's embedding row is gathered on the device); the host reads token n while they run, builds the
             # repeat-penalty list that includes it and only then issues the step's LM head and sampling ops.
@@ -1069,13 +1338,13 @@ class DecodeEngine:
                 if nt in config.eos_token_ids:
                     return False
                 out.append(nt)
-                hist.append(nt)
+                fed.append(nt)
                 return True
             for step in range(config.max_tokens):
                 t0 = time.perf_counter()
                 n_before = len(out)
-                self._forward(None, len(token_ids) + step, sample=True, sample_cfg=config, sample_prev=hist,
-                              from_device=True, on_token=seen)
+                self._forward(None, len(token_ids) + step, sample=True, sample_cfg=config, sample_prev=prev,
+                              from_device=True, on_token=seen, sample_mode=mode)
                 if len(out) == n_before:
                     break
                 ttimes.append(time.perf_counter() - t0)
@@ -1085,30 +1354,43 @@ class DecodeEngine:
             # is therefore noticed after one step too many was issued (its KV row is never read).
             for step in range(config.max_tokens):
                 t0 = time.perf_counter()
-                self._forward(None, len(token_ids) + step, from_device=True)
+                self._forward(None, len(token_ids) + step, from_device=True, sample_mode=mode)
                 nt = self._wait_tokens(self._feed_ticket)[0]       # the token that step consumes
                 if nt in config.eos_token_ids:
                     break
                 out.append(nt)
-                hist.append(nt)
+                fed.append(nt)
                 ttimes.append(time.perf_counter() - t0)
         for step in range(0 if not ahead else config.max_tokens, config.max_tokens):
             t0 = time.perf_counter()
-            nt = self.read_token()
+            nt = self._next_token(mode, config, logits, prev())
             if nt in config.eos_token_ids:
                 break
             out.append(nt)
-            feed = nt if forced is None else int(forced[step])
-            hist.append(feed)
-            self._forward(feed, len(token_ids) + step, sample=True, sample_cfg=config, sample_prev=hist)
+            fed.append(nt if forced is None else int(forced[step]))
+            logits = self._forward(fed[-1], len(token_ids) + step, sample=True, sample_cfg=config, sample_prev=prev,
+                                   sample_mode=mode)
             ttimes.append(time.perf_counter() - t0)
         self.gpu.sync()
         t_dec = time.perf_counter() - td
-        n_p, n_g = len(token_ids), len(out)
+        n_p, n_g = len(token_ids) - n_reused, len(out)
         return out, {
-            'n_prompt': n_p, 'n_gen': n_g, 'prefill_s': t_pre, 'decode_s': t_dec,
+            'n_prompt': n_p, 'n_prompt_total': len(token_ids), 'n_prompt_reused': n_reused, 'n_prompt_prefilled': n_p,
+            'n_gen': n_g, 'prefill_s': t_pre, 'decode_s': t_dec,
             'prefill_tps': n_p / t_pre if t_pre > 0 else 0.0,
             'decode_tps': n_g / t_dec if t_dec > 0 else 0.0,
             'avg_ms': float(np.mean(ttimes) * 1000) if ttimes else 0.0,
-            'sampling_mode': 'gpu_fused_topk' if sampled else 'gpu_matvec_argmax',
+            'sampling_mode': mode,
         }
+
+    def _next_token(self, mode, cfg, logits, prev):
+        """The token the last forward pass chose, per mode (reference engine.py:3856-3875)."""
+        ready, self._sample_token_ready = self._sample_token_ready, False
+        if mode == 'gpu_approx_rerank':
+            return self._sample_approx_rerank(cfg)
+        if mode == 'cpu':
+            return self._sample_host(logits, cfg, prev)
+        if mode == 'gpu_topk' and not ready:                 # deterministic: the head of the top-k list
+            pos = self._ws['sample_topk_idx'][2]
+            return int(self.gpu.gather(self.WS_MAP, np.array([pos], np.uint32)).view(np.float32)[0])
+        return self.read_token()

@@ -22,8 +22,8 @@ f32 = np.float32
 class CpuModel:
     def __init__(self, cfg, tensors, kv_cap, kv_fp16=False, acc64=True):
         """tensors: name -> float32 ndarray ([N,K] matrices, 1-D norms); the untied embedding may be
-        an object with .row(tok).  acc64=False keeps every matrix product in float32 BLAS, which is
-        how the reference's forward_cpu runs (used when this model is timed as the CPU baseline)."""
+        an object with .row(tok).  acc64=False keeps every matrix product (attention included) in float32
+        BLAS, which is how the reference's forward_cpu runs (used when this model is timed as the CPU baseline)."""
         self.c = cfg
         self.acc64 = acc64
         self.t = tensors
@@ -99,13 +99,20 @@ class CpuModel:
             for h in range(c.n_head):
                 Kh = self.k_cache[L, h // gs, :seq]
                 Vh = self.v_cache[L, h // gs, :seq]
-                sc = ((Kh.astype(np.float64) @ q[h].astype(np.float64)).astype(np.float32) * scale).astype(np.float32)
+                if self.acc64:
+                    sc = ((Kh.astype(np.float64) @ q[h].astype(np.float64)).astype(np.float32) * scale).astype(np.float32)
+                else:                                   # the timed baseline: float32 BLAS here too, no conversions
+                    sc = ((Kh @ q[h]) * scale).astype(np.float32)
                 if c.attn_softcap > 0:
                     cap = f32(c.attn_softcap)
                     sc = (np.tanh(sc / cap) * cap).astype(np.float32)
-                w_ = np.exp((sc - sc.max()).astype(np.float64))
-                w_ /= w_.sum()
-                attn[h] = (w_ @ Vh.astype(np.float64)).astype(np.float32)
+                if self.acc64:
+                    w_ = np.exp((sc - sc.max()).astype(np.float64))
+                    w_ /= w_.sum()
+                    attn[h] = (w_ @ Vh.astype(np.float64)).astype(np.float32)
+                else:
+                    w_ = np.exp(sc - sc.max())
+                    attn[h] = (w_ @ Vh) / w_.sum()
             o = self.mv(f'{p}.attn_output.weight', attn.reshape(-1))
             pan = f'{p}.post_attention_norm.weight'
             if pan in t:

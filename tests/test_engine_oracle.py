@@ -78,13 +78,13 @@ def test_sampled_generation_draws_from_the_top_k_of_the_reference_logits(arch):
         runs.append(out)
     assert runs[0] == runs[1] and runs[0] != runs[2]
     ref = CpuModel(cfg, dequant_tensors(tensors), kv_cap=32)
-    hist = list(prompt)
+    hist = []                                  # the penalty looks at the generated tokens (repeat_on_prompt is off)
     logits = None
     for i, t in enumerate(prompt):
         logits = ref.forward(int(t), i)
     for step, tok in enumerate(runs[0]):
         lg = np.array(logits, np.float32)
-        for r in set(hist):
+        for r in set(hist[-64:]):
             lg[r] = lg[r] / np.float32(1.2) if lg[r] > 0 else lg[r] * np.float32(1.2)
         top = np.argsort(-lg, kind="stable")[:8]
         assert tok in top, (step, tok, top)
