@@ -185,3 +185,81 @@ def test_gemv_error_codes(hip):
     assert hip.scatter_q4_packed_contiguous(1, 1, np.zeros(2, np.uint8), 4) == (1 << 64) - 3   # odd start: -3
     h, _ = hip.upload_dev(np.zeros(4, np.uint32))
     assert hip.upload_dev(np.zeros(5, np.uint32), handle=h)[0] == 0               # size change -> 0
+
+
+# ---- guard for the cross-lane moves of the Q4 GEMV -----------------------------------------------------
+def _integer_weights(N, K, seed):
+    """Q4_0 blocks with scale 1: the weights are the integers q - 8."""
+    q = np.random.default_rng(seed).integers(0, 16, (N, K), dtype=np.uint8)
+    codes = (q[:, 0::2] | (q[:, 1::2] << 4)).astype(np.uint8).reshape(-1)
+    return quant.QTensor('q4_0', (N, K), np.ones(N * K // 32, np.float16), codes), q.astype(np.float64) - 8.0
+
+
+@pytest.mark.parametrize("K,N", [(4096, 515), (1152, 1024), (6912, 1152)])
+@pytest.mark.parametrize("pro", ["none", "rmsnorm", "norm2", "combine"])
+def test_unit_scale_integer_weights_give_exact_sums(hip, pro, K, N):
+    """Guard for the cross-lane moves of the matrix-instruction GEMV: the kernel hands blocks, scales, block maxima
+    and integer sums from lane to lane (ds_bpermute, DPP), and every such move is kept an instruction of its own
+    because, folded by the compiler into its consumer, the kernel once returned wrong sums without any other sign.
+    With weights q - 8 at scale 1 and activations that are small integers (or integers over a power of two) every
+    product and every partial sum is exact in int32 and in float32, whichever order the lanes add them in: the
+    result must EQUAL the integer dot products, for every staging variant of the kernel -- plain, RMSNorm folded in,
+    both norms of a layer boundary folded in, merge of the attention slices folded in (operands chosen so that the
+    norms' factors are 1/2 and 1/4 and the softmax is uniform over 1024 rows)."""
+    rng = np.random.default_rng(K + N)
+    if pro == "combine":
+        K = 1024                                       # 4 heads x 256 over one KV head: the merge in the GEMV's staging
+    qt, W = _integer_weights(N, K, K * 3 + N)
+    load_qtensor(hip, 1, qt)
+    assert hip.map_layout(1) == 1
+    note(f"gemv exact integer sums pro={pro} {N}x{K}")
+    if pro == "combine":
+        ctx, Hq, d = 1024, 4, 256
+        V = rng.integers(-1, 2, (ctx, d)).astype(np.float32)
+        Kc = rng.standard_normal((ctx, d)).astype(np.float32)
+        q_pos, out_pos, y_pos = Hq * ctx, Hq * ctx + Hq * d, Hq * ctx + 2 * Hq * d
+        kv = (y_pos + N + d - 1) // d * d
+        f32map(hip, 0, kv + 2 * ctx * d, None)
+        hip.kv_cache_fp16(0, kv, 2 * ctx * d)
+        hip.scatter_contiguous(0, q_pos, np.zeros(Hq * d, np.float32))        # q = 0: every score is 0
+        hip.scatter_contiguous(0, kv, Kc.reshape(-1)); hip.scatter_contiguous(0, kv + ctx * d, V.reshape(-1))
+        s_rows, o_rows = up(hip, np.arange(Hq) * ctx), up(hip, out_pos + np.arange(Hq) * d)
+        hip.batch_begin()
+        hip.map_matmul_t_dev(0, up(hip, q_pos + np.arange(Hq) * d), up(hip, [kv] * Hq), s_rows, 1, d, ctx, Hq)
+        hip.map_attn_softmax_value_dev(0, s_rows, up(hip, [kv + ctx * d] * Hq), o_rows, Hq, ctx, d, float(1 / 16), 0.0)
+        hip.fusion_flush()
+        hip.map_matmul_t_xq4_dev(0, 1, up(hip, [out_pos]), up(hip, [0]), up(hip, [y_pos]), 1, K, N)
+        hip.batch_end()
+        x = np.tile(V.astype(np.float64).sum(0) / ctx, Hq)
+        assert np.array_equal(read(hip, 0, out_pos, K), x.astype(np.float32))
+        assert hip.get_last_barrier_count() == 2                              # attention, GEMV with the merge
+        y = read(hip, 0, y_pos, N)
+    else:
+        src = rng.choice([-2.0, 2.0], K).astype(np.float32)
+        w1 = np.full(K, 2.0, np.float32)
+        w2 = rng.choice([1.0, 2.0, 4.0], K).astype(np.float32)
+        o = {"src": 0, "w1": K, "w2": 2 * K, "res": 3 * K, "x": 4 * K, "y": 5 * K}
+        f32map(hip, 0, 5 * K + N + 8, np.concatenate([src, w1, w2, src]))      # residual = source
+        h = lambda n: up(hip, [o[n]])
+        hip.batch_begin()
+        if pro == "none":
+            x = rng.integers(-4, 5, K).astype(np.float32)
+            hip.scatter_contiguous(0, o["x"], x)
+        elif pro == "rmsnorm":                                                 # mean(src^2) = 4, eps 0: factor 1/2
+            hip.map_rmsnorm_dev(0, h("src"), h("w2"), h("x"), 1, K, 0.0)
+            x = src * 0.5 * w2
+        else:                                   # t = src/2 * 2 + src = +-4; mean(t^2) = 16, eps 0: factor 1/4
+            hip.map_rmsnorm_add_dev(0, h("src"), h("w1"), h("res"), h("res"), 1, K, 0.0)
+            hip.map_rmsnorm_dev(0, h("res"), h("w2"), h("x"), 1, K, 0.0)
+            x = 2.0 * src * 0.25 * w2
+        hip.map_matmul_t_xq4_dev(0, 1, h("x"), up(hip, [0]), h("y"), 1, K, N)
+        hip.batch_end()
+        if K <= 4096:                           # (longer rows do not fit the staging's registers: the norms run apart)
+            assert hip.get_last_barrier_count() == 1                          # the norms rode in the GEMV's staging
+        assert np.array_equal(read(hip, 0, o["x"], K), x.astype(np.float32))
+        if pro == "norm2":
+            assert np.array_equal(read(hip, 0, o["res"], K), 2.0 * src)
+        y = read(hip, 0, o["y"], N)
+    want = W @ x.astype(np.float64)
+    assert np.all(np.abs(want) < 2 ** 24 / 1024)
+    assert np.array_equal(y, want.astype(np.float32))
