@@ -234,6 +234,215 @@ k_attn_prefill(const float* data, float* out, const __half* kv, uint64_t kv_shif
   }
 }
 
+// ---- the same chunk with both products on the matrix cores ------------------------------------------------
+// k_attn_prefill above accumulates softmax . V with vector multiply-adds (16 queries x D/64 dims per lane and cache
+// row) and walks the cache once per query head.  The form below keeps everything in v_mfma_f32_16x16x32_f16:
+//
+//   * a wave owns one query head and a tile of 16 consecutive tokens and walks the cache in tiles of 32 rows; the
+//     four waves of a workgroup are four heads of the same token tile -- with grouped queries, the heads of one KV
+//     head, so their K / V tiles come out of the L1 after the first wave has asked for them;
+//   * scores transposed, S^T = K . Q^T: A = K tile (row = cache row, 8 consecutive dims per lane: one 16-byte load
+//     of the row-major cache), B = the queries as exact hi + lo fp16 pairs after a power-of-two scale (held in
+//     registers for the whole walk).  The result leaves lane (query l % 16, g = l / 16) with cache rows 4g..4g+3 of
+//     both 16-row halves of the tile: all eight values of a lane belong to ONE query, so the softmax statistics
+//     are one (max, sum) pair per lane and the row maximum needs two cross-lane steps;
+//   * that is also the A-operand layout of P . V with the contraction index (g, j) standing for cache row
+//     4g + j (j < 4) or 16 + 4g + j - 4: P goes into the second product as it is (hi + lo fp16, so its products
+//     with the fp16 values are exact), no transposition;
+//   * the B operand of P . V needs eight cache ROWS per lane at one dim.  k_v_tile_transpose writes the visible
+//     part of the fp16 V cache once per launch into a scratch laid out [KV head][tile][16-dim block][g][dim][8 rows]
+//     so that this operand is one 16-byte load, too (rows past the end: zeros);
+//   * no LDS, no barrier: the accumulators (queries 4g..4g+3 x dim l % 16 per 16-dim block) are rescaled only in
+//     tiles where some query's maximum moved, the factors fetched across lanes.
+// Workgroup b serves head quad b % (H / 4): with eight KV heads, XCD x (workgroups x, x + 8, ...) walks the cache of
+// KV head x only, which fits its L2; the token tiles with the longest walks come first.
+typedef _Float16 h8p_t __attribute__((ext_vector_type(8)));
+typedef float f4pu_t __attribute__((ext_vector_type(4), aligned(4)));
+struct AttpVt { uint32_t grp[ATTP_MAX_HEADS]; };   // head -> index of its KV head's part of the transposed scratch
+struct AttpVtSrc { uint32_t vb[ATTP_MAX_HEADS]; };  // group -> base of its V cache (element offset in the map)
+
+template <int D>
+__global__ void __launch_bounds__(256)
+k_v_tile_transpose(const __half* kv, uint64_t kv_shift, const AttpVtSrc src, uint32_t nkeys, uint32_t tiles, uint4* vt) {
+  constexpr uint32_t NB = D / 16;
+  const uint32_t T = blockIdx.x, grp = blockIdx.y;
+  const unsigned short* v = (const unsigned short*)(kv + ((uint64_t)src.vb[grp] - kv_shift));
+  for (uint32_t idx = threadIdx.x; idx < NB * 64u; idx += 256u) {
+    const uint32_t b = idx >> 6, g = (idx >> 4) & 3u, n = idx & 15u;
+    uint32_t w[4];
+#pragma unroll
+    for (uint32_t j = 0; j < 8; j++) {
+      const uint32_t key = 32u * T + (j < 4u ? 4u * g + j : 16u + 4u * g + (j - 4u));
+      const uint32_t x = key < nkeys ? (uint32_t)v[(uint64_t)key * D + 16u * b + n] : 0u;
+      if (j & 1u) w[j >> 1] |= x << 16; else w[j >> 1] = x;
+    }
+    vt[((((uint64_t)grp * tiles + T) * NB + b) * 4u + g) * 16u + n] = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
+
+#define ATTP_MFMA32(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0)
+
+template <int D>
+__global__ void __launch_bounds__(256)
+k_attn_prefill_mfma(const float* data, float* out, const __half* kv, uint64_t kv_shift, const uint4* __restrict__ vt,
+                    const AttpBases bs, const AttpVt gv, uint32_t H, uint32_t n_quads, uint32_t n_ttiles, uint32_t m,
+                    uint32_t seq0, uint32_t q_stride, uint32_t o_stride, float scale, float cap, uint32_t vt_tiles) {
+  constexpr int KS = D / 32;           // 32-dim steps of the score product
+  constexpr int NB = D / 16;           // 16-dim blocks of the output
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const uint32_t n = lane & 15u, g = lane >> 4;
+  const uint32_t head = (blockIdx.x % n_quads) * 4u + wave;
+  const uint32_t t0 = (n_ttiles - 1u - blockIdx.x / n_quads) * 16u;
+  if (head >= H) return;               // (no barrier in this kernel)
+  const uint32_t rows = min(16u, m - t0);
+  const uint32_t nkeys = seq0 + t0 + rows - 1u;          // cache rows the tile's last query sees
+  const uint32_t n_tiles = (nkeys + 31u) >> 5;
+  const char* kbase = (const char*)(kv + ((uint64_t)bs.kb[head] - kv_shift));
+  const uint4* vbase = vt + (uint64_t)gv.grp[head] * vt_tiles * (NB * 64u) + g * 16u + n;
+
+  // this lane's query (n): dims 32 step + 8g .. + 7, scaled by a power of two into fp16 range, hi + lo
+  h8p_t qh[KS], ql[KS];
+  float inv_s;
+  {
+    float x[KS][8], mx = 0.f;
+    const float* qp = data + (uint64_t)bs.q[head] + (uint64_t)(t0 + min(n, rows - 1u)) * q_stride + 8u * g;
+#pragma unroll
+    for (int st = 0; st < KS; st++) {
+      const f4pu_t a = *(const f4pu_t*)(qp + 32 * st), b = *(const f4pu_t*)(qp + 32 * st + 4);
+      x[st][0] = a.x; x[st][1] = a.y; x[st][2] = a.z; x[st][3] = a.w; x[st][4] = b.x; x[st][5] = b.y; x[st][6] = b.z; x[st][7] = b.w;
+#pragma unroll
+      for (int t = 0; t < 8; t++) { if (n >= rows) x[st][t] = 0.f; mx = fmaxf(mx, fabsf(x[st][t])); }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64)); mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const uint32_t e = (__float_as_uint(mx) >> 23) & 0xFFu;
+    float s = 1.f;
+    inv_s = 1.f;
+    if (e >= 14u && e <= 254u) { s = __uint_as_float((267u - e) << 23); inv_s = __uint_as_float((e - 13u) << 23); }
+#pragma unroll
+    for (int st = 0; st < KS; st++)
+#pragma unroll
+      for (int t = 0; t < 8; t++) {
+        const float xs = x[st][t] * s;
+        const _Float16 hi = (_Float16)xs;
+        qh[st][t] = hi;
+        ql[st][t] = (_Float16)(xs - (float)hi);
+      }
+  }
+  const uint32_t lim = n < rows ? seq0 + t0 + n : 0u;     // cache rows this lane's query sees
+  const bool last = n < rows && t0 + n == m - 1u;
+  const uint64_t sc_row = bs.sc[head];
+
+  f4p_t acc[NB];
+#pragma unroll
+  for (int b = 0; b < NB; b++) acc[b] = (f4p_t){0.f, 0.f, 0.f, 0.f};
+  float m_run = ATTP_NEG, l_run = 0.f;
+
+  struct Tile { uint4 k[2][KS]; uint4 v[NB]; };
+  auto fetch = [&](Tile& t, uint32_t T) {
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) {
+      const uint32_t key = min(32u * T + 16u * kb + n, nkeys - 1u);
+#pragma unroll
+      for (int st = 0; st < KS; st++) t.k[kb][st] = *(const uint4*)(kbase + (uint64_t)key * (2u * D) + 64u * st + 16u * g);
+    }
+#pragma unroll
+    for (int b = 0; b < NB; b++) t.v[b] = vbase[((uint64_t)T * NB + b) * 64u];
+  };
+  auto compute = [&](const Tile& t, uint32_t T) {
+    f4p_t s[2][2];
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) { s[kb][0] = (f4p_t){0.f, 0.f, 0.f, 0.f}; s[kb][1] = s[kb][0]; }
+#pragma unroll
+    for (int st = 0; st < KS; st++)
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++) {
+        const h8p_t ka = __builtin_bit_cast(h8p_t, t.k[kb][st]);
+        s[kb][0] = ATTP_MFMA32(ka, qh[st], s[kb][0]);
+        s[kb][1] = ATTP_MFMA32(ka, ql[st], s[kb][1]);
+      }
+    float v[8], mt = ATTP_NEG;
+    bool ok[8];
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const uint32_t key = 32u * T + 16u * kb + 4u * g + r;
+        const float raw = (s[kb][0][r] + s[kb][1][r]) * inv_s;
+        ok[4 * kb + r] = key < lim;
+        if (ok[4 * kb + r] && last) out[sc_row + key] = raw;
+        v[4 * kb + r] = ok[4 * kb + r] ? prep(raw, scale, cap) : ATTP_NEG;
+        mt = fmaxf(mt, v[4 * kb + r]);
+      }
+    mt = fmaxf(mt, __shfl_xor(mt, 16, 64)); mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float m_new = fmaxf(m_run, mt);
+    const float alpha = __expf(m_run - m_new);
+    const bool moved = m_new > m_run;
+    m_run = m_new;
+    h8p_t ph, pl;
+    float psum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const float pj = ok[j] ? __expf(v[j] - m_new) : 0.f;
+      psum += pj;
+      const _Float16 hi = (_Float16)pj;
+      ph[j] = hi;
+      pl[j] = (_Float16)(pj - (float)hi);
+    }
+    l_run = l_run * alpha + psum;
+    if (__any(moved)) {                 // wave-uniform: most tiles after the first few leave every maximum where it was
+      float a4[4];
+#pragma unroll
+      for (int r = 0; r < 4; r++) a4[r] = __shfl(alpha, (int)(4u * g + r), 64);
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[b][r] *= a4[r];
+    }
+#pragma unroll
+    for (int b = 0; b < NB; b++) {
+      const h8p_t vb = __builtin_bit_cast(h8p_t, t.v[b]);
+      acc[b] = ATTP_MFMA32(ph, vb, acc[b]);
+      acc[b] = ATTP_MFMA32(pl, vb, acc[b]);
+    }
+  };
+
+  Tile A, B;
+  fetch(A, 0u);
+  for (uint32_t T = 0; T < n_tiles; T += 2u) {
+    fetch(B, min(T + 1u, n_tiles - 1u));                 // (past the end: the last tile again, not used)
+    __builtin_amdgcn_sched_barrier(0);
+    compute(A, T);
+    if (T + 1u >= n_tiles) break;
+    fetch(A, min(T + 2u, n_tiles - 1u));
+    __builtin_amdgcn_sched_barrier(0);
+    compute(B, T + 1u);
+  }
+
+  float l_tot = l_run + __shfl_xor(l_run, 16, 64);
+  l_tot += __shfl_xor(l_tot, 32, 64);
+  const float inv_l = 1.0f / l_tot;
+  float il[4];
+#pragma unroll
+  for (int r = 0; r < 4; r++) il[r] = __shfl(inv_l, (int)(4u * g + r), 64);
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    const uint32_t qr = 4u * g + r;
+    if (qr >= rows) continue;
+    float* dst = out + (uint64_t)bs.o[head] + (uint64_t)(t0 + qr) * o_stride + n;
+#pragma unroll
+    for (int b = 0; b < NB; b++) dst[16 * b] = acc[b][r] * il[r];
+  }
+}
+
+// transposed V tiles of the chunk launches: grown on demand, released at shutdown
+static uint4* g_vt = nullptr;
+static size_t g_vt_bytes = 0;
+void attn_prefill_release() {
+  if (g_vt) hipFree(g_vt);
+  g_vt = nullptr; g_vt_bytes = 0;
+}
+
 static bool disjoint_iv(uint64_t a0, uint64_t a1, uint64_t b0, uint64_t b1) { return a1 <= b0 || b1 <= a0; }
 
 // The run of (scores, softmax . V) pairs that starts at q[i]: launches it as one chunk and returns the
@@ -300,6 +509,43 @@ size_t launch_attn_chunk(const std::vector<PendOp>& q, size_t i, int* rc) {
   AttpBases bs;
   for (uint32_t h = 0; h < H; h++) { bs.q[h] = q0[h]; bs.sc[h] = sc[h]; bs.o[h] = o0[h]; bs.kb[h] = kb[h]; bs.vb[h] = vb[h]; }
   float* d = (float*)mp->buf;
+  if (tuning("ADAMAH_ATTN_PREFILL_MFMA", 1) != 0) {
+    // both products on the matrix cores: the visible V rows of every KV head transposed into tiles first
+    AttpVt gv; AttpVtSrc src;
+    uint32_t n_grp = 0;
+    for (uint32_t h = 0; h < H; h++) {
+      uint32_t gi = 0;
+      while (gi < n_grp && src.vb[gi] != vb[h]) gi++;
+      if (gi == n_grp) src.vb[n_grp++] = vb[h];
+      gv.grp[h] = gi;
+    }
+    const uint32_t tiles = cdiv(seq_last, 32u);
+    const size_t need = (size_t)n_grp * tiles * 32u * D * sizeof(__half);
+    bool ok = true;
+    if (need > g_vt_bytes) {
+      hipStreamSynchronize(g.stream);
+      if (g_vt) hipFree(g_vt);
+      g_vt = nullptr; g_vt_bytes = 0;
+      const size_t want = std::max(need + need / 2, (size_t)8 << 20);
+      if (hipMalloc((void**)&g_vt, want) == hipSuccess) g_vt_bytes = want;
+      else { (void)hipGetLastError(); ok = false; }
+      layout_changed();
+    }
+    if (ok) {
+      const uint32_t n_quads = cdiv(H, 4u), n_tt = cdiv(m, 16u);
+#define APM(DD)                                                                                                   \
+  do {                                                                                                            \
+    k_v_tile_transpose<DD><<<dim3(tiles, n_grp), 256, 0, g.stream>>>(mp->kv16, mp->kv_start, src, seq_last, tiles, g_vt); \
+    k_attn_prefill_mfma<DD><<<n_quads * n_tt, 256, 0, g.stream>>>(d, d, mp->kv16, mp->kv_start, g_vt, bs, gv, H, n_quads, n_tt, m, \
+                                                                  s0.n, qs, os, a0.eps, a0.f2, tiles);           \
+  } while (0)
+      if (D == 64) APM(64); else if (D == 128) APM(128); else APM(256);
+#undef APM
+      count_launch(2);
+      *rc = check_launch();
+      return 2 * (size_t)m;
+    }
+  }
   dim3 grid(cdiv(m, 16u), H);
 #define APL(DD, NW) k_attn_prefill<DD, NW><<<grid, NW * 64, 0, g.stream>>>(d, d, mp->kv16, mp->kv_start, bs, m, s0.n, qs, os, a0.eps, a0.f2)
   if (D == 64) APL(64, 4); else if (D == 128) APL(128, 4); else APL(256, 2);

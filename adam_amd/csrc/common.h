@@ -200,6 +200,7 @@ size_t launch_attn_batch(const std::vector<PendOp>& q, size_t i, int* rc);   // 
 int launch_attn_combine_dev(Map* m, const float* partial, const uint32_t* lo_dev, uint32_t n_ops, uint32_t value_dim,
                             uint32_t n_splits);
 void attn_decode_release();
+void attn_prefill_release();   // attn_prefill.hip: the transposed V tiles (shutdown)
 void token_feed_release();      // frees the pinned ring tokens reach the host through (shutdown)
 
 inline void layout_changed() { g.layout_gen++; }

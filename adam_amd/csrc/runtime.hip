@@ -405,6 +405,7 @@ void adamah_shutdown(void) { ADAMAH_API();
   topk_fused_release();
   sampling_release();
   attn_decode_release();
+  attn_prefill_release();
   token_feed_release();
   g.pend.clear();
   for (int i = 0; i < MAX_PLANS; i++) { g.plans[i].clear(); g.plan_active[i] = false; plan_graph_reset(i); }
