@@ -509,8 +509,13 @@ size_t launch_attn_chunk(const std::vector<PendOp>& q, size_t i, int* rc) {
   AttpBases bs;
   for (uint32_t h = 0; h < H; h++) { bs.q[h] = q0[h]; bs.sc[h] = sc[h]; bs.o[h] = o0[h]; bs.kb[h] = kb[h]; bs.vb[h] = vb[h]; }
   float* d = (float*)mp->buf;
-  if (tuning("ADAMAH_ATTN_PREFILL_MFMA", 1) != 0) {
-    // both products on the matrix cores: the visible V rows of every KV head transposed into tiles first
+  // Both products on the matrix cores (a wave per head and 16-token tile) when that gives at least half the CUs a
+  // workgroup; a chunk with few heads or few tokens (Gemma-3-1B: 4 heads, 32 workgroups for 512 tokens) spreads wider on
+  // the kernel above, whose workgroups are one head each and split the cache between their waves.
+  // ADAMAH_ATTN_PREFILL_MFMA: 0 never, 1 by that rule (default), 2 always.
+  const int mfma_mode = tuning("ADAMAH_ATTN_PREFILL_MFMA", 1);
+  if (mfma_mode == 2 || (mfma_mode == 1 && cdiv(H, 4u) * cdiv(m, 16u) * 2u >= (uint32_t)g.n_cu)) {
+    // the visible V rows of every KV head transposed into tiles first
     AttpVt gv; AttpVtSrc src;
     uint32_t n_grp = 0;
     for (uint32_t h = 0; h < H; h++) {

@@ -104,7 +104,15 @@ def test_gqa_heads_with_equal_queries_agree(hip):
             assert np.array_equal(out[g0 * 4], out[g0 * 4 + j])
 
 
-CHUNK_LAUNCHES = 2      # a chunk's attention: the V tiles' transposing pass, then the causal kernel
+# a chunk's attention: one causal kernel -- or, on the matrix-core form (taken by itself for chunks that fill the chip:
+# ADAMAH_ATTN_PREFILL_MFMA=1, the default; forced with 2, off with 0), the V tiles' transposing pass and then the kernel
+CHUNK_LAUNCHES = {"0": 1, "2": 2}
+
+
+@pytest.fixture(params=["0", "2"], ids=["vector-pv", "matrix-pv"])
+def chunk_impl(request, monkeypatch):
+    monkeypatch.setenv("ADAMAH_ATTN_PREFILL_MFMA", request.param)
+    return request.param
 
 
 def chunk_case(g, q, K, V, seq0, cap_len, scale, softcap, gap=0, one_call=False):
@@ -149,7 +157,7 @@ def chunk_case(g, q, K, V, seq0, cap_len, scale, softcap, gap=0, one_call=False)
     (17, 3, 8, 2, 64, 0.0, 8),          # head size 64, padded output rows
     (2, 5, 4, 4, 128, 30.0, 0),         # the shortest run
 ])
-def test_prefill_chunk_is_one_causal_launch(hip, m, seq0, Hq, Hkv, d, softcap, gap):
+def test_prefill_chunk_is_one_causal_launch(hip, chunk_impl, m, seq0, Hq, Hkv, d, softcap, gap):
     """The per-token pairs of a prompt chunk, issued in one batch, run as one causal launch (behind the pass that
     lays the visible V rows out in tiles for the matrix cores) and give what the oracle gives token by token: outputs per token and head within 1e-3 relative L2, and the score rows
     hold the last token's raw scores."""
@@ -162,14 +170,14 @@ def test_prefill_chunk_is_one_causal_launch(hip, m, seq0, Hq, Hkv, d, softcap, g
     note(f"attention chunk m={m} seq0={seq0} {Hq}q/{Hkv}kv d={d}")
     out, scores, launches = chunk_case(hip, q, K, V, seq0, cap_len, scale, softcap, gap)
     ref, ref_scores, _ = chunk_case(oracle.init(), q, K, V, seq0, cap_len, scale, softcap, gap)
-    assert launches == CHUNK_LAUNCHES, launches
+    assert launches == CHUNK_LAUNCHES[chunk_impl], launches
     for t in range(m):
         for h in range(Hq):
             assert rel_l2(out[t, h], ref[t, h]) < TOL, (t, h)
     assert rel_l2(scores, ref_scores) < 1e-5
 
 
-def test_causal_rows_entry_point_equals_the_pairs_issued_one_by_one(hip):
+def test_causal_rows_entry_point_equals_the_pairs_issued_one_by_one(hip, chunk_impl):
     """adamah_attn_causal_rows_dev (an extension: m pairs in one native call) leaves the words the 2 m calls
     leave, in as many launches; the oracle's form of it agrees within the attention bar; bad arguments fail."""
     rng = np.random.default_rng(77)
@@ -182,7 +190,7 @@ def test_causal_rows_entry_point_equals_the_pairs_issued_one_by_one(hip):
     note("attention causal rows entry point")
     a = chunk_case(hip, q, K, V, seq0, cap_len, scale, 20.0, one_call=True)
     b = chunk_case(hip, q, K, V, seq0, cap_len, scale, 20.0)
-    assert a[2] == b[2] == CHUNK_LAUNCHES
+    assert a[2] == b[2] == CHUNK_LAUNCHES[chunk_impl]
     assert np.array_equal(a[0].view(np.uint32), b[0].view(np.uint32)) and np.array_equal(a[1].view(np.uint32), b[1].view(np.uint32))
     ref = chunk_case(oracle.init(), q, K, V, seq0, cap_len, scale, 20.0, one_call=True)
     assert rel_l2(a[0], ref[0]) < TOL and rel_l2(a[1], ref[1]) < 1e-5
@@ -192,7 +200,7 @@ def test_causal_rows_entry_point_equals_the_pairs_issued_one_by_one(hip):
 
 
 @pytest.mark.parametrize("layout,expect", [("hole", 2), ("irregular", 3)])
-def test_prefill_chunk_splits_or_falls_back_when_tokens_do_not_line_up(hip, layout, expect):
+def test_prefill_chunk_splits_or_falls_back_when_tokens_do_not_line_up(hip, chunk_impl, layout, expect):
     """A hole in the query rows after the third token: two chunk launches.  No common stride at all: the
     tokens pair up (any two tokens have a stride), three launches.  Same results either way."""
     rng = np.random.default_rng(9)
@@ -228,7 +236,7 @@ def test_prefill_chunk_splits_or_falls_back_when_tokens_do_not_line_up(hip, layo
                                          0.1, 0.0)
         g.batch_end()
         if g is hip:
-            assert g.get_last_barrier_count() == expect * CHUNK_LAUNCHES
+            assert g.get_last_barrier_count() == expect * CHUNK_LAUNCHES[chunk_impl]
         outs.append(read(g, 0, out_pos, m * Hq * d))
     assert rel_l2(outs[0], outs[1]) < TOL
 
