@@ -156,6 +156,8 @@ def chunk_case(g, q, K, V, seq0, cap_len, scale, softcap, gap=0, one_call=False)
     (64, 200, 32, 8, 128, 0.0, 0),      # Llama-3-8B heads, second chunk of a prompt
     (17, 3, 8, 2, 64, 0.0, 8),          # head size 64, padded output rows
     (2, 5, 4, 4, 128, 30.0, 0),         # the shortest run
+    (33, 100, 6, 3, 64, 0.0, 0),        # heads not a multiple of four; a quad of waves straddles two KV heads
+    (50, 4000, 8, 2, 128, 0.0, 0),      # a short chunk deep into a long context
 ])
 def test_prefill_chunk_is_one_causal_launch(hip, chunk_impl, m, seq0, Hq, Hkv, d, softcap, gap):
     """The per-token pairs of a prompt chunk, issued in one batch, run as one causal launch (behind the pass that
