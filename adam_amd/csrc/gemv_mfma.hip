@@ -111,18 +111,24 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
   // ks > 1 (store only, short matrices with long rows): ks neighbouring waves share one bundle and take
   // every ks-th step of K each; a workgroup holds nwav / ks bundles, one round.
   uint32_t grp = blockIdx.x, first, stride, seg_end;
-  const uint32_t kpart = ks > 1u ? wave % ks : 0u;
+  const uint32_t ksh = ks >> 1;                        // ks is 1, 2 or 4: its logarithm
+  const uint32_t kpart = wave & (ks - 1u);
   if (EPI == EPI_STORE && ks > 1u) {
-    const uint32_t bundle = blockIdx.x * (nwav / ks) + wave / ks;
+    const uint32_t bundle = blockIdx.x * (nwav >> ksh) + (wave >> ksh);
     first = bundle * 4u;
     seg_end = kpart < C ? min(N, first + 4u) : 0u;      // nothing to do: no bundle, or no step of K left for this wave
     if (first >= N) seg_end = 0u;
     stride = 4u;
   } else if (EPI == EPI_STORE) {
     const uint32_t slot = (wave & 3u) * (nwav >> 2) + (wave >> 2);
-    const uint64_t n_q = (N + 3u) / 4u, gw = (uint64_t)blockIdx.x * nwav + slot, wt = (uint64_t)gridDim.x * nwav;
-    first = (uint32_t)(gw * n_q / wt) * 4u;
-    seg_end = min(N, (uint32_t)((gw + 1) * n_q / wt) * 4u);
+    // balanced shares without a division (see GemvFuse::sh_q): a 64-bit quotient here is a few hundred instructions
+    // and two jumps to the far end of the kernel, in front of the wave's first loads and with a cold instruction cache
+    const uint32_t gw = blockIdx.x * nwav + slot;
+    auto share = [&](uint32_t gq) -> uint32_t {
+      return gq * fz.sh_q + (uint32_t)(((uint64_t)(gq * fz.sh_r) * fz.sh_m) >> fz.sh_s);
+    };
+    first = share(gw) * 4u;
+    seg_end = min(N, share(gw + 1u) * 4u);
     stride = 4u;
   } else {
     first = grp * rows_per_group + wave * 4u;
@@ -565,8 +571,9 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
       // steps t = 0..T-1 in (row bundle, chunk) order; register set A holds step 0 on entry.  The
       // prefetch of the following step is issued unconditionally (past the end it re-reads the last
       // rows, clamped in load()), so the number of loads in flight at every wait is known statically.
-      const uint32_t Cw = (C - kpart + ks - 1u) / ks;     // steps of K this wave takes per bundle
-      const uint32_t T = ((seg_end - first + stride - 1u) / stride) * Cw;
+      const uint32_t Cw = (C - kpart + ks - 1u) >> ksh;     // steps of K this wave takes per bundle
+      // (stride is 4 or 4 * waves per workgroup: a power of two)
+      const uint32_t T = ((seg_end - first + stride - 1u) >> (EPI == EPI_STORE ? 2u : (uint32_t)__builtin_ctz(stride))) * Cw;
       uint32_t row_a = first, ch_a = kpart, row_b, ch_b, row_n = first, ch_n = kpart;
       if ((ch_n += ks) >= C) { ch_n = kpart; row_n += stride; }
       if (T == 1) compute(A, first, kpart, seg_end);   // nothing to prefetch
@@ -670,9 +677,18 @@ static void launch_mfma_p(int fmt, uint32_t grid, uint32_t threads, const Map* m
   const bool norm = PRO == PRO_RMSNORM || PRO == PRO_NORM2;
   const uint32_t x_src = norm ? fz.p_src : a;
   const float* n_wt = norm ? fz.p_wt : act;
+  GemvFuse fzs = fz;
+  if (EPI == EPI_STORE && ks == 1u) {   // the shares of the bundles (GemvFuse::sh_q)
+    while (grid * (threads >> 6) > 16384u) grid >>= 1;   // keeps g * sh_r below 2^28 (no launch shape comes near)
+    const uint32_t n_q = cdiv(N, 4u), wt = grid * (threads >> 6);
+    uint32_t lg = 0;
+    while ((1u << lg) < wt) lg++;
+    fzs.sh_q = n_q / wt; fzs.sh_r = n_q % wt; fzs.sh_s = 28u + lg;
+    fzs.sh_m = (uint32_t)((((uint64_t)1 << fzs.sh_s) + wt - 1u) / wt);
+  }
 #define MK(F, R, UU)                                                                                              \
   k_gemv_mfma<F, EPI, R, PRO, UU><<<grid, threads, smem, g.stream>>>(act, mw->buf, mw->d16, K, N, ks, x_src, b, n_wt, fz.p_src2, act_out, c, \
-                                                                     mw->qp, lidx, lval, rpg, n_groups, fz)
+                                                                     mw->qp, lidx, lval, rpg, n_groups, fzs)
   // (the shorter steps exist in the clamping form only: they are chosen for rows that do not fill steps of 64)
   if (fmt == FMT_Q4_B16) {
     if (U == 3u) MK(FMT_Q4_B16, true, 3);
