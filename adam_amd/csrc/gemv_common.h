@@ -107,11 +107,6 @@ struct GemvFuse {
   // EPIX_GEGLU / SWIGLU: the matrix is [gate rows; up rows], e_dst[i] = act(y[i]) * y[N/2 + i]
   uint32_t e_mode;
   uint32_t e_res, e_dst;
-  // Set by the launcher (store variant with one wave per bundle): the 4-row bundles are dealt out to the launch's wt
-  // waves in contiguous balanced shares, wave g taking bundles [f(g), f(g + 1)), f(g) = floor(g * n_q / wt) =
-  // g * sh_q + floor(g * sh_r / wt) with sh_q = n_q / wt, sh_r = n_q % wt, and the last quotient as a multiplication
-  // by sh_m = ceil(2^sh_s / wt) and a shift (exact for g * sh_r < 2^28): the kernel divides nothing.
-  uint32_t sh_q, sh_r, sh_m, sh_s;
 };
 // Threads per workgroup the launchers will use for a matrix with N rows (store variant).
 uint32_t mfma_store_threads(uint32_t K, uint32_t N);

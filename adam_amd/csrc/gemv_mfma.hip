@@ -79,15 +79,17 @@ struct PreMT {
 // stages the activations; their results are also stored where the unfused ops would have put them.
 template <int FMT, int EPI, bool RAGGED, int PRO, int MF_U>
 __global__ void __launch_bounds__(1024)
-k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __restrict__ d16, uint32_t K, uint32_t N, uint32_t ks,
-            uint32_t x_src, uint32_t b_off, const float* n_wt, uint32_t n_w,
-            float* act_out, uint32_t c_out, const float2* __restrict__ qp, const uint32_t* __restrict__ lidx,
-            const uint32_t* __restrict__ lval, uint32_t rows_per_group, uint32_t n_groups, GemvFuse fz) {
-  // The first 14 dwords of the arguments are in registers when a wave starts (the rest is fetched from the argument
-  // block, a trip to memory): what the first loads need stands in front -- the activations and where they start
-  // (x_src: the vector itself, or the source of the first folded norm, whose weights are n_wt + n_w), the weights,
-  // K, N and the K split.
-  const uint32_t a = x_src;
+k_gemv_mfma(const float* xp, const uint8_t* __restrict__ W, const __half* __restrict__ d16, const float* nwp, uint32_t K, uint32_t N,
+            uint32_t cfg, uint32_t w0, uint32_t w1, uint32_t w2,
+            const float* act, float* act_out, uint32_t c_out, const float2* __restrict__ qp, const uint32_t* __restrict__ lidx,
+            const uint32_t* __restrict__ lval, uint32_t n_groups, GemvFuse fz) {
+  // The first 14 dwords of the arguments are in registers when a wave starts; the rest is fetched from the argument
+  // block, a trip to memory that nothing in front of a wave's first loads may wait for.  So everything those loads
+  // need stands in front, with the offsets folded into the pointers by the launcher: xp = the activation vector (or
+  // the source of the first folded norm, whose weights start at nwp), W / d16 (and, behind, qp) = the matrix's first
+  // block, K, N, cfg = ks | threads per workgroup << 3 | epilogue << 14 | share shift << 16, and w0..w2 = the
+  // multiply-and-shift form of the waves' row shares (store) or, w0, the rows per group (argmax).
+  const uint32_t ks = cfg & 7u, e_mode = (cfg >> 14) & 3u;
   using PreM = PreMT<MF_U>;
   constexpr uint32_t SB = 16u * MF_U;                 // blocks per step
   constexpr bool B16 = (FMT == FMT_Q4_B16);
@@ -100,10 +102,9 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
   const uint32_t nblk = K >> 5;
   const uint32_t C = (nblk + SB - 1u) / SB;           // steps per row bundle
 
-  const uint32_t tid = threadIdx.x, lane = tid & 63u, nthr = blockDim.x, nwav = nthr >> 6;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, nthr = (cfg >> 3) & 0x7FFu, nwav = nthr >> 6;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t l = lane & 3u, bcol = lane >> 2;      // row in bundle, block column 0..15
-  const uint64_t gbase = (uint64_t)b_off >> 5;
 
   // ---- this wave's rows: store = contiguous balanced share of the 4-row bundles (waves that share
   // a SIMD, w % 4, take neighbouring shares so that every SIMD gets the same load); argmax = the
@@ -121,24 +122,27 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
     stride = 4u;
   } else if (EPI == EPI_STORE) {
     const uint32_t slot = (wave & 3u) * (nwav >> 2) + (wave >> 2);
-    // balanced shares without a division (see GemvFuse::sh_q): a 64-bit quotient here is a few hundred instructions
+    // balanced shares without a division: a 64-bit quotient here is a few hundred instructions
     // and two jumps to the far end of the kernel, in front of the wave's first loads and with a cold instruction cache
     const uint32_t gw = blockIdx.x * nwav + slot;
+    // wave g takes bundles [f(g), f(g + 1)), f(g) = floor(g * n_q / wt) = g * w0 + floor(g * w1 / wt) with
+    // w0 = n_q / wt, w1 = n_q % wt and the last quotient as a multiplication by w2 = ceil(2^s / wt) and a shift
+    // (exact for g * w1 < 2^28)
     auto share = [&](uint32_t gq) -> uint32_t {
-      return gq * fz.sh_q + (uint32_t)(((uint64_t)(gq * fz.sh_r) * fz.sh_m) >> fz.sh_s);
+      return gq * w0 + (uint32_t)(((uint64_t)(gq * w1) * w2) >> (cfg >> 16));
     };
     first = share(gw) * 4u;
     seg_end = min(N, share(gw + 1u) * 4u);
     stride = 4u;
   } else {
-    first = grp * rows_per_group + wave * 4u;
-    seg_end = min(N, (grp + 1) * rows_per_group);
+    first = grp * w0 + wave * 4u;
+    seg_end = min(N, (grp + 1) * w0);
     stride = 4u * nwav;
   }
 
   // Row of lane-row l in the bundle that starts at row0.  With the gated-activation epilogue the
   // matrix is [gate rows; up rows] (N/2 each) and a bundle pairs two gate rows with their up rows.
-  const bool glu = EPI == EPI_STORE && (fz.e_mode == EPIX_GEGLU || fz.e_mode == EPIX_SWIGLU);
+  const bool glu = EPI == EPI_STORE && (e_mode == EPIX_GEGLU || e_mode == EPIX_SWIGLU);
   auto row_of = [&](uint32_t row0, uint32_t end) -> uint32_t {
     if (glu) return (row0 >> 1) + (l & 1u) + (l >> 1) * (N >> 1);
     return min(row0 + l, end - 1u);
@@ -150,13 +154,13 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
   const uint32_t ll = lane >> 4, lbcol = lane & 15u;
   auto load = [&](PreM& R, uint32_t row0, uint32_t chunk, uint32_t end) {
     const uint32_t row = glu ? (row0 >> 1) + (ll & 1u) + (ll >> 1) * (N >> 1) : min(row0 + ll, end - 1u);
-    const uint64_t g0 = gbase + (uint64_t)row * nblk + chunk * SB + lbcol;
+    const uint64_t g0 = (uint64_t)row * nblk + chunk * SB + lbcol;
 #pragma unroll
     for (uint32_t u = 0; u < MF_U; u++) {
       uint64_t gi = g0 + u * 16u;
       // blocks past the end of the row are clamped, not skipped: the number of loads per step has to be
       // fixed for the prefetch to stay ahead (see the step loop)
-      if (RAGGED) gi = gbase + (uint64_t)row * nblk + min(chunk * SB + u * 16u + lbcol, nblk - 1u);
+      if (RAGGED) gi = (uint64_t)row * nblk + min(chunk * SB + u * 16u + lbcol, nblk - 1u);
       // the codes are read once per launch and not again before the next token: non-temporal, so that they do not
       // push the step's small, re-read data (activations, KV rows, slice partials) out of the L2
       const u4v_t t = __builtin_nontemporal_load((const u4v_t*)(W + (gi << 4)));
@@ -168,7 +172,7 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
     // 4 * column + row, column 0 stores), so it has arrived long before the row sum is complete.  Every lane asks at
     // every step (without the epilogue: for a word of the activations, not used): a load under a branch would leave
     // the compiler unable to count the loads in flight, and it then waits for all of them wherever it waits for one.
-    if (EPI == EPI_STORE) R.res = act[fz.e_mode == EPIX_ADD ? (uint64_t)fz.e_res + min(row0 + l, end - 1u) : (uint64_t)a];
+    if (EPI == EPI_STORE) R.res = *(e_mode == EPIX_ADD ? act + ((uint64_t)fz.e_res + min(row0 + l, end - 1u)) : xp);
   };
 
   PreM A, B;   // A's first loads stay in flight while the activations are staged
@@ -247,7 +251,7 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
     auto x_round = [&](uint32_t i0, bool with_weights) {
       float x[4][8];
 #pragma unroll
-      for (uint32_t u = 0; u < 4; u++) load8(act + a + (uint64_t)min(i0 + u * nthr + tid, nw - 1u) * 8u, x[u]);
+      for (uint32_t u = 0; u < 4; u++) load8(xp + (uint64_t)min(i0 + u * nthr + tid, nw - 1u) * 8u, x[u]);
       if (with_weights) {
         __builtin_amdgcn_sched_barrier(0);
         first_loads();
@@ -361,8 +365,8 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
       for (int k = 0; k < 8; k++) { v[u][k] = 0.f; wv[u][k] = 0.f; rv[u][k] = 0.f; w2v[u][k] = 0.f; }
       // (waves without words of their own load the row's last word: every path issues the same loads)
       const uint64_t e0 = (uint64_t)min(i, nw - 1u) * 8u;
-      load8(act + x_src + e0, v[u]);
-      load8(n_wt + n_w + e0, wv[u]);
+      load8(xp + e0, v[u]);
+      load8(nwp + e0, wv[u]);
       if (PRO == PRO_NORM2) { load8(act + fz.p_res + e0, rv[u]); load8(fz.p_wt2 + fz.p_w2 + e0, w2v[u]); }
     }
     __builtin_amdgcn_sched_barrier(0);   // activation loads first: they are waited for first
@@ -530,7 +534,7 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
           const uint32_t row = row_of(row0, end);
           act_out[(uint64_t)c_out + row] = y;
           if (lane < 2u) {
-            const float t = fz.e_mode == EPIX_GEGLU ? gelu_tanh(y) * yu : (y / (1.0f + expf(-y))) * yu;
+            const float t = e_mode == EPIX_GEGLU ? gelu_tanh(y) * yu : (y / (1.0f + expf(-y))) * yu;
             act_out[(uint64_t)fz.e_dst + row] = t;
           }
         }
@@ -539,7 +543,7 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
         if (row < end && bcol == 0u) {
           if (EPI == EPI_STORE) {
             act_out[(uint64_t)c_out + row] = y;
-            if (fz.e_mode == EPIX_ADD) act_out[(uint64_t)fz.e_dst + row] = Rl.res + y;
+            if (e_mode == EPIX_ADD) act_out[(uint64_t)fz.e_dst + row] = Rl.res + y;
           } else if (better(y, row, best_v, best_i)) { best_v = y; best_i = row; }
         }
       }
@@ -604,7 +608,7 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
         const uint32_t row = first + l;
         if (row < N && bcol == 0u) {
           act_out[(uint64_t)c_out + row] = y;
-          if (fz.e_mode == EPIX_ADD) act_out[(uint64_t)fz.e_dst + row] = res_keep + y;
+          if (e_mode == EPIX_ADD) act_out[(uint64_t)fz.e_dst + row] = res_keep + y;
         }
       }
       break;
@@ -615,8 +619,8 @@ k_gemv_mfma(const float* act, const uint8_t* __restrict__ W, const __half* __res
     grp += gridDim.x;
     const bool more = grp < n_groups;
     if (more) {
-      first = grp * rows_per_group + wave * 4u;
-      seg_end = min(N, (grp + 1) * rows_per_group);
+      first = grp * w0 + wave * 4u;
+      seg_end = min(N, (grp + 1) * w0);
       if (first < seg_end) load(A, first, 0, seg_end);
     }
     // lanes 0..3 hold the best of their own rows
@@ -677,18 +681,24 @@ static void launch_mfma_p(int fmt, uint32_t grid, uint32_t threads, const Map* m
   const bool norm = PRO == PRO_RMSNORM || PRO == PRO_NORM2;
   const uint32_t x_src = norm ? fz.p_src : a;
   const float* n_wt = norm ? fz.p_wt : act;
-  GemvFuse fzs = fz;
-  if (EPI == EPI_STORE && ks == 1u) {   // the shares of the bundles (GemvFuse::sh_q)
-    while (grid * (threads >> 6) > 16384u) grid >>= 1;   // keeps g * sh_r below 2^28 (no launch shape comes near)
+  // (the kernel's argument list says what goes where and why)
+  uint32_t w0 = rpg, w1 = 0, w2 = 0, sh = 0;
+  if (EPI == EPI_STORE && ks == 1u) {   // the shares of the bundles
+    while (grid * (threads >> 6) > 16384u) grid >>= 1;   // keeps g * w1 below 2^28 (no launch shape comes near)
     const uint32_t n_q = cdiv(N, 4u), wt = grid * (threads >> 6);
     uint32_t lg = 0;
     while ((1u << lg) < wt) lg++;
-    fzs.sh_q = n_q / wt; fzs.sh_r = n_q % wt; fzs.sh_s = 28u + lg;
-    fzs.sh_m = (uint32_t)((((uint64_t)1 << fzs.sh_s) + wt - 1u) / wt);
+    sh = 28u + lg;
+    w0 = n_q / wt; w1 = n_q % wt; w2 = (uint32_t)((((uint64_t)1 << sh) + wt - 1u) / wt);
   }
+  const uint32_t cfg = ks | (threads << 3) | ((EPI == EPI_STORE ? fz.e_mode : 0u) << 14) | (sh << 16);
+  const uint64_t blk0 = (uint64_t)b >> 5;
+  const uint8_t* Wp = (const uint8_t*)mw->buf + (blk0 << 4);
+  const __half* d16p = mw->d16 ? mw->d16 + blk0 : nullptr;
+  const float2* qpp = mw->qp ? mw->qp + blk0 : nullptr;
 #define MK(F, R, UU)                                                                                              \
-  k_gemv_mfma<F, EPI, R, PRO, UU><<<grid, threads, smem, g.stream>>>(act, mw->buf, mw->d16, K, N, ks, x_src, b, n_wt, fz.p_src2, act_out, c, \
-                                                                     mw->qp, lidx, lval, rpg, n_groups, fzs)
+  k_gemv_mfma<F, EPI, R, PRO, UU><<<grid, threads, smem, g.stream>>>(act + x_src, Wp, d16p, n_wt + fz.p_src2, K, N, cfg, w0, w1, w2,    \
+                                                                     act, act_out, c, qpp, lidx, lval, n_groups, fz)
   // (the shorter steps exist in the clamping form only: they are chosen for rows that do not fill steps of 64)
   if (fmt == FMT_Q4_B16) {
     if (U == 3u) MK(FMT_Q4_B16, true, 3);
