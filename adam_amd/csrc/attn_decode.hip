@@ -115,8 +115,15 @@ k_attn_decode(const float* data, const __half* kv, uint64_t kv_shift, uint32_t r
   // 0xFFFFFFFF is not stored.
   const uint32_t n_all = gridDim.y * (uint32_t)G;
   const uint32_t *e_q = ext, *e_sc = ext + n_all, *e_o = ext + 2u * n_all, *e_kb = ext + 3u * n_all, *e_vb = e_kb + gridDim.y;
-  const char* kbase = (const char*)(kv + ((uint64_t)(EXT ? e_kb[group] : bs.kb[group]) - kv_shift));
-  const char* vbase = (const char*)(kv + ((uint64_t)(EXT ? e_vb[group] : bs.vb[group]) - kv_shift));
+  // (set where the first tile is asked for: with the row preparation the bases come from the part of the argument
+  // block that is not in registers at the start, and the raw rows' loads go out before anything waits for it)
+  const char *kbase = nullptr, *vbase = nullptr;
+  const uint32_t kb_g = EXT ? e_kb[group] : bs.kb[group], vb_g = EXT ? e_vb[group] : bs.vb[group];   // asked for here
+  auto set_bases = [&]() {                                                                           // waited for here
+    kbase = (const char*)(kv + ((uint64_t)kb_g - kv_shift));
+    vbase = (const char*)(kv + ((uint64_t)vb_g - kv_shift));
+  };
+  if (!RP) set_bases();
   const uint32_t klane = 16u * kc, vlane = 2u * (uint32_t)DPL * lane;
 
   auto fetch = [&](uint4 (&kr)[NI], uint32_t (&vr)[16][DW], uint32_t rb) {
@@ -188,6 +195,13 @@ k_attn_decode(const float* data, const __half* kv, uint64_t kv_shift, uint32_t r
         vraw = data[(uint64_t)rp_v_src + (uint64_t)group * D + d];
       }
       float fr[PN], wq[PN][2], wk[2];
+#pragma unroll
+      for (uint32_t u = 0; u < PN; u++) fr[u] = rp_inv_freq[(tid + u * NT) % half];
+      // Everything above is addressed from the arguments that are in registers when the wave starts; what follows
+      // needs the rest of the argument block (a trip to memory), and the fence keeps that wait from being scheduled
+      // in front of the raw rows' loads.
+      __builtin_amdgcn_sched_barrier(0);
+      set_bases();
       const bool nrm = (rp.flags & 1u) != 0u;
       {
         const float* wqp = nrm ? data + rp.q_w : rp_inv_freq;     // no norm: any readable address, the value is not used
@@ -196,7 +210,6 @@ k_attn_decode(const float* data, const __half* kv, uint64_t kv_shift, uint32_t r
 #pragma unroll
         for (uint32_t u = 0; u < PN; u++) {
           const uint32_t i = (tid + u * NT) % half;
-          fr[u] = rp_inv_freq[i];
           wq[u][0] = wqp[i]; wq[u][1] = wqp[i + hs];
         }
         wk[0] = wkp[tid % half]; wk[1] = wkp[tid % half + hs];
