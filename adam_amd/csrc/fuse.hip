@@ -345,7 +345,7 @@ void flush_pending() {
       if (ai + 1 < n && q[ai + 1].kind == PK_GEMV && q[ai + 1].map_act == at.map_act) {
         const PendOp& gp = q[ai + 1];
         const uint32_t* oh = res_host(at.h[2], at.rpg);
-        fold = oh && gp.a == oh[0] && gp.k == at.rpg * at.k && (at.k & 7u) == 0 && disjoint(gp.c, gp.n, gp.a, gp.k);
+        fold = oh && gp.a == oh[0] && gp.k == at.rpg * at.k && (at.k & 7u) == 0 && at.k <= 8184u && disjoint(gp.c, gp.n, gp.a, gp.k);
         for (uint32_t h = 1; fold && h < at.rpg; h++) fold = oh[h] == oh[0] + h * at.k;
         // a merging GEMV may also have to put the token's prepared queries in place (workgroup 0, while others
         // already store result rows): its results must lie clear of those rows

@@ -87,9 +87,12 @@ k_gemv_mfma(const float* xp, const uint8_t* __restrict__ W, const __half* __rest
   // block, a trip to memory that nothing in front of a wave's first loads may wait for.  So everything those loads
   // need stands in front, with the offsets folded into the pointers by the launcher: xp = the activation vector (or
   // the source of the first folded norm, whose weights start at nwp), W / d16 (and, behind, qp) = the matrix's first
-  // block, K, N, cfg = ks | threads per workgroup << 3 | epilogue << 14 | share shift << 16, and w0..w2 = the
-  // multiply-and-shift form of the waves' row shares (store) or, w0, the rows per group (argmax).
-  const uint32_t ks = cfg & 7u, e_mode = (cfg >> 14) & 3u;
+  // block, K, N, cfg = ks | waves per workgroup << 3 | epilogue << 8 | (share shift - 28) << 10 | (slices - 1) << 14 |
+  // value_dim / 8 << 22 (the last two: PRO_COMBINE, whose partials start at nwp), and w0..w2 = the multiply-and-shift
+  // form of the waves' row shares (store) or, w0, the rows per group (argmax).
+  const uint32_t ks = cfg & 7u, e_mode = (cfg >> 8) & 3u;
+  const float* c_partial = nwp;
+  const uint32_t c_splits = ((cfg >> 14) & 0xFFu) + 1u, c_vd = (cfg >> 22) << 3;
   using PreM = PreMT<MF_U>;
   constexpr uint32_t SB = 16u * MF_U;                 // blocks per step
   constexpr bool B16 = (FMT == FMT_Q4_B16);
@@ -102,7 +105,7 @@ k_gemv_mfma(const float* xp, const uint8_t* __restrict__ W, const __half* __rest
   const uint32_t nblk = K >> 5;
   const uint32_t C = (nblk + SB - 1u) / SB;           // steps per row bundle
 
-  const uint32_t tid = threadIdx.x, lane = tid & 63u, nthr = (cfg >> 3) & 0x7FFu, nwav = nthr >> 6;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, nwav = (cfg >> 3) & 31u, nthr = nwav << 6;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t l = lane & 3u, bcol = lane >> 2;      // row in bundle, block column 0..15
 
@@ -129,7 +132,7 @@ k_gemv_mfma(const float* xp, const uint8_t* __restrict__ W, const __half* __rest
     // w0 = n_q / wt, w1 = n_q % wt and the last quotient as a multiplication by w2 = ceil(2^s / wt) and a shift
     // (exact for g * w1 < 2^28)
     auto share = [&](uint32_t gq) -> uint32_t {
-      return gq * w0 + (uint32_t)(((uint64_t)(gq * w1) * w2) >> (cfg >> 16));
+      return gq * w0 + (uint32_t)(((uint64_t)(gq * w1) * w2) >> (28u + ((cfg >> 10) & 15u)));
     };
     first = share(gw) * 4u;
     seg_end = min(N, share(gw + 1u) * 4u);
@@ -267,7 +270,7 @@ k_gemv_mfma(const float* xp, const uint8_t* __restrict__ W, const __half* __rest
   } else if (PRO == PRO_COMBINE) {
     // Folded merge of the attention partials (same arithmetic as the stand-alone merge kernel):
     // M = max m_s, w_s = e^(m_s - M), L = sum l_s w_s, x = sum_s o_s w_s / L, per head.
-    const uint32_t stride = fz.c_vd + 2u;
+    const uint32_t stride = c_vd + 2u;
     // At most eight slices and two threads per word: straight-line form.  A thread merges four elements: every value
     // it needs and the slices' (max, sum) pairs are asked for in one round, ahead of the first weights (loads return
     // in order: behind the weights they would wait for the weights' trip to memory as well).  Slices past the last
@@ -275,10 +278,10 @@ k_gemv_mfma(const float* xp, const uint8_t* __restrict__ W, const __half* __rest
     // the thread's group of eight lanes, which all work on the same head (value_dim a multiple of 32).  The merged
     // elements meet in LDS (in the digits' place, before there are digits), where each word's thread picks them up.
     // Same order of operations per element as the loops below.
-    const bool few = EPI == EPI_STORE && fz.c_splits <= 8u && 2u * nw <= nthr && fz.c_vd % 32u == 0u;
+    const bool few = EPI == EPI_STORE && c_splits <= 8u && 2u * nw <= nthr && c_vd % 32u == 0u;
     if (few) {
-      const uint32_t e0 = min(tid, 2u * nw - 1u) * 4u, head = e0 / fz.c_vd, j0 = e0 % fz.c_vd, last = fz.c_splits - 1u;
-      const float* pp = fz.c_partial + (uint64_t)head * fz.c_splits * stride;
+      const uint32_t e0 = min(tid, 2u * nw - 1u) * 4u, head = e0 / c_vd, j0 = e0 % c_vd, last = c_splits - 1u;
+      const float* pp = c_partial + (uint64_t)head * c_splits * stride;
       const float* pm = pp + (uint64_t)min(lane & 7u, last) * stride;
       const float m_own = pm[0], l_own = pm[1];
       f4u_t o[8];
@@ -294,12 +297,12 @@ k_gemv_mfma(const float* xp, const uint8_t* __restrict__ W, const __half* __rest
         lv[sp] = __shfl(l_own, (int)((lane & ~7u) + sp), 64);
       }
 #pragma unroll
-      for (uint32_t sp = 0; sp < 8u; sp++) M = sp < fz.c_splits ? fmaxf(M, mv[sp]) : M;
+      for (uint32_t sp = 0; sp < 8u; sp++) M = sp < c_splits ? fmaxf(M, mv[sp]) : M;
       f4u_t x4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (uint32_t sp = 0; sp < 8u; sp++) {
         const float wgt = expf(mv[sp] - M);
-        const bool on = sp < fz.c_splits;
+        const bool on = sp < c_splits;
         L = on ? fmaf(lv[sp], wgt, L) : L;
         x4.x = on ? fmaf(o[sp].x, wgt, x4.x) : x4.x; x4.y = on ? fmaf(o[sp].y, wgt, x4.y) : x4.y;
         x4.z = on ? fmaf(o[sp].z, wgt, x4.z) : x4.z; x4.w = on ? fmaf(o[sp].w, wgt, x4.w) : x4.w;
@@ -320,12 +323,12 @@ k_gemv_mfma(const float* xp, const uint8_t* __restrict__ W, const __half* __rest
       first_loads();
       for (uint32_t i0 = 0; i0 < nw; i0 += nthr) {
         const uint32_t i = i0 + tid, ic = min(i, nw - 1u);
-        const uint32_t head = (ic * 8u) / fz.c_vd, j0 = (ic * 8u) % fz.c_vd;
-        const float* pp = fz.c_partial + (uint64_t)head * fz.c_splits * stride;
+        const uint32_t head = (ic * 8u) / c_vd, j0 = (ic * 8u) % c_vd;
+        const float* pp = c_partial + (uint64_t)head * c_splits * stride;
         float M = -9.99999968e+37f;
-        for (uint32_t sp = 0; sp < fz.c_splits; sp++) M = fmaxf(M, pp[(uint64_t)sp * stride]);
+        for (uint32_t sp = 0; sp < c_splits; sp++) M = fmaxf(M, pp[(uint64_t)sp * stride]);
         float L = 0.f, x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (uint32_t sp = 0; sp < fz.c_splits; sp++) {
+        for (uint32_t sp = 0; sp < c_splits; sp++) {
           const float wgt = expf(pp[(uint64_t)sp * stride] - M);
           L = fmaf(pp[(uint64_t)sp * stride + 1], wgt, L);
           float o[8];
@@ -367,7 +370,17 @@ k_gemv_mfma(const float* xp, const uint8_t* __restrict__ W, const __half* __rest
       const uint64_t e0 = (uint64_t)min(i, nw - 1u) * 8u;
       load8(xp + e0, v[u]);
       load8(nwp + e0, wv[u]);
-      if (PRO == PRO_NORM2) { load8(act + fz.p_res + e0, rv[u]); load8(fz.p_wt2 + fz.p_w2 + e0, w2v[u]); }
+    }
+    if (PRO == PRO_NORM2) {
+      // the second norm's operands are addressed from the part of the argument block that is fetched from memory:
+      // behind a fence, so that the loads above do not wait for it
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (uint32_t u = 0; u < PRO_WPT; u++) {
+        const uint64_t e0 = (uint64_t)min(u * nthr + tid, nw - 1u) * 8u;
+        load8(act + fz.p_res + e0, rv[u]);
+        load8(fz.p_wt2 + fz.p_w2 + e0, w2v[u]);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);   // activation loads first: they are waited for first
     first_loads();
@@ -688,16 +701,18 @@ static void launch_mfma_p(int fmt, uint32_t grid, uint32_t threads, const Map* m
     const uint32_t n_q = cdiv(N, 4u), wt = grid * (threads >> 6);
     uint32_t lg = 0;
     while ((1u << lg) < wt) lg++;
-    sh = 28u + lg;
-    w0 = n_q / wt; w1 = n_q % wt; w2 = (uint32_t)((((uint64_t)1 << sh) + wt - 1u) / wt);
+    sh = lg;
+    w0 = n_q / wt; w1 = n_q % wt; w2 = (uint32_t)((((uint64_t)1 << (28u + lg)) + wt - 1u) / wt);
   }
-  const uint32_t cfg = ks | (threads << 3) | ((EPI == EPI_STORE ? fz.e_mode : 0u) << 14) | (sh << 16);
+  uint32_t cfg = ks | ((threads >> 6) << 3) | ((EPI == EPI_STORE ? fz.e_mode : 0u) << 8) | (sh << 10);
+  if (PRO == PRO_COMBINE) cfg |= ((fz.c_splits - 1u) & 0xFFu) << 14 | (fz.c_vd >> 3) << 22;   // (the fold checks the ranges)
+  const float* nwp = PRO == PRO_COMBINE ? fz.c_partial : n_wt + fz.p_src2;
   const uint64_t blk0 = (uint64_t)b >> 5;
   const uint8_t* Wp = (const uint8_t*)mw->buf + (blk0 << 4);
   const __half* d16p = mw->d16 ? mw->d16 + blk0 : nullptr;
   const float2* qpp = mw->qp ? mw->qp + blk0 : nullptr;
 #define MK(F, R, UU)                                                                                              \
-  k_gemv_mfma<F, EPI, R, PRO, UU><<<grid, threads, smem, g.stream>>>(act + x_src, Wp, d16p, n_wt + fz.p_src2, K, N, cfg, w0, w1, w2,    \
+  k_gemv_mfma<F, EPI, R, PRO, UU><<<grid, threads, smem, g.stream>>>(act + x_src, Wp, d16p, nwp, K, N, cfg, w0, w1, w2,    \
                                                                      act, act_out, c, qpp, lidx, lval, n_groups, fz)
   // (the shorter steps exist in the clamping form only: they are chosen for rows that do not fill steps of 64)
   if (fmt == FMT_Q4_B16) {
