@@ -93,6 +93,11 @@ k_gemv_mfma(const float* xp, const uint8_t* __restrict__ W, const __half* __rest
   const uint32_t ks = cfg & 7u, e_mode = (cfg >> 8) & 3u;
   const float* c_partial = nwp;
   const uint32_t c_splits = ((cfg >> 14) & 0xFFu) + 1u, c_vd = (cfg >> 22) << 3;
+  // Gated activation, split form (bit 14 of cfg where the prologue is not the merge): half of a workgroup's waves take
+  // gate rows, the other half the matching up rows, plain bundles of four neighbouring rows each; the results meet in
+  // LDS at the end of the workgroup.  (In the paired form a bundle is two gate rows and their two up rows, and every
+  // wave reads from both halves of the matrix, which costs about a microsecond at 28672 x 4096.)
+  const bool glu_split = EPI == EPI_STORE && PRO != PRO_COMBINE && ((cfg >> 14) & 1u) != 0u;
   using PreM = PreMT<MF_U>;
   constexpr uint32_t SB = 16u * MF_U;                 // blocks per step
   constexpr bool B16 = (FMT == FMT_Q4_B16);
@@ -115,6 +120,7 @@ k_gemv_mfma(const float* xp, const uint8_t* __restrict__ W, const __half* __rest
   // ks > 1 (store only, short matrices with long rows): ks neighbouring waves share one bundle and take
   // every ks-th step of K each; a workgroup holds nwav / ks bundles, one round.
   uint32_t grp = blockIdx.x, first, stride, seg_end;
+  uint32_t glu_base = 0, glu_slot = 0, glu_rows = 0;   // split gated form: first row of the workgroup's region, LDS slot, rows
   const uint32_t ksh = ks >> 1;                        // ks is 1, 2 or 4: its logarithm
   const uint32_t kpart = wave & (ks - 1u);
   if (EPI == EPI_STORE && ks > 1u) {
@@ -123,6 +129,29 @@ k_gemv_mfma(const float* xp, const uint8_t* __restrict__ W, const __half* __rest
     seg_end = kpart < C ? min(N, first + 4u) : 0u;      // nothing to do: no bundle, or no step of K left for this wave
     if (first >= N) seg_end = 0u;
     stride = 4u;
+  } else if (glu_split) {
+    // workgroup b: gate bundles [F(b), F(b + 1)), F(b) = floor(b * n_gb / workgroups) in the multiply-and-shift form
+    // (w0..w2 are for the grid here); its waves: region r (0 gate, 1 up) and part p of the region's `half` parts,
+    // waves that share a SIMD (w % 4) taking parts of both regions that differ in size as little as possible
+    auto share = [&](uint32_t gq) -> uint32_t {
+      return gq * w0 + (uint32_t)(((uint64_t)(gq * w1) * w2) >> (28u + ((cfg >> 10) & 15u)));
+    };
+    const uint32_t f0 = share(blockIdx.x), nb = share(blockIdx.x + 1u) - f0;
+    const uint32_t half = nwav >> 1, hsh = (uint32_t)__builtin_ctz(half);
+    uint32_t r, p;
+    if (nwav == 4u) { r = wave >> 1; p = wave & 1u; }
+    else {
+      const uint32_t sd = wave & 3u, q = wave >> 2, per = nwav >> 3;   // per: q-levels per region (1 or 2)
+      r = q / per;
+      p = (q % per) * 4u + ((sd + 2u * r) & 3u);
+    }
+    const uint32_t rb = r * (N >> 1), re = rb + (N >> 1);
+    first = rb + (f0 + ((p * nb) >> hsh)) * 4u;
+    seg_end = min(re, rb + (f0 + (((p + 1u) * nb) >> hsh)) * 4u);
+    stride = 4u;
+    glu_base = rb + f0 * 4u;
+    glu_slot = r * 512u;
+    glu_rows = nb * 4u;
   } else if (EPI == EPI_STORE) {
     const uint32_t slot = (wave & 3u) * (nwav >> 2) + (wave >> 2);
     // balanced shares without a division: a 64-bit quotient here is a few hundred instructions
@@ -145,7 +174,7 @@ k_gemv_mfma(const float* xp, const uint8_t* __restrict__ W, const __half* __rest
 
   // Row of lane-row l in the bundle that starts at row0.  With the gated-activation epilogue the
   // matrix is [gate rows; up rows] (N/2 each) and a bundle pairs two gate rows with their up rows.
-  const bool glu = EPI == EPI_STORE && (e_mode == EPIX_GEGLU || e_mode == EPIX_SWIGLU);
+  const bool glu = EPI == EPI_STORE && !glu_split && (e_mode == EPIX_GEGLU || e_mode == EPIX_SWIGLU);
   auto row_of = [&](uint32_t row0, uint32_t end) -> uint32_t {
     if (glu) return (row0 >> 1) + (l & 1u) + (l >> 1) * (N >> 1);
     return min(row0 + l, end - 1u);
@@ -556,6 +585,7 @@ k_gemv_mfma(const float* xp, const uint8_t* __restrict__ W, const __half* __rest
         if (row < end && bcol == 0u) {
           if (EPI == EPI_STORE) {
             act_out[(uint64_t)c_out + row] = y;
+            if (glu_split) part[glu_slot + (row - glu_base)] = y;
             if (e_mode == EPIX_ADD) act_out[(uint64_t)fz.e_dst + row] = Rl.res + y;
           } else if (better(y, row, best_v, best_i)) { best_v = y; best_i = row; }
         }
@@ -623,6 +653,18 @@ k_gemv_mfma(const float* xp, const uint8_t* __restrict__ W, const __half* __rest
           act_out[(uint64_t)c_out + row] = y;
           if (e_mode == EPIX_ADD) act_out[(uint64_t)fz.e_dst + row] = res_keep + y;
         }
+      }
+      break;
+    }
+    if (EPI == EPI_STORE && glu_split) {
+      // gate and up results of the workgroup's rows meet: act(gate) * up, one row per thread
+      __syncthreads();
+      const uint32_t g0 = glu_base - (glu_slot ? (N >> 1) : 0u);          // the workgroup's first gate row
+      const uint32_t f1 = min(N >> 1, g0 + 512u);
+      for (uint32_t i = tid; g0 + i < f1 && i < glu_rows; i += nthr) {
+        const float y = part[i], yu = part[512u + i];
+        const float t = e_mode == EPIX_GEGLU ? gelu_tanh(y) * yu : (y / (1.0f + expf(-y))) * yu;
+        act_out[(uint64_t)fz.e_dst + g0 + i] = t;
       }
       break;
     }
@@ -704,7 +746,25 @@ static void launch_mfma_p(int fmt, uint32_t grid, uint32_t threads, const Map* m
     sh = lg;
     w0 = n_q / wt; w1 = n_q % wt; w2 = (uint32_t)((((uint64_t)1 << (28u + lg)) + wt - 1u) / wt);
   }
-  uint32_t cfg = ks | ((threads >> 6) << 3) | ((EPI == EPI_STORE ? fz.e_mode : 0u) << 8) | (sh << 10);
+  // gated activation: the split form (see the kernel) where a workgroup's rows fit its LDS slots and the average
+  // wave has two steps or more (Llama shape, 28672 x 4096, 3.5 steps per wave: 594 -> 612 tok/s; Gemma shape,
+  // 13824 x 1152, under one step per wave: the closing barrier costs more than the rows' order gains, 1154 -> 1150)
+  const bool gated = EPI == EPI_STORE && (fz.e_mode == EPIX_GEGLU || fz.e_mode == EPIX_SWIGLU);
+  const int split_mode = tuning("ADAMAH_GLU_SPLIT", 1);
+  const uint64_t wave_steps = (uint64_t)cdiv(N, 4u) * cdiv(K, 512u * U);
+  bool glu_split = gated && ks == 1u && PRO != PRO_COMBINE && (N & 7u) == 0 &&
+                   (split_mode == 2 || (split_mode == 1 && wave_steps >= 2ull * grid * (threads >> 6)));
+  if (glu_split) {
+    const uint32_t n_gb = N >> 3;                       // bundles of four gate rows
+    if (grid > 16384u || 4u * (n_gb / grid + 1u) > 512u) glu_split = false;
+    else {
+      uint32_t lg = 0;
+      while ((1u << lg) < grid) lg++;
+      sh = lg;
+      w0 = n_gb / grid; w1 = n_gb % grid; w2 = (uint32_t)((((uint64_t)1 << (28u + lg)) + grid - 1u) / grid);
+    }
+  }
+  uint32_t cfg = ks | ((threads >> 6) << 3) | ((EPI == EPI_STORE ? fz.e_mode : 0u) << 8) | (sh << 10) | (glu_split ? 1u << 14 : 0u);
   if (PRO == PRO_COMBINE) cfg |= ((fz.c_splits - 1u) & 0xFFu) << 14 | (fz.c_vd >> 3) << 22;   // (the fold checks the ranges)
   const float* nwp = PRO == PRO_COMBINE ? fz.c_partial : n_wt + fz.p_src2;
   const uint64_t blk0 = (uint64_t)b >> 5;

@@ -461,7 +461,7 @@ def main():
         if args.only == "roofline":
             out = {"gemv_shapes": measure_gemv(gpu, A, LLAMA_GEMV_SHAPES[:1], rounds=8)}
         elif args.only == "gemv":
-            out = {"gemv_shapes": measure_gemv(gpu, A, LLAMA_GEMV_SHAPES[:1] + LLAMA_GEMV_SHAPES[3:], rounds=3)}
+            out = {"gemv_shapes": measure_gemv(gpu, A, LLAMA_GEMV_SHAPES, rounds=3)}
         elif args.only == "attention":
             out = {"attention": measure_attention(gpu, A)}
         elif args.only == "gemm":

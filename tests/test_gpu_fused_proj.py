@@ -65,6 +65,39 @@ def test_fused_qkv(hip, kind, K, rows, gap, batch):
         assert launches == (1 if gap == 0 else n_proj), launches
 
 
+@pytest.fixture(params=["0", "2"], ids=["paired-rows", "split-rows"])
+def glu_form(request, monkeypatch):
+    """Both ways the gate / up GEMV with the folded gated activation deals out its rows (the default chooses by size)."""
+    monkeypatch.setenv("ADAMAH_GLU_SPLIT", request.param)
+    return request.param
+
+
+@pytest.mark.parametrize("K,ff,act", [(1152, 6912, "geglu"), (4096, 14336, "swiglu"), (2048, 1028, "swiglu"), (512, 36, "geglu"),
+                                      (1536, 2050, "swiglu")])
+def test_folded_gated_activation_in_both_row_orders(hip, glu_form, K, ff, act):
+    """Gate and up rows, and act(gate) * up, from one launch in either form: whole bundles, a last workgroup with few
+    rows, fewer bundles than waves, and a row count the split form cannot take (ff not a multiple of four)."""
+    qt, bases = stacked("q4", (ff, ff), K, ff)
+    x = np.random.default_rng(ff).standard_normal(K).astype(np.float32)
+    outs, launches = [], None
+    for g in (hip, oracle.init()):
+        note(f"fused_gateup q4 K={K} ff={ff} act={act} form={glu_form}")
+        load_qtensor(g, 1, qt)
+        f32map(g, 0, K + 3 * ff + 64, x)
+        g.batch_begin()
+        g.map_fused_gateup_t_xq4_dev(0, 1, up(g, [0]), up(g, [bases[0]]), up(g, [bases[1]]), up(g, [K]), up(g, [K + ff]), K, ff, ff)
+        g.map_op2_dev(0, A.OP_GEGLU if act == "geglu" else A.OP_SWIGLU, up(g, K + np.arange(ff)), up(g, K + ff + np.arange(ff)),
+                      up(g, K + 2 * ff + np.arange(ff)), ff)
+        g.batch_end()
+        if g is hip:
+            launches = g.get_last_barrier_count()
+        outs.append(read(g, 0, K, 3 * ff + 8))
+    for part in range(3):
+        assert rel_l2(outs[0][part * ff:(part + 1) * ff], outs[1][part * ff:(part + 1) * ff]) < TOL, part
+    assert np.array_equal(outs[0][3 * ff:], outs[1][3 * ff:])      # nothing written past the results
+    assert launches == 1, launches
+
+
 @pytest.mark.parametrize("kind,K,ff,act", [("q4", 1152, 6912, "geglu"), ("q4", 4096, 14336, "swiglu"), ("q4", 4096, 1024, None),
                                            ("q8", 1152, 512, None)])
 def test_fused_gateup_and_folded_activation(hip, kind, K, ff, act):
