@@ -41,9 +41,9 @@ HBM_PEAK_GBPS = 8000.0
 LLAMA_GEMV_SHAPES = [(28672, 4096), (14336, 4096), (6144, 4096), (4096, 4096), (4096, 14336)]
 CONFIG1_GEMV_SHAPE = (6912, 1152)      # BASELINE config 1 (Gemma-3-1B FFN up): launch-bound, reported beside the others
 # HBM bytes per 28672x4096 Q4_0 GEMV launch from rocprofv3 --pmc (profiles/gemv_q4_0_llama_shapes_pmc_
-# fetch_write.txt): FETCH_SIZE 33,575.0 counts x 1.999 KiB (factor from a plain read kernel of known
-# size) + WRITE_SIZE 112.1 counts x 1.000 KiB (factor from a plain copy kernel).
-GEMV_TRAFFIC_BYTES = int(33575.0 * 1.999 * 1024 + 112.1 * 1.000 * 1024)
+# fetch_write.txt): FETCH_SIZE 33,535.3 counts x 1.999 KiB (factor from a plain read kernel of known
+# size) + WRITE_SIZE 112.2 counts x 1.000 KiB (factor from a plain copy kernel).
+GEMV_TRAFFIC_BYTES = int(33535.3 * 1.999 * 1024 + 112.2 * 1.000 * 1024)
 GEMV_TRAFFIC_SOURCE = ("profiles/gemv_q4_0_llama_shapes_pmc_fetch_write.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of "
                        "`bench.py --only gemv`, scaled by the same counters of `bench.py --only probe`; a figure of that "
                        "profile, not of this run")
