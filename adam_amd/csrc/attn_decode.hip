@@ -81,9 +81,14 @@ __device__ __forceinline__ float row16_sum(float v) {
 
 template <int D, int G, int NW, bool PF, bool EXT, bool RP>
 __global__ void __launch_bounds__(NW * 64)
-k_attn_decode(const float* data, const __half* kv, uint64_t kv_shift, uint32_t row_size, uint32_t chunk, uint32_t n_splits,
+k_attn_decode(const float* data, const __half* kv, uint64_t kv_shift, uint32_t row_size, uint32_t chunk, uint32_t splits_share,
               uint32_t rp_q_src, uint32_t rp_k_src, uint32_t rp_v_src, const void* early_ptr,
               float* out, float scale, float cap, float* partial, const AttdBases bs, const AttdRowPrep rp) {
+  // splits_share = slices | log2(share) << 16.  share > 1: the launch's groups are narrower than the KV groups --
+  // `share` consecutive groups of G heads read the same K / V rows (a short launch spread over more workgroups, each
+  // with fewer heads to work through between its barriers); with the row preparation they share one raw K / V row,
+  // every one of them prepares it for its own use and the first of them stores it to the cache.
+  const uint32_t n_splits = splits_share & 0xFFFFu, share_log = splits_share >> 16;
   // (the first 14 dwords of the arguments are in registers when a wave starts: what the first loads need stands in
   // front -- with the row preparation the raw rows' places and the frequency table, copies of rp's fields; with
   // the operand bases in device memory, the table's address)
@@ -108,6 +113,8 @@ k_attn_decode(const float* data, const __half* kv, uint64_t kv_shift, uint32_t r
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));   // scalar: row numbers below are too
   const uint32_t c = lane & 15u, kc = lane >> 4;
   const uint32_t split = blockIdx.x, group = blockIdx.y, op0 = group * G;
+  const uint32_t kvg = group >> share_log;                          // RP: index of the raw K / V row
+  const bool kv_writer = (group & ((1u << share_log) - 1u)) == 0u;  // RP: stores the new rows to the cache
   const uint32_t t0 = split * chunk, t1 = min(row_size, t0 + chunk);
   // wave-uniform bases plus 32-bit byte offsets: the V row of a load is the same for all lanes
   // EXT (several sets of heads in one launch, too many for the argument block): the bases come from
@@ -191,8 +198,8 @@ k_attn_decode(const float* data, const __half* kv, uint64_t kv_shift, uint32_t r
         qraw[u] = data[(uint64_t)rp_q_src + (uint64_t)op0 * D + min(tid + u * NT, (uint32_t)(G * D) - 1u)];
       {
         const uint32_t d = min(tid, (uint32_t)D - 1u);
-        kraw = data[(uint64_t)rp_k_src + (uint64_t)group * D + d];
-        vraw = data[(uint64_t)rp_v_src + (uint64_t)group * D + d];
+        kraw = data[(uint64_t)rp_k_src + (uint64_t)kvg * D + d];
+        vraw = data[(uint64_t)rp_v_src + (uint64_t)kvg * D + d];
       }
       float fr[PN], wq[PN][2], wk[2];
 #pragma unroll
@@ -241,8 +248,10 @@ k_attn_decode(const float* data, const __half* kv, uint64_t kv_shift, uint32_t r
         // the V row: rounded to fp16 for the copy, and the rounded value into the float32 row
         const __half vh = __float2half(vraw);
         const uint64_t vo = (uint64_t)bs.vb[group] + (uint64_t)(row_size - 1u) * D + tid;
-        const_cast<__half*>(kv)[vo - kv_shift] = vh;
-        out[vo] = __half2float(vh);
+        if (kv_writer) {
+          const_cast<__half*>(kv)[vo - kv_shift] = vh;
+          out[vo] = __half2float(vh);
+        }
         vnew[tid] = vh;
       }
       __syncthreads();
@@ -283,14 +292,16 @@ k_attn_decode(const float* data, const __half* kv, uint64_t kv_shift, uint32_t r
               k1 = k1 * inv * wk[1];
             }
             const float kr0 = k0 * cs - k1 * sn, kr1 = k0 * sn + k1 * cs;
-            if (rp.k_dst != ROWT_NONE) {
-              out[(uint64_t)rp.k_dst + (uint64_t)group * D + i] = kr0;
-              out[(uint64_t)rp.k_dst + (uint64_t)group * D + i + half] = kr1;
+            if (rp.k_dst != ROWT_NONE && kv_writer) {
+              out[(uint64_t)rp.k_dst + (uint64_t)kvg * D + i] = kr0;
+              out[(uint64_t)rp.k_dst + (uint64_t)kvg * D + i + half] = kr1;
             }
             const __half h0 = __float2half(kr0), h1 = __float2half(kr1);
             const uint64_t ko = (uint64_t)bs.kb[group] + (uint64_t)(row_size - 1u) * D + i;
-            const_cast<__half*>(kv)[ko - kv_shift] = h0; const_cast<__half*>(kv)[ko - kv_shift + half] = h1;
-            out[ko] = __half2float(h0); out[ko + half] = __half2float(h1);
+            if (kv_writer) {
+              const_cast<__half*>(kv)[ko - kv_shift] = h0; const_cast<__half*>(kv)[ko - kv_shift + half] = h1;
+              out[ko] = __half2float(h0); out[ko + half] = __half2float(h1);
+            }
             knew[i] = h0; knew[i + half] = h1;
           }
         }
@@ -630,11 +641,25 @@ bool launch_attn_decode(const AttnDecodeArgs& a, AttnPartials* ap, bool* left, i
   const bool pf = chunk > nw * 16u;
   const uint32_t n_splits = cdiv(a.row_size, chunk);
   if ((uint64_t)n_ops * n_splits * (D + 2) > g.attn_scratch_floats) return false;
+  // A launch of few workgroups (short context, few KV heads): one query head per workgroup instead of the whole
+  // group -- G times the workgroups, each with a G-th of the vector work between its barriers; the heads of a group
+  // ask for the same K / V tiles (Gemma shape at context 640: 5 -> 20 workgroups).
+  uint32_t Gl = G, share_log = 0;
+  {
+    const int hs = tuning("ADAMAH_ATTN_HEADSPLIT", 1);
+    const bool small = (uint64_t)n_ops * cdiv(a.row_size, chunk) <= (uint64_t)g.n_cu;
+    if (G > 1 && n_ops <= ATTD_MAX_GROUPS && (hs == 2 || (hs == 1 && small))) {
+      Gl = 1;
+      while ((1u << share_log) < G) share_log++;
+    }
+  }
+  const uint32_t n_groups_l = n_ops / Gl;
   AttdBases bs;
   for (uint32_t op = 0; op < n_ops; op++) { bs.q[op] = a.ha[op]; bs.sc[op] = a.hc[op]; bs.o[op] = a.ho[op]; }
-  for (uint32_t gi = 0; gi < n_groups; gi++) { bs.kb[gi] = a.hb[gi * G]; bs.vb[gi] = a.hv[gi * G]; }
+  for (uint32_t gi = 0; gi < n_groups_l; gi++) { bs.kb[gi] = a.hb[gi * Gl]; bs.vb[gi] = a.hv[gi * Gl]; }
   // the slices are merged by the consumer (leave) or by the caller's merge kernel
-  dim3 grid(n_splits, n_groups);
+  dim3 grid(n_splits, n_groups_l);
+  const uint32_t splits_share = n_splits | (share_log << 16);
   const AttdRowPrep* rpp = a.prep ? &rp : nullptr;
   // the prepared queries wait behind the partials until the merge copies them to their rows
   const uint64_t part_floats = (uint64_t)n_ops * n_splits * (D + 2);
@@ -642,9 +667,9 @@ bool launch_attn_decode(const AttnDecodeArgs& a, AttnPartials* ap, bool* left, i
     if (part_floats + (uint64_t)n_ops * D > g.attn_scratch_floats) return false;
     rp.q_scratch = g.attn_scratch + part_floats;
   }
-  if (D == 64) launch_d<64>(G, nw, pf, grid, a, bs, n_splits, chunk);
-  else if (D == 128) launch_d<128>(G, nw, pf, grid, a, bs, n_splits, chunk, nullptr, rpp);
-  else launch_d<256>(G, nw, pf, grid, a, bs, n_splits, chunk, nullptr, rpp);
+  if (D == 64) launch_d<64>(Gl, nw, pf, grid, a, bs, splits_share, chunk);
+  else if (D == 128) launch_d<128>(Gl, nw, pf, grid, a, bs, splits_share, chunk, nullptr, rpp);
+  else launch_d<256>(Gl, nw, pf, grid, a, bs, splits_share, chunk, nullptr, rpp);
   if (a.prep) *a.prep_done = true;
   count_launch();
   *rc = check_launch();
