@@ -263,3 +263,24 @@ def test_unit_scale_integer_weights_give_exact_sums(hip, pro, K, N):
     want = W @ x.astype(np.float64)
     assert np.all(np.abs(want) < 2 ** 24 / 1024)
     assert np.array_equal(y, want.astype(np.float32))
+
+
+@pytest.mark.parametrize("N,K", [(3, 4096), (5, 512), (1021, 4096), (4100, 4096), (7170, 2048), (16389, 4096), (28676, 512),
+                                 (65537, 512), (100003, 512)])
+def test_every_row_belongs_to_exactly_one_wave(hip, N, K):
+    """The launcher deals the 4-row bundles out to the waves as floor(g * bundles / waves), which the kernel evaluates
+    with a multiplication and a shift prepared on the host instead of a division: row counts on either side of
+    multiples of 4, of the wave count and of the workgroup count, with and without a K split.  Integer weights at
+    scale 1 and small integer activations make every row's result exact, so a row that no wave took (its place still
+    holds the marker) or that was summed from another row's blocks fails equality."""
+    qt, W = _integer_weights(N, K, N + K)
+    x = np.random.default_rng(N).integers(-3, 4, K).astype(np.float32)
+    load_qtensor(hip, 1, qt)
+    f32map(hip, 0, K + N + 8, np.concatenate([x, np.full(N + 8, -12345.0, np.float32)]))
+    note(f"gemv row shares {N}x{K}")
+    hip.batch_begin()
+    hip.map_matmul_t_xq4_dev(0, 1, up(hip, [0]), up(hip, [0]), up(hip, [K]), 1, K, N)
+    hip.batch_end()
+    got = read(hip, 0, K, N + 8)
+    assert np.array_equal(got[:N], (W @ x.astype(np.float64)).astype(np.float32))
+    assert np.all(got[N:] == -12345.0)                    # and nothing past the last row
