@@ -73,10 +73,11 @@ def glu_form(request, monkeypatch):
 
 
 @pytest.mark.parametrize("K,ff,act", [(1152, 6912, "geglu"), (4096, 14336, "swiglu"), (2048, 1028, "swiglu"), (512, 36, "geglu"),
-                                      (1536, 2050, "swiglu")])
+                                      (1536, 2050, "swiglu"), (8192, 8192, "swiglu")])
 def test_folded_gated_activation_in_both_row_orders(hip, glu_form, K, ff, act):
     """Gate and up rows, and act(gate) * up, from one launch in either form: whole bundles, a last workgroup with few
-    rows, fewer bundles than waves, and a row count the split form cannot take (ff not a multiple of four)."""
+    rows, fewer bundles than waves, a row count the split form cannot take (ff not a multiple of four), and rows long
+    and many enough for workgroups of 16 waves."""
     qt, bases = stacked("q4", (ff, ff), K, ff)
     x = np.random.default_rng(ff).standard_normal(K).astype(np.float32)
     outs, launches = [], None
