@@ -149,19 +149,23 @@ __global__ void __launch_bounds__(64 * NW)
 k_gemm_q4_f16_tiled(const uint8_t* __restrict__ W, const __half* __restrict__ d16, const u4q_t* __restrict__ xh, const u4q_t* __restrict__ xl,
                      uint32_t K, uint32_t N, uint32_t M, uint32_t b_val, uint32_t c_val, uint32_t by_val, float* out,
                      const uint32_t* __restrict__ lb, const uint32_t* __restrict__ lc, const float* __restrict__ scale,
-                     GemmSegs segs) {
+                     GemmSegs segs, uint32_t ksplit, uint32_t kper, float* __restrict__ part) {
   // (the first 14 dwords of the arguments are in registers when a wave starts; by_val bit 0 / 1: the weights' / the
   // result's element offset of op 0 is b_val / c_val -- known on the host -- instead of a load from lb / lc, which
   // the first weight loads would have to wait for)
+  // ksplit > 1 (one op): blockIdx.z is a share of K -- kper blocks, a multiple of 4 -- and the tile's raw sums go to
+  // part[share][row][n] for k_gemm_splitk_sum; wide tiles then still give every CU a workgroup on a narrow matrix.
   constexpr uint32_t BM = 16u * MT, ROWB = 272u;
   __shared__ __attribute__((aligned(16))) uint8_t xs[2u * BM * ROWB];   // first plane, then second plane
   uint8_t* const xs2 = xs + BM * ROWB;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
   const uint32_t r16 = lane & 15u, g = lane >> 4;
   constexpr uint32_t NT = 64u * NW, NP = 256u * MT / NT;       // threads; 16-byte pieces per thread, plane and step
-  const uint32_t n0 = blockIdx.x * (16u * NW * R) + wave * (16u * R), m0 = blockIdx.y * BM, op = blockIdx.z;
+  const uint32_t n0 = blockIdx.x * (16u * NW * R) + wave * (16u * R), m0 = blockIdx.y * BM;
+  const uint32_t op = ksplit > 1u ? 0u : blockIdx.z, kz = ksplit > 1u ? blockIdx.z : 0u;
   const uint64_t c_off = (by_val & 2u) ? (uint64_t)c_val : (uint64_t)lc[op], gbase = ((by_val & 1u) ? (uint64_t)b_val : (uint64_t)lb[op]) >> 5;
   const uint32_t nblk = K >> 5, kw = K >> 3;                   // blocks and 16-byte pieces per row
+  const uint32_t kb_lo = kz * kper, kb_hi = min(nblk, kb_lo + kper);   // this workgroup's blocks of K
   uint32_t nrow[R];
 #pragma unroll
   for (int r = 0; r < R; r++) nrow[r] = min(n0 + r * 16u + r16, N - 1u);   // rows past N: clamped, not stored
@@ -185,7 +189,7 @@ k_gemm_q4_f16_tiled(const uint8_t* __restrict__ W, const __half* __restrict__ d1
   // always executed; the step past K re-reads the last one and is not used
 #define GEMM_FETCH(kb_raw)                                                        \
   do {                                                                            \
-    const uint32_t kb_ = min((kb_raw), nblk - 4u);                                \
+    const uint32_t kb_ = min((kb_raw), kb_hi - 4u);                               \
     _Pragma("unroll") for (int r = 0; r < R; r++) {                               \
       const uint64_t gi = gbase + (uint64_t)nrow[r] * nblk + kb_ + g;             \
       qn[r] = *(const u4q_t*)(W + (gi << 4));                                     \
@@ -196,9 +200,9 @@ k_gemm_q4_f16_tiled(const uint8_t* __restrict__ W, const __half* __restrict__ d1
       xln[u] = xl[xoff[u] + kb_ * 4u];                                            \
     }                                                                             \
   } while (0)
-  GEMM_FETCH(0u);
+  GEMM_FETCH(kb_lo);
 
-  for (uint32_t kb0 = 0; kb0 < nblk; kb0 += 4u) {
+  for (uint32_t kb0 = kb_lo; kb0 < kb_hi; kb0 += 4u) {
 #pragma unroll
     for (uint32_t u = 0; u < NP; u++) {
       const uint32_t w = tid + u * NT;
@@ -255,6 +259,15 @@ k_gemm_q4_f16_tiled(const uint8_t* __restrict__ W, const __half* __restrict__ d1
     for (int i = 0; i < 4; i++) {
       const uint32_t row = m0 + t * 16u + 4u * g + i;
       if (row >= M) continue;
+      if (ksplit > 1u) {   // raw sums of this share of K; scale and placement are k_gemm_splitk_sum's
+        float* pr = part + ((uint64_t)kz * M + row) * N;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+          const uint32_t n = n0 + r * 16u + r16;
+          if (n < N) pr[n] = acc[r][t][i];
+        }
+        continue;
+      }
       const float inv = scale[2 * ((uint64_t)op * M + row) + 1];
       float* c = out + c_off + (uint64_t)row * N;
 #pragma unroll
@@ -272,6 +285,46 @@ k_gemm_q4_f16_tiled(const uint8_t* __restrict__ W, const __half* __restrict__ d1
 }
 
 #undef GEMM_FETCH
+
+// The shares of K of a split launch of the kernel above, summed in the order of the shares, scaled by the row's factor
+// and stored where the unsplit launch would have stored them (one op).  Four results per thread.
+__global__ void __launch_bounds__(256)
+k_gemm_splitk_sum(const float* __restrict__ part, uint32_t ksplit, uint32_t M, uint32_t N, float* out, uint32_t c_val,
+                  uint32_t by_val, const uint32_t* __restrict__ lc, const float* __restrict__ scale, GemmSegs segs) {
+  const uint64_t total = (uint64_t)M * N, i0 = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * 4u;
+  if (i0 >= total) return;
+  const uint64_t c_off = (by_val & 2u) ? (uint64_t)c_val : (uint64_t)lc[0];
+  float v[4];
+  const bool whole = (N & 3u) == 0u;      // the four are one row's: one 16-byte load per share
+  if (whole) {
+    f4q_t a = *(const f4q_t*)(part + i0);
+    for (uint32_t z = 1; z < ksplit; z++) {
+      const f4q_t b = *(const f4q_t*)(part + z * total + i0);
+      a[0] += b[0]; a[1] += b[1]; a[2] += b[2]; a[3] += b[3];
+    }
+    v[0] = a[0]; v[1] = a[1]; v[2] = a[2]; v[3] = a[3];
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      float a = i0 + e < total ? part[i0 + e] : 0.f;
+      for (uint32_t z = 1; z < ksplit; z++) a += i0 + e < total ? part[z * total + i0 + e] : 0.f;
+      v[e] = a;
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    const uint64_t i = i0 + e;
+    if (i >= total) break;
+    const uint32_t row = (uint32_t)(i / N), n = (uint32_t)(i % N);
+    const float y = v[e] * scale[2 * (uint64_t)row + 1];
+    if (segs.count) {
+      uint32_t sgi = 0;
+#pragma unroll
+      for (uint32_t q = 1; q < 4; q++) sgi += (q < segs.count && n >= segs.begin[q]) ? 1u : 0u;
+      out[segs.c[sgi] + (uint64_t)row * segs.n[sgi] + (n - segs.begin[sgi])] = y;
+    } else out[c_off + (uint64_t)row * N + n] = y;
+  }
+}
 
 // Few activation rows (M <= 32): the weights are read once and nothing is reused, so the work is
 // bound by how fast they stream.  The NWV waves of a workgroup share R tiles of 16 weight rows and
@@ -734,6 +787,17 @@ static size_t g_scale_cap = 0;
 // offset of the second plane those rows were written with.
 static struct { const void* buf; uint64_t a; uint32_t M, K; uint64_t dispatch, mem_gen; size_t plane; bool valid; } g_xh_key = {};
 
+static float* g_part_buf = nullptr;   // raw sums of the shares of a K-split launch
+static size_t g_part_cap = 0;
+static bool ensure_part_buf(size_t floats) {
+  if (floats <= g_part_cap) return true;
+  layout_changed();
+  if (g_part_buf) { hipStreamSynchronize(g.stream); hipFree(g_part_buf); }
+  g_part_cap = floats;
+  if (hipMalloc((void**)&g_part_buf, g_part_cap * sizeof(float)) != hipSuccess) { (void)hipGetLastError(); g_part_buf = nullptr; g_part_cap = 0; return false; }
+  return true;
+}
+
 static bool ensure_act_bufs(size_t scale_floats, size_t xh_bytes) {
   if (scale_floats > g_scale_cap) {
     layout_changed();
@@ -985,9 +1049,31 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
   NW = (uint32_t)knob("ADAMAH_GEMM_NW", (int)NW) >= 8 ? 8 : 4;
   R = R >= 4 && mt == 4 ? 4 : R >= 2 ? 2 : 1;
   if (mt == 4 && NW == 8 && R == 1) R = 2;
-  dim3 grid(cdiv(N, 16 * NW * R), cdiv(M, 16 * mt), n_ops);
-#define GT(T, RR, W) k_gemm_q4_f16_tiled<T, RR, W><<<grid, 64 * W, 0, g.stream>>>(mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, K, N, M, b_val, c_val, by_val, act, lb, lc, g_scale_buf, sg)
-  if (mt == 4 && NW == 8) { if (R == 4) GT(4, 4, 8); else GT(4, 2, 8); }
+  // A narrow matrix under many rows (N = 4096 / 6144 at M = 512) gives the widest tile (256 weight rows x 128 rows)
+  // too few workgroups for the chip, and the smaller tiles that do fill it re-stage more activations per flop: there
+  // the widest tile is launched over 2 .. 4 shares of K, raw sums into scratch, and a second launch adds the shares.
+  uint32_t ksplit = 1, kper = K >> 5;
+  if (M >= 128 && n_ops == 1 && tuning("ADAMAH_GEMM_SPLITK", 1) != 0) {
+    const uint64_t w256 = wgs(256, 8);
+    if (w256 * 4 < 3ull * (uint64_t)g.n_cu) {
+      uint32_t sp = (uint32_t)std::min<uint64_t>(4, (uint64_t)g.n_cu / std::max<uint64_t>(1, w256));
+      while (sp > 1 && K / sp < 1024u) sp--;
+      if (sp > 1 && w256 * sp * 4 >= 3ull * (uint64_t)g.n_cu && ensure_part_buf((size_t)sp * M * N)) {
+        ksplit = sp; mt = 8; R = 2; NW = 8;
+        kper = cdiv(cdiv(K >> 5, ksplit), 4u) * 4u;
+        ksplit = cdiv(K >> 5, kper);
+      }
+    }
+  }
+  dim3 grid(cdiv(N, 16 * NW * R), cdiv(M, 16 * mt), ksplit > 1 ? ksplit : n_ops);
+#define GT(T, RR, W) k_gemm_q4_f16_tiled<T, RR, W><<<grid, 64 * W, 0, g.stream>>>(mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, K, N, M, b_val, c_val, by_val, act, lb, lc, g_scale_buf, sg, ksplit, kper, g_part_buf)
+  if (ksplit > 1) {
+    GT(8, 2, 8);
+    count_launch();
+    const uint64_t quads = ((uint64_t)M * N + 3) / 4;
+    k_gemm_splitk_sum<<<cdiv(quads, 256), 256, 0, g.stream>>>(g_part_buf, ksplit, M, N, act, c_val, by_val, lc, g_scale_buf, sg);
+  }
+  else if (mt == 4 && NW == 8) { if (R == 4) GT(4, 4, 8); else GT(4, 2, 8); }
   else if (mt == 4) { if (R == 4) GT(4, 4, 4); else if (R == 2) GT(4, 2, 4); else GT(4, 1, 4); }
   else if (NW == 8) { if (R == 2) GT(8, 2, 8); else GT(8, 1, 8); }
   else { if (R == 2) GT(8, 2, 4); else GT(8, 1, 4); }
@@ -1005,6 +1091,9 @@ void gemm_q4_mfma_release() {
   g_xh_buf = nullptr;
   g_xh_cap = 0;
   g_xh_key.valid = false;
+  if (g_part_buf) hipFree(g_part_buf);
+  g_part_buf = nullptr;
+  g_part_cap = 0;
 }
 
 }  // namespace adamah

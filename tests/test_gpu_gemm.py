@@ -213,11 +213,14 @@ def test_rmsnorm_rows_feed_the_matmul_without_a_conversion_launch(hip, dim, rows
 @pytest.mark.parametrize("kind,M,K,Ns", [("q4", 16, 4096, (4096, 1024, 1024)), ("q4", 5, 256, (40, 24)), ("q8", 16, 512, (100, 60, 33, 7)),
                                          ("q4", 32, 1152, (1024, 256, 256)), ("q4", 100, 256, (200, 72, 72)),
                                          ("q4", 512, 4096, (4096, 1024, 1024))])
-def test_stacked_matmuls_place_every_result_where_its_op_asked(hip, kind, M, K, Ns):
+def test_stacked_matmuls_place_every_result_where_its_op_asked(hip, monkeypatch, kind, M, K, Ns):
     """Matmuls over the same rows with weight matrices back to back but results at unrelated places and of
     different widths (not multiples of 16 either): one launch, each [M, N_i] result at its own base, equal
-    bit for bit to the ops run one by one (ADAMAH_GEMM_MERGE=0)."""
+    bit for bit to the ops run one by one (ADAMAH_GEMM_MERGE=0).  (With the split over K off: how many shares of K
+    a launch is cut into goes by its width, so the stacked launch and the single ones add in different orders;
+    test_narrow_matrix_under_many_rows_split_over_k covers that path.)"""
     import os
+    monkeypatch.setenv("ADAMAH_GEMM_SPLITK", "0")
     rng = np.random.default_rng(sum(Ns) + M)
     Nt = sum(Ns)
     w = rng.standard_normal((Nt, K), dtype=np.float32) * np.float32(0.05)
@@ -398,3 +401,47 @@ def test_gated_activation_stored_by_the_stacked_gate_up_matmul(hip, kind, op, M,
     if down_ok:
         assert rel_l2(fused[y0:y0 + M * N2], want[y0:y0 + M * N2]) < TOL
     assert not fused[y0 + M * N2:].any()
+
+
+@pytest.mark.parametrize("M,N,K,Ns", [(512, 4096, 4096, None), (487, 4096, 14336, None), (512, 6144, 4096, (4096, 1024, 1024)),
+                                      (400, 4100, 4096, None)])
+def test_narrow_matrix_under_many_rows_split_over_k(hip, monkeypatch, M, N, K, Ns):
+    """Matrices too narrow for the widest tile to fill the chip are run as shares of K whose raw sums a second launch
+    adds: same product as the unsplit launch (and the reference's) for whole and ragged tiles, a last share shorter
+    than the others, and stacked matrices with results in three places."""
+    rng = np.random.default_rng(M + N + K)
+    qt = quant.quantize_q4_0((rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.02)))
+    x = rng.standard_normal((M, K), dtype=np.float32)
+    want = x.astype(np.float64) @ qt.dequant().astype(np.float64).T
+
+    def once():
+        load_qtensor(hip, 1, qt)
+        f32map(hip, 0, M * K + M * N + 64, x.reshape(-1))
+        hip.batch_begin()
+        if Ns is None:
+            hip.map_matmul_t_xq4_dev(0, 1, up(hip, [0]), up(hip, [0]), up(hip, [M * K]), M, K, N, 1)
+        else:                            # storage order: one launch over the stacked rows
+            r = 0
+            for n in Ns:
+                hip.map_matmul_t_xq4_dev(0, 1, up(hip, [0]), up(hip, [r * K]), up(hip, [M * K + M * r]), M, K, n, 1)
+                r += n
+        hip.batch_end()
+        return read(hip, 0, M * K, M * N), hip.get_last_barrier_count()
+
+    note(f"gemm q4 split-K M={M} N={N} K={K}")
+    y1, l1 = once()
+    monkeypatch.setenv("ADAMAH_GEMM_SPLITK", "0")
+    y0, l0 = once()
+    if Ns is None:
+        got1, got0 = y1.reshape(M, N), y0.reshape(M, N)
+    else:
+        got1, got0 = np.empty((M, N), np.float32), np.empty((M, N), np.float32)
+        r = 0
+        for n in Ns:
+            got1[:, r:r + n] = y1[M * r:M * (r + n)].reshape(M, n)
+            got0[:, r:r + n] = y0[M * r:M * (r + n)].reshape(M, n)
+            r += n
+    for m in range(0, M, 7):
+        assert rel_l2(got1[m], want[m]) < TOL_Q4 and rel_l2(got0[m], want[m]) < TOL_Q4, m
+    assert rel_l2(got1, got0) < 1e-5
+    assert l1 == l0 + 1, (l1, l0)        # the launch that adds the shares
