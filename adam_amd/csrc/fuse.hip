@@ -272,7 +272,9 @@ void flush_pending() {
       // one matrix followed by the add that consumes its result (hidden += projection): stored by the matmul.
       // The matmul reads its fp16 copy of the rows, so only the result and the residual have to lie clear.
       size_t used = m;
-      if (m == 1 && M <= 32 && i + 1 < n && q[i + 1].kind == PK_OP2 && q[i + 1].op == 0 && q[i + 1].map_act == p.map_act &&
+      // (many rows: only where the matmul runs over shares of K, whose adding launch stores the add as well)
+      if (m == 1 && (M <= 32 || (p.op != (uint32_t)FMT_Q8_B16 && gemm_q4_k_shares((uint32_t)M, p.k, p.n) > 1)) && i + 1 < n &&
+          q[i + 1].kind == PK_OP2 && q[i + 1].op == 0 && q[i + 1].map_act == p.map_act &&
           q[i + 1].n == M * p.n && tuning("ADAMAH_GEMM_EPI", 1) != 0) {
         const PendOp& e = q[i + 1];
         if ((e.a == p.c) != (e.b == p.c)) {

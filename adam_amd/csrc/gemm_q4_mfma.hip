@@ -322,7 +322,10 @@ k_gemm_splitk_sum(const float* __restrict__ part, uint32_t ksplit, uint32_t M, u
 #pragma unroll
       for (uint32_t q = 1; q < 4; q++) sgi += (q < segs.count && n >= segs.begin[q]) ? 1u : 0u;
       out[segs.c[sgi] + (uint64_t)row * segs.n[sgi] + (n - segs.begin[sgi])] = y;
-    } else out[c_off + (uint64_t)row * N + n] = y;
+    } else {
+      out[c_off + (uint64_t)row * N + n] = y;
+      if (segs.add) out[segs.dst + (uint64_t)row * N + n] = out[segs.res + (uint64_t)row * N + n] + y;   // the add behind it
+    }
   }
 }
 
@@ -951,13 +954,26 @@ void gemm_act_forget() { g_xh_key.valid = false; }
 // Preconditions (checked by the caller against the host copies of the handles): Q4 map whose blocks
 // in range are in the block16 layout, K a multiple of 128, weight bases block aligned, all operands
 // in range.
+// Shares of K a one-op Q4 matmul of M rows is cut into (1: one launch): 2 .. 4 where the widest tile (256 weight rows
+// x 128 rows) would give fewer than three quarters of the CUs a workgroup and the shares fill them, each share at
+// least 1024 elements long.
+uint32_t gemm_q4_k_shares(uint32_t M, uint32_t K, uint32_t N) {
+  if (M < 128 || tuning("ADAMAH_GEMM_SPLITK", 1) == 0) return 1;
+  const uint64_t w256 = (uint64_t)cdiv(N, 256) * cdiv(M, 128);
+  if (w256 * 4 >= 3ull * (uint64_t)g.n_cu) return 1;
+  uint32_t sp = (uint32_t)std::min<uint64_t>(4, (uint64_t)g.n_cu / std::max<uint64_t>(1, w256));
+  while (sp > 1 && K / sp < 1024u) sp--;
+  return sp > 1 && w256 * sp * 4 >= 3ull * (uint64_t)g.n_cu ? sp : 1u;
+}
+
 int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb, const uint32_t* lc,
                         uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops, bool q8, float* out, int64_t a_host,
                         int64_t c_host, const GemmSegs* segs, int64_t b_host) {
   // offsets of op 0 the host knows go to the kernels by value
   const uint32_t b_val = b_host >= 0 ? (uint32_t)b_host : 0u, c_val = c_host >= 0 ? (uint32_t)c_host : 0u;
   const uint32_t by_val = n_ops == 1 ? ((b_host >= 0 ? 1u : 0u) | (c_host >= 0 ? 2u : 0u)) : 0u;
-  if (((q8 || out) && M > 32) || ((out || segs) && n_ops != 1) || (out && segs) || (segs && (segs->add || segs->glu) && M > 32))
+  if (((q8 || out) && M > 32) || ((out || segs) && n_ops != 1) || (out && segs) || (segs && segs->glu && M > 32) ||
+      (segs && segs->add && M > 32 && (n_ops != 1 || q8 || gemm_q4_k_shares(M, K, N) < 2)))
     return ADAMAH_ERR_INVALID;
   GemmSegs sg = {};
   if (segs) sg = *segs;
@@ -1053,17 +1069,13 @@ int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const 
   // too few workgroups for the chip, and the smaller tiles that do fill it re-stage more activations per flop: there
   // the widest tile is launched over 2 .. 4 shares of K, raw sums into scratch, and a second launch adds the shares.
   uint32_t ksplit = 1, kper = K >> 5;
-  if (M >= 128 && n_ops == 1 && tuning("ADAMAH_GEMM_SPLITK", 1) != 0) {
-    const uint64_t w256 = wgs(256, 8);
-    if (w256 * 4 < 3ull * (uint64_t)g.n_cu) {
-      uint32_t sp = (uint32_t)std::min<uint64_t>(4, (uint64_t)g.n_cu / std::max<uint64_t>(1, w256));
-      while (sp > 1 && K / sp < 1024u) sp--;
-      if (sp > 1 && w256 * sp * 4 >= 3ull * (uint64_t)g.n_cu && ensure_part_buf((size_t)sp * M * N)) {
-        ksplit = sp; mt = 8; R = 2; NW = 8;
-        kper = cdiv(cdiv(K >> 5, ksplit), 4u) * 4u;
-        ksplit = cdiv(K >> 5, kper);
-      }
-    }
+  {
+    const uint32_t sp = n_ops == 1 && !q8 && !out ? gemm_q4_k_shares(M, K, N) : 1u;
+    if (sp > 1 && ensure_part_buf((size_t)sp * M * N)) {
+      ksplit = sp; mt = 8; R = 2; NW = 8;
+      kper = cdiv(cdiv(K >> 5, ksplit), 4u) * 4u;
+      ksplit = cdiv(K >> 5, kper);
+    } else if (sg.add && M > 32) return ADAMAH_ERR_MEMORY;   // (only the split launch stores the add of many rows)
   }
   dim3 grid(cdiv(N, 16 * NW * R), cdiv(M, 16 * mt), ksplit > 1 ? ksplit : n_ops);
 #define GT(T, RR, W) k_gemm_q4_f16_tiled<T, RR, W><<<grid, 64 * W, 0, g.stream>>>(mw->buf, mw->d16, (const u4q_t*)xh, (const u4q_t*)xl, K, N, M, b_val, c_val, by_val, act, lb, lc, g_scale_buf, sg, ksplit, kper, g_part_buf)

@@ -139,6 +139,7 @@ struct GemmSegs {
 // host knows them (n_ops == 1): lets consecutive matmuls over the same rows share one conversion.  b_host: likewise
 // the element offset of op 0's weights; known offsets go to the kernels by value (no load in front of their first loads).
 // segs (M <= 32, one op): the weights are several matrices back to back, results placed per segment.
+uint32_t gemm_q4_k_shares(uint32_t M, uint32_t K, uint32_t N);   // > 1: the matmul runs over shares of K and may store an add
 int launch_gemm_q4_mfma(const Map* ma, const Map* mw, const uint32_t* la, const uint32_t* lb, const uint32_t* lc,
                         uint32_t M, uint32_t K, uint32_t N, uint32_t n_ops, bool q8 = false, float* out = nullptr,
                         int64_t a_host = -1, int64_t c_host = -1, const GemmSegs* segs = nullptr, int64_t b_host = -1);

@@ -265,11 +265,13 @@ def test_stacked_matmuls_place_every_result_where_its_op_asked(hip, monkeypatch,
     assert not merged[M * K:M * K + 8].any()       # nothing outside the results was written
 
 
-@pytest.mark.parametrize("M,K,N,in_place", [(16, 4096, 4096, True), (7, 256, 50, False), (32, 1152, 72, True)])
+@pytest.mark.parametrize("M,K,N,in_place", [(16, 4096, 4096, True), (7, 256, 50, False), (32, 1152, 72, True),
+                                            (512, 4096, 4096, True), (400, 4096, 4100, False)])
 def test_residual_add_stored_by_the_matmul(hip, M, K, N, in_place):
     """hidden += X W^T issued as matmul then add: the matmul's store also writes residual + result (two launches
     with the conversion instead of three); the projection itself still lands in its own rows.  All words equal
-    the unfused sequence's (ADAMAH_GEMM_EPI=0)."""
+    the unfused sequence's (ADAMAH_GEMM_EPI=0).  With many rows the add rides in the launch that adds the shares
+    of a matmul run over shares of K (three launches instead of four)."""
     import os
     rng = np.random.default_rng(M + N)
     qt = quant.quantize_q4_0(rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.05))
@@ -297,10 +299,15 @@ def test_residual_add_stored_by_the_matmul(hip, M, K, N, in_place):
         apart, n_apart = go(hip)
     finally:
         del os.environ["ADAMAH_GEMM_EPI"]
-    assert (n_fused, n_apart) == (2, 3)
+    assert (n_fused, n_apart) == ((2, 3) if M <= 32 else (3, 4))
     assert np.array_equal(fused.view(np.uint32), apart.view(np.uint32))
-    want, _ = go(oracle.init())
-    assert rel_l2(fused[y0:], want[y0:]) < TOL
+    if M <= 32:
+        want, _ = go(oracle.init())
+        assert rel_l2(fused[y0:], want[y0:]) < TOL
+    else:                                  # (the oracle's op surface takes minutes over this many rows)
+        y = x.astype(np.float64) @ qt.dequant().astype(np.float64).T
+        assert rel_l2(fused[y0:h0].reshape(M, N), y) < TOL
+        assert rel_l2(fused[d0:d0 + M * N].reshape(M, N), y + hid) < TOL
 
 
 @pytest.mark.parametrize("op,M,K,N,in_place", [("swiglu", 16, 14336, 96, False), ("geglu", 5, 6912, 64, False), ("swiglu", 40, 256, 50, False),
