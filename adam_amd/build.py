@@ -16,7 +16,11 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", 
          "-Wno-unused-result", "-Wno-unused-value"]
 # gemv_mfma.hip draws a ticket with one atomic per workgroup and looks at it much later; the
 # compiler's wave-level aggregation of uniform-address atomics would wait for the result at once.
-EXTRA = {"gemv_mfma.hip": ["-mllvm", "-amdgpu-atomic-optimizer-strategy=None"]}
+# attn_prefill.hip: the matrix instructions' results in ordinary vector registers.  With the accumulator registers the
+# compiler otherwise picks, the chunk attention's 32 running output values moved to vector registers and back in every
+# key tile (64 of ~300 vector instructions per tile) because the score products wanted the same accumulator registers.
+EXTRA = {"gemv_mfma.hip": ["-mllvm", "-amdgpu-atomic-optimizer-strategy=None"],
+         "attn_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def _hipcc():

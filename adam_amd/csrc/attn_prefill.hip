@@ -282,7 +282,7 @@ k_v_tile_transpose(const __half* kv, uint64_t kv_shift, const AttpVtSrc src, uin
 
 #define ATTP_MFMA32(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0)
 
-template <int D>
+template <int D, bool CAP>
 __global__ void __launch_bounds__(256)
 k_attn_prefill_mfma(const float* data, float* out, const __half* kv, uint64_t kv_shift, const uint4* __restrict__ vt,
                     const AttpBases bs, const AttpVt gv, uint32_t H, uint32_t n_quads, uint32_t n_ttiles, uint32_t m,
@@ -330,6 +330,7 @@ k_attn_prefill_mfma(const float* data, float* out, const __half* kv, uint64_t kv
       }
   }
   const uint32_t lim = n < rows ? seq0 + t0 + n : 0u;     // cache rows this lane's query sees
+  const float c2 = inv_s * scale * 1.44269504f;          // (inv_s is a power of two)
   const bool last = n < rows && t0 + n == m - 1u;
   const uint64_t sc_row = bs.sc[head];
 
@@ -361,36 +362,47 @@ k_attn_prefill_mfma(const float* data, float* out, const __half* kv, uint64_t kv
         s[kb][0] = ATTP_MFMA32(ka, qh[st], s[kb][0]);
         s[kb][1] = ATTP_MFMA32(ka, ql[st], s[kb][1]);
       }
+    // The softmax runs on base-2 exponents: without a soft cap the scores' power-of-two scale, the softmax scale and
+    // log2(e) are one factor (one rounding, as scale alone would take), a masked score is a large negative number
+    // whose power is exactly 0, and the only branches of a tile are wave-uniform and rarely taken (the raw scores
+    // of the chunk's last token, a maximum that moved).
     float v[8], mt = ATTP_NEG;
-    bool ok[8];
+    const uint32_t key0 = 32u * T + 4u * g;
 #pragma unroll
     for (int kb = 0; kb < 2; kb++)
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        const uint32_t key = 32u * T + 16u * kb + 4u * g + r;
-        const float raw = (s[kb][0][r] + s[kb][1][r]) * inv_s;
-        ok[4 * kb + r] = key < lim;
-        if (ok[4 * kb + r] && last) out[sc_row + key] = raw;
-        v[4 * kb + r] = ok[4 * kb + r] ? prep(raw, scale, cap) : ATTP_NEG;
+        const float sum = s[kb][0][r] + s[kb][1][r];
+        const float x = CAP ? prep(sum * inv_s, scale, cap) * 1.44269504f : sum * c2;
+        v[4 * kb + r] = key0 + 16u * kb + r < lim ? x : ATTP_NEG;
         mt = fmaxf(mt, v[4 * kb + r]);
       }
+    if (__builtin_expect(__any(last), 0)) {
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const uint32_t key = key0 + 16u * kb + r;
+          if (key < lim && last) out[sc_row + key] = (s[kb][0][r] + s[kb][1][r]) * inv_s;
+        }
+    }
     mt = fmaxf(mt, __shfl_xor(mt, 16, 64)); mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
     const float m_new = fmaxf(m_run, mt);
-    const float alpha = __expf(m_run - m_new);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     const bool moved = m_new > m_run;
     m_run = m_new;
     h8p_t ph, pl;
     float psum = 0.f;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
-      const float pj = ok[j] ? __expf(v[j] - m_new) : 0.f;
+      const float pj = __builtin_amdgcn_exp2f(v[j] - m_new);
       psum += pj;
       const _Float16 hi = (_Float16)pj;
       ph[j] = hi;
       pl[j] = (_Float16)(pj - (float)hi);
     }
     l_run = l_run * alpha + psum;
-    if (__any(moved)) {                 // wave-uniform: most tiles after the first few leave every maximum where it was
+    if (__builtin_expect(__any(moved), 0)) {   // wave-uniform: most tiles after the first few leave every maximum where it was
       float a4[4];
 #pragma unroll
       for (int r = 0; r < 4; r++) a4[r] = __shfl(alpha, (int)(4u * g + r), 64);
@@ -541,8 +553,12 @@ size_t launch_attn_chunk(const std::vector<PendOp>& q, size_t i, int* rc) {
 #define APM(DD)                                                                                                   \
   do {                                                                                                            \
     k_v_tile_transpose<DD><<<dim3(tiles, n_grp), 256, 0, g.stream>>>(mp->kv16, mp->kv_start, src, seq_last, tiles, g_vt); \
-    k_attn_prefill_mfma<DD><<<n_quads * n_tt, 256, 0, g.stream>>>(d, d, mp->kv16, mp->kv_start, g_vt, bs, gv, H, n_quads, n_tt, m, \
-                                                                  s0.n, qs, os, a0.eps, a0.f2, tiles);           \
+    if (a0.f2 > 0.0f)                                                                                             \
+      k_attn_prefill_mfma<DD, true><<<n_quads * n_tt, 256, 0, g.stream>>>(d, d, mp->kv16, mp->kv_start, g_vt, bs, gv, H, n_quads, n_tt, \
+                                                                          m, s0.n, qs, os, a0.eps, a0.f2, tiles); \
+    else                                                                                                          \
+      k_attn_prefill_mfma<DD, false><<<n_quads * n_tt, 256, 0, g.stream>>>(d, d, mp->kv16, mp->kv_start, g_vt, bs, gv, H, n_quads, n_tt, \
+                                                                           m, s0.n, qs, os, a0.eps, a0.f2, tiles); \
   } while (0)
       if (D == 64) APM(64); else if (D == 128) APM(128); else APM(256);
 #undef APM
