@@ -241,15 +241,20 @@ k_attn_prefill(const float* data, float* out, const __half* kv, uint64_t kv_shif
 //   * a wave owns one query head and a tile of 16 consecutive tokens and walks the cache in tiles of 32 rows; the
 //     four waves of a workgroup are four heads of the same token tile -- with grouped queries, the heads of one KV
 //     head, so their K / V tiles come out of the L1 after the first wave has asked for them;
-//   * scores transposed, S^T = K . Q^T: A = K tile (row = cache row, 8 consecutive dims per lane: one 16-byte load
-//     of the row-major cache), B = the queries as exact hi + lo fp16 pairs after a power-of-two scale (held in
-//     registers for the whole walk).  The result leaves lane (query l % 16, g = l / 16) with cache rows 4g..4g+3 of
+//   * scores transposed, S^T = K . Q^T: A = K tile (row = cache row, 8 consecutive dims per lane: one 16-byte
+//     piece), B = the queries as exact hi + lo fp16 pairs after a power-of-two scale (held in registers for the
+//     whole walk).  Read from the row-major cache, the sixteen pieces of neighbouring lanes lie in sixteen
+//     different rows, and the L1 takes a load instruction's lanes four at a time only where they are neighbours in
+//     memory: 64 tag look-ups per instruction instead of 16, which made the K loads (eight of a tile's sixteen) four
+//     fifths of the CU's L1 time and the L1 the bound of the launch.  k_kv_tile_arrange therefore also writes the
+//     visible K rows once per launch in operand order, [KV head][tile][32-dim step][16-row half][lane], and a
+//     K load is 1 KB of consecutive memory like a V load;  The result leaves lane (query l % 16, g = l / 16) with cache rows 4g..4g+3 of
 //     both 16-row halves of the tile: all eight values of a lane belong to ONE query, so the softmax statistics
 //     are one (max, sum) pair per lane and the row maximum needs two cross-lane steps;
 //   * that is also the A-operand layout of P . V with the contraction index (g, j) standing for cache row
 //     4g + j (j < 4) or 16 + 4g + j - 4: P goes into the second product as it is (hi + lo fp16, so its products
 //     with the fp16 values are exact), no transposition;
-//   * the B operand of P . V needs eight cache ROWS per lane at one dim.  k_v_tile_transpose writes the visible
+//   * the B operand of P . V needs eight cache ROWS per lane at one dim.  k_kv_tile_arrange writes the visible
 //     part of the fp16 V cache once per launch into a scratch laid out [KV head][tile][16-dim block][g][dim][8 rows]
 //     so that this operand is one 16-byte load, too (rows past the end: zeros);
 //   * no LDS, no barrier: the accumulators (queries 4g..4g+3 x dim l % 16 per 16-dim block) are rescaled only in
@@ -259,12 +264,12 @@ k_attn_prefill(const float* data, float* out, const __half* kv, uint64_t kv_shif
 typedef _Float16 h8p_t __attribute__((ext_vector_type(8)));
 typedef float f4pu_t __attribute__((ext_vector_type(4), aligned(4)));
 struct AttpVt { uint32_t grp[ATTP_MAX_HEADS]; };   // head -> index of its KV head's part of the transposed scratch
-struct AttpVtSrc { uint32_t vb[ATTP_MAX_HEADS]; };  // group -> base of its V cache (element offset in the map)
+struct AttpVtSrc { uint32_t vb[ATTP_MAX_HEADS], kb[ATTP_MAX_HEADS]; };  // group -> bases of its V and K cache (element offsets in the map)
 
 template <int D>
 __global__ void __launch_bounds__(256)
-k_v_tile_transpose(const __half* kv, uint64_t kv_shift, const AttpVtSrc src, uint32_t nkeys, uint32_t tiles, uint4* vt) {
-  constexpr uint32_t NB = D / 16;
+k_kv_tile_arrange(const __half* kv, uint64_t kv_shift, const AttpVtSrc src, uint32_t nkeys, uint32_t tiles, uint4* vt, uint4* kt) {
+  constexpr uint32_t NB = D / 16, KS = D / 32;
   const uint32_t T = blockIdx.x, grp = blockIdx.y;
   const unsigned short* v = (const unsigned short*)(kv + ((uint64_t)src.vb[grp] - kv_shift));
   for (uint32_t idx = threadIdx.x; idx < NB * 64u; idx += 256u) {
@@ -278,13 +283,21 @@ k_v_tile_transpose(const __half* kv, uint64_t kv_shift, const AttpVtSrc src, uin
     }
     vt[((((uint64_t)grp * tiles + T) * NB + b) * 4u + g) * 16u + n] = make_uint4(w[0], w[1], w[2], w[3]);
   }
+  // K: piece (step st, half kb, lane (g, n)) = dims 32 st + 8 g .. + 7 of row 32 T + 16 kb + n (rows past the end: zeros)
+  const uint4* k = (const uint4*)(kv + ((uint64_t)src.kb[grp] - kv_shift));
+  for (uint32_t idx = threadIdx.x; idx < 2u * KS * 64u; idx += 256u) {
+    const uint32_t st = idx >> 7, kb = (idx >> 6) & 1u, g = (idx >> 4) & 3u, n = idx & 15u;
+    const uint32_t key = 32u * T + 16u * kb + n;
+    kt[((uint64_t)grp * tiles + T) * (2u * KS * 64u) + idx] =
+        key < nkeys ? k[(uint64_t)key * (D / 8) + 4u * st + g] : make_uint4(0u, 0u, 0u, 0u);
+  }
 }
 
 #define ATTP_MFMA32(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0)
 
 template <int D, bool CAP>
 __global__ void __launch_bounds__(256)
-k_attn_prefill_mfma(const float* data, float* out, const __half* kv, uint64_t kv_shift, const uint4* __restrict__ vt,
+k_attn_prefill_mfma(const float* data, float* out, const uint4* __restrict__ kt, const uint4* __restrict__ vt,
                     const AttpBases bs, const AttpVt gv, uint32_t H, uint32_t n_quads, uint32_t n_ttiles, uint32_t m,
                     uint32_t seq0, uint32_t q_stride, uint32_t o_stride, float scale, float cap, uint32_t vt_tiles) {
   constexpr int KS = D / 32;           // 32-dim steps of the score product
@@ -298,7 +311,7 @@ k_attn_prefill_mfma(const float* data, float* out, const __half* kv, uint64_t kv
   const uint32_t rows = min(16u, m - t0);
   const uint32_t nkeys = seq0 + t0 + rows - 1u;          // cache rows the tile's last query sees
   const uint32_t n_tiles = (nkeys + 31u) >> 5;
-  const char* kbase = (const char*)(kv + ((uint64_t)bs.kb[head] - kv_shift));
+  const uint4* kbase = kt + (uint64_t)gv.grp[head] * vt_tiles * (2u * KS * 64u) + lane;
   const uint4* vbase = vt + (uint64_t)gv.grp[head] * vt_tiles * (NB * 64u) + g * 16u + n;
 
   // this lane's query (n): dims 32 step + 8g .. + 7, scaled by a power of two into fp16 range, hi + lo
@@ -342,25 +355,32 @@ k_attn_prefill_mfma(const float* data, float* out, const __half* kv, uint64_t kv
   struct Tile { uint4 k[2][KS]; uint4 v[NB]; };
   auto fetch = [&](Tile& t, uint32_t T) {
 #pragma unroll
-    for (int kb = 0; kb < 2; kb++) {
-      const uint32_t key = min(32u * T + 16u * kb + n, nkeys - 1u);
+    for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-      for (int st = 0; st < KS; st++) t.k[kb][st] = *(const uint4*)(kbase + (uint64_t)key * (2u * D) + 64u * st + 16u * g);
-    }
+      for (int st = 0; st < KS; st++) t.k[kb][st] = kbase[((uint64_t)T * (2 * KS) + 2 * st + kb) * 64u];
 #pragma unroll
     for (int b = 0; b < NB; b++) t.v[b] = vbase[((uint64_t)T * NB + b) * 64u];
   };
-  auto compute = [&](const Tile& t, uint32_t T) {
+  // One tile's arithmetic, with the loads of tile Tn (into nx) spread between its matrix instructions, one 16-byte
+  // load per lane in front of every pair: a wave issues in order, and sixteen loads in a row ahead of the arithmetic
+  // keep it at its load instructions for as long as the CU's one address unit, shared by the four waves, takes to
+  // accept them (16 clocks each: ~1000 clocks per tile during which no wave of the CU multiplies).
+  auto compute = [&](const Tile& t, uint32_t T, Tile& nx, uint32_t Tn) {
     f4p_t s[2][2];
 #pragma unroll
     for (int kb = 0; kb < 2; kb++) { s[kb][0] = (f4p_t){0.f, 0.f, 0.f, 0.f}; s[kb][1] = s[kb][0]; }
+    const uint4* kn = kbase + (uint64_t)Tn * (2 * KS) * 64u;
+    const uint4* vn = vbase + (uint64_t)Tn * NB * 64u;
 #pragma unroll
     for (int st = 0; st < KS; st++)
 #pragma unroll
       for (int kb = 0; kb < 2; kb++) {
+        nx.k[kb][st] = kn[(2 * st + kb) * 64];
+        __builtin_amdgcn_sched_barrier(0);
         const h8p_t ka = __builtin_bit_cast(h8p_t, t.k[kb][st]);
         s[kb][0] = ATTP_MFMA32(ka, qh[st], s[kb][0]);
         s[kb][1] = ATTP_MFMA32(ka, ql[st], s[kb][1]);
+        __builtin_amdgcn_sched_barrier(0);
       }
     // The softmax runs on base-2 exponents: without a soft cap the scores' power-of-two scale, the softmax scale and
     // log2(e) are one factor (one rounding, as scale alone would take), a masked score is a large negative number
@@ -413,22 +433,21 @@ k_attn_prefill_mfma(const float* data, float* out, const __half* kv, uint64_t kv
     }
 #pragma unroll
     for (int b = 0; b < NB; b++) {
+      nx.v[b] = vn[b * 64];
+      __builtin_amdgcn_sched_barrier(0);
       const h8p_t vb = __builtin_bit_cast(h8p_t, t.v[b]);
       acc[b] = ATTP_MFMA32(ph, vb, acc[b]);
       acc[b] = ATTP_MFMA32(pl, vb, acc[b]);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
   Tile A, B;
   fetch(A, 0u);
   for (uint32_t T = 0; T < n_tiles; T += 2u) {
-    fetch(B, min(T + 1u, n_tiles - 1u));                 // (past the end: the last tile again, not used)
-    __builtin_amdgcn_sched_barrier(0);
-    compute(A, T);
+    compute(A, T, B, min(T + 1u, n_tiles - 1u));         // (past the end: the last tile again, not used)
     if (T + 1u >= n_tiles) break;
-    fetch(A, min(T + 2u, n_tiles - 1u));
-    __builtin_amdgcn_sched_barrier(0);
-    compute(B, T + 1u);
+    compute(B, T + 1u, A, min(T + 2u, n_tiles - 1u));
   }
 
   float l_tot = l_run + __shfl_xor(l_run, 16, 64);
@@ -532,12 +551,13 @@ size_t launch_attn_chunk(const std::vector<PendOp>& q, size_t i, int* rc) {
     uint32_t n_grp = 0;
     for (uint32_t h = 0; h < H; h++) {
       uint32_t gi = 0;
-      while (gi < n_grp && src.vb[gi] != vb[h]) gi++;
-      if (gi == n_grp) src.vb[n_grp++] = vb[h];
+      while (gi < n_grp && (src.vb[gi] != vb[h] || src.kb[gi] != kb[h])) gi++;
+      if (gi == n_grp) { src.vb[n_grp] = vb[h]; src.kb[n_grp++] = kb[h]; }
       gv.grp[h] = gi;
     }
     const uint32_t tiles = cdiv(seq_last, 32u);
-    const size_t need = (size_t)n_grp * tiles * 32u * D * sizeof(__half);
+    const size_t plane = (size_t)n_grp * tiles * 32u * D * sizeof(__half);   // V tiles, then K tiles
+    const size_t need = 2 * plane;
     bool ok = true;
     if (need > g_vt_bytes) {
       hipStreamSynchronize(g.stream);
@@ -550,14 +570,15 @@ size_t launch_attn_chunk(const std::vector<PendOp>& q, size_t i, int* rc) {
     }
     if (ok) {
       const uint32_t n_quads = cdiv(H, 4u), n_tt = cdiv(m, 16u);
+      uint4* const g_kt = (uint4*)((char*)g_vt + plane);
 #define APM(DD)                                                                                                   \
   do {                                                                                                            \
-    k_v_tile_transpose<DD><<<dim3(tiles, n_grp), 256, 0, g.stream>>>(mp->kv16, mp->kv_start, src, seq_last, tiles, g_vt); \
+    k_kv_tile_arrange<DD><<<dim3(tiles, n_grp), 256, 0, g.stream>>>(mp->kv16, mp->kv_start, src, seq_last, tiles, g_vt, g_kt); \
     if (a0.f2 > 0.0f)                                                                                             \
-      k_attn_prefill_mfma<DD, true><<<n_quads * n_tt, 256, 0, g.stream>>>(d, d, mp->kv16, mp->kv_start, g_vt, bs, gv, H, n_quads, n_tt, \
+      k_attn_prefill_mfma<DD, true><<<n_quads * n_tt, 256, 0, g.stream>>>(d, d, g_kt, g_vt, bs, gv, H, n_quads, n_tt, \
                                                                           m, s0.n, qs, os, a0.eps, a0.f2, tiles); \
     else                                                                                                          \
-      k_attn_prefill_mfma<DD, false><<<n_quads * n_tt, 256, 0, g.stream>>>(d, d, mp->kv16, mp->kv_start, g_vt, bs, gv, H, n_quads, n_tt, \
+      k_attn_prefill_mfma<DD, false><<<n_quads * n_tt, 256, 0, g.stream>>>(d, d, g_kt, g_vt, bs, gv, H, n_quads, n_tt, \
                                                                            m, s0.n, qs, os, a0.eps, a0.f2, tiles); \
   } while (0)
       if (D == 64) APM(64); else if (D == 128) APM(128); else APM(256);
