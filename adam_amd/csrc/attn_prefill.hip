@@ -295,8 +295,8 @@ k_kv_tile_arrange(const __half* kv, uint64_t kv_shift, const AttpVtSrc src, uint
 
 #define ATTP_MFMA32(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0)
 
-template <int D, bool CAP>
-__global__ void __launch_bounds__(256)
+template <int D, bool CAP, int WPH>
+__global__ void __launch_bounds__(256 * WPH)
 k_attn_prefill_mfma(const float* data, float* out, const uint4* __restrict__ kt, const uint4* __restrict__ vt,
                     const AttpBases bs, const AttpVt gv, uint32_t H, uint32_t n_quads, uint32_t n_ttiles, uint32_t m,
                     uint32_t seq0, uint32_t q_stride, uint32_t o_stride, float scale, float cap, uint32_t vt_tiles) {
@@ -305,12 +305,20 @@ k_attn_prefill_mfma(const float* data, float* out, const uint4* __restrict__ kt,
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const uint32_t n = lane & 15u, g = lane >> 4;
-  const uint32_t head = (blockIdx.x % n_quads) * 4u + wave;
+  // WPH = 2 (a launch that gives every CU one workgroup at most): two waves per head, the second four waves of the
+  // workgroup walk the second half of the key tiles and hand their running state over in LDS at the end -- two waves
+  // per SIMD, so that one's loads are served while the other one multiplies.
+  const uint32_t half = WPH == 2 ? wave >> 2 : 0u;
+  const uint32_t head_raw = (blockIdx.x % n_quads) * 4u + (wave & 3u);
+  const bool live = head_raw < H;
+  if (WPH == 1 && !live) return;       // (no barrier in the one-wave form)
+  const uint32_t head = min(head_raw, H - 1u);
   const uint32_t t0 = (n_ttiles - 1u - blockIdx.x / n_quads) * 16u;
-  if (head >= H) return;               // (no barrier in this kernel)
   const uint32_t rows = min(16u, m - t0);
   const uint32_t nkeys = seq0 + t0 + rows - 1u;          // cache rows the tile's last query sees
   const uint32_t n_tiles = (nkeys + 31u) >> 5;
+  const uint32_t t_split = WPH == 2 ? (n_tiles + 1u) >> 1 : n_tiles;
+  const uint32_t T_lo = !live ? 0u : half ? t_split : 0u, T_hi = !live ? 0u : half ? n_tiles : t_split;
   const uint4* kbase = kt + (uint64_t)gv.grp[head] * vt_tiles * (2u * KS * 64u) + lane;
   const uint4* vbase = vt + (uint64_t)gv.grp[head] * vt_tiles * (NB * 64u) + g * 16u + n;
 
@@ -344,7 +352,7 @@ k_attn_prefill_mfma(const float* data, float* out, const uint4* __restrict__ kt,
   }
   const uint32_t lim = n < rows ? seq0 + t0 + n : 0u;     // cache rows this lane's query sees
   const float c2 = inv_s * scale * 1.44269504f;          // (inv_s is a power of two)
-  const bool last = n < rows && t0 + n == m - 1u;
+  const bool last = live && n < rows && t0 + n == m - 1u;
   const uint64_t sc_row = bs.sc[head];
 
   f4p_t acc[NB];
@@ -443,11 +451,38 @@ k_attn_prefill_mfma(const float* data, float* out, const uint4* __restrict__ kt,
   };
 
   Tile A, B;
-  fetch(A, 0u);
-  for (uint32_t T = 0; T < n_tiles; T += 2u) {
-    compute(A, T, B, min(T + 1u, n_tiles - 1u));         // (past the end: the last tile again, not used)
-    if (T + 1u >= n_tiles) break;
-    compute(B, T + 1u, A, min(T + 2u, n_tiles - 1u));
+  if (T_lo < T_hi) fetch(A, T_lo);
+  for (uint32_t T = T_lo; T < T_hi; T += 2u) {
+    compute(A, T, B, min(T + 1u, T_hi - 1u));            // (past the end: the last tile again, not used)
+    if (T + 1u >= T_hi) break;
+    compute(B, T + 1u, A, min(T + 2u, T_hi - 1u));
+  }
+
+  if (WPH == 2) {
+    // the second wave of a head hands (maximum, sum, accumulators) to the first, which merges: both rescaled to the
+    // common maximum (a wave without tiles hands over maximum -1e30, sum 0: factor exactly 0)
+    __shared__ float xch[4 * (2 + 4 * NB) * 64];
+    float* mine = xch + (wave & 3u) * ((2 + 4 * NB) * 64) + lane;
+    if (half) {
+      mine[0] = m_run; mine[64] = l_run;
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) mine[(2 + 4 * b + r) * 64] = acc[b][r];
+    }
+    __syncthreads();
+    if (half || !live) return;
+    const float m1 = mine[0], l1 = mine[64];
+    const float mm = fmaxf(m_run, m1);
+    const float f0 = __builtin_amdgcn_exp2f(m_run - mm), f1 = __builtin_amdgcn_exp2f(m1 - mm);
+    l_run = l_run * f0 + l1 * f1;
+    float g0[4], g1[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) { g0[r] = __shfl(f0, (int)(4u * g + r), 64); g1[r] = __shfl(f1, (int)(4u * g + r), 64); }
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) acc[b][r] = acc[b][r] * g0[r] + mine[(2 + 4 * b + r) * 64] * g1[r];
   }
 
   float l_tot = l_run + __shfl_xor(l_run, 16, 64);
@@ -571,18 +606,26 @@ size_t launch_attn_chunk(const std::vector<PendOp>& q, size_t i, int* rc) {
     if (ok) {
       const uint32_t n_quads = cdiv(H, 4u), n_tt = cdiv(m, 16u);
       uint4* const g_kt = (uint4*)((char*)g_vt + plane);
+      // two waves per head where the launch has at most one workgroup per CU (ADAMAH_ATTN_PREFILL_WPH: 1 / 2 force)
+      const int wph_mode = tuning("ADAMAH_ATTN_PREFILL_WPH", 0);
+      const int wph = wph_mode == 1 || wph_mode == 2 ? wph_mode : (n_quads * n_tt <= (uint32_t)g.n_cu ? 2 : 1);
+#define APM_ARGS d, d, g_kt, g_vt, bs, gv, H, n_quads, n_tt, m, s0.n, qs, os, a0.eps, a0.f2, tiles
 #define APM(DD)                                                                                                   \
   do {                                                                                                            \
     k_kv_tile_arrange<DD><<<dim3(tiles, n_grp), 256, 0, g.stream>>>(mp->kv16, mp->kv_start, src, seq_last, tiles, g_vt, g_kt); \
-    if (a0.f2 > 0.0f)                                                                                             \
-      k_attn_prefill_mfma<DD, true><<<n_quads * n_tt, 256, 0, g.stream>>>(d, d, g_kt, g_vt, bs, gv, H, n_quads, n_tt, \
-                                                                          m, s0.n, qs, os, a0.eps, a0.f2, tiles); \
-    else                                                                                                          \
-      k_attn_prefill_mfma<DD, false><<<n_quads * n_tt, 256, 0, g.stream>>>(d, d, g_kt, g_vt, bs, gv, H, n_quads, n_tt, \
-                                                                           m, s0.n, qs, os, a0.eps, a0.f2, tiles); \
+    const dim3 gr_(n_quads * n_tt);                                                                               \
+    if (wph == 2 && DD <= 128) {   /* (D = 256 needs more registers than two waves per SIMD have) */              \
+      constexpr int D2_ = DD <= 128 ? DD : 128;                                                                   \
+      if (a0.f2 > 0.0f) k_attn_prefill_mfma<D2_, true, 2><<<gr_, 512, 0, g.stream>>>(APM_ARGS);                  \
+      else k_attn_prefill_mfma<D2_, false, 2><<<gr_, 512, 0, g.stream>>>(APM_ARGS);                              \
+    } else {                                                                                                      \
+      if (a0.f2 > 0.0f) k_attn_prefill_mfma<DD, true, 1><<<gr_, 256, 0, g.stream>>>(APM_ARGS);                   \
+      else k_attn_prefill_mfma<DD, false, 1><<<gr_, 256, 0, g.stream>>>(APM_ARGS);                               \
+    }                                                                                                             \
   } while (0)
       if (D == 64) APM(64); else if (D == 128) APM(128); else APM(256);
 #undef APM
+#undef APM_ARGS
       count_launch(2);
       *rc = check_launch();
       return 2 * (size_t)m;

@@ -109,10 +109,15 @@ def test_gqa_heads_with_equal_queries_agree(hip):
 CHUNK_LAUNCHES = {"0": 1, "2": 2}
 
 
-@pytest.fixture(params=["0", "2"], ids=["vector-pv", "matrix-pv"])
+@pytest.fixture(params=["0", "2/1", "2/2"], ids=["vector-pv", "matrix-pv", "matrix-pv-two-waves-per-head"])
 def chunk_impl(request, monkeypatch):
-    monkeypatch.setenv("ADAMAH_ATTN_PREFILL_MFMA", request.param)
-    return request.param
+    """The chunk's attention on vector multiply-adds, on the matrix cores with one wave per head, and with two waves
+    per head sharing the key tiles (by itself the form of launches with at most one workgroup per CU)."""
+    impl, _, wph = request.param.partition("/")
+    monkeypatch.setenv("ADAMAH_ATTN_PREFILL_MFMA", impl)
+    if wph:
+        monkeypatch.setenv("ADAMAH_ATTN_PREFILL_WPH", wph)
+    return impl
 
 
 def chunk_case(g, q, K, V, seq0, cap_len, scale, softcap, gap=0, one_call=False):

@@ -23,7 +23,7 @@ pytestmark = pytest.mark.gpu
 SWITCHES = [("ADAMAH_NO_FUSE", "1"), ("ADAMAH_PLAN_GRAPH", "0"), ("ADAMAH_GEMV_IMPL", "0"), ("ADAMAH_GEMV_IMPL", "1"), ("ADAMAH_GEMV_IMPL", "3"),
             ("ADAMAH_GLU_SPLIT", "0"), ("ADAMAH_GLU_SPLIT", "2"), ("ADAMAH_GEMM_IMPL", "0"), ("ADAMAH_GEMM_MERGE", "0"), ("ADAMAH_GEMM_SPLITK", "0"), ("ADAMAH_GEMM_EPI", "0"), ("ADAMAH_GEMM_REUSE", "0"), ("ADAMAH_GLU_EMIT", "0"), ("ADAMAH_GEMM_ROWS16", "0"),
             ("ADAMAH_RMSNORM_EMIT", "0"), ("ADAMAH_RMSNORM_ROWS", "0"), ("ADAMAH_ARGMAX_RUN", "0"),
-            ("ADAMAH_ATTN_CHUNK", "0"), ("ADAMAH_ATTN_PREFILL_MFMA", "0"), ("ADAMAH_ATTN_PREFILL_MFMA", "2"), ("ADAMAH_ATTN_HEADSPLIT", "0"), ("ADAMAH_ATTN_HEADSPLIT", "2"), ("ADAMAH_ATTN_BATCH", "0"), ("ADAMAH_ATTN_MERGE_EMIT", "0"), ("ADAMAH_ATTN_IMPL", "0"), ("ADAMAH_ATTN_ROWPREP", "0"), ("ADAMAH_ROWS_WIDE", "0"), ("ADAMAH_NORM2_PARK", "0"), ("ADAMAH_TOPK_RANK", "0"),
+            ("ADAMAH_ATTN_CHUNK", "0"), ("ADAMAH_ATTN_PREFILL_MFMA", "0"), ("ADAMAH_ATTN_PREFILL_MFMA", "2"), ("ADAMAH_ATTN_PREFILL_WPH", "1"), ("ADAMAH_ATTN_PREFILL_WPH", "2"), ("ADAMAH_ATTN_HEADSPLIT", "0"), ("ADAMAH_ATTN_HEADSPLIT", "2"), ("ADAMAH_ATTN_BATCH", "0"), ("ADAMAH_ATTN_MERGE_EMIT", "0"), ("ADAMAH_ATTN_IMPL", "0"), ("ADAMAH_ATTN_ROWPREP", "0"), ("ADAMAH_ROWS_WIDE", "0"), ("ADAMAH_NORM2_PARK", "0"), ("ADAMAH_TOPK_RANK", "0"),
             ("ADAMAH_TOPK_RANK", "1"), ("ADAMAH_TOPK_SELECT", "0"), ("ADAMAH_TOPK_BLOCK", "0")]
 
 _REF = {}
