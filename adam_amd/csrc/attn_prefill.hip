@@ -257,8 +257,8 @@ k_attn_prefill(const float* data, float* out, const __half* kv, uint64_t kv_shif
 //   * the B operand of P . V needs eight cache ROWS per lane at one dim.  k_kv_tile_arrange writes the visible
 //     part of the fp16 V cache once per launch into a scratch laid out [KV head][tile][16-dim block][g][dim][8 rows]
 //     so that this operand is one 16-byte load, too (rows past the end: zeros);
-//   * no LDS, no barrier: the accumulators (queries 4g..4g+3 x dim l % 16 per 16-dim block) are rescaled only in
-//     tiles where some query's maximum moved, the factors fetched across lanes.
+//   * no LDS and no barrier in the walk: the accumulators (queries 4g..4g+3 x dim l % 16 per 16-dim block) are
+//     rescaled only in tiles where some query's maximum moved, the factors fetched across lanes.
 // Workgroup b serves head quad b % (H / 4): with eight KV heads, XCD x (workgroups x, x + 8, ...) walks the cache of
 // KV head x only, which fits its L2; the token tiles with the longest walks come first.
 typedef _Float16 h8p_t __attribute__((ext_vector_type(8)));

@@ -105,7 +105,7 @@ def test_gqa_heads_with_equal_queries_agree(hip):
 
 
 # a chunk's attention: one causal kernel -- or, on the matrix-core form (taken by itself for chunks that fill the chip:
-# ADAMAH_ATTN_PREFILL_MFMA=1, the default; forced with 2, off with 0), the V tiles' transposing pass and then the kernel
+# ADAMAH_ATTN_PREFILL_MFMA=1, the default; forced with 2, off with 0), the pass that arranges the K / V tiles and then the kernel
 CHUNK_LAUNCHES = {"0": 1, "2": 2}
 
 
